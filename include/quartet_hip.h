@@ -1,0 +1,103 @@
+/*
+ * quartet_hip.h -- C ABI of libquartet_hip.so: the MI355X (gfx950) kernels behind Quartet's
+ * MXFP4 quantized-linear path.
+ *
+ * Conventions
+ *   - every tensor pointer is a DEVICE pointer owned by the caller; outputs are pre-allocated;
+ *   - `stream` is a hipStream_t (NULL = default stream); calls are asynchronous on it;
+ *   - return value: 0 = ok, < 0 = rejected arguments (nothing was launched; qm_last_error()
+ *     holds the reason, thread-local), > 0 = a hipError_t from the launch;
+ *   - packed MXFP4 tensor of logical shape [R, C] (C % 32 == 0):
+ *       codes  uint8 [R, C/2]   E2M1, element 2i in the low nibble of byte i, sign in bit 3
+ *       scales uint8 [R, C/32]  E8M0 (value 2^(byte-127)), one per 32 consecutive elements
+ *       mask   uint8 [R, C/8]   bit i of byte j = clip mask of element 8j+i
+ *   - `sign_bits`: HOST pointer to ceil(hd/32) uint32 words, bit j set = rotated column j is
+ *     negated (the accumulated +-1 diagonal of re_randomize), or NULL for no sign flips.
+ *
+ * The reference has no FFI; each entry point below names the Python/Triton call it replaces
+ * (paths relative to the reference checkout).
+ */
+#ifndef QUARTET_HIP_H
+#define QUARTET_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { QM_BF16 = 0, QM_F32 = 1 };
+/* scale rule + rounding: quest = std-based scale (QuestMXFP4Quantizer), absmax = max/(3/4)
+ * (AlbertTsengQuantizer); RTN = ties toward zero, SR = stochastic rounding */
+enum { QM_QUEST_RTN = 0, QM_ABSMAX_RTN = 1, QM_ABSMAX_SR = 2, QM_QUEST_SR = 3 };
+
+#define QM_ERR_INVALID (-1)
+#define QM_ERR_UNALIGNED (-2)
+
+int qm_version(void);
+/* message of the last failed call on this thread ("" if none) */
+const char* qm_last_error(void);
+
+/*
+ * Fused block-Hadamard rotation + MXFP4 quantization of a logical [rows, cols] tensor along cols.
+ * Replaces mxfp4_forward_kernel_wrapper (src/models/quantization/quantizers/mxfp4_triton.py:177-220)
+ * as called by QuestMXFP4QuantizerFn.forward (quantizers/mxfp4.py:129-140, mode QM_QUEST_RTN with
+ * maskbits) and AlbertTsengQuantizerFn.forward (quantizers/mxfp4.py:17-28, QM_ABSMAX_RTN/SR).
+ *   x            input, dtype x_dtype; row-major [rows, cols], or, when transposed_in != 0,
+ *                row-major [cols, rows] (the kernel quantizes its transpose: this is
+ *                `e.T.contiguous()` + quantize of backward.py:81 in one pass)
+ *   hadamard_dim 32, 64 or 128; cols % hadamard_dim == 0
+ *   u            SR modes: device floats in [0,1) indexed by logical flat offset, or NULL to draw
+ *                them in-kernel from Philox4x32-10 keyed by (seed, offset)
+ *   codes/scales outputs (required); maskbits, dequant optional (NULL to skip); dequant has
+ *                x_dtype and logical shape and holds what the reference kernel returns
+ */
+int qm_quantize_mxfp4(const void* x, int x_dtype, int64_t rows, int64_t cols, int hadamard_dim,
+                      const uint32_t* sign_bits, int mode, int transposed_in, const float* u,
+                      uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits,
+                      void* dequant, void* stream);
+
+/*
+ * De-quantize a packed [R, C] tensor, transpose it, rotate and re-quantize along R:
+ * outputs codes_out [C, R/2], scales_out [C, R/32].  Replaces
+ * `g_quantizer(wq.T.contiguous())` / `g_quantizer(xq.T.contiguous())`
+ * (src/models/quantization/backward.py:73,82) on the saved quantized operand, and the role of
+ * backward_qt_bf16 in notebooks/benchmark_mxfp4.ipynb.
+ *   post       1.0 if the input was quest-coded, fl32(4/3) if absmax-coded
+ *   val_dtype  dtype the reference would hold the de-quantized tensor in (selects the rounding
+ *              of the Hadamard constant and of the de-quantized values)
+ */
+int qm_requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R,
+                                   int64_t C, float post, int val_dtype, int hadamard_dim,
+                                   const uint32_t* sign_bits, int mode, const float* u,
+                                   uint64_t seed, uint8_t* codes_out, uint8_t* scales_out,
+                                   void* dequant, void* stream);
+
+/*
+ * C[M, N] = alpha * A[M, K] . B[N, K]^T on packed MXFP4 operands, fp32 accumulation.
+ * Replaces F.linear / einsum on de-quantized operands (src/models/quantization/backward.py:62,
+ * 71-75, 79-83) and matmul_mxf4_bf16_tn of notebooks/benchmark_mxfp4.ipynb.  K % 32 == 0.
+ * alpha carries the per-operand constants of absmax coding (fl32(4/3) each).
+ */
+int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                     const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c,
+                     int c_dtype, void* stream);
+
+/*
+ * out = ((g * mask).view(-1, hd)) @ H^T: the straight-through backward of the forward quantizer,
+ * QuestMXFP4QuantizerFn.backward (src/models/quantization/quantizers/mxfp4.py:143-146); with
+ * maskbits == NULL it is AlbertTsengQuantizerFn.backward (mxfp4.py:31-34).
+ *   scale_dtype  dtype whose rounding of hd^-1/2 the matrix H carries
+ */
+int qm_masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t cols,
+                           int hadamard_dim, int scale_dtype, const uint32_t* sign_bits,
+                           const uint8_t* maskbits, void* out, int out_dtype, void* stream);
+
+/* out[r, c] = e2m1(code) * post * 2^(scale-127); the tensor the reference's pseudo-quantizer returns */
+int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, int64_t C,
+                        float post, void* out, int out_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QUARTET_HIP_H */

@@ -1,0 +1,62 @@
+"""ctypes binding of libquartet_hip.so (the C ABI declared in include/quartet_hip.h).
+
+There is no fallback: if the shared library is missing the import of this module's ``lib()``
+raises, so no caller can silently run without the HIP kernels."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libquartet_hip.so")
+
+QM_BF16, QM_F32 = 0, 1
+QM_QUEST_RTN, QM_ABSMAX_RTN, QM_ABSMAX_SR, QM_QUEST_SR = 0, 1, 2, 3
+
+EXPORTS = (
+    "qm_version",
+    "qm_last_error",
+    "qm_quantize_mxfp4",
+    "qm_requantize_transposed_mxfp4",
+    "qm_gemm_mxfp4_tn",
+    "qm_masked_hadamard_bwd",
+    "qm_dequantize_mxfp4",
+)
+
+_lib = None
+
+
+class QuartetHipError(RuntimeError):
+    pass
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise QuartetHipError(
+            f"{LIB_PATH} is missing: build it with `make -C quartet_amd/csrc` (or __graft_entry__.build()); "
+            "there is no CPU fallback for the quantized-linear path")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, i32, i64, u64, f32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_uint64, ctypes.c_float
+    L.qm_version.restype = i32
+    L.qm_version.argtypes = []
+    L.qm_last_error.restype = ctypes.c_char_p
+    L.qm_last_error.argtypes = []
+    L.qm_quantize_mxfp4.restype = i32
+    L.qm_quantize_mxfp4.argtypes = [vp, i32, i64, i64, i32, vp, i32, i32, vp, u64, vp, vp, vp, vp, vp]
+    L.qm_requantize_transposed_mxfp4.restype = i32
+    L.qm_requantize_transposed_mxfp4.argtypes = [vp, vp, i64, i64, f32, i32, i32, vp, i32, vp, u64, vp, vp, vp, vp]
+    L.qm_gemm_mxfp4_tn.restype = i32
+    L.qm_gemm_mxfp4_tn.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, vp]
+    L.qm_masked_hadamard_bwd.restype = i32
+    L.qm_masked_hadamard_bwd.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp, i32, vp]
+    L.qm_dequantize_mxfp4.restype = i32
+    L.qm_dequantize_mxfp4.argtypes = [vp, vp, i64, i64, f32, vp, i32, vp]
+    _lib = L
+    return L
+
+
+def check(rc, what):
+    if rc != 0:
+        msg = lib().qm_last_error().decode("utf-8", "replace")
+        raise QuartetHipError(f"{what} failed (rc={rc}): {msg}")

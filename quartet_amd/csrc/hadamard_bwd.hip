@@ -1,0 +1,164 @@
+// Straight-through backward of the forward quantizer (K3) and the MXFP4 de-quantizer.
+//
+// masked_hadamard_bwd replaces src/models/quantization/quantizers/mxfp4.py:143-146
+//     grad_in = ((grad_out * mask).view(-1, hd)) @ H^T,   H = c * S * diag(signs)
+// with the mask read as packed bits (bit i of byte j <-> element 8j+i).  Signs are applied to the
+// input column, then the ascending-stride butterfly, then c: the same canonical order the forward
+// rotation uses.  HBM traffic per element (bf16): 2 B in + 1/8 B mask + 2 B out.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "qm_kernels.h"
+#include "qm_math.h"
+
+namespace qm {
+
+namespace {
+
+__device__ __forceinline__ float dpp_quad_xor1(float v) {
+    return u2f((uint32_t)__builtin_amdgcn_mov_dpp((int)f2u(v), 0xB1, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_quad_xor2(float v) {
+    return u2f((uint32_t)__builtin_amdgcn_mov_dpp((int)f2u(v), 0x4E, 0xF, 0xF, true));
+}
+template <int LANE_MASK>
+__device__ __forceinline__ float lane_xor(float v) {
+    if constexpr (LANE_MASK == 1) return dpp_quad_xor1(v);
+    else if constexpr (LANE_MASK == 2) return dpp_quad_xor2(v);
+    else return __shfl_xor(v, LANE_MASK, 64);
+}
+template <int LANE_MASK>
+__device__ __forceinline__ void cross_lane_stage(float (&v)[8], int lane_in_chunk) {
+    const bool upper = (lane_in_chunk & LANE_MASK) != 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float p = lane_xor<LANE_MASK>(v[i]);
+        v[i] = upper ? (p - v[i]) : (v[i] + p);
+    }
+}
+
+template <typename TIn, typename TOut, int HD>
+__global__ __launch_bounds__(256) void masked_hadamard_bwd_kernel(const TIn* __restrict__ g, int64_t n_octets,
+                                                                  float c, SignBits sb,
+                                                                  const uint8_t* __restrict__ maskbits,
+                                                                  TOut* __restrict__ out) {
+    const int64_t octet = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (octet >= n_octets) return;
+    const int lic = (int)(octet & (HD / 8 - 1));
+    float v[8];
+    if constexpr (sizeof(TIn) == 2) {
+        uint4 raw = *reinterpret_cast<const uint4*>(g + octet * 8);
+        uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = u2f(w[i] << 16);
+            v[2 * i + 1] = u2f(w[i] & 0xffff0000u);
+        }
+    } else {
+        float4 a = *reinterpret_cast<const float4*>(g + octet * 8);
+        float4 b = *reinterpret_cast<const float4*>(g + octet * 8 + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+    const uint32_t keep = maskbits ? (uint32_t)maskbits[octet] : 0xffu;
+    const int j0 = lic * 8;
+    const uint32_t sign8 = (sb.w[j0 >> 5] >> (j0 & 31)) & 0xffu;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float x = v[i] * (float)((keep >> i) & 1u);  // g * mask, as the reference multiplies
+        v[i] = ((sign8 >> i) & 1u) ? -x : x;
+    }
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (i & h) continue;
+            float a = v[i], b = v[i + h];
+            v[i] = a + b;
+            v[i + h] = a - b;
+        }
+    }
+    cross_lane_stage<1>(v, lic);
+    cross_lane_stage<2>(v, lic);
+    if constexpr (HD >= 64) cross_lane_stage<4>(v, lic);
+    if constexpr (HD >= 128) cross_lane_stage<8>(v, lic);
+    if constexpr (sizeof(TOut) == 2) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            w[i] = (uint32_t)f32_to_bf16(v[2 * i] * c) | ((uint32_t)f32_to_bf16(v[2 * i + 1] * c) << 16);
+        *reinterpret_cast<uint4*>(out + octet * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+        *reinterpret_cast<float4*>(out + octet * 8) = make_float4(v[0] * c, v[1] * c, v[2] * c, v[3] * c);
+        *reinterpret_cast<float4*>(out + octet * 8 + 4) = make_float4(v[4] * c, v[5] * c, v[6] * c, v[7] * c);
+    }
+}
+
+template <typename TOut>
+__global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t* __restrict__ codes,
+                                                         const uint8_t* __restrict__ scales, int64_t n_octets,
+                                                         float post, TOut* __restrict__ out) {
+    const int64_t octet = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (octet >= n_octets) return;
+    const uint32_t w = codes[octet];
+    const float scale = scale_pow2(post, (int)scales[octet >> 2] - 127);
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        uint32_t nib = (w >> (4 * i)) & 15u;
+        float q = e2m1_value((int)(nib & 7u));
+        v[i] = ((nib & 8u) ? -q : q) * scale;
+    }
+    if constexpr (sizeof(TOut) == 2) {
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = (uint32_t)f32_to_bf16(v[2 * i]) | ((uint32_t)f32_to_bf16(v[2 * i + 1]) << 16);
+        *reinterpret_cast<uint4*>(out + octet * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+    } else {
+        *reinterpret_cast<float4*>(out + octet * 8) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4*>(out + octet * 8 + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+}
+
+template <typename TIn, typename TOut>
+void launch_bwd(int hd, const void* g, int64_t n, float c, const SignBits& sb, const uint8_t* maskbits, void* out,
+                hipStream_t stream) {
+    const int64_t n_octets = n / 8;
+    dim3 grid((unsigned)((n_octets + 255) / 256)), block(256);
+    const TIn* gp = reinterpret_cast<const TIn*>(g);
+    TOut* op = reinterpret_cast<TOut*>(out);
+    if (hd == 32) masked_hadamard_bwd_kernel<TIn, TOut, 32><<<grid, block, 0, stream>>>(gp, n_octets, c, sb, maskbits, op);
+    else if (hd == 64) masked_hadamard_bwd_kernel<TIn, TOut, 64><<<grid, block, 0, stream>>>(gp, n_octets, c, sb, maskbits, op);
+    else masked_hadamard_bwd_kernel<TIn, TOut, 128><<<grid, block, 0, stream>>>(gp, n_octets, c, sb, maskbits, op);
+}
+
+}  // namespace
+
+hipError_t masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t cols, int hd, int scale_dtype,
+                               const SignBits& sb, const uint8_t* maskbits, void* out, int out_dtype,
+                               hipStream_t stream) {
+    if (rows == 0 || cols == 0) return hipSuccess;
+    const float c = hadamard_scale(hd, scale_dtype);
+    const int64_t n = rows * cols;
+    if (g_dtype == BF16 && out_dtype == BF16) launch_bwd<uint16_t, uint16_t>(hd, g, n, c, sb, maskbits, out, stream);
+    else if (g_dtype == BF16) launch_bwd<uint16_t, float>(hd, g, n, c, sb, maskbits, out, stream);
+    else if (out_dtype == BF16) launch_bwd<float, uint16_t>(hd, g, n, c, sb, maskbits, out, stream);
+    else launch_bwd<float, float>(hd, g, n, c, sb, maskbits, out, stream);
+    return hipGetLastError();
+}
+
+hipError_t dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, int64_t C, float post, void* out,
+                            int out_dtype, hipStream_t stream) {
+    if (R == 0 || C == 0) return hipSuccess;
+    const int64_t n_octets = R * C / 8;
+    dim3 grid((unsigned)((n_octets + 255) / 256)), block(256);
+    if (out_dtype == BF16)
+        dequantize_kernel<uint16_t><<<grid, block, 0, stream>>>(reinterpret_cast<const uint32_t*>(codes), scales, n_octets, post, reinterpret_cast<uint16_t*>(out));
+    else
+        dequantize_kernel<float><<<grid, block, 0, stream>>>(reinterpret_cast<const uint32_t*>(codes), scales, n_octets, post, reinterpret_cast<float*>(out));
+    return hipGetLastError();
+}
+
+}  // namespace qm

@@ -1,0 +1,118 @@
+"""Tensor-level wrappers over the C ABI: allocate outputs with torch, pass raw device pointers and
+the current HIP stream.  PyTorch is only the allocator and stream provider here."""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import QM_ABSMAX_RTN, QM_ABSMAX_SR, QM_BF16, QM_F32, QM_QUEST_RTN, QM_QUEST_SR  # noqa: F401
+
+FOUR_THIRDS = float(torch.tensor(1.0 / 0.75, dtype=torch.float32))
+
+
+def _dtype_code(dt):
+    if dt == torch.bfloat16:
+        return QM_BF16
+    if dt == torch.float32:
+        return QM_F32
+    raise TypeError(f"quartet_amd kernels take bfloat16 or float32 tensors, got {dt}")
+
+
+def _torch_dtype(code):
+    return torch.bfloat16 if code == QM_BF16 else torch.float32
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise _lib.QuartetHipError("quartet_amd kernels need tensors on the GPU (no CPU path exists)")
+
+
+def sign_words(sign_bits):
+    """sign_bits: python int bit mask (bit j = column j negated) or None -> ctypes uint32[4] or None."""
+    if sign_bits is None or sign_bits == 0:
+        return None
+    return (ctypes.c_uint32 * 4)(*[(sign_bits >> (32 * i)) & 0xFFFFFFFF for i in range(4)])
+
+
+def quantize_mxfp4(x, hadamard_dim=32, sign_bits=None, mode=QM_QUEST_RTN, transposed_in=False, u=None, seed=0,
+                   want_mask=False, want_dequant=False):
+    """x: 2-D contiguous tensor.  Returns (codes [R,C/2] u8, scales [R,C/32] u8, maskbits [R,C/8] u8 | None,
+    dequant [R,C] like x | None) for the logical [R,C] tensor (x, or x.T when transposed_in)."""
+    _require_cuda(x, u)
+    assert x.dim() == 2 and x.is_contiguous()
+    rows, cols = (x.shape[1], x.shape[0]) if transposed_in else x.shape
+    dev = x.device
+    codes = torch.empty((rows, cols // 2), dtype=torch.uint8, device=dev)
+    scales = torch.empty((rows, cols // 32), dtype=torch.uint8, device=dev)
+    mask = torch.empty((rows, cols // 8), dtype=torch.uint8, device=dev) if want_mask else None
+    deq = torch.empty((rows, cols), dtype=x.dtype, device=dev) if want_dequant else None
+    if u is not None:
+        assert u.dtype == torch.float32 and u.is_contiguous() and u.numel() == rows * cols
+    rc = _lib.lib().qm_quantize_mxfp4(_ptr(x), _dtype_code(x.dtype), rows, cols, hadamard_dim, sign_words(sign_bits),
+                                      mode, int(transposed_in), _ptr(u), seed, _ptr(codes), _ptr(scales), _ptr(mask),
+                                      _ptr(deq), _stream())
+    _lib.check(rc, "qm_quantize_mxfp4")
+    return codes, scales, mask, deq
+
+
+def requantize_transposed_mxfp4(codes, scales, post=1.0, val_dtype=torch.bfloat16, hadamard_dim=32, sign_bits=None,
+                                mode=QM_ABSMAX_SR, u=None, seed=0, want_dequant=False):
+    """codes [R,C/2], scales [R,C/32] -> (codes [C,R/2], scales [C,R/32], dequant [C,R] | None)."""
+    _require_cuda(codes, scales, u)
+    assert codes.is_contiguous() and scales.is_contiguous()
+    R, C = codes.shape[0], codes.shape[1] * 2
+    dev = codes.device
+    codes_out = torch.empty((C, R // 2), dtype=torch.uint8, device=dev)
+    scales_out = torch.empty((C, R // 32), dtype=torch.uint8, device=dev)
+    deq = torch.empty((C, R), dtype=val_dtype, device=dev) if want_dequant else None
+    rc = _lib.lib().qm_requantize_transposed_mxfp4(_ptr(codes), _ptr(scales), R, C, post, _dtype_code(val_dtype),
+                                                   hadamard_dim, sign_words(sign_bits), mode, _ptr(u), seed,
+                                                   _ptr(codes_out), _ptr(scales_out), _ptr(deq), _stream())
+    _lib.check(rc, "qm_requantize_transposed_mxfp4")
+    return codes_out, scales_out, deq
+
+
+def gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, alpha=1.0, out_dtype=torch.bfloat16):
+    """[M,K/2],[M,K/32] x [N,K/2],[N,K/32] -> alpha * A @ B^T as [M,N] of out_dtype."""
+    _require_cuda(a_codes, a_scales, b_codes, b_scales)
+    M, K = a_codes.shape[0], a_codes.shape[1] * 2
+    N = b_codes.shape[0]
+    if b_codes.shape[1] * 2 != K:
+        raise _lib.QuartetHipError(f"gemm_mxfp4_tn: contraction sizes differ ({K} vs {b_codes.shape[1] * 2})")
+    c = torch.empty((M, N), dtype=out_dtype, device=a_codes.device)
+    rc = _lib.lib().qm_gemm_mxfp4_tn(_ptr(a_codes), _ptr(a_scales), _ptr(b_codes), _ptr(b_scales), M, N, K, alpha,
+                                     _ptr(c), _dtype_code(out_dtype), _stream())
+    _lib.check(rc, "qm_gemm_mxfp4_tn")
+    return c
+
+
+def masked_hadamard_bwd(g, hadamard_dim=32, scale_dtype=torch.bfloat16, sign_bits=None, maskbits=None, out_dtype=None):
+    """g [R,C] -> ((g*mask).view(-1,hd) @ H^T) as [R,C] of out_dtype (default g.dtype)."""
+    _require_cuda(g, maskbits)
+    assert g.dim() == 2 and g.is_contiguous()
+    out_dtype = g.dtype if out_dtype is None else out_dtype
+    out = torch.empty(g.shape, dtype=out_dtype, device=g.device)
+    rc = _lib.lib().qm_masked_hadamard_bwd(_ptr(g), _dtype_code(g.dtype), g.shape[0], g.shape[1], hadamard_dim,
+                                           _dtype_code(scale_dtype), sign_words(sign_bits), _ptr(maskbits), _ptr(out),
+                                           _dtype_code(out_dtype), _stream())
+    _lib.check(rc, "qm_masked_hadamard_bwd")
+    return out
+
+
+def dequantize_mxfp4(codes, scales, post=1.0, out_dtype=torch.float32):
+    _require_cuda(codes, scales)
+    R, C = codes.shape[0], codes.shape[1] * 2
+    out = torch.empty((R, C), dtype=out_dtype, device=codes.device)
+    rc = _lib.lib().qm_dequantize_mxfp4(_ptr(codes), _ptr(scales), R, C, post, _ptr(out), _dtype_code(out_dtype),
+                                        _stream())
+    _lib.check(rc, "qm_dequantize_mxfp4")
+    return out

@@ -1,0 +1,74 @@
+"""GPU parity of the MXFP4 x MXFP4 GEMM (K2) against the oracle's fp64 matmul of the de-quantized
+operands: relative Frobenius error <= 1e-3 (the tolerance the target states); bit-exact in the
+special cases where every partial sum is exactly representable."""
+import numpy as np
+import pytest
+import torch
+
+from tests.util import make_input, to_oracle
+
+pytestmark = pytest.mark.gpu
+REL_FRO_TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def K():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from quartet_amd import kernels
+    return kernels
+
+
+def _quant(oracle, rows, cols, mode, seed, scale=1.0):
+    x = make_input(rows, cols, torch.bfloat16, seed=seed, scale=scale)
+    q = oracle.quantize(to_oracle(x), 32, mode=mode)
+    return q["codes"], q["scales"]
+
+
+@pytest.mark.parametrize("M,N,K_", [(128, 128, 128), (256, 384, 512), (96, 160, 224), (32, 32, 32), (1000, 72, 1728)])
+def test_gemm_against_fp64_matmul(oracle, K, M, N, K_):
+    print(f"case gemm {M}x{N}x{K_}", flush=True)
+    dev = torch.device("cuda:0")
+    ac, as_ = _quant(oracle, M, K_, oracle.QUEST_RTN, 1)
+    bc, bs = _quant(oracle, N, K_, oracle.ABSMAX_RTN, 2, scale=0.02)
+    d = float(oracle.FOUR_THIRDS)
+    want = oracle.gemm_tn(ac, as_, bc, bs, alpha=1.0, b_post=d)
+    args = [torch.from_numpy(t).to(dev) for t in (ac, as_, bc, bs)]
+    got32 = K.gemm_mxfp4_tn(*args, alpha=d, out_dtype=torch.float32)
+    got16 = K.gemm_mxfp4_tn(*args, alpha=d, out_dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    g = got32.cpu().numpy().astype(np.float64)
+    rel = np.linalg.norm(g - want) / np.linalg.norm(want)
+    assert rel <= REL_FRO_TOL, rel
+    assert rel <= 1e-5, rel  # fp32 accumulation of exact products: far inside the stated tolerance
+    # the bf16 output is the same accumulator rounded once
+    assert torch.equal(got16.cpu(), got32.cpu().to(torch.bfloat16))
+
+
+def test_gemm_bit_exact_when_sums_are_exact(oracle, K):
+    # all scales equal: products are multiples of 1/4 below 2^24 -> every fp32 partial sum is exact
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(0)
+    M, N, K_ = 160, 96, 640
+    ac = rng.integers(0, 256, (M, K_ // 2), dtype=np.uint8)
+    bc = rng.integers(0, 256, (N, K_ // 2), dtype=np.uint8)
+    as_ = np.full((M, K_ // 32), 127, dtype=np.uint8)
+    bs = np.full((N, K_ // 32), 126, dtype=np.uint8)
+    want = oracle.gemm_tn(ac, as_, bc, bs)
+    got = K.gemm_mxfp4_tn(*[torch.from_numpy(t).to(dev) for t in (ac, as_, bc, bs)], alpha=1.0, out_dtype=torch.float32)
+    assert np.array_equal(got.cpu().numpy().astype(np.float64), want)
+
+
+def test_gemm_one_hot_operand_selects_single_products(oracle, K):
+    dev = torch.device("cuda:0")
+    M, N, K_ = 64, 64, 256
+    bc, bs = _quant(oracle, N, K_, oracle.QUEST_RTN, 7)
+    ac = np.zeros((M, K_ // 2), dtype=np.uint8)
+    as_ = np.full((M, K_ // 32), 127, dtype=np.uint8)
+    ks = [(3 * m + 5) % K_ for m in range(M)]
+    for m, k in enumerate(ks):
+        ac[m, k // 2] = 0x2 << (4 * (k & 1))  # +1.0 at column k
+    got = K.gemm_mxfp4_tn(*[torch.from_numpy(t).to(dev) for t in (ac, as_, bc, bs)], alpha=1.0, out_dtype=torch.float32)
+    B = oracle.dequantize(bc, bs)
+    want = np.stack([B[:, k] for k in ks], axis=0)
+    assert np.array_equal(got.cpu().numpy(), want)

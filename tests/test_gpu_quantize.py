@@ -1,0 +1,151 @@
+"""GPU parity of the K1 quantizer family against the CPU oracle: FP4 codes, E8M0 scales, clip-mask
+bits and the de-quantized tensor must be bit-exact (integer/byte work), through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from tests.util import make_input, sign_int, to_oracle
+
+pytestmark = pytest.mark.gpu
+
+MODES = {"quest_rtn": 0, "absmax_rtn": 1, "absmax_sr": 2, "quest_sr": 3}
+
+
+@pytest.fixture(scope="module")
+def K():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from quartet_amd import kernels
+    return kernels
+
+
+def _check(oracle, K, x, hd, mode, signs, transposed, u, seed, tag):
+    dev = torch.device("cuda:0")
+    sb = None if signs is None else sign_int(signs)
+    want_mask = mode in (0, 3)
+    codes, scales, mask, deq = K.quantize_mxfp4(x.to(dev), hd, sb, mode, transposed, None if u is None else u.to(dev),
+                                                seed, want_mask=want_mask, want_dequant=True)
+    torch.cuda.synchronize()
+    ref = oracle.quantize(to_oracle(x), hd, signs=None if signs is None else signs.numpy(), mode=mode,
+                          transposed_in=transposed, u=None if u is None else u.numpy(), seed=seed,
+                          want_mask=want_mask, want_dequant=True)
+    for name, got, want in (("scales", scales, ref["scales"]), ("codes", codes, ref["codes"]),
+                            ("mask", mask, ref["mask"]), ("dequant", deq, ref["dequant"])):
+        if want is None:
+            continue
+        g = to_oracle(got)
+        if g.dtype == np.float32:
+            g, want = g.view(np.uint32), want.view(np.uint32)
+        bad = int((g != want).sum())
+        assert bad == 0, f"{tag}: {name} differs in {bad} of {want.size} entries"
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("hd", [32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rowmajor_bit_exact(oracle, K, mode, hd, dtype):
+    print(f"case rowmajor mode={mode} hd={hd} dtype={dtype}", flush=True)
+    x = make_input(96, 1024, dtype, seed=hd + MODES[mode], zero_rows=2)
+    g = torch.Generator().manual_seed(1)
+    signs = torch.randint(0, 2, (hd,), generator=g) * 2 - 1
+    u = torch.rand(x.shape, generator=g) if "sr" in mode else None
+    _check(oracle, K, x, hd, MODES[mode], signs, False, u, 0, f"rowmajor/{mode}/{hd}/{dtype}")
+
+
+@pytest.mark.parametrize("mode", ["absmax_sr", "quest_sr"])
+@pytest.mark.parametrize("hd", [32, 128])
+def test_philox_stream_bit_exact(oracle, K, mode, hd):
+    print(f"case philox mode={mode} hd={hd}", flush=True)
+    x = make_input(64, 512, torch.bfloat16, seed=3)
+    _check(oracle, K, x, hd, MODES[mode], None, False, None, 0x1234_5678_9ABC, f"philox/{mode}/{hd}")
+
+
+@pytest.mark.parametrize("mode", ["absmax_sr", "absmax_rtn", "quest_rtn"])
+@pytest.mark.parametrize("hd", [32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_transposed_input_bit_exact(oracle, K, mode, hd, dtype):
+    print(f"case transposed mode={mode} hd={hd} dtype={dtype}", flush=True)
+    # physical [P=384, Q=200]: ragged against the 128x64 tile in both directions
+    x = make_input(384, 200, dtype, seed=hd, zero_rows=1)
+    g = torch.Generator().manual_seed(2)
+    signs = torch.randint(0, 2, (hd,), generator=g) * 2 - 1
+    u = torch.rand(200, 384, generator=g) if "sr" in mode else None
+    _check(oracle, K, x, hd, MODES[mode], signs, True, u, 0, f"transposed/{mode}/{hd}/{dtype}")
+
+
+@pytest.mark.parametrize("hd", [32, 64, 128])
+@pytest.mark.parametrize("val_dtype", [torch.bfloat16, torch.float32])
+def test_requantize_transposed_bit_exact(oracle, K, hd, val_dtype):
+    print(f"case requant hd={hd} val_dtype={val_dtype}", flush=True)
+    dev = torch.device("cuda:0")
+    x = make_input(384, 160, torch.bfloat16, seed=5, zero_rows=1)
+    q = oracle.quantize(to_oracle(x), 32, mode=oracle.QUEST_RTN)
+    g = torch.Generator().manual_seed(3)
+    signs = torch.randint(0, 2, (hd,), generator=g) * 2 - 1
+    u = torch.rand(160, 384, generator=g)
+    vd = oracle.BF16 if val_dtype == torch.bfloat16 else oracle.F32
+    for mode, post in ((2, 1.0), (1, 1.0), (2, float(oracle.FOUR_THIRDS))):
+        ref = oracle.requantize_transposed(q["codes"], q["scales"], post=post, val_dtype=vd, hd=hd,
+                                           signs=signs.numpy(), mode=mode, u=u.numpy(), want_dequant=True)
+        co, so, dq = K.requantize_transposed_mxfp4(torch.from_numpy(q["codes"]).to(dev),
+                                                   torch.from_numpy(q["scales"]).to(dev), post, val_dtype, hd,
+                                                   sign_int(signs), mode, u.to(dev), 0, want_dequant=True)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_oracle(so), ref["scales"])
+        assert np.array_equal(to_oracle(co), ref["codes"])
+        a, b = to_oracle(dq), ref["dequant"]
+        if a.dtype == np.float32:
+            a, b = a.view(np.uint32), b.view(np.uint32)
+        assert np.array_equal(a, b)
+
+
+def test_order_independent_integer_fixture(oracle, K):
+    # x = S @ g with small integers and hd = 64: every partial sum is exact, so the expected
+    # rotated values (8*g) and hence codes/scales do not depend on any summation order.
+    import scipy.linalg
+    rng = np.random.default_rng(0)
+    g = rng.integers(-3, 4, size=(32, 64)).astype(np.float64)
+    x = torch.from_numpy((g @ scipy.linalg.hadamard(64)).astype(np.float32))
+    for mode in (0, 1):
+        _check(oracle, K, x, 64, mode, None, False, None, 0, f"integer/{mode}")
+        _check(oracle, K, x.to(torch.bfloat16), 64, mode, None, False, None, 0, f"integer-bf16/{mode}")
+
+
+def test_dequantize_and_hadamard_bwd(oracle, K):
+    dev = torch.device("cuda:0")
+    x = make_input(64, 512, torch.bfloat16, seed=9)
+    for mode, post in ((0, 1.0), (1, float(oracle.FOUR_THIRDS))):
+        q = oracle.quantize(to_oracle(x), 32, mode=mode, want_mask=True)
+        for od, oc in ((torch.float32, oracle.F32), (torch.bfloat16, oracle.BF16)):
+            got = K.dequantize_mxfp4(torch.from_numpy(q["codes"]).to(dev), torch.from_numpy(q["scales"]).to(dev), post, od)
+            want = oracle.dequantize(q["codes"], q["scales"], post, oc)
+            a = to_oracle(got)
+            assert np.array_equal(a.view(np.uint32) if a.dtype == np.float32 else a,
+                                  want.view(np.uint32) if want.dtype == np.float32 else want)
+    gen = torch.Generator().manual_seed(4)
+    for hd in (32, 64, 128):
+        signs = torch.randint(0, 2, (hd,), generator=gen) * 2 - 1
+        maskbits = torch.randint(0, 256, (64, 512 // 8), generator=gen, dtype=torch.uint8)
+        for gd, od in ((torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32), (torch.bfloat16, torch.float32)):
+            g = make_input(64, 512, gd, seed=hd)
+            for mb in (maskbits, None):
+                got = K.masked_hadamard_bwd(g.to(dev), hd, torch.bfloat16, sign_int(signs), None if mb is None else mb.to(dev), od)
+                want = oracle.masked_hadamard_bwd(to_oracle(g), hd, oracle.BF16, signs.numpy(),
+                                                  None if mb is None else mb.numpy(),
+                                                  oracle.BF16 if od == torch.bfloat16 else oracle.F32)
+                a = to_oracle(got)
+                assert np.array_equal(a.view(np.uint32) if a.dtype == np.float32 else a,
+                                      want.view(np.uint32) if want.dtype == np.float32 else want), (hd, gd, od)
+
+
+def test_empty_and_rejected_inputs(K):
+    dev = torch.device("cuda:0")
+    from quartet_amd._lib import QuartetHipError
+    c, s, m, d = K.quantize_mxfp4(torch.empty(0, 64, dtype=torch.bfloat16, device=dev), want_mask=True, want_dequant=True)
+    assert c.shape == (0, 32) and s.shape == (0, 2)
+    with pytest.raises(QuartetHipError, match="multiple of hadamard_dim"):
+        K.quantize_mxfp4(torch.zeros(4, 48, dtype=torch.bfloat16, device=dev))
+    with pytest.raises(QuartetHipError, match="hadamard_dim"):
+        K.quantize_mxfp4(torch.zeros(4, 64, dtype=torch.bfloat16, device=dev), hadamard_dim=16)
+    with pytest.raises(QuartetHipError):
+        K.quantize_mxfp4(torch.zeros(4, 64, dtype=torch.bfloat16))  # CPU tensor: no fallback
