@@ -1,0 +1,106 @@
+"""QuantizedLinear (API of the reference's src/models/quantization/__init__.py:11-42) and the fused
+packed-MXFP4 autograd Function behind its production configuration.
+
+Production configuration (main_setup.sh:77-93 of the reference): QuestMXFP4Quantizer on weights and
+activations, AlbertTsengQuantizer on gradients, scheme "Q(E)Q(Wt)t_Q(Et)Q(Xt)t".  For it the layer
+never materialises de-quantized tensors: operands stay packed (E2M1 codes + E8M0 scales + mask
+bits, the tensors notebooks/benchmark_mxfp4.ipynb's CudaGemm saves) and the three products run on
+the block-scaled FP4 MFMA.  Any other mix of quantizers/schemes takes the generic path through the
+quantizer modules and library GEMMs, as the reference does."""
+import torch
+import torch.nn as nn
+
+from . import kernels as K
+from .backward import BACKWARD_SCHEMES, EW_EtX_Scheme, QEQWtt_QEtQXtt_Scheme  # noqa: F401
+from .quantizers import QUANTIZER_CLASSES, AlbertTsengQuantizer, NoQuantizer, QuestMXFP4Quantizer  # noqa: F401
+from .quantizers.mxfp4 import _autocast_bf16, _fresh_seed
+
+
+class QuartetLinearFn(torch.autograd.Function):
+    """y = Q(x) Q(W)^T with the fully quantized backward of backward.py:57-85, on packed operands.
+
+    forward : F1/F2 quantize (quest RTN + mask) -> F3 FP4 GEMM
+    backward: re-randomise signs; B1 Q(e); B2 Q(Q(W)^T); B3 GEMM -> grad wrt Q(x);
+              B4 Q(e^T); B5 Q(Q(x)^T); B6 GEMM -> grad wrt Q(W);
+              B7/B8 masked inverse rotation (straight-through estimators of F1/F2)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, a_q, w_q, g_q):
+        in_features = weight.shape[1]
+        x2 = x.reshape(-1, in_features).contiguous()
+        w2 = weight.contiguous()
+        out_dtype = torch.bfloat16 if _autocast_bf16() else x.dtype
+        xc, xs, xm, _ = K.quantize_mxfp4(x2, a_q.hadamard_dim, a_q.sign_bits, K.QM_QUEST_RTN, want_mask=True)
+        wc, ws, wm, _ = K.quantize_mxfp4(w2, w_q.hadamard_dim, w_q.sign_bits, K.QM_QUEST_RTN, want_mask=True)
+        y = K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, out_dtype)
+        ctx.save_for_backward(xc, xs, xm, wc, ws, wm)
+        ctx.g_q = g_q
+        ctx.fwd = (a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits)
+        ctx.x_shape, ctx.x_dtype, ctx.w_dtype = x.shape, x.dtype, weight.dtype
+        return y.view(*x.shape[:-1], weight.shape[0])
+
+    @staticmethod
+    def backward(ctx, e):
+        xc, xs, xm, wc, ws, wm = ctx.saved_tensors
+        g_q = ctx.g_q
+        a_hd, a_signs, w_hd, w_signs = ctx.fwd
+        g_q.re_randomize()
+        hd, signs = g_q.hadamard_dim, g_q.sign_bits
+        mode = K.QM_ABSMAX_SR if g_q.stochastic else K.QM_ABSMAX_RTN
+        seed = (lambda: _fresh_seed()) if g_q.stochastic else (lambda: 0)
+        e2 = e.reshape(-1, e.shape[-1]).contiguous()
+        low = _autocast_bf16() or e2.dtype == torch.bfloat16
+        mid_dtype = torch.bfloat16 if low else e2.dtype
+        alpha = K.FOUR_THIRDS * K.FOUR_THIRDS  # both operands are absmax-coded: value = code * 2^k * 4/3
+
+        ec, es, _, _ = K.quantize_mxfp4(e2, hd, signs, mode, seed=seed())
+        wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, ctx.w_dtype, hd, signs, mode, seed=seed())
+        gxq = K.gemm_mxfp4_tn(ec, es, wtc, wts, alpha, mid_dtype)
+
+        etc, ets, _, _ = K.quantize_mxfp4(e2, hd, signs, mode, transposed_in=True, seed=seed())
+        xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, ctx.x_dtype, hd, signs, mode, seed=seed())
+        gwq = K.gemm_mxfp4_tn(etc, ets, xtc, xts, alpha, mid_dtype)
+
+        sd_x = torch.bfloat16 if low else ctx.x_dtype
+        sd_w = torch.bfloat16 if low else ctx.w_dtype
+        gx = K.masked_hadamard_bwd(gxq, a_hd, sd_x, a_signs, xm, mid_dtype).to(ctx.x_dtype)
+        gw = K.masked_hadamard_bwd(gwq, w_hd, sd_w, w_signs, wm, mid_dtype).to(ctx.w_dtype)
+        return gx.view(ctx.x_shape), gw, None, None, None
+
+
+class QuantizedLinear(nn.Linear):
+    """nn.Linear whose forward is scheme(act_q(x), weight_q(W)); the bias parameter, if requested,
+    is never applied -- exactly as in the reference (the scheme calls F.linear(x, w, None))."""
+
+    def __init__(self, in_features, out_features, weight_quantizer=None, activation_quantizer=None,
+                 gradient_quantizer=None, backward_scheme=None, **kwargs):
+        super().__init__(in_features, out_features, **kwargs)
+        if weight_quantizer is None:
+            weight_quantizer = NoQuantizer()
+        if activation_quantizer is None:
+            activation_quantizer = NoQuantizer()
+        if gradient_quantizer is None:
+            gradient_quantizer = NoQuantizer()
+        if backward_scheme is None:
+            backward_scheme = EW_EtX_Scheme()
+        self.weight_quantizer = weight_quantizer
+        self.activation_quantizer = activation_quantizer
+        self.backward_scheme = backward_scheme
+        self.backward_scheme.g_quantizer = gradient_quantizer
+        self.use_packed_path = True
+
+    def _is_production_config(self):
+        g_q = self.backward_scheme.g_quantizer
+        return (self.use_packed_path
+                and type(self.activation_quantizer) is QuestMXFP4Quantizer
+                and type(self.weight_quantizer) is QuestMXFP4Quantizer
+                and type(g_q) is AlbertTsengQuantizer
+                and type(self.backward_scheme) is QEQWtt_QEtQXtt_Scheme)
+
+    def forward(self, x):
+        if self._is_production_config():
+            return QuartetLinearFn.apply(x, self.weight, self.activation_quantizer, self.weight_quantizer,
+                                         self.backward_scheme.g_quantizer)
+        xq = self.activation_quantizer(x)
+        wq = self.weight_quantizer(self.weight)
+        return self.backward_scheme(xq, wq)

@@ -1,0 +1,180 @@
+"""GPU parity of the whole Quartet linear (QuantizedLinear in its production configuration and the
+per-quantizer modules) against the oracle pipeline on identical inputs, seeds and sign flips."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from tests.util import make_input, to_oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def q():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import quartet_amd
+    return quartet_amd
+
+
+def rel(a, b):
+    a, b = np.asarray(a, dtype=np.float64), np.asarray(b, dtype=np.float64)
+    return float(np.linalg.norm(a - b) / np.linalg.norm(b))
+
+
+def production_layer(q, I, O, stochastic, rerotate, dtype):
+    return q.QuantizedLinear(I, O, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(),
+                             activation_quantizer=q.QuestMXFP4Quantizer(),
+                             gradient_quantizer=q.AlbertTsengQuantizer(stochastic=stochastic, rerotate=rerotate),
+                             backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]()).to("cuda:0", dtype)
+
+
+def oracle_step(o, x, w, dy, signs, seeds, mode, val_dtype):
+    d = float(o.FOUR_THIRDS)
+    qx = o.quantize(to_oracle(x), 32, mode=o.QUEST_RTN, want_mask=True)
+    qw = o.quantize(to_oracle(w), 32, mode=o.QUEST_RTN, want_mask=True)
+    y = o.gemm_tn(qx["codes"], qx["scales"], qw["codes"], qw["scales"])
+    qe = o.quantize(to_oracle(dy), 32, signs=signs, mode=mode, seed=seeds[0])
+    qwt = o.requantize_transposed(qw["codes"], qw["scales"], val_dtype=val_dtype, hd=32, signs=signs, mode=mode, seed=seeds[1])
+    gxq = o.gemm_tn(qe["codes"], qe["scales"], qwt["codes"], qwt["scales"], a_post=d, b_post=d)
+    qet = o.quantize(to_oracle(dy), 32, signs=signs, mode=mode, transposed_in=True, seed=seeds[2])
+    qxt = o.requantize_transposed(qx["codes"], qx["scales"], val_dtype=val_dtype, hd=32, signs=signs, mode=mode, seed=seeds[3])
+    gwq = o.gemm_tn(qet["codes"], qet["scales"], qxt["codes"], qxt["scales"], a_post=d, b_post=d)
+    return y, gxq, gwq, qx["mask"], qw["mask"]
+
+
+def test_config1_forward_with_outlier_columns(oracle, q):
+    # X [4096 x 512] ~ N(0,1) with 4 outlier columns x20, W [2048 x 512] ~ N(0, 0.02), seed 0
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(4096, 512, generator=g)
+    cols = torch.randperm(512, generator=g)[:4]
+    x[:, cols] *= 20
+    w = 0.02 * torch.randn(2048, 512, generator=g)
+    x, w = x.to(torch.bfloat16), w.to(torch.bfloat16)
+    from quartet_amd import kernels as K
+    dev = "cuda:0"
+    xc, xs, xm, _ = K.quantize_mxfp4(x.to(dev), 32, None, K.QM_QUEST_RTN, want_mask=True)
+    wc, ws, wm, _ = K.quantize_mxfp4(w.to(dev), 32, None, K.QM_QUEST_RTN, want_mask=True)
+    qx = oracle.quantize(to_oracle(x), 32, mode=oracle.QUEST_RTN, want_mask=True)
+    qw = oracle.quantize(to_oracle(w), 32, mode=oracle.QUEST_RTN, want_mask=True)
+    for got, want in ((xc, qx["codes"]), (xs, qx["scales"]), (xm, qx["mask"]), (wc, qw["codes"]), (ws, qw["scales"]), (wm, qw["mask"])):
+        assert np.array_equal(to_oracle(got), want)
+    y = K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.float32)
+    y_ref = oracle.gemm_tn(qx["codes"], qx["scales"], qw["codes"], qw["scales"])
+    assert rel(y.cpu().numpy(), y_ref) <= 1e-3
+    # and through the module (bf16 output = one extra rounding of 2^-9 relative per element)
+    layer = production_layer(q, 512, 2048, False, None, torch.bfloat16)
+    with torch.no_grad():
+        layer.weight.copy_(w.to(dev))
+        ym = layer(x.to(dev))
+    assert torch.equal(ym.cpu(), y.cpu().to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("stochastic,rerotate", [(False, None), (True, "signs")])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_production_step_against_oracle(oracle, q, stochastic, rerotate, dtype):
+    print(f"case linear step stochastic={stochastic} rerotate={rerotate} dtype={dtype}", flush=True)
+    T, I, O = 384, 256, 160
+    x = make_input(T, I, dtype, seed=1, outlier_frac=0.01)
+    w = make_input(O, I, dtype, seed=2, outlier_frac=0, scale=0.02)
+    dy = make_input(T, O, dtype, seed=3, outlier_frac=0, scale=1e-3)
+    layer = production_layer(q, I, O, stochastic, rerotate, dtype)
+    with torch.no_grad():
+        layer.weight.copy_(w.to("cuda:0"))
+    xd = x.to("cuda:0").view(2, T // 2, I).requires_grad_(True)  # leading dims are flattened by the layer
+    torch.manual_seed(5)
+    random.seed(5)
+    y = layer(xd)
+    y.backward(dy.to("cuda:0").view(2, T // 2, O))
+    torch.cuda.synchronize()
+
+    torch.manual_seed(5)
+    random.seed(5)
+    signs = None
+    if rerotate == "signs":
+        signs = np.where(torch.randint(0, 2, (32,)).numpy() == 0, -1, 1)
+    seeds = [random.getrandbits(63) for _ in range(4)] if stochastic else [0, 0, 0, 0]
+    mode = oracle.ABSMAX_SR if stochastic else oracle.ABSMAX_RTN
+    vd = oracle.BF16 if dtype == torch.bfloat16 else oracle.F32
+    y_ref, gxq, gwq, xm, wm = oracle_step(oracle, x, w, dy, signs, seeds, mode, vd)
+    gx_ref = oracle.masked_hadamard_bwd(gxq.astype(np.float32), 32, vd, None, xm, out_dtype=oracle.F32)
+    gw_ref = oracle.masked_hadamard_bwd(gwq.astype(np.float32), 32, vd, None, wm, out_dtype=oracle.F32)
+    # fp32 end to end: only accumulation order differs -> the 1e-3 Frobenius tolerance of the target,
+    # with a wide margin.  bf16: each stored tensor adds one rounding of relative size 2^-9.
+    tol_y, tol_g = (1e-5, 1e-5) if dtype == torch.float32 else (3e-3, 5e-3)
+    assert y.dtype == dtype and xd.grad.dtype == dtype and layer.weight.grad.dtype == dtype
+    assert rel(y.detach().float().cpu().numpy().reshape(T, O), y_ref) <= tol_y
+    assert rel(xd.grad.float().cpu().numpy().reshape(T, I), gx_ref) <= tol_g
+    assert rel(layer.weight.grad.float().cpu().numpy(), gw_ref) <= tol_g
+
+
+def test_generic_module_path_matches_packed_path(q):
+    # the reference-shaped path (quantizer modules -> de-quantized tensors -> library GEMMs) and the
+    # packed FP4 path compute the same function when the backward is deterministic
+    T, I, O = 256, 128, 96
+    x = make_input(T, I, torch.float32, seed=4)
+    w = make_input(O, I, torch.float32, seed=5, outlier_frac=0, scale=0.02)
+    dy = make_input(T, O, torch.float32, seed=6, outlier_frac=0, scale=1e-3)
+    outs = []
+    for packed in (True, False):
+        layer = production_layer(q, I, O, False, None, torch.float32)
+        layer.use_packed_path = packed
+        with torch.no_grad():
+            layer.weight.copy_(w.to("cuda:0"))
+        xd = x.to("cuda:0").requires_grad_(True)
+        y = layer(xd)
+        y.backward(dy.to("cuda:0"))
+        outs.append((y.detach().cpu().numpy(), xd.grad.cpu().numpy(), layer.weight.grad.cpu().numpy()))
+    for a, b in zip(*outs):
+        assert rel(a, b) <= 1e-3
+
+
+def test_quantizer_modules_match_oracle(oracle, q):
+    dev = "cuda:0"
+    x = make_input(64, 256, torch.bfloat16, seed=7)
+    xd = x.to(dev).requires_grad_(True)
+    quest = q.QuestMXFP4Quantizer()
+    out = quest(xd)
+    ref = oracle.quantize(to_oracle(x), 32, mode=oracle.QUEST_RTN, want_mask=True, want_dequant=True)
+    assert np.array_equal(to_oracle(out), ref["dequant"])
+    g = make_input(64, 256, torch.bfloat16, seed=8, outlier_frac=0)
+    out.backward(g.to(dev))
+    want = oracle.masked_hadamard_bwd(to_oracle(g), 32, oracle.BF16, None, ref["mask"])
+    assert np.array_equal(to_oracle(xd.grad), want)
+    # kernel wrapper with the reference's signature, matrix carrying sign flips
+    tseng = q.AlbertTsengQuantizer(stochastic=False, rerotate="signs")
+    torch.manual_seed(3)
+    tseng.re_randomize()
+    tseng._note_input(xd)
+    deq, clip = q.mxfp4_forward_kernel_wrapper(x.to(dev), tseng.hadamard_matrix, return_clip_mask=True, quest=False)
+    signs = np.array([-1 if (tseng.sign_bits >> j) & 1 else 1 for j in range(32)])
+    ref2 = oracle.quantize(to_oracle(x), 32, signs=signs, mode=oracle.ABSMAX_RTN, want_mask=True, want_dequant=True)
+    assert np.array_equal(to_oracle(deq), ref2["dequant"])
+    assert np.array_equal(clip.cpu().numpy(), oracle.unpack_mask(ref2["mask"]))
+    assert np.array_equal(to_oracle(tseng(x.to(dev))), ref2["dequant"])
+    aligned = q.AlignedAlbertTsengQuantizer()
+    got = aligned(x.to(dev)).float().cpu().numpy()
+    base = oracle.bf16_bits_to_f32(oracle.quantize(to_oracle(x), 32, mode=oracle.ABSMAX_RTN, want_dequant=True)["dequant"])
+    np.testing.assert_allclose(got, base * 1.009276, rtol=2 ** -7)
+
+
+def test_notebook_error_bands_on_gpu(q):
+    # notebooks/benchmark_mxfp4.ipynb: x = randn(1,128,4096), w = randn(128,4096) bf16, deterministic
+    # backward: 2e-2 < fwd rel^2 err < 6e-2 and 6e-2 < wgrad rel^2 err < 15e-2 against plain bf16 linear
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(1, 128, 4096, generator=g).to(torch.bfloat16).to("cuda:0").requires_grad_(True)
+    w = torch.randn(128, 4096, generator=g).to(torch.bfloat16).to("cuda:0")
+    dy = torch.randn(1, 128, 128, generator=g).to(torch.bfloat16).to("cuda:0")
+    layer = production_layer(q, 4096, 128, False, None, torch.bfloat16)
+    with torch.no_grad():
+        layer.weight.copy_(w)
+    y = layer(x)
+    y.backward(dy)
+    wref = w.clone().float().requires_grad_(True)
+    yref = torch.nn.functional.linear(x.detach().float(), wref)
+    yref.backward(dy.float())
+    err = lambda a, b: float(((a.float() - b.float()) ** 2).sum() / (b.float() ** 2).sum())
+    assert 2e-2 < err(y, yref) < 6e-2
+    assert 6e-2 < err(layer.weight.grad, wref.grad) < 15e-2
