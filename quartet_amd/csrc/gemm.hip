@@ -204,6 +204,466 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tn_kernel(const uint8_t* __res
         }
 }
 
+
+// ---- large-tile kernel: 256 x 256 macro tile, one wave per SIMD owning 128 x 128 -----------------
+// Requires M % 256 == 0, N % 256 == 0, K % 128 == 0.
+//
+// Per K step of 128 a wave issues 32 MFMAs (2 sub-steps x 4 x 4 tiles) against 16 fragment reads of
+// 16 bytes.  Operands go global -> LDS directly (global_load_lds_dwordx4: each wave instruction drops
+// 64 x 16 B contiguously into LDS, no staging registers, no ds_write), into a ring of four stages, so
+// a tile is requested three K steps before it is consumed.  LDS rows are 64 bytes; the 16-byte column
+// of (row, c) is stored at c ^ ((row >> 2) & 3), applied on the global-address side of the load and on
+// the fragment read, which keeps the 16-byte fragment reads of 32 consecutive rows off each other's banks.
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+
+// acc element e of a 32x32 tile is row 8*(e/4) + 4*half + e%4, column lane%32: per store instruction the
+// two half-waves each write one 64-byte (bf16) row segment.  (Making a lane's 4 values contiguous along n by
+// swapping the MFMA operand roles was measured slower: 64 scattered 8-byte pieces per instruction.)
+template <typename OutT>
+__device__ __forceinline__ void store_tile(const v16f& t, float alpha, OutT* __restrict__ c, int64_t row0, int64_t col,
+                                           int64_t N, int half) {
+#pragma unroll
+    for (int e = 0; e < 16; e += 2) {
+        const int64_t r = row0 + 8 * (e / 4) + 4 * half + (e & 3);
+        const float v0 = t[e] * alpha, v1 = t[e + 1] * alpha;
+        if constexpr (sizeof(OutT) == 2) {
+            // v_cvt_pk_bf16_f32: round-to-nearest-even, two values per instruction
+            const v2bf p = __builtin_convertvector(v2f{v0, v1}, v2bf);
+            const uint32_t bits = __builtin_bit_cast(uint32_t, p);
+            c[r * N + col] = (uint16_t)(bits & 0xffffu);
+            c[(r + 1) * N + col] = (uint16_t)(bits >> 16);
+        } else {
+            c[r * N + col] = v0;
+            c[(r + 1) * N + col] = v1;
+        }
+    }
+}
+
+constexpr int kBigM = 256, kBigN = 256;
+constexpr int kStages = 4;
+constexpr int kStageBytes = (kBigM + kBigN) * kRowBytes + (kBigM + kBigN) * 4;  // 32 KiB codes + 2 KiB scales
+constexpr int kBOff = kBigM * kRowBytes;
+constexpr int kSAOff = (kBigM + kBigN) * kRowBytes;
+constexpr int kSBOff = kSAOff + kBigM * 4;
+constexpr int kBigSmemBytes = kStages * kStageBytes;
+constexpr int kLoadsPerStep = 10;  // VMEM instructions per wave per K step
+
+// Tile order: workgroup ids are dealt round-robin to the 8 XCDs by the hardware; give each XCD a
+// contiguous run of tiles in an order that walks 8-row groups column by column, so the tiles that
+// share an L2 also share A and B panels.
+__device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int total = tiles_m * tiles_n;
+    int t = bid;
+    if ((total & 7) == 0) t = (bid & 7) * (total >> 3) + (bid >> 3);
+    constexpr int GM = 8;
+    const int per_group = GM * tiles_n;
+    const int group = t / per_group;
+    const int first_m = group * GM;
+    const int gm = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
+    const int r = t - group * per_group;
+    tm = first_m + r % gm;
+    tn = r / gm;
+}
+
+struct BigLoadPlan {
+    const uint8_t* a;   // this lane's A source for wave-load 0 at K step 0 (+ j * 16 rows, + ks * 64 bytes)
+    const uint8_t* b;
+    const uint8_t* sa;  // this lane's A scale dword source at K step 0 (+ ks * 4 bytes)
+    const uint8_t* sb;
+    int64_t row16_bytes;   // 16 rows of codes
+    uint32_t lds_codes;    // wave-uniform LDS byte address of this wave's first A wave-load in stage 0
+    uint32_t lds_scales;   // likewise for its A scale wave-load
+};
+
+// global -> LDS without passing through registers.  Written as inline assembly on purpose: the
+// compiler's wait-count insertion treats every LDS read as possibly aliasing an outstanding
+// global_load_lds and would drain all loads (vmcnt(0)) before each fragment read, which defeats the
+// prefetch ring; the kernel waits explicitly for the one tile it is about to read instead.
+// LDS destination = lds_base (wave-uniform, via M0) + lane * size.
+__device__ __forceinline__ void load_lds_b128(const uint8_t* gsrc, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gsrc), "s"(lds_base));
+}
+__device__ __forceinline__ void load_lds_b32(const uint8_t* gsrc, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gsrc), "s"(lds_base));
+}
+
+// issue the ten loads of K step ks into ring stage `stage`
+__device__ __forceinline__ void big_issue_loads(const BigLoadPlan& p, int stage, int ks) {
+    const uint32_t base = p.lds_codes + stage * kStageBytes;
+    const int kb = ks * kRowBytes;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        load_lds_b128(p.a + j * p.row16_bytes + kb, base + j * 1024);
+        load_lds_b128(p.b + j * p.row16_bytes + kb, base + kBOff + j * 1024);
+    }
+#ifndef QM_DBG_NO_SCALES
+    load_lds_b32(p.sa + ks * 4, p.lds_scales + stage * kStageBytes);
+    load_lds_b32(p.sb + ks * 4, p.lds_scales + stage * kStageBytes + (kSBOff - kSAOff));
+#endif
+}
+
+struct SubFrags {
+    uint4 a[4], b[4];  // one K sub-step (64 values): four A tiles, four B tiles
+};
+
+// frag_off = byte offset of this lane's 16 bytes for the wanted sub-step within tile 0 of its operand
+__device__ __forceinline__ void big_read_sub(const uint8_t* __restrict__ stage, int a_off, int b_off, SubFrags& f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f.a[i] = *reinterpret_cast<const uint4*>(stage + a_off + i * 32 * kRowBytes);
+        f.b[i] = *reinterpret_cast<const uint4*>(stage + kBOff + b_off + i * 32 * kRowBytes);
+    }
+}
+
+// Scales in LDS: per operand, dword [(row / 128) * 32 + row % 32][(row / 32) % 4] is the row's four E8M0
+// bytes of this K step, so one 16-byte read fetches the scale dwords of a lane's four tiles.
+__device__ __forceinline__ void big_read_scales(const uint8_t* __restrict__ stage, int a_off, int b_off, uint4& sa4,
+                                                uint4& sb4) {
+    sa4 = *reinterpret_cast<const uint4*>(stage + kSAOff + a_off);
+    sb4 = *reinterpret_cast<const uint4*>(stage + kSBOff + b_off);
+}
+
+template <int SUB>
+__device__ __forceinline__ void big_mfma_sub(const SubFrags& f, const uint32_t (&sca)[4], const uint32_t (&scb)[4],
+                                             v16f (&acc)[4][4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const v8i av = v8i{(int)f.a[i].x, (int)f.a[i].y, (int)f.a[i].z, (int)f.a[i].w, 0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const v8i bv = v8i{(int)f.b[j].x, (int)f.b[j].y, (int)f.b[j].z, (int)f.b[j].w, 0, 0, 0, 0};
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[i][j], 4, 4, SUB, (int)sca[i], SUB, (int)scb[j]);
+        }
+    }
+}
+
+// one MFMA, then one memory instruction of the given class, n times: keeps the matrix pipe fed while the
+// wave issues its LDS / VMEM instructions
+#define QM_SCHED_PAIR(mask, n)                                   \
+    for (int _i = 0; _i < (n); ++_i) {                           \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);       \
+        __builtin_amdgcn_sched_group_barrier((mask), 1, 0);      \
+    }
+
+// Pipeline, K step ks (tile ks lives in ring stage ks % 4); one barrier per step:
+//   phase 1: read sub-step-1 fragments of tile ks | 16 MFMAs on its sub-step-0 fragments (in registers);
+//   wait until this wave's loads of tile ks+1 have landed, barrier (tile ks+1 visible to all, stage ks%4 free);
+//   phase 2: request tile ks+4 into stage ks%4; read scales and sub-step-0 fragments of tile ks+1 |
+//            16 MFMAs on sub-step 1 of tile ks.
+template <typename OutT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mxfp4_tn_big_kernel(
+    const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ b_codes,
+    const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c) {
+    extern __shared__ uint32_t smem[];
+    uint8_t* smem_bytes = reinterpret_cast<uint8_t*>(smem);
+    const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)smem;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lrow = lane & 31, half = lane >> 5;
+    int tm, tn;
+    tile_of_block((int)blockIdx.x, M / kBigM, N / kBigN, tm, tn);
+    const int64_t m0 = (int64_t)tm * kBigM, n0 = (int64_t)tn * kBigN;
+    const int code_pitch = K / 2, groups = K / 32;
+    const int nk = K / kBK;
+
+    BigLoadPlan plan;
+    {
+        // codes: wave-load j of wave w fills LDS rows (w*4+j)*16 .. +15; lane l -> row + l/4, slot l%4
+        const int row = wave * 64 + (lane >> 2);
+        const int cv = (lane & 3) ^ ((row >> 2) & 3);
+        plan.a = a_codes + (m0 + row) * code_pitch + cv * 16;
+        plan.b = b_codes + (n0 + row) * code_pitch + cv * 16;
+        plan.row16_bytes = (int64_t)16 * code_pitch;
+        // scales: LDS dword p = wave*64 + lane holds operand row (p>>7)*128 + (p&3)*32 + ((p>>2)&31)
+        const int p = wave * 64 + lane;
+        const int srow = (p >> 7) * 128 + (p & 3) * 32 + ((p >> 2) & 31);
+        plan.sa = a_scales + (m0 + srow) * groups;
+        plan.sb = b_scales + (n0 + srow) * groups;
+        plan.lds_codes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + wave * 4096));
+        plan.lds_scales = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + kSAOff + wave * 256));
+    }
+
+    v16f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    const int swz = (lrow >> 2) & 3;
+    const int a_off0 = (wm * 128 + lrow) * kRowBytes + (((2 * half) ^ swz) * 16);
+    const int a_off1 = (wm * 128 + lrow) * kRowBytes + (((2 * half + 1) ^ swz) * 16);
+    const int b_off0 = (wn * 128 + lrow) * kRowBytes + (((2 * half) ^ swz) * 16);
+    const int b_off1 = (wn * 128 + lrow) * kRowBytes + (((2 * half + 1) ^ swz) * 16);
+    const int a_sc_off = (wm * 32 + lrow) * 16, b_sc_off = (wn * 32 + lrow) * 16;
+    const int sh = 16 * half;
+
+    // prologue: request the first four tiles, wait for tile 0
+#pragma unroll
+    for (int t = 0; t < kStages; ++t)
+        if (t < nk) big_issue_loads(plan, t, t);
+    if (nk >= kStages) __builtin_amdgcn_s_waitcnt(0x0f70 | (3 * kLoadsPerStep & 0xf) | (((3 * kLoadsPerStep) >> 4) << 14));
+    else __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    __syncthreads();
+    SubFrags f0, f1;
+    uint4 sa4, sb4;
+    big_read_sub(smem_bytes, a_off0, b_off0, f0);
+    big_read_scales(smem_bytes, a_sc_off, b_sc_off, sa4, sb4);
+
+    int ks = 0;
+    // steady state: tiles up to ks+4 exist; no conditionals inside the scheduling regions
+    for (; ks + kStages < nk; ++ks) {
+        const uint8_t* cur = smem_bytes + (ks & 3) * kStageBytes;
+        const uint8_t* nxt = smem_bytes + ((ks + 1) & 3) * kStageBytes;
+        const uint32_t sca[4] = {sa4.x >> sh, sa4.y >> sh, sa4.z >> sh, sa4.w >> sh};
+        const uint32_t scb[4] = {sb4.x >> sh, sb4.y >> sh, sb4.z >> sh, sb4.w >> sh};
+#ifndef QM_DBG_NO_LDSREAD
+        big_read_sub(cur, a_off1, b_off1, f1);
+#endif
+        big_mfma_sub<0>(f0, sca, scb, acc);
+        QM_SCHED_PAIR(0x100, 8)
+        __builtin_amdgcn_sched_barrier(0);
+        // this wave's loads of tile ks+1 are older than those of tiles ks+2, ks+3: allow 20 outstanding
+        __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * kLoadsPerStep & 0xf) | (((2 * kLoadsPerStep) >> 4) << 14));
+#ifndef QM_DBG_NO_BARRIER
+        __syncthreads();
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+#ifndef QM_DBG_NO_LDSREAD
+        big_read_scales(nxt, a_sc_off, b_sc_off, sa4, sb4);
+        big_read_sub(nxt, a_off0, b_off0, f0);
+#endif
+#ifndef QM_DBG_NO_GLOBAL
+        big_issue_loads(plan, ks & 3, ks + kStages);
+#endif
+        big_mfma_sub<1>(f1, sca, scb, acc);
+        QM_SCHED_PAIR(0x100, 10)
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // drain: the last (up to four) tiles, nothing left to request
+    for (; ks < nk; ++ks) {
+        const uint8_t* cur = smem_bytes + (ks & 3) * kStageBytes;
+        const uint8_t* nxt = smem_bytes + ((ks + 1) & 3) * kStageBytes;
+        const bool has_next = ks + 1 < nk;
+        const uint32_t sca[4] = {sa4.x >> sh, sa4.y >> sh, sa4.z >> sh, sa4.w >> sh};
+        const uint32_t scb[4] = {sb4.x >> sh, sb4.y >> sh, sb4.z >> sh, sb4.w >> sh};
+        big_read_sub(cur, a_off1, b_off1, f1);
+        big_mfma_sub<0>(f0, sca, scb, acc);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): everything requested has landed
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        if (has_next) {
+            big_read_scales(nxt, a_sc_off, b_sc_off, sa4, sb4);
+            big_read_sub(nxt, a_off0, b_off0, f0);
+        }
+        big_mfma_sub<1>(f1, sca, scb, acc);
+    }
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            store_tile<OutT>(acc[i][j], alpha, c, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
+}
+
+// ---- variant for K % 512 == 0: scales travel in blocks of four K steps -----------------------------
+// Fetching one scale dword per row per K step costs as many L2 requests as the codes themselves (each
+// row's 4 bytes sit in a different cache line).  Here a wave-load brings 16 bytes per row = the scales of
+// four K steps, into a small double-buffered LDS area behind the four code stages; a lane reads the
+// scale vectors of its eight tile rows once per block and keeps them in registers.
+constexpr int kCodeStageBytes = (kBigM + kBigN) * kRowBytes;            // 32 KiB
+constexpr int kScaleAreaOff = kStages * kCodeStageBytes;                // 128 KiB
+constexpr int kScaleBufBytes = (kBigM + kBigN) * 16;                    // 8 KiB per block of four K steps
+constexpr int kBig4SmemBytes = kScaleAreaOff + 2 * kScaleBufBytes;      // 144 KiB
+
+struct Big4Plan {
+    const uint8_t* a;
+    const uint8_t* b;
+    const uint8_t* sa;  // this lane's scale source of block 0: row (wave*64 + lane), 16 bytes per block
+    const uint8_t* sb;
+    int64_t row16_bytes;
+    uint32_t lds_codes;   // wave-uniform LDS address of this wave's first A wave-load in stage 0
+    uint32_t lds_scales;  // wave-uniform LDS address of this wave's A scale wave-load in buffer 0
+};
+
+__device__ __forceinline__ void big4_issue_codes(const Big4Plan& p, int stage, int ks) {
+    const uint32_t base = p.lds_codes + stage * kCodeStageBytes;
+    const int kb = ks * kRowBytes;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        load_lds_b128(p.a + j * p.row16_bytes + kb, base + j * 1024);
+        load_lds_b128(p.b + j * p.row16_bytes + kb, base + kBOff + j * 1024);
+    }
+}
+__device__ __forceinline__ void big4_issue_scales(const Big4Plan& p, int qb) {
+    const uint32_t base = p.lds_scales + (qb & 1) * kScaleBufBytes;
+    load_lds_b128(p.sa + qb * 16, base);
+    load_lds_b128(p.sb + qb * 16, base + kBigM * 16);
+}
+
+struct ScaleRegs {
+    uint4 a[4], b[4];  // per tile: the row's scale dwords of the block's four K steps
+};
+__device__ __forceinline__ void big4_read_scales(const uint8_t* __restrict__ sbuf, int a_off, int b_off, ScaleRegs& r) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        r.a[i] = *reinterpret_cast<const uint4*>(sbuf + a_off + i * 32 * 16);
+        r.b[i] = *reinterpret_cast<const uint4*>(sbuf + kBigM * 16 + b_off + i * 32 * 16);
+    }
+}
+template <int Q>
+__device__ __forceinline__ uint32_t pick(const uint4& v) {
+    return Q == 0 ? v.x : (Q == 1 ? v.y : (Q == 2 ? v.z : v.w));
+}
+
+constexpr int vmcnt_imm(int n) { return 0x0f70 | (n & 0xf) | ((n >> 4) << 14); }
+
+struct Big4State {
+    SubFrags f0, f1;
+    ScaleRegs sr;
+};
+
+// K step ks = 4*qb + Q.  ISSUE: steady state (tile ks+4 and, for Q == 0, scale block qb+1 are requested).
+template <int Q, bool ISSUE>
+__device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_bytes, int ks, bool has_next, int a_off0,
+                                          int a_off1, int b_off0, int b_off1, int a_sc_off, int b_sc_off, int sh,
+                                          Big4State& st, v16f (&acc)[4][4]) {
+    const uint8_t* cur = smem_bytes + (ks & 3) * kCodeStageBytes;
+    const uint8_t* nxt = smem_bytes + ((ks + 1) & 3) * kCodeStageBytes;
+    const uint32_t sca[4] = {pick<Q>(st.sr.a[0]) >> sh, pick<Q>(st.sr.a[1]) >> sh, pick<Q>(st.sr.a[2]) >> sh, pick<Q>(st.sr.a[3]) >> sh};
+    const uint32_t scb[4] = {pick<Q>(st.sr.b[0]) >> sh, pick<Q>(st.sr.b[1]) >> sh, pick<Q>(st.sr.b[2]) >> sh, pick<Q>(st.sr.b[3]) >> sh};
+    big_read_sub(cur, a_off1, b_off1, st.f1);
+    big_mfma_sub<0>(st.f0, sca, scb, acc);
+    if constexpr (ISSUE) { QM_SCHED_PAIR(0x100, 8) }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (ISSUE) {
+        // loads younger than the codes of tile ks+1: codes of tiles ks+2, ks+3 (16) and, for Q = 1, 2, the two
+        // scale loads issued since; for Q = 3 the scale block read below is older than those and must be in
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((Q == 1 || Q == 2) ? 18 : 16));
+    } else {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    }
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    if (ISSUE || has_next) {
+        if constexpr (Q == 3) big4_read_scales(smem_bytes + kScaleAreaOff + (((ks + 1) >> 2) & 1) * kScaleBufBytes, a_sc_off, b_sc_off, st.sr);
+        big_read_sub(nxt, a_off0, b_off0, st.f0);
+    }
+    if constexpr (ISSUE) {
+        big4_issue_codes(plan, ks & 3, ks + kStages);
+        if constexpr (Q == 0) big4_issue_scales(plan, (ks >> 2) + 1);
+    }
+    big_mfma_sub<1>(st.f1, sca, scb, acc);
+    if constexpr (ISSUE) { QM_SCHED_PAIR(0x100, (Q == 3 ? 16 : 8)) }
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <typename OutT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mxfp4_tn_big4_kernel(
+    const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ b_codes,
+    const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c) {
+    extern __shared__ uint32_t smem[];
+    uint8_t* smem_bytes = reinterpret_cast<uint8_t*>(smem);
+    const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)smem;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lrow = lane & 31, half = lane >> 5;
+    int tm, tn;
+    tile_of_block((int)blockIdx.x, M / kBigM, N / kBigN, tm, tn);
+    const int64_t m0 = (int64_t)tm * kBigM, n0 = (int64_t)tn * kBigN;
+    const int code_pitch = K / 2, groups = K / 32;
+    const int nk = K / kBK;  // a multiple of 4
+
+    Big4Plan plan;
+    {
+        const int row = wave * 64 + (lane >> 2);
+        const int cv = (lane & 3) ^ ((row >> 2) & 3);
+        plan.a = a_codes + (m0 + row) * code_pitch + cv * 16;
+        plan.b = b_codes + (n0 + row) * code_pitch + cv * 16;
+        plan.row16_bytes = (int64_t)16 * code_pitch;
+        plan.sa = a_scales + (m0 + wave * 64 + lane) * groups;
+        plan.sb = b_scales + (n0 + wave * 64 + lane) * groups;
+        plan.lds_codes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + wave * 4096));
+        plan.lds_scales = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + kScaleAreaOff + wave * 1024));
+    }
+
+    v16f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    const int swz = (lrow >> 2) & 3;
+    const int a_off0 = (wm * 128 + lrow) * kRowBytes + (((2 * half) ^ swz) * 16);
+    const int a_off1 = (wm * 128 + lrow) * kRowBytes + (((2 * half + 1) ^ swz) * 16);
+    const int b_off0 = (wn * 128 + lrow) * kRowBytes + (((2 * half) ^ swz) * 16);
+    const int b_off1 = (wn * 128 + lrow) * kRowBytes + (((2 * half + 1) ^ swz) * 16);
+    const int a_sc_off = (wm * 128 + lrow) * 16, b_sc_off = (wn * 128 + lrow) * 16;
+    const int sh = 16 * half;
+
+    // prologue: scale block 0, code tiles 0..3; wait for the scales and tile 0 (24 younger loads may be pending)
+    big4_issue_scales(plan, 0);
+#pragma unroll
+    for (int t = 0; t < kStages; ++t) big4_issue_codes(plan, t, t);
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(24));
+    __syncthreads();
+    Big4State st;
+    big4_read_scales(smem_bytes + kScaleAreaOff, a_sc_off, b_sc_off, st.sr);
+    big_read_sub(smem_bytes, a_off0, b_off0, st.f0);
+
+    int ks = 0;
+    for (; ks + 8 <= nk; ks += 4) {
+        big4_step<0, true>(plan, smem_bytes, ks, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+        big4_step<1, true>(plan, smem_bytes, ks + 1, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+        big4_step<2, true>(plan, smem_bytes, ks + 2, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+        big4_step<3, true>(plan, smem_bytes, ks + 3, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+    }
+    // last block: everything has been requested
+    big4_step<0, false>(plan, smem_bytes, ks, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+    big4_step<1, false>(plan, smem_bytes, ks + 1, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+    big4_step<2, false>(plan, smem_bytes, ks + 2, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+    big4_step<3, false>(plan, smem_bytes, ks + 3, false, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            store_tile<OutT>(acc[i][j], alpha, c, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
+}
+
+template <typename OutT>
+hipError_t launch_big4(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                       const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c,
+                       hipStream_t stream) {
+    auto kern = gemm_mxfp4_tn_big4_kernel<OutT>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kBig4SmemBytes);
+    if (e != hipSuccess) return e;
+    dim3 grid((unsigned)((M / kBigM) * (N / kBigN))), block(256);
+    kern<<<grid, block, kBig4SmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
+                                                  reinterpret_cast<OutT*>(c));
+    return hipGetLastError();
+}
+
+template <typename OutT>
+hipError_t launch_big(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                      const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c,
+                      hipStream_t stream) {
+    auto kern = gemm_mxfp4_tn_big_kernel<OutT>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kBigSmemBytes);
+    if (e != hipSuccess) return e;
+    dim3 grid((unsigned)((M / kBigM) * (N / kBigN))), block(256);
+    kern<<<grid, block, kBigSmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
+                                                 reinterpret_cast<OutT*>(c));
+    return hipGetLastError();
+}
+
 template <int BM, int BN, int WM, int WN>
 hipError_t launch_gemm(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                        const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
@@ -234,6 +694,15 @@ hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const 
                          const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
                          hipStream_t stream) {
     if (M == 0 || N == 0) return hipSuccess;
+    const bool big_ok = M % kBigM == 0 && N % kBigN == 0 && K > 0 && M < (1 << 30) && N < (1 << 30) && K < (1 << 30);
+    if (big_ok && K % 512 == 0 && (reinterpret_cast<uintptr_t>(a_scales) & 15) == 0 && (reinterpret_cast<uintptr_t>(b_scales) & 15) == 0) {
+        if (c_dtype == BF16) return launch_big4<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, stream);
+        return launch_big4<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, stream);
+    }
+    if (big_ok && K % kBK == 0) {
+        if (c_dtype == BF16) return launch_big<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, stream);
+        return launch_big<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, stream);
+    }
     return launch_gemm<128, 128, 64, 64>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, c_dtype, stream);
 }
 
