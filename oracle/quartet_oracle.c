@@ -98,7 +98,10 @@ void qo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out
  * Uniform for the element at flat offset o of the tensor being quantized (the role of
  * tl.rand(seed, offsets), mxfp4_triton.py:124).  One Philox call serves eight consecutive
  * elements: counter = (o/8 low, o/8 high, 0, 0), key = (seed low, seed high); element o takes
- * 16 bits: word (o%8)/2, low half for even o, high half for odd o; u = r16 * 2^-16.
+ * 16 bits r16: word (o%8)/2, high half for even o, low half for odd o.  The uniform is the
+ * largest float below (64*r16 + 1) * 2^-22, so that "u < p" holds exactly when
+ * p >= (64*r16 + 1) * 2^-22: a comparison at 22 fractional bits, which is what gfx950's
+ * stochastic-rounding convert evaluates; u is uniform on a 2^-16 grid (shifted by < 2^-22).
  */
 float qo_philox_uniform16(uint64_t seed, uint64_t o) {
     uint32_t ctr[4] = {(uint32_t)(o >> 3), (uint32_t)((o >> 3) >> 32), 0u, 0u};
@@ -106,8 +109,9 @@ float qo_philox_uniform16(uint64_t seed, uint64_t o) {
     uint32_t w[4];
     qo_philox4x32_10(ctr, key, w);
     uint32_t word = w[(o & 7) >> 1];
-    uint32_t r16 = (o & 1) ? (word >> 16) : (word & 0xffffu);
-    return (float)r16 * (1.0f / 65536.0f);
+    uint32_t r16 = (o & 1) ? (word & 0xffffu) : (word >> 16);
+    float bound = (float)(64u * r16 + 1u) * (1.0f / 4194304.0f); /* exact: 22 significant bits */
+    return bits_to_f32(f32_to_bits(bound) - 1u);
 }
 
 void qo_philox_uniform16_fill(uint64_t seed, int64_t n, float* u) {
@@ -226,7 +230,9 @@ static void quantize_group(const float* g, int mode, const float* u, uint8_t* co
     }
     for (int i = 0; i < 32; ++i) {
         float A = fabsf(t[i]);
-        int neg = !(t[i] > 0.0f);
+        /* sign = "not (t > 0)" (mxfp4_triton.py:65-69); t and g have the same sign, and taking it
+           from g keeps it defined when t underflows */
+        int neg = !(g[i] > 0.0f);
         int mag = sr ? sr_code(A, u[i]) : rtn_code(A);
         code[i] = (uint8_t)(mag | (neg << 3));
         keep[i] = (uint8_t)(A < 6.0f);

@@ -15,6 +15,11 @@ hipError_t quantize_mxfp4(const void* x, int dtype, int64_t rows, int64_t cols, 
                           bool transposed_in, const float* u, uint64_t seed, uint8_t* codes, uint8_t* scales,
                           uint8_t* maskbits, void* dequant, hipStream_t stream);
 
+// hd = 32 fast path (one MX group per lane, hardware FP4 converts); row-major input, RTN or Philox SR
+hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t n, uint32_t sign_word, int mode, uint64_t seed,
+                                  uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
+                                  hipStream_t stream);
+
 hipError_t requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C,
                                        float post, int val_dtype, int hd, const SignBits& sb, int mode, const float* u,
                                        uint64_t seed, uint8_t* codes_out, uint8_t* scales_out, void* dequant,

@@ -138,7 +138,7 @@ __device__ __forceinline__ void quantize_octet(const float (&g)[8], const float 
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         float A = fabsf(t[i]);
-        uint32_t neg = !(t[i] > 0.0f);
+        uint32_t neg = !(g[i] > 0.0f);  // sign of t, taken from g so that it survives underflow
         int mag;
         if constexpr (kSR) mag = sr_code(A, u[i]);
         else mag = rtn_code(A);
@@ -220,7 +220,7 @@ __device__ __forceinline__ void process_octet(float (&v)[8], int lane_in_chunk, 
         } else {
             Philox4 ph = philox_for_octet(seed, (uint64_t)octet);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) uu[i] = (float)philox_r16(ph, i) * (1.0f / 65536.0f);
+            for (int i = 0; i < 8; ++i) uu[i] = uniform_from_r16(philox_r16(ph, i));
         }
     }
     OctetResult r;
@@ -398,6 +398,10 @@ hipError_t quantize_mxfp4(const void* x, int dtype, int64_t rows, int64_t cols, 
                           bool transposed_in, const float* u, uint64_t seed, uint8_t* codes, uint8_t* scales,
                           uint8_t* maskbits, void* dequant, hipStream_t stream) {
     if (rows == 0 || cols == 0) return hipSuccess;
+    const bool rtn = (mode == QUEST_RTN || mode == ABSMAX_RTN);
+    const auto al = [](const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
+    if (hd == 32 && !transposed_in && (rtn || u == nullptr) && al(codes, 16) && al(maskbits, 4))
+        return quantize_rowmajor_hd32(x, dtype, rows * cols, sb.w[0], mode, seed, codes, scales, maskbits, dequant, stream);
     QuantOut out{reinterpret_cast<uint32_t*>(codes), scales, maskbits, dequant};
     const float c = hadamard_scale(hd, dtype);
     dispatch_hd(hd, [&](auto HDc) {

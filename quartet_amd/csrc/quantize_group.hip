@@ -1,0 +1,278 @@
+// Fast path of the fused block-Hadamard + MXFP4 quantizer for Hadamard block 32 (K1, "group layout").
+//
+// Same arithmetic as quantize.hip (the reference kernel
+// src/models/quantization/quantizers/mxfp4_triton.py:19-174), different work decomposition: one lane
+// owns a whole MX group of 32 values in registers, so
+//   - the five butterfly stages, the group statistics and the scale are computed without any
+//     cross-lane traffic and the per-group scalar work (sqrt, exponent extraction) is done once
+//     instead of once per quarter group;
+//   - the column sign of rotated element j is the same for every lane (j is a register index), so it
+//     folds into the multiply by hd^-1/2;
+//   - rounding, sign and nibble packing are done by gfx950's FP4 converts:
+//       RTN  v_cvt_scalef32_pk_fp4_f32 is round-to-nearest-even; the reference rounds ties toward
+//            zero, which differs exactly at .75, 1.75, 3.5.  Replacing the operand's bit pattern b by
+//            (b - 1) | 1 moves every tie just below itself and nothing else across a boundary.
+//       SR   v_cvt_scalef32_sr_pk_fp4_f32 rounds up iff floor(p * 2^22) + R >= 2^22 with p the position
+//            inside the bracket and R = bits 31..10 of the random operand for the pair's first element,
+//            bits 30..9 for its second (measured).  With R = 2^22 - 1 - 64 * r16 this is "u < p" for
+//            the uniform the Philox stream defines (qm_math.h), bit for bit.  Each element gets its
+//            own random word (two converts per pair, merged with one mask), so pairs are not correlated.
+//     The reference's sign rule "negative unless t > 0" makes +0 negative: adding -2^-149 first turns
+//     both zeros into a negative denormal and changes no other value's code.
+// Outputs are one 16-byte code store, one scale byte and one mask dword per lane, all contiguous across
+// lanes; the input is read as 64 (bf16) or 128 (fp32) contiguous bytes per lane.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "qm_kernels.h"
+#include "qm_math.h"
+
+namespace qm {
+
+namespace {
+
+typedef float v2f __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void butterfly32(float (&v)[32]) {
+#pragma unroll
+    for (int h = 1; h < 32; h <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            if (i & h) continue;
+            const float a = v[i], b = v[i + h];
+            v[i] = a + b;
+            v[i + h] = a - b;
+        }
+    }
+}
+
+// pairwise tree: adjacent pairs, then pairs of pairs, ... (the canonical order of the group sums)
+__device__ __forceinline__ float tree_sum32(const float (&p)[32]) {
+    float t[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) t[i] = p[2 * i] + p[2 * i + 1];
+#pragma unroll
+    for (int n = 8; n >= 1; n >>= 1)
+#pragma unroll
+        for (int i = 0; i < n; ++i) t[i] = t[2 * i] + t[2 * i + 1];
+    return t[0];
+}
+
+struct GroupCodes {
+    uint32_t w[4];        // 32 nibbles, element i in bits [4(i%8), +4) of word i/8
+    uint32_t scale_byte;  // E8M0
+    uint32_t keep;        // bit i = |t_i| < 6
+    float deq_scale;      // what a code value is multiplied by in the de-quantized tensor
+};
+
+#define kNegTiny (u2f(0x80000001u))  // -2^-149
+
+// v_cvt_scalef32_sr_pk_fp4_f32 replaces byte SEL of its destination and keeps the other three, but the
+// compiler builtin of this toolchain does not tie the destination to its `old` operand (the untouched bytes
+// come back as whatever the allocated register held), so the instruction is issued directly.
+template <int SEL>
+__device__ __forceinline__ void sr_convert_pair(uint32_t& dst, v2f pair, uint32_t rnd, float scale) {
+    if constexpr (SEL == 0) asm("v_cvt_scalef32_sr_pk_fp4_f32 %0, %1, %2, %3" : "+v"(dst) : "v"(pair), "v"(rnd), "v"(scale));
+    else if constexpr (SEL == 1) asm("v_cvt_scalef32_sr_pk_fp4_f32 %0, %1, %2, %3 op_sel:[0,0,1,0]" : "+v"(dst) : "v"(pair), "v"(rnd), "v"(scale));
+    else if constexpr (SEL == 2) asm("v_cvt_scalef32_sr_pk_fp4_f32 %0, %1, %2, %3 op_sel:[0,0,0,1]" : "+v"(dst) : "v"(pair), "v"(rnd), "v"(scale));
+    else asm("v_cvt_scalef32_sr_pk_fp4_f32 %0, %1, %2, %3 op_sel:[0,0,1,1]" : "+v"(dst) : "v"(pair), "v"(rnd), "v"(scale));
+}
+
+// ties-toward-zero via the round-to-nearest-even convert (see the file comment)
+__device__ __forceinline__ float tie_nudge(float v) {
+    return u2f(__builtin_elementwise_sub_sat(f2u(v), 1u) | 1u);
+}
+
+template <int MODE>
+__device__ __forceinline__ void quantize_group_regs(const float (&g)[32], uint64_t seed, int64_t group_index,
+                                                    GroupCodes& o) {
+    constexpr bool kQuest = (MODE == QUEST_RTN || MODE == QUEST_SR);
+    constexpr bool kSR = (MODE == ABSMAX_SR || MODE == QUEST_SR);
+    float hw_scale;   // power of two the convert divides by
+    uint32_t thr_bits;  // bit pattern of 6 * scale: |g| < thr  <=>  |t| < 6
+    float t[32];
+    bool all_zero = false;
+    if constexpr (kQuest) {
+        float sq[32];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) sq[i] = g[i] * g[i];
+        const float ms = tree_sum32(sq) * 0.03125f;
+        const float m = tree_sum32(g) * 0.03125f;
+        const float mm = m * m;
+        float var = ms - mm;
+        var = var > 0.0f ? var : 0.0f;
+        const float sd = __builtin_sqrtf(var);
+        const float gs = kQuestG * sd;
+        const float s = gs + 1e-8f;
+        int E = (int)((f2u(s) >> 23) & 0xffu) - 127;
+        E = E > 127 ? 127 : E;
+        o.scale_byte = (uint32_t)(E + 127);
+        hw_scale = pow2i(E);
+        o.deq_scale = hw_scale;
+        thr_bits = f2u(6.0f * hw_scale);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) t[i] = g[i];
+    } else {
+        float a = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) a = fmaxf(a, fabsf(g[i]));
+        all_zero = (a == 0.0f);
+        int k = (int)((f2u(a) >> 23) & 0xffu) - 129;
+        k = k < -127 ? -127 : (k > 127 ? 127 : k);
+        o.scale_byte = (uint32_t)(k + 127);
+        hw_scale = pow2i(k);
+        o.deq_scale = scale_pow2(kFourThirds, k);
+        // |t| < 6 with t = RN(g 2^-k / d): evaluated on the quotient h = RN(g / d) against 6 * 2^k
+        thr_bits = f2u(6.0f * hw_scale);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) t[i] = div_four_thirds(g[i]);
+    }
+    // clip mask, most significant element first so that element 0 lands in bit 0
+    uint32_t keep = 0u;
+#pragma unroll
+    for (int i = 31; i >= 0; --i) keep = (keep << 1) | (((f2u(t[i]) & 0x7fffffffu) < thr_bits) ? 1u : 0u);
+    o.keep = all_zero ? 0u : keep;
+
+    // the converts' byte selector must be a literal, hence the macros
+#define QM_RTN_PAIR(B)                                                                                   \
+    w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, tie_nudge(t[wi * 8 + 2 * (B)] + kNegTiny),           \
+                                                 tie_nudge(t[wi * 8 + 2 * (B) + 1] + kNegTiny), hw_scale, (B));
+#define QM_SR_PAIR(B)                                                                                    \
+    {                                                                                                    \
+        const uint32_t nw = ~ph.w[(B)];                                                                  \
+        const uint32_t r_even = nw | 0xffffu;           /* first element: bits 31..10, r16 = high half */  \
+        const uint32_t r_odd = (nw << 15) | 0x7fffu;    /* second element: bits 30..9, r16 = low half  */  \
+        const v2f pr = {t[wi * 8 + 2 * (B)] + kNegTiny, t[wi * 8 + 2 * (B) + 1] + kNegTiny};             \
+        sr_convert_pair<(B)>(even, pr, r_even, hw_scale);                                                \
+        sr_convert_pair<(B)>(odd, pr, r_odd, hw_scale);                                                  \
+    }
+    if constexpr (!kSR) {
+#pragma unroll
+        for (int wi = 0; wi < 4; ++wi) {
+            uint32_t w = 0u;
+            QM_RTN_PAIR(0) QM_RTN_PAIR(1) QM_RTN_PAIR(2) QM_RTN_PAIR(3)
+            o.w[wi] = w;
+        }
+    } else {
+#pragma unroll
+        for (int wi = 0; wi < 4; ++wi) {
+            const Philox4 ph = philox_for_octet(seed, (uint64_t)(group_index * 4 + wi));
+            uint32_t even = 0u, odd = 0u;  // converts driven by the even / odd element's random word
+            QM_SR_PAIR(0) QM_SR_PAIR(1) QM_SR_PAIR(2) QM_SR_PAIR(3)
+            o.w[wi] = (even & 0x0f0f0f0fu) | (odd & 0xf0f0f0f0u);
+        }
+    }
+#undef QM_RTN_PAIR
+#undef QM_SR_PAIR
+}
+
+template <typename T>
+__device__ __forceinline__ void load_group(const T* __restrict__ p, float (&v)[32]) {
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint4 raw = reinterpret_cast<const uint4*>(p)[q];
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[q * 8 + 2 * i] = u2f(w[i] << 16);
+                v[q * 8 + 2 * i + 1] = u2f(w[i] & 0xffff0000u);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const float4 f = reinterpret_cast<const float4*>(p)[q];
+            v[q * 4] = f.x; v[q * 4 + 1] = f.y; v[q * 4 + 2] = f.z; v[q * 4 + 3] = f.w;
+        }
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ void store_dequant(T* __restrict__ p, const GroupCodes& o) {
+    float v[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        const uint32_t nib = (o.w[i >> 3] >> (4 * (i & 7))) & 15u;
+        const float q = e2m1_value((int)(nib & 7u));
+        v[i] = ((nib & 8u) ? -q : q) * o.deq_scale;
+    }
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                w[i] = (uint32_t)f32_to_bf16(v[q * 8 + 2 * i]) | ((uint32_t)f32_to_bf16(v[q * 8 + 2 * i + 1]) << 16);
+            reinterpret_cast<uint4*>(p)[q] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+            reinterpret_cast<float4*>(p)[q] = make_float4(v[q * 4], v[q * 4 + 1], v[q * 4 + 2], v[q * 4 + 3]);
+    }
+}
+
+struct GroupOut {
+    uint4* codes;        // [n_groups]
+    uint8_t* scales;     // [n_groups]
+    uint32_t* maskbits;  // [n_groups] or null
+    void* dequant;       // [n_groups * 32] of T or null
+};
+
+// rotate (hd = 32) + quantize the group in v, write its outputs at group index gi
+template <typename T, int MODE>
+__device__ __forceinline__ void finish_group(float (&v)[32], int64_t gi, float c, uint32_t sign_word, uint64_t seed,
+                                             const GroupOut& out) {
+    butterfly32(v);
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+        const float cj = ((sign_word >> j) & 1u) ? -c : c;  // wave-uniform: folds into the multiply
+        v[j] = v[j] * cj;
+    }
+    GroupCodes o;
+    quantize_group_regs<MODE>(v, seed, gi, o);
+    out.codes[gi] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
+    out.scales[gi] = (uint8_t)o.scale_byte;
+    if (out.maskbits) out.maskbits[gi] = o.keep;
+    if (out.dequant) store_dequant<T>(reinterpret_cast<T*>(out.dequant) + gi * 32, o);
+}
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void quantize_rowmajor_g32_kernel(const T* __restrict__ x, int64_t n_groups, float c,
+                                                                    uint32_t sign_word, uint64_t seed, GroupOut out) {
+    const int64_t gi = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (gi >= n_groups) return;
+    float v[32];
+    load_group<T>(x + gi * 32, v);
+    finish_group<T, MODE>(v, gi, c, sign_word, seed, out);
+}
+
+template <typename T>
+void launch_rowmajor_g32(int mode, const void* x, int64_t n, float c, uint32_t sign_word, uint64_t seed,
+                         const GroupOut& out, hipStream_t stream) {
+    const int64_t n_groups = n / 32;
+    dim3 grid((unsigned)((n_groups + 255) / 256)), block(256);
+    const T* xp = reinterpret_cast<const T*>(x);
+    switch (mode) {
+        case QUEST_RTN: quantize_rowmajor_g32_kernel<T, QUEST_RTN><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
+        case ABSMAX_RTN: quantize_rowmajor_g32_kernel<T, ABSMAX_RTN><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
+        case ABSMAX_SR: quantize_rowmajor_g32_kernel<T, ABSMAX_SR><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
+        default: quantize_rowmajor_g32_kernel<T, QUEST_SR><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
+    }
+}
+
+}  // namespace
+
+// hd = 32, row-major input, RTN or Philox-driven SR (explicit uniforms take the generic path)
+hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t n, uint32_t sign_word, int mode, uint64_t seed,
+                                  uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
+                                  hipStream_t stream) {
+    GroupOut out{reinterpret_cast<uint4*>(codes), scales, reinterpret_cast<uint32_t*>(maskbits), dequant};
+    const float c = hadamard_scale(32, dtype);
+    if (dtype == BF16) launch_rowmajor_g32<uint16_t>(mode, x, n, c, sign_word, seed, out, stream);
+    else launch_rowmajor_g32<float>(mode, x, n, c, sign_word, seed, out, stream);
+    return hipGetLastError();
+}
+
+}  // namespace qm

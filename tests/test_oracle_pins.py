@@ -147,16 +147,27 @@ def test_philox_known_answer_vectors(oracle):
 
 
 def test_philox_uniform16_mapping(oracle):
+    # u(r16) = largest float below (64*r16 + 1) / 2^22, r16 = 16-bit slices of Philox words
     seed = 0x1234_5678_9ABC
     u = oracle.philox_uniform16(seed, 64)
     for blk in range(8):
         w = oracle.philox4x32_10([blk, 0, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
         want = []
         for word in w.tolist():
-            want += [(word & 0xFFFF) / 65536.0, (word >> 16) / 65536.0]
+            for r16 in (word >> 16, word & 0xFFFF):  # even element: high half, odd element: low half
+                bound = np.float32((64 * r16 + 1) / 4194304.0)
+                assert float(bound) == (64 * r16 + 1) / 4194304.0  # exactly representable
+                want.append(float(np.nextafter(bound, np.float32(0))))
         assert u[8 * blk:8 * blk + 8].tolist() == want
     big = oracle.philox_uniform16(7, 1 << 16)
     assert 0 <= big.min() and big.max() < 1 and abs(big.mean() - 0.5) < 5e-3
+    # "u < p" is the 22-bit comparison "floor(p * 2^22) > 64 * r16" for every float p in [0, 1]
+    rng = np.random.default_rng(0)
+    r16 = rng.integers(0, 65536, 20000)
+    bound = ((64 * r16 + 1) / 4194304.0).astype(np.float32)
+    uu = np.nextafter(bound, np.float32(0))
+    p = np.concatenate([rng.random(10000, dtype=np.float32), bound[:5000], uu[:2500], np.nextafter(bound[:2500], np.float32(2))])
+    assert np.array_equal(uu < p, np.floor(p.astype(np.float64) * 4194304.0) > 64 * r16)
 
 
 # ---- scales, codes, mask, packing ---------------------------------------------------------------
