@@ -20,6 +20,12 @@ hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t n, uint32_t 
                                   uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
                                   hipStream_t stream);
 
+hipError_t quantize_transposed_hd32(const void* x, int dtype, int64_t P, int64_t Q, uint32_t sign_word, int mode,
+                                    uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant, hipStream_t stream);
+hipError_t requantize_transposed_hd32(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C, float post,
+                                      int val_dtype, uint32_t sign_word, int mode, uint64_t seed, uint8_t* codes,
+                                      uint8_t* scales, void* dequant, hipStream_t stream);
+
 hipError_t requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C,
                                        float post, int val_dtype, int hd, const SignBits& sb, int mode, const float* u,
                                        uint64_t seed, uint8_t* codes_out, uint8_t* scales_out, void* dequant,

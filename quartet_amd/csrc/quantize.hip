@@ -218,9 +218,10 @@ __device__ __forceinline__ void process_octet(float (&v)[8], int lane_in_chunk, 
         if (u != nullptr) {
             load_octet<float>(u + octet * 8, uu);
         } else {
-            Philox4 ph = philox_for_octet(seed, (uint64_t)octet);
+            // sixteen elements share one Philox call: the two octets of a pair compute it twice
+            Philox4 ph = philox_for_hexadecad(seed, (uint64_t)(octet >> 1));
 #pragma unroll
-            for (int i = 0; i < 8; ++i) uu[i] = uniform_from_r16(philox_r16(ph, i));
+            for (int i = 0; i < 8; ++i) uu[i] = uniform_from_r8(philox_r8(ph, (int)(octet & 1) * 8 + i));
         }
     }
     OctetResult r;
@@ -402,6 +403,10 @@ hipError_t quantize_mxfp4(const void* x, int dtype, int64_t rows, int64_t cols, 
     const auto al = [](const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
     if (hd == 32 && !transposed_in && (rtn || u == nullptr) && al(codes, 16) && al(maskbits, 4))
         return quantize_rowmajor_hd32(x, dtype, rows * cols, sb.w[0], mode, seed, codes, scales, maskbits, dequant, stream);
+    // logical [rows, cols] = physical [P = cols, Q = rows]
+    if (hd == 32 && transposed_in && (rtn || u == nullptr) && maskbits == nullptr && al(codes, 16) && al(scales, 4) &&
+        cols % 128 == 0)
+        return quantize_transposed_hd32(x, dtype, cols, rows, sb.w[0], mode, seed, codes, scales, dequant, stream);
     QuantOut out{reinterpret_cast<uint32_t*>(codes), scales, maskbits, dequant};
     const float c = hadamard_scale(hd, dtype);
     dispatch_hd(hd, [&](auto HDc) {
@@ -423,6 +428,11 @@ hipError_t requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* s
                                        uint64_t seed, uint8_t* codes_out, uint8_t* scales_out, void* dequant,
                                        hipStream_t stream) {
     if (R == 0 || C == 0) return hipSuccess;
+    const bool rtn = (mode == QUEST_RTN || mode == ABSMAX_RTN);
+    const auto al = [](const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
+    if (hd == 32 && (rtn || u == nullptr) && al(codes_out, 16) && al(scales_out, 4) && R % 128 == 0)
+        return requantize_transposed_hd32(codes_in, scales_in, R, C, post, val_dtype, sb.w[0], mode, seed, codes_out,
+                                          scales_out, dequant, stream);
     QuantOut out{reinterpret_cast<uint32_t*>(codes_out), scales_out, nullptr, dequant};
     const float c = hadamard_scale(hd, val_dtype);
     dispatch_hd(hd, [&](auto HDc) {

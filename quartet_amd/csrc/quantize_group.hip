@@ -14,15 +14,17 @@
 //            (b - 1) | 1 moves every tie just below itself and nothing else across a boundary.
 //       SR   v_cvt_scalef32_sr_pk_fp4_f32 rounds up iff floor(p * 2^22) + R >= 2^22 with p the position
 //            inside the bracket and R = bits 31..10 of the random operand for the pair's first element,
-//            bits 30..9 for its second (measured).  With R = 2^22 - 1 - 64 * r16 this is "u < p" for
+//            bits 30..9 for its second (measured).  With R = 2^22 - 1 - r8 2^14 - 2^13 this is "u < p" for
 //            the uniform the Philox stream defines (qm_math.h), bit for bit.  Each element gets its
-//            own random word (two converts per pair, merged with one mask), so pairs are not correlated.
+//            own random byte (two converts per pair, merged with one mask), so pairs are not correlated.
 //     The reference's sign rule "negative unless t > 0" makes +0 negative: adding -2^-149 first turns
 //     both zeros into a negative denormal and changes no other value's code.
 // Outputs are one 16-byte code store, one scale byte and one mask dword per lane, all contiguous across
 // lanes; the input is read as 64 (bf16) or 128 (fp32) contiguous bytes per lane.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "qm_kernels.h"
 #include "qm_math.h"
@@ -137,14 +139,18 @@ __device__ __forceinline__ void quantize_group_regs(const float (&g)[32], uint64
 #define QM_RTN_PAIR(B)                                                                                   \
     w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, tie_nudge(t[wi * 8 + 2 * (B)] + kNegTiny),           \
                                                  tie_nudge(t[wi * 8 + 2 * (B) + 1] + kNegTiny), hw_scale, (B));
-#define QM_SR_PAIR(B)                                                                                    \
-    {                                                                                                    \
-        const uint32_t nw = ~ph.w[(B)];                                                                  \
-        const uint32_t r_even = nw | 0xffffu;           /* first element: bits 31..10, r16 = high half */  \
-        const uint32_t r_odd = (nw << 15) | 0x7fffu;    /* second element: bits 30..9, r16 = low half  */  \
-        const v2f pr = {t[wi * 8 + 2 * (B)] + kNegTiny, t[wi * 8 + 2 * (B) + 1] + kNegTiny};             \
-        sr_convert_pair<(B)>(even, pr, r_even, hw_scale);                                                \
-        sr_convert_pair<(B)>(odd, pr, r_odd, hw_scale);                                                  \
+    // element j of a Philox call (16 elements): byte j%4 of word j/4.  r for the pair's first element carries
+    // ~r8 in bits 31..24 above the constant 0x7fffff (R = 2^22 - 1 - r8 2^14 - 2^13 in bits 31..10); the second
+    // element reads bits 30..9, i.e. the same pattern shifted right by one.  v_perm_b32 builds the pattern:
+    // selector bytes pick {~word byte, 0x7f, 0xff, 0xff}.
+#define QM_SR_PAIR(B, J0)                                                                                 \
+    {                                                                                                     \
+        const uint32_t nw = ~ph.w[(J0) >> 2];                                                             \
+        const uint32_t r_even = __builtin_amdgcn_perm(nw, 0x7f7f7f7fu, 0x0000ffffu | ((4u + ((J0) & 3)) << 24));                \
+        const uint32_t r_odd = __builtin_amdgcn_perm(nw, 0x7f7f7f7fu, 0x0000ffffu | ((4u + (((J0) + 1) & 3)) << 24)) >> 1;  \
+        const v2f pr = {t[wi * 8 + 2 * (B)] + kNegTiny, t[wi * 8 + 2 * (B) + 1] + kNegTiny};              \
+        sr_convert_pair<(B)>(even, pr, r_even, hw_scale);                                                 \
+        sr_convert_pair<(B)>(odd, pr, r_odd, hw_scale);                                                   \
     }
     if constexpr (!kSR) {
 #pragma unroll
@@ -154,11 +160,14 @@ __device__ __forceinline__ void quantize_group_regs(const float (&g)[32], uint64
             o.w[wi] = w;
         }
     } else {
+        Philox4 ph;
 #pragma unroll
         for (int wi = 0; wi < 4; ++wi) {
-            const Philox4 ph = philox_for_octet(seed, (uint64_t)(group_index * 4 + wi));
-            uint32_t even = 0u, odd = 0u;  // converts driven by the even / odd element's random word
-            QM_SR_PAIR(0) QM_SR_PAIR(1) QM_SR_PAIR(2) QM_SR_PAIR(3)
+            // words 0,1 of the call serve the even octet of the pair, words 2,3 the odd one
+            if ((wi & 1) == 0) ph = philox_for_hexadecad(seed, (uint64_t)(group_index * 2 + (wi >> 1)));
+            uint32_t even = 0u, odd = 0u;  // converts driven by the even / odd element's random byte
+            if ((wi & 1) == 0) { QM_SR_PAIR(0, 0) QM_SR_PAIR(1, 2) QM_SR_PAIR(2, 4) QM_SR_PAIR(3, 6) }
+            else { QM_SR_PAIR(0, 8) QM_SR_PAIR(1, 10) QM_SR_PAIR(2, 12) QM_SR_PAIR(3, 14) }
             o.w[wi] = (even & 0x0f0f0f0fu) | (odd & 0xf0f0f0f0u);
         }
     }
@@ -220,16 +229,21 @@ struct GroupOut {
     void* dequant;       // [n_groups * 32] of T or null
 };
 
+// x @ H for one chunk of 32: butterfly, then hd^-1/2 with the column sign folded in (wave-uniform)
+__device__ __forceinline__ void rotate_group(float (&v)[32], float c, uint32_t sign_word) {
+    butterfly32(v);
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+        const float cj = ((sign_word >> j) & 1u) ? -c : c;
+        v[j] = v[j] * cj;
+    }
+}
+
 // rotate (hd = 32) + quantize the group in v, write its outputs at group index gi
 template <typename T, int MODE>
 __device__ __forceinline__ void finish_group(float (&v)[32], int64_t gi, float c, uint32_t sign_word, uint64_t seed,
                                              const GroupOut& out) {
-    butterfly32(v);
-#pragma unroll
-    for (int j = 0; j < 32; ++j) {
-        const float cj = ((sign_word >> j) & 1u) ? -c : c;  // wave-uniform: folds into the multiply
-        v[j] = v[j] * cj;
-    }
+    rotate_group(v, c, sign_word);
     GroupCodes o;
     quantize_group_regs<MODE>(v, seed, gi, o);
     out.codes[gi] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
@@ -262,6 +276,245 @@ void launch_rowmajor_g32(int mode, const void* x, int64_t n, float c, uint32_t s
     }
 }
 
+// ---- transposed input: x is [P, Q] row-major, output is the [Q, P] tensor quantized along P ----------
+// Tile = 128 p x TQ q staged in LDS exactly as it lies in memory (rows of 256 bytes).  Wave w then owns
+// p-group w of the tile; a lane reads its column (bf16: two adjacent columns per 32-bit read) at 32
+// successive rows, so every LDS read of a wave is one full 256-byte row: conflict free.  Codes and scales go
+// back through LDS so that each q row leaves as one contiguous 64-byte (codes) / 4-byte (scales) piece.
+template <typename T>
+struct TrTile {
+    static constexpr int kQ = 256 / (int)sizeof(T);      // 128 columns of bf16, 64 of fp32
+    static constexpr int kGroupsPerLane = kQ / 64;       // 2 for bf16, 1 for fp32
+};
+constexpr int kTrP = 128;
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void quantize_transposed_g32_kernel(const T* __restrict__ x, int64_t P, int64_t Q,
+                                                                      float c, uint32_t sign_word, uint64_t seed,
+                                                                      uint8_t* __restrict__ codes,
+                                                                      uint8_t* __restrict__ scales,
+                                                                      void* __restrict__ dequant) {
+    constexpr int TQ = TrTile<T>::kQ;
+    constexpr int GPL = TrTile<T>::kGroupsPerLane;
+    __shared__ uint4 tile4[kTrP * 16];  // 128 rows x 256 bytes
+    uint32_t* tile = reinterpret_cast<uint32_t*>(tile4);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t p0 = (int64_t)blockIdx.x * kTrP, q0 = (int64_t)blockIdx.y * TQ;
+    constexpr int kVec = 16 / (int)sizeof(T);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int idx = tid + j * 256, row = idx >> 4, cv = idx & 15;
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (p0 + row < P && q0 + cv * kVec < Q)
+            raw = *reinterpret_cast<const uint4*>(x + (p0 + row) * Q + q0 + cv * kVec);
+        tile4[idx] = raw;
+    }
+    __syncthreads();
+    const int64_t pbase = p0 + wave * 32;       // this wave's group along p
+    const int64_t qa = q0 + lane * GPL;         // this lane's first column
+    const bool active = pbase < P && qa < Q;    // P % 32 == 0 and Q % 8 == 0: all of a lane's groups or none
+    GroupCodes res[GPL];
+    if (active) {
+        float v[GPL][32];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const uint32_t w = tile[(wave * 32 + i) * 64 + lane];
+            if constexpr (sizeof(T) == 2) {
+                v[0][i] = u2f(w << 16);
+                v[1][i] = u2f(w & 0xffff0000u);
+            } else {
+                v[0][i] = u2f(w);
+            }
+        }
+#pragma unroll
+        for (int gq = 0; gq < GPL; ++gq) {
+            const int64_t gi = (qa + gq) * (P / 32) + pbase / 32;
+            rotate_group(v[gq], c, sign_word);
+            quantize_group_regs<MODE>(v[gq], seed, gi, res[gq]);
+            if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res[gq]);
+        }
+    }
+    __syncthreads();  // every wave is done reading the input tile: reuse it as the output stage
+    // stage: codes [TQ][4 groups x 16 B], then scales [TQ][4 B]
+    uint4* ocodes = tile4;
+    uint8_t* oscales = reinterpret_cast<uint8_t*>(tile4 + TQ * 4);
+    if (active) {
+#pragma unroll
+        for (int gq = 0; gq < GPL; ++gq) {
+            ocodes[(lane * GPL + gq) * 4 + wave] = make_uint4(res[gq].w[0], res[gq].w[1], res[gq].w[2], res[gq].w[3]);
+            oscales[(lane * GPL + gq) * 4 + wave] = (uint8_t)res[gq].scale_byte;
+        }
+    }
+    __syncthreads();
+    const int64_t code_pitch = P / 2, scale_pitch = P / 32;
+    for (int idx = tid; idx < TQ * 4; idx += 256) {
+        const int ql = idx >> 2, part = idx & 3;
+        if (q0 + ql < Q && p0 + part * 32 < P)
+            *reinterpret_cast<uint4*>(codes + (q0 + ql) * code_pitch + p0 / 2 + part * 16) = ocodes[idx];
+    }
+    if (tid < TQ && q0 + tid < Q) {
+        const uint32_t sw = reinterpret_cast<const uint32_t*>(oscales)[tid];
+        uint8_t* dst = scales + (q0 + tid) * scale_pitch + p0 / 32;
+        if (p0 + kTrP <= P) {
+            *reinterpret_cast<uint32_t*>(dst) = sw;
+        } else {
+            for (int b = 0; b < 4; ++b)
+                if (p0 + b * 32 < P) dst[b] = (uint8_t)(sw >> (8 * b));
+        }
+    }
+}
+
+// ---- packed MXFP4 in, transposed + rotated + re-quantized out --------------------------------------------
+// in: codes [R, C/2], scales [R, C/32]; out: the [C, R] tensor quantized along R.  Tile = 128 r x 256 c
+// (rows of 128 code bytes + 8 scale bytes).  Wave w owns r-group w; a lane handles one byte column = two
+// adjacent c, 32 rows deep; the hardware FP4 de-quantizing convert turns each byte into two floats.
+constexpr int kRqR = 128, kRqC = 256;
+
+template <int VAL_DTYPE, int MODE>
+__global__ __launch_bounds__(256) void requantize_transposed_g32_kernel(const uint8_t* __restrict__ codes_in,
+                                                                        const uint8_t* __restrict__ scales_in,
+                                                                        int64_t R, int64_t C, float post, float c,
+                                                                        uint32_t sign_word, uint64_t seed,
+                                                                        uint8_t* __restrict__ codes,
+                                                                        uint8_t* __restrict__ scales,
+                                                                        void* __restrict__ dequant) {
+    using T = typename std::conditional<VAL_DTYPE == BF16, uint16_t, float>::type;
+    __shared__ uint4 ctile4[kRqR * 8];   // 128 rows x 128 bytes of codes; later the output stage (16 KiB)
+    __shared__ uint2 stile2[kRqR];       // 8 scale bytes per row
+    const uint8_t* ctile = reinterpret_cast<const uint8_t*>(ctile4);
+    const uint8_t* stile = reinterpret_cast<const uint8_t*>(stile2);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t r0 = (int64_t)blockIdx.x * kRqR, c0 = (int64_t)blockIdx.y * kRqC;
+    const int64_t in_code_pitch = C / 2, in_scale_pitch = C / 32;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int idx = tid + j * 256, row = idx >> 3, cv = idx & 7;
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (r0 + row < R && c0 + cv * 32 < C)
+            raw = *reinterpret_cast<const uint4*>(codes_in + (r0 + row) * in_code_pitch + c0 / 2 + cv * 16);
+        ctile4[idx] = raw;
+    }
+    if (tid < kRqR) {
+        uint2 s = make_uint2(0, 0);
+        if (r0 + tid < R) {
+            const uint8_t* sp = scales_in + (r0 + tid) * in_scale_pitch + c0 / 32;
+            if (c0 + kRqC <= C && (in_scale_pitch & 7) == 0) {
+                s = *reinterpret_cast<const uint2*>(sp);
+            } else {
+                uint32_t lo = 0, hi = 0;
+                for (int b = 0; b < 8; ++b)
+                    if (c0 + b * 32 < C) (b < 4 ? lo : hi) |= (uint32_t)sp[b] << (8 * (b & 3));
+                s = make_uint2(lo, hi);
+            }
+        }
+        stile2[tid] = s;
+    }
+    __syncthreads();
+    const int64_t rbase = r0 + wave * 32;
+    GroupCodes res[2][2];  // [pass][column of the pair]
+    bool active[2];
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int bcol = pass * 64 + lane;           // byte column within the tile: c = c0 + 2*bcol, +1
+        const int64_t ca = c0 + 2 * bcol;
+        active[pass] = rbase < R && ca < C;          // C % 32 == 0: both columns of the pair or none
+        if (!active[pass]) continue;
+        float v[2][32];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const int row = wave * 32 + i;
+            const uint32_t byte = ctile[row * 128 + bcol];
+            const uint32_t sbyte = stile[row * 8 + (bcol >> 4)];
+            const v2f pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(byte, u2f(sbyte << 23), 0);
+            float a = pr.x, b = pr.y;
+            if (post != 1.0f) {  // absmax-coded input: value = code * 2^k * post, held in val_dtype
+                a *= post;
+                b *= post;
+                if constexpr (VAL_DTYPE == BF16) {
+                    a = bf16_to_f32(f32_to_bf16(a));
+                    b = bf16_to_f32(f32_to_bf16(b));
+                }
+            }
+            v[0][i] = a;
+            v[1][i] = b;
+        }
+#pragma unroll
+        for (int gq = 0; gq < 2; ++gq) {
+            const int64_t gi = (ca + gq) * (R / 32) + rbase / 32;
+            rotate_group(v[gq], c, sign_word);
+            quantize_group_regs<MODE>(v[gq], seed, gi, res[pass][gq]);
+            if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res[pass][gq]);
+        }
+    }
+    __syncthreads();
+    // output stage: codes [256 c][4 groups x 16 B] = 16 KiB over the code tile, scales [256 c][4 B] over ... a
+    // second pass: the scale tile is only 1 KiB, so scales are staged after the codes have been written out
+    uint4* ocodes = ctile4;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        if (!active[pass]) continue;
+#pragma unroll
+        for (int gq = 0; gq < 2; ++gq) {
+            const int cl = 2 * (pass * 64 + lane) + gq;
+            const GroupCodes& g = res[pass][gq];
+            ocodes[cl * 4 + wave] = make_uint4(g.w[0], g.w[1], g.w[2], g.w[3]);
+        }
+    }
+    __syncthreads();
+    const int64_t code_pitch = R / 2, scale_pitch = R / 32;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int idx = tid + j * 256, cl = idx >> 2, part = idx & 3;
+        if (c0 + cl < C && r0 + part * 32 < R)
+            *reinterpret_cast<uint4*>(codes + (c0 + cl) * code_pitch + r0 / 2 + part * 16) = ocodes[idx];
+    }
+    __syncthreads();
+    uint8_t* oscales = reinterpret_cast<uint8_t*>(ctile4);
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        if (!active[pass]) continue;
+#pragma unroll
+        for (int gq = 0; gq < 2; ++gq) oscales[(2 * (pass * 64 + lane) + gq) * 4 + wave] = (uint8_t)res[pass][gq].scale_byte;
+    }
+    __syncthreads();
+    if (c0 + tid < C) {
+        const uint32_t sw = reinterpret_cast<const uint32_t*>(oscales)[tid];
+        uint8_t* dst = scales + (c0 + tid) * scale_pitch + r0 / 32;
+        if (r0 + kRqR <= R) {
+            *reinterpret_cast<uint32_t*>(dst) = sw;
+        } else {
+            for (int b = 0; b < 4; ++b)
+                if (r0 + b * 32 < R) dst[b] = (uint8_t)(sw >> (8 * b));
+        }
+    }
+}
+
+template <typename T>
+void launch_transposed_g32(int mode, const void* x, int64_t P, int64_t Q, float c, uint32_t sign_word, uint64_t seed,
+                           uint8_t* codes, uint8_t* scales, void* dequant, hipStream_t stream) {
+    dim3 grid((unsigned)((P + kTrP - 1) / kTrP), (unsigned)((Q + TrTile<T>::kQ - 1) / TrTile<T>::kQ)), block(256);
+    const T* xp = reinterpret_cast<const T*>(x);
+    switch (mode) {
+        case QUEST_RTN: quantize_transposed_g32_kernel<T, QUEST_RTN><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant); break;
+        case ABSMAX_RTN: quantize_transposed_g32_kernel<T, ABSMAX_RTN><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant); break;
+        case ABSMAX_SR: quantize_transposed_g32_kernel<T, ABSMAX_SR><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant); break;
+        default: quantize_transposed_g32_kernel<T, QUEST_SR><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant); break;
+    }
+}
+
+template <int VAL_DTYPE>
+void launch_requant_g32(int mode, const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C, float post,
+                        float c, uint32_t sign_word, uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant,
+                        hipStream_t stream) {
+    dim3 grid((unsigned)((R + kRqR - 1) / kRqR), (unsigned)((C + kRqC - 1) / kRqC)), block(256);
+    switch (mode) {
+        case QUEST_RTN: requantize_transposed_g32_kernel<VAL_DTYPE, QUEST_RTN><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant); break;
+        case ABSMAX_RTN: requantize_transposed_g32_kernel<VAL_DTYPE, ABSMAX_RTN><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant); break;
+        case ABSMAX_SR: requantize_transposed_g32_kernel<VAL_DTYPE, ABSMAX_SR><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant); break;
+        default: requantize_transposed_g32_kernel<VAL_DTYPE, QUEST_SR><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant); break;
+    }
+}
+
 }  // namespace
 
 // hd = 32, row-major input, RTN or Philox-driven SR (explicit uniforms take the generic path)
@@ -272,6 +525,24 @@ hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t n, uint32_t 
     const float c = hadamard_scale(32, dtype);
     if (dtype == BF16) launch_rowmajor_g32<uint16_t>(mode, x, n, c, sign_word, seed, out, stream);
     else launch_rowmajor_g32<float>(mode, x, n, c, sign_word, seed, out, stream);
+    return hipGetLastError();
+}
+
+// hd = 32, x is [P, Q] row-major and the output is its transpose quantized along P; no clip mask
+hipError_t quantize_transposed_hd32(const void* x, int dtype, int64_t P, int64_t Q, uint32_t sign_word, int mode,
+                                    uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant, hipStream_t stream) {
+    const float c = hadamard_scale(32, dtype);
+    if (dtype == BF16) launch_transposed_g32<uint16_t>(mode, x, P, Q, c, sign_word, seed, codes, scales, dequant, stream);
+    else launch_transposed_g32<float>(mode, x, P, Q, c, sign_word, seed, codes, scales, dequant, stream);
+    return hipGetLastError();
+}
+
+hipError_t requantize_transposed_hd32(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C, float post,
+                                      int val_dtype, uint32_t sign_word, int mode, uint64_t seed, uint8_t* codes,
+                                      uint8_t* scales, void* dequant, hipStream_t stream) {
+    const float c = hadamard_scale(32, val_dtype);
+    if (val_dtype == BF16) launch_requant_g32<BF16>(mode, codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, stream);
+    else launch_requant_g32<F32>(mode, codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, stream);
     return hipGetLastError();
 }
 

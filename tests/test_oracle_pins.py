@@ -147,27 +147,32 @@ def test_philox_known_answer_vectors(oracle):
 
 
 def test_philox_uniform16_mapping(oracle):
-    # u(r16) = largest float below (64*r16 + 1) / 2^22, r16 = 16-bit slices of Philox words
+    # u(r8) = largest float below (r8 * 2^14 + 2^13 + 1) / 2^22, r8 = bytes of Philox words, 16 elements per call
     seed = 0x1234_5678_9ABC
     u = oracle.philox_uniform16(seed, 64)
-    for blk in range(8):
+    for blk in range(4):
         w = oracle.philox4x32_10([blk, 0, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
         want = []
         for word in w.tolist():
-            for r16 in (word >> 16, word & 0xFFFF):  # even element: high half, odd element: low half
-                bound = np.float32((64 * r16 + 1) / 4194304.0)
-                assert float(bound) == (64 * r16 + 1) / 4194304.0  # exactly representable
+            for b in range(4):
+                r8 = (word >> (8 * b)) & 0xFF
+                bound = np.float32((16384 * r8 + 8193) / 4194304.0)
+                assert float(bound) == (16384 * r8 + 8193) / 4194304.0  # exactly representable
                 want.append(float(np.nextafter(bound, np.float32(0))))
-        assert u[8 * blk:8 * blk + 8].tolist() == want
+        assert u[16 * blk:16 * blk + 16].tolist() == want
     big = oracle.philox_uniform16(7, 1 << 16)
     assert 0 <= big.min() and big.max() < 1 and abs(big.mean() - 0.5) < 5e-3
-    # "u < p" is the 22-bit comparison "floor(p * 2^22) > 64 * r16" for every float p in [0, 1]
+    # "u < p" is the 22-bit comparison "floor(p * 2^22) > r8 * 2^14 + 2^13" for every float p in [0, 1]
     rng = np.random.default_rng(0)
-    r16 = rng.integers(0, 65536, 20000)
-    bound = ((64 * r16 + 1) / 4194304.0).astype(np.float32)
+    r8 = rng.integers(0, 256, 20000)
+    bound = ((16384 * r8 + 8193) / 4194304.0).astype(np.float32)
     uu = np.nextafter(bound, np.float32(0))
     p = np.concatenate([rng.random(10000, dtype=np.float32), bound[:5000], uu[:2500], np.nextafter(bound[:2500], np.float32(2))])
-    assert np.array_equal(uu < p, np.floor(p.astype(np.float64) * 4194304.0) > 64 * r16)
+    assert np.array_equal(uu < p, np.floor(p.astype(np.float64) * 4194304.0) > 16384 * r8 + 8192)
+    # centred bins: averaged over r8 the round-up probability of p is p to within 2^-9
+    for pv in (0.1, 0.37, 0.5, 0.93):
+        allu = np.nextafter(((16384 * np.arange(256) + 8193) / 4194304.0).astype(np.float32), np.float32(0))
+        assert abs(np.mean(allu < np.float32(pv)) - pv) <= 1 / 512 + 1e-9
 
 
 # ---- scales, codes, mask, packing ---------------------------------------------------------------
