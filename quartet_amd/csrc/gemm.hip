@@ -284,6 +284,10 @@ struct BigLoadPlan {
 __device__ __forceinline__ void load_lds_b128(const uint8_t* gsrc, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gsrc), "s"(lds_base));
 }
+// same, addressed as uniform 64-bit base (SGPR pair) + per-lane 32-bit byte offset: no 64-bit VGPR address math
+__device__ __forceinline__ void load_lds_b128_s(const uint8_t* base, uint32_t lane_off, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(lds_base));
+}
 __device__ __forceinline__ void load_lds_b32(const uint8_t* gsrc, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gsrc), "s"(lds_base));
 }
@@ -297,10 +301,8 @@ __device__ __forceinline__ void big_issue_loads(const BigLoadPlan& p, int stage,
         load_lds_b128(p.a + j * p.row16_bytes + kb, base + j * 1024);
         load_lds_b128(p.b + j * p.row16_bytes + kb, base + kBOff + j * 1024);
     }
-#ifndef QM_DBG_NO_SCALES
     load_lds_b32(p.sa + ks * 4, p.lds_scales + stage * kStageBytes);
     load_lds_b32(p.sb + ks * 4, p.lds_scales + stage * kStageBytes + (kSBOff - kSAOff));
-#endif
 }
 
 struct SubFrags {
@@ -324,7 +326,10 @@ __device__ __forceinline__ void big_read_scales(const uint8_t* __restrict__ stag
     sb4 = *reinterpret_cast<const uint4*>(stage + kSBOff + b_off);
 }
 
-template <int SUB>
+// SWAP = false: A rows become result rows.  SWAP = true: B's rows (n) are fed as the MFMA's first operand and
+// A's rows (m) as its second, so a lane ends up with 4 consecutive n of one m (contiguous in row-major C),
+// which the bf16 epilogue packs into 8-byte LDS writes.
+template <int SUB, bool SWAP>
 __device__ __forceinline__ void big_mfma_sub(const SubFrags& f, const uint32_t (&sca)[4], const uint32_t (&scb)[4],
                                              v16f (&acc)[4][4]) {
 #pragma unroll
@@ -333,7 +338,53 @@ __device__ __forceinline__ void big_mfma_sub(const SubFrags& f, const uint32_t (
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const v8i bv = v8i{(int)f.b[j].x, (int)f.b[j].y, (int)f.b[j].z, (int)f.b[j].w, 0, 0, 0, 0};
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[i][j], 4, 4, SUB, (int)sca[i], SUB, (int)scb[j]);
+            if constexpr (SWAP)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, acc[i][j], 4, 4, SUB, (int)scb[j], SUB, (int)sca[i]);
+            else
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[i][j], 4, 4, SUB, (int)sca[i], SUB, (int)scb[j]);
+        }
+    }
+}
+
+// Epilogue of the 256x256 kernels.  fp32: direct stores (acc element e of tile (i,j) is row 8*(e/4)+4*half+e%4,
+// column lane%32).  bf16 (SWAP layout: element e is n = 8*(e/4)+4*half+e%4 of m = lane%32): each wave packs its
+// 128x128 block into its own LDS region (rows of 256 bytes, pitch 272 so the 8-byte writes of 32 consecutive
+// rows spread over the banks), then writes it out as 16-byte pieces, four full 256-byte row segments per
+// instruction.  The LDS used is the operand ring, free once every wave has passed the final barrier.
+constexpr int kEpiPitch = 272;
+template <typename OutT>
+__device__ __forceinline__ void big_epilogue(v16f (&acc)[4][4], float alpha, OutT* __restrict__ c, int64_t m0, int64_t n0,
+                                             int64_t N, int wm, int wn, int wave, int lane, uint8_t* smem_bytes) {
+    const int lrow = lane & 31, half = lane >> 5;
+    if constexpr (sizeof(OutT) == 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                store_tile<OutT>(acc[i][j], alpha, c, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
+    } else {
+        uint8_t* region = smem_bytes + wave * (128 * kEpiPitch);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const v16f& t = acc[i][j];
+                    const v2bf p0 = __builtin_convertvector(v2f{t[4 * b] * alpha, t[4 * b + 1] * alpha}, v2bf);
+                    const v2bf p1 = __builtin_convertvector(v2f{t[4 * b + 2] * alpha, t[4 * b + 3] * alpha}, v2bf);
+                    *reinterpret_cast<uint2*>(region + (i * 32 + lrow) * kEpiPitch + (j * 32 + 8 * b + 4 * half) * 2) =
+                        make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
+                }
+        // the region is private to the wave: its own writes are ordered before its own reads
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+        const int chunk = lane & 15, rsub = lane >> 4;
+        uint8_t* cbase = reinterpret_cast<uint8_t*>(c + (m0 + wm * 128) * N + n0 + wn * 128) + chunk * 16;
+#pragma unroll 8
+        for (int r4 = 0; r4 < 32; ++r4) {
+            const int row = r4 * 4 + rsub;
+            const uint4 v = *reinterpret_cast<const uint4*>(region + row * kEpiPitch + chunk * 16);
+            *reinterpret_cast<uint4*>(cbase + (int64_t)row * N * 2) = v;
         }
     }
 }
@@ -420,26 +471,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         const uint8_t* nxt = smem_bytes + ((ks + 1) & 3) * kStageBytes;
         const uint32_t sca[4] = {sa4.x >> sh, sa4.y >> sh, sa4.z >> sh, sa4.w >> sh};
         const uint32_t scb[4] = {sb4.x >> sh, sb4.y >> sh, sb4.z >> sh, sb4.w >> sh};
-#ifndef QM_DBG_NO_LDSREAD
         big_read_sub(cur, a_off1, b_off1, f1);
-#endif
-        big_mfma_sub<0>(f0, sca, scb, acc);
+        big_mfma_sub<0, sizeof(OutT) == 2>(f0, sca, scb, acc);
         QM_SCHED_PAIR(0x100, 8)
         __builtin_amdgcn_sched_barrier(0);
         // this wave's loads of tile ks+1 are older than those of tiles ks+2, ks+3: allow 20 outstanding
         __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * kLoadsPerStep & 0xf) | (((2 * kLoadsPerStep) >> 4) << 14));
-#ifndef QM_DBG_NO_BARRIER
         __syncthreads();
-#endif
         __builtin_amdgcn_sched_barrier(0);
-#ifndef QM_DBG_NO_LDSREAD
         big_read_scales(nxt, a_sc_off, b_sc_off, sa4, sb4);
         big_read_sub(nxt, a_off0, b_off0, f0);
-#endif
-#ifndef QM_DBG_NO_GLOBAL
         big_issue_loads(plan, ks & 3, ks + kStages);
-#endif
-        big_mfma_sub<1>(f1, sca, scb, acc);
+        big_mfma_sub<1, sizeof(OutT) == 2>(f1, sca, scb, acc);
         QM_SCHED_PAIR(0x100, 10)
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -451,7 +494,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         const uint32_t sca[4] = {sa4.x >> sh, sa4.y >> sh, sa4.z >> sh, sa4.w >> sh};
         const uint32_t scb[4] = {sb4.x >> sh, sb4.y >> sh, sb4.z >> sh, sb4.w >> sh};
         big_read_sub(cur, a_off1, b_off1, f1);
-        big_mfma_sub<0>(f0, sca, scb, acc);
+        big_mfma_sub<0, sizeof(OutT) == 2>(f0, sca, scb, acc);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): everything requested has landed
         __syncthreads();
@@ -460,14 +503,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             big_read_scales(nxt, a_sc_off, b_sc_off, sa4, sb4);
             big_read_sub(nxt, a_off0, b_off0, f0);
         }
-        big_mfma_sub<1>(f1, sca, scb, acc);
+        big_mfma_sub<1, sizeof(OutT) == 2>(f1, sca, scb, acc);
     }
 
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            store_tile<OutT>(acc[i][j], alpha, c, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
+    __syncthreads();  // every wave has finished reading the operand ring: it becomes the epilogue stage
+    big_epilogue<OutT>(acc, alpha, c, m0, n0, N, wm, wn, wave, lane, smem_bytes);
 }
 
 // ---- variant for K % 512 == 0: scales travel in blocks of four K steps -----------------------------
@@ -478,16 +518,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 constexpr int kCodeStageBytes = (kBigM + kBigN) * kRowBytes;            // 32 KiB
 constexpr int kScaleAreaOff = kStages * kCodeStageBytes;                // 128 KiB
 constexpr int kScaleBufBytes = (kBigM + kBigN) * 16;                    // 8 KiB per block of four K steps
-constexpr int kBig4SmemBytes = kScaleAreaOff + 2 * kScaleBufBytes;      // 144 KiB
+constexpr int kEpiAreaOff = kScaleAreaOff + 2 * kScaleBufBytes;     // 144 KiB
+constexpr int kEpiWaveBytes = 4096;                                  // 32 rows x 64 bf16 per wave
+constexpr int kBig4SmemBytes = kEpiAreaOff + 4 * kEpiWaveBytes;      // 160 KiB
 
 struct Big4Plan {
-    const uint8_t* a;
+    const uint8_t* a;   // uniform: first code byte of this tile's A panel (row m0, K step 0)
     const uint8_t* b;
-    const uint8_t* sa;  // this lane's scale source of block 0: row (wave*64 + lane), 16 bytes per block
+    const uint8_t* sa;  // uniform: first scale byte of this tile's A panel
     const uint8_t* sb;
-    int64_t row16_bytes;
-    uint32_t lds_codes;   // wave-uniform LDS address of this wave's first A wave-load in stage 0
-    uint32_t lds_scales;  // wave-uniform LDS address of this wave's A scale wave-load in buffer 0
+    int64_t row16_bytes;    // 16 rows of codes
+    uint32_t lane_codes;    // this lane's byte offset inside a panel for wave-load 0: row wave*64 + lane/4, swizzled 16-byte column
+    uint32_t lane_scales;   // this lane's byte offset inside a panel's scales: row wave*64 + lane
+    uint32_t lds_codes;     // wave-uniform LDS address of this wave's first A wave-load in stage 0
+    uint32_t lds_scales;    // wave-uniform LDS address of this wave's A scale wave-load in buffer 0
 };
 
 __device__ __forceinline__ void big4_issue_codes(const Big4Plan& p, int stage, int ks) {
@@ -495,14 +539,14 @@ __device__ __forceinline__ void big4_issue_codes(const Big4Plan& p, int stage, i
     const int kb = ks * kRowBytes;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        load_lds_b128(p.a + j * p.row16_bytes + kb, base + j * 1024);
-        load_lds_b128(p.b + j * p.row16_bytes + kb, base + kBOff + j * 1024);
+        load_lds_b128_s(p.a + j * p.row16_bytes + kb, p.lane_codes, base + j * 1024);
+        load_lds_b128_s(p.b + j * p.row16_bytes + kb, p.lane_codes, base + kBOff + j * 1024);
     }
 }
-__device__ __forceinline__ void big4_issue_scales(const Big4Plan& p, int qb) {
-    const uint32_t base = p.lds_scales + (qb & 1) * kScaleBufBytes;
-    load_lds_b128(p.sa + qb * 16, base);
-    load_lds_b128(p.sb + qb * 16, base + kBigM * 16);
+__device__ __forceinline__ void big4_issue_scales(const Big4Plan& p, int qb, int buf) {
+    const uint32_t base = p.lds_scales + buf * kScaleBufBytes;
+    load_lds_b128_s(p.sa + qb * 16, p.lane_scales, base);
+    load_lds_b128_s(p.sb + qb * 16, p.lane_scales, base + kBigM * 16);
 }
 
 struct ScaleRegs {
@@ -527,41 +571,82 @@ struct Big4State {
     ScaleRegs sr;
 };
 
-// K step ks = 4*qb + Q.  ISSUE: steady state (tile ks+4 and, for Q == 0, scale block qb+1 are requested).
-template <int Q, bool ISSUE>
-__device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_bytes, int ks, bool has_next, int a_off0,
+// One K step of the flat (tile, K step) stream; the step's index in its tile is congruent to Q mod 4, so
+// the ring stage it consumes is Q.  `lks` is the K step (of the tile `plan` points at) whose codes it
+// requests into the stage it has just freed; `par` selects the scale buffer the current block lives in.
+template <int Q, bool SWAP>
+__device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_bytes, int lks, int par, int a_off0,
                                           int a_off1, int b_off0, int b_off1, int a_sc_off, int b_sc_off, int sh,
                                           Big4State& st, v16f (&acc)[4][4]) {
-    const uint8_t* cur = smem_bytes + (ks & 3) * kCodeStageBytes;
-    const uint8_t* nxt = smem_bytes + ((ks + 1) & 3) * kCodeStageBytes;
+    const uint8_t* cur = smem_bytes + Q * kCodeStageBytes;
+    const uint8_t* nxt = smem_bytes + ((Q + 1) & 3) * kCodeStageBytes;
     const uint32_t sca[4] = {pick<Q>(st.sr.a[0]) >> sh, pick<Q>(st.sr.a[1]) >> sh, pick<Q>(st.sr.a[2]) >> sh, pick<Q>(st.sr.a[3]) >> sh};
     const uint32_t scb[4] = {pick<Q>(st.sr.b[0]) >> sh, pick<Q>(st.sr.b[1]) >> sh, pick<Q>(st.sr.b[2]) >> sh, pick<Q>(st.sr.b[3]) >> sh};
     big_read_sub(cur, a_off1, b_off1, st.f1);
-    big_mfma_sub<0>(st.f0, sca, scb, acc);
-    if constexpr (ISSUE) { QM_SCHED_PAIR(0x100, 8) }
+    big_mfma_sub<0, SWAP>(st.f0, sca, scb, acc);
+    QM_SCHED_PAIR(0x100, 8)
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (ISSUE) {
-        // loads younger than the codes of tile ks+1: codes of tiles ks+2, ks+3 (16) and, for Q = 1, 2, the two
-        // scale loads issued since; for Q = 3 the scale block read below is older than those and must be in
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm((Q == 1 || Q == 2) ? 18 : 16));
-    } else {
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-    }
+    // loads younger than the codes of the next step: the codes of the two steps after it (16) and, for Q = 1, 2,
+    // the two scale loads issued since; for Q = 3 the scale block read below is older than those and must be in
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm((Q == 1 || Q == 2) ? 18 : 16));
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-    if (ISSUE || has_next) {
-        if constexpr (Q == 3) big4_read_scales(smem_bytes + kScaleAreaOff + (((ks + 1) >> 2) & 1) * kScaleBufBytes, a_sc_off, b_sc_off, st.sr);
-        big_read_sub(nxt, a_off0, b_off0, st.f0);
-    }
-    if constexpr (ISSUE) {
-        big4_issue_codes(plan, ks & 3, ks + kStages);
-        if constexpr (Q == 0) big4_issue_scales(plan, (ks >> 2) + 1);
-    }
-    big_mfma_sub<1>(st.f1, sca, scb, acc);
-    if constexpr (ISSUE) { QM_SCHED_PAIR(0x100, (Q == 3 ? 16 : 8)) }
+    if constexpr (Q == 3) big4_read_scales(smem_bytes + kScaleAreaOff + (par ^ 1) * kScaleBufBytes, a_sc_off, b_sc_off, st.sr);
+    big_read_sub(nxt, a_off0, b_off0, st.f0);
+    big4_issue_codes(plan, Q, lks);
+    if constexpr (Q == 0) big4_issue_scales(plan, lks >> 2, par ^ 1);
+    big_mfma_sub<1, SWAP>(st.f1, sca, scb, acc);
+    QM_SCHED_PAIR(0x100, (Q == 3 ? 16 : 8))
     __builtin_amdgcn_sched_barrier(0);
 }
 
+// bf16 epilogue (operand roles swapped: a lane's accumulator quads run along n).  Eight passes of 32 rows x 64
+// columns per wave through a private 4 KiB LDS stage outside the operand ring, so the next tile's operands
+// keep streaming in underneath; 16-byte chunks are XOR-swizzled by row so that writes and reads spread over
+// all banks.
+__device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alpha, uint16_t* __restrict__ c, int64_t m0,
+                                                   int64_t n0, int64_t N, int wm, int wn, int wave, int lane_in,
+                                                   uint8_t* smem_bytes) {
+    // The opaque copy keeps the address arithmetic below inside the (rarely executed) epilogue instead of being
+    // hoisted out of the K loop, where it would hold dozens of registers across the MFMA schedule.
+    int lane = lane_in;
+    asm volatile("" : "+v"(lane));
+    const int lrow = lane & 31, half = lane >> 5;
+    uint8_t* region = smem_bytes + kEpiAreaOff + wave * kEpiWaveBytes;
+    const int chunk = lane & 7, rsub = lane >> 3;
+    uint8_t* wr = region + lrow * 128 + half * 8;
+    const int wsw = (lrow & 7) * 16;
+    const uint8_t* rd = region + rsub * 128 + ((chunk ^ rsub) * 16);  // rows rsub + 8k share rsub's swizzle
+    const int64_t pitch8 = N * 16;                                   // eight rows of bf16
+    uint8_t* out = reinterpret_cast<uint8_t*>(c + (m0 + wm * 128 + rsub) * N + n0 + wn * 128) + chunk * 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int jp = 0; jp < 2; ++jp) {
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const v16f& t = acc[i][2 * jp + jj];
+                    const v2bf p0 = __builtin_convertvector(v2f{t[4 * b] * alpha, t[4 * b + 1] * alpha}, v2bf);
+                    const v2bf p1 = __builtin_convertvector(v2f{t[4 * b + 2] * alpha, t[4 * b + 3] * alpha}, v2bf);
+                    *reinterpret_cast<uint2*>(wr + (((jj * 4 + b) * 16) ^ wsw)) =
+                        make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
+                }
+            // the region is private to the wave; LDS operations of one wave complete in order
+#pragma unroll
+            for (int r8 = 0; r8 < 4; ++r8) {
+                const uint4 v = *reinterpret_cast<const uint4*>(rd + r8 * 1024);
+                *reinterpret_cast<uint4*>(out + r8 * pitch8 + jp * 128) = v;
+            }
+        }
+        out += 4 * pitch8;
+    }
+}
+
+// Persistent: the grid is one workgroup per CU (or fewer); each workgroup walks tiles bid, bid + grid, ... as one
+// flat stream of K steps.  The loads that refill a freed ring stage simply continue into the next tile, so the
+// pipeline never drains between tiles and the epilogue runs while the next tile's first four stages arrive.
 template <typename OutT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mxfp4_tn_big4_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ b_codes,
@@ -573,32 +658,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int lrow = lane & 31, half = lane >> 5;
-    int tm, tn;
-    tile_of_block((int)blockIdx.x, M / kBigM, N / kBigN, tm, tn);
-    const int64_t m0 = (int64_t)tm * kBigM, n0 = (int64_t)tn * kBigN;
+    const int tiles_m = M / kBigM, tiles_n = N / kBigN, total = tiles_m * tiles_n;
     const int code_pitch = K / 2, groups = K / 32;
     const int nk = K / kBK;  // a multiple of 4
-
-    Big4Plan plan;
-    {
-        const int row = wave * 64 + (lane >> 2);
-        const int cv = (lane & 3) ^ ((row >> 2) & 3);
-        plan.a = a_codes + (m0 + row) * code_pitch + cv * 16;
-        plan.b = b_codes + (n0 + row) * code_pitch + cv * 16;
-        plan.row16_bytes = (int64_t)16 * code_pitch;
-        plan.sa = a_scales + (m0 + wave * 64 + lane) * groups;
-        plan.sb = b_scales + (n0 + wave * 64 + lane) * groups;
-        plan.lds_codes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + wave * 4096));
-        plan.lds_scales = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + kScaleAreaOff + wave * 1024));
-    }
-
-    v16f acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+    const int stride = (int)gridDim.x;
 
     const int swz = (lrow >> 2) & 3;
     const int a_off0 = (wm * 128 + lrow) * kRowBytes + (((2 * half) ^ swz) * 16);
@@ -608,34 +671,81 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int a_sc_off = (wm * 128 + lrow) * 16, b_sc_off = (wn * 128 + lrow) * 16;
     const int sh = 16 * half;
 
-    // prologue: scale block 0, code tiles 0..3; wait for the scales and tile 0 (24 younger loads may be pending)
-    big4_issue_scales(plan, 0);
-#pragma unroll
-    for (int t = 0; t < kStages; ++t) big4_issue_codes(plan, t, t);
+    Big4Plan plan;
+    plan.row16_bytes = (int64_t)16 * code_pitch;
+    plan.lds_codes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + wave * 4096));
+    plan.lds_scales = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + kScaleAreaOff + wave * 1024));
+    {
+        const int prow = lane >> 2;  // the wave's 64-row offset is folded into the uniform part below
+        const int pcv = (lane & 3) ^ ((prow >> 2) & 3);
+        plan.lane_codes = (uint32_t)(prow * code_pitch + pcv * 16);
+        plan.lane_scales = (uint32_t)(lane * groups);
+    }
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    int load_tm, load_tn;  // tile the load stream is in
+    auto plan_tile = [&](int t) {
+        tile_of_block(t, tiles_m, tiles_n, load_tm, load_tn);
+        const int64_t m0 = (int64_t)load_tm * kBigM + wave_u * 64, n0 = (int64_t)load_tn * kBigN + wave_u * 64;
+        plan.a = a_codes + m0 * code_pitch;
+        plan.b = b_codes + n0 * code_pitch;
+        plan.sa = a_scales + m0 * groups;
+        plan.sb = b_scales + n0 * groups;
+    };
+
+    plan_tile((int)blockIdx.x);
+    big4_issue_scales(plan, 0, 0);
+    big4_issue_codes(plan, 0, 0);
+    big4_issue_codes(plan, 1, 1);
+    big4_issue_codes(plan, 2, 2);
+    big4_issue_codes(plan, 3, 3);
+
+    // scale block 0 and code stage 0 must be in; stages 1..3 (24 loads, the youngest) may be pending
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(24));
     __syncthreads();
     Big4State st;
     big4_read_scales(smem_bytes + kScaleAreaOff, a_sc_off, b_sc_off, st.sr);
     big_read_sub(smem_bytes, a_off0, b_off0, st.f0);
 
-    int ks = 0;
-    for (; ks + 8 <= nk; ks += 4) {
-        big4_step<0, true>(plan, smem_bytes, ks, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
-        big4_step<1, true>(plan, smem_bytes, ks + 1, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
-        big4_step<2, true>(plan, smem_bytes, ks + 2, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
-        big4_step<3, true>(plan, smem_bytes, ks + 3, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+    int par = 0;
+    for (int t = (int)blockIdx.x; t < total; t += stride) {
+        v16f acc[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+        const int64_t m0 = (int64_t)load_tm * kBigM, n0 = (int64_t)load_tn * kBigN;  // the load stream is still in tile t
+        for (int ks = 0; ks < nk; ks += 4) {
+            // where the load stream is: four K steps ahead, rolling over into the next tile; after the last tile
+            // it re-requests the current steps (never consumed), which keeps the outstanding-load counts uniform
+            int lks = ks + 4;
+            if (lks == nk) {
+                if (t + stride < total) {
+                    plan_tile(t + stride);
+                    lks = 0;
+                } else {
+                    lks = ks;
+                }
+            }
+            big4_step<0, sizeof(OutT) == 2>(plan, smem_bytes, lks, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+            big4_step<1, sizeof(OutT) == 2>(plan, smem_bytes, lks + 1, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+            big4_step<2, sizeof(OutT) == 2>(plan, smem_bytes, lks + 2, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+            big4_step<3, sizeof(OutT) == 2>(plan, smem_bytes, lks + 3, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+            par ^= 1;
+        }
+        if constexpr (sizeof(OutT) == 2) {
+            big4_epilogue_bf16(acc, alpha, reinterpret_cast<uint16_t*>(c), m0, n0, N, wm, wn, wave, lane, smem_bytes);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    store_tile<OutT>(acc[i][j], alpha, c, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
+        }
     }
-    // last block: everything has been requested
-    big4_step<0, false>(plan, smem_bytes, ks, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
-    big4_step<1, false>(plan, smem_bytes, ks + 1, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
-    big4_step<2, false>(plan, smem_bytes, ks + 2, true, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
-    big4_step<3, false>(plan, smem_bytes, ks + 3, false, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
-
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            store_tile<OutT>(acc[i][j], alpha, c, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
+    // direct-to-LDS loads must not outlive the workgroup's LDS allocation
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
 }
 
 template <typename OutT>
@@ -645,7 +755,18 @@ hipError_t launch_big4(const uint8_t* a_codes, const uint8_t* a_scales, const ui
     auto kern = gemm_mxfp4_tn_big4_kernel<OutT>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kBig4SmemBytes);
     if (e != hipSuccess) return e;
-    dim3 grid((unsigned)((M / kBigM) * (N / kBigN))), block(256);
+    const int64_t tiles = (M / kBigM) * (N / kBigN);
+    int cus = 256;
+    {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+    }
+    // one workgroup per CU, and a grid that is a multiple of 8 so that tile t and t + grid land on the same XCD
+    int64_t g = tiles < cus ? tiles : cus;
+    if (g > 8) g -= g % 8;
+    dim3 grid((unsigned)g), block(256);
     kern<<<grid, block, kBig4SmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
                                                   reinterpret_cast<OutT*>(c));
     return hipGetLastError();

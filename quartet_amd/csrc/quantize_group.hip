@@ -85,7 +85,7 @@ __device__ __forceinline__ float tie_nudge(float v) {
     return u2f(__builtin_elementwise_sub_sat(f2u(v), 1u) | 1u);
 }
 
-template <int MODE>
+template <int MODE, bool WANT_MASK>
 __device__ __forceinline__ void quantize_group_regs(const float (&g)[32], uint64_t seed, int64_t group_index,
                                                     GroupCodes& o) {
     constexpr bool kQuest = (MODE == QUEST_RTN || MODE == QUEST_SR);
@@ -129,11 +129,14 @@ __device__ __forceinline__ void quantize_group_regs(const float (&g)[32], uint64
 #pragma unroll
         for (int i = 0; i < 32; ++i) t[i] = div_four_thirds(g[i]);
     }
-    // clip mask, most significant element first so that element 0 lands in bit 0
-    uint32_t keep = 0u;
+    o.keep = 0u;
+    if constexpr (WANT_MASK) {
+        // clip mask, most significant element first so that element 0 lands in bit 0
+        uint32_t keep = 0u;
 #pragma unroll
-    for (int i = 31; i >= 0; --i) keep = (keep << 1) | (((f2u(t[i]) & 0x7fffffffu) < thr_bits) ? 1u : 0u);
-    o.keep = all_zero ? 0u : keep;
+        for (int i = 31; i >= 0; --i) keep = (keep << 1) | (((f2u(t[i]) & 0x7fffffffu) < thr_bits) ? 1u : 0u);
+        o.keep = all_zero ? 0u : keep;
+    }
 
     // the converts' byte selector must be a literal, hence the macros
 #define QM_RTN_PAIR(B)                                                                                   \
@@ -240,47 +243,48 @@ __device__ __forceinline__ void rotate_group(float (&v)[32], float c, uint32_t s
 }
 
 // rotate (hd = 32) + quantize the group in v, write its outputs at group index gi
-template <typename T, int MODE>
+template <typename T, int MODE, bool WANT_MASK>
 __device__ __forceinline__ void finish_group(float (&v)[32], int64_t gi, float c, uint32_t sign_word, uint64_t seed,
                                              const GroupOut& out) {
     rotate_group(v, c, sign_word);
     GroupCodes o;
-    quantize_group_regs<MODE>(v, seed, gi, o);
+    quantize_group_regs<MODE, WANT_MASK>(v, seed, gi, o);
     out.codes[gi] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
     out.scales[gi] = (uint8_t)o.scale_byte;
-    if (out.maskbits) out.maskbits[gi] = o.keep;
+    if constexpr (WANT_MASK) out.maskbits[gi] = o.keep;
     if (out.dequant) store_dequant<T>(reinterpret_cast<T*>(out.dequant) + gi * 32, o);
 }
 
-template <typename T, int MODE>
+template <typename T, int MODE, bool WANT_MASK>
 __global__ __launch_bounds__(256) void quantize_rowmajor_g32_kernel(const T* __restrict__ x, int64_t n_groups, float c,
                                                                     uint32_t sign_word, uint64_t seed, GroupOut out) {
     const int64_t gi = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (gi >= n_groups) return;
     float v[32];
     load_group<T>(x + gi * 32, v);
-    finish_group<T, MODE>(v, gi, c, sign_word, seed, out);
+    finish_group<T, MODE, WANT_MASK>(v, gi, c, sign_word, seed, out);
 }
 
-template <typename T>
+template <typename T, bool WANT_MASK>
 void launch_rowmajor_g32(int mode, const void* x, int64_t n, float c, uint32_t sign_word, uint64_t seed,
                          const GroupOut& out, hipStream_t stream) {
     const int64_t n_groups = n / 32;
     dim3 grid((unsigned)((n_groups + 255) / 256)), block(256);
     const T* xp = reinterpret_cast<const T*>(x);
     switch (mode) {
-        case QUEST_RTN: quantize_rowmajor_g32_kernel<T, QUEST_RTN><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
-        case ABSMAX_RTN: quantize_rowmajor_g32_kernel<T, ABSMAX_RTN><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
-        case ABSMAX_SR: quantize_rowmajor_g32_kernel<T, ABSMAX_SR><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
-        default: quantize_rowmajor_g32_kernel<T, QUEST_SR><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
+        case QUEST_RTN: quantize_rowmajor_g32_kernel<T, QUEST_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
+        case ABSMAX_RTN: quantize_rowmajor_g32_kernel<T, ABSMAX_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
+        case ABSMAX_SR: quantize_rowmajor_g32_kernel<T, ABSMAX_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
+        default: quantize_rowmajor_g32_kernel<T, QUEST_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
     }
 }
 
 // ---- transposed input: x is [P, Q] row-major, output is the [Q, P] tensor quantized along P ----------
-// Tile = 128 p x TQ q staged in LDS exactly as it lies in memory (rows of 256 bytes).  Wave w then owns
-// p-group w of the tile; a lane reads its column (bf16: two adjacent columns per 32-bit read) at 32
-// successive rows, so every LDS read of a wave is one full 256-byte row: conflict free.  Codes and scales go
-// back through LDS so that each q row leaves as one contiguous 64-byte (codes) / 4-byte (scales) piece.
+// A workgroup owns a strip of 256 bytes of columns (128 bf16 / 64 fp32) by 128 rows; wave w owns p-group w.
+// A lane reads its column (bf16: two adjacent columns per 32-bit load) at 32 successive rows straight from
+// global memory: each wave load is one contiguous 256-byte row segment, 8 KiB in flight per wave, no LDS and
+// no barrier on the input side.  Codes and scales go through LDS so that each q row leaves the workgroup as
+// one contiguous 64-byte (codes) / 4-byte (scales) piece.
 template <typename T>
 struct TrTile {
     static constexpr int kQ = 256 / (int)sizeof(T);      // 128 columns of bf16, 64 of fp32
@@ -296,29 +300,20 @@ __global__ __launch_bounds__(256) void quantize_transposed_g32_kernel(const T* _
                                                                       void* __restrict__ dequant) {
     constexpr int TQ = TrTile<T>::kQ;
     constexpr int GPL = TrTile<T>::kGroupsPerLane;
-    __shared__ uint4 tile4[kTrP * 16];  // 128 rows x 256 bytes
-    uint32_t* tile = reinterpret_cast<uint32_t*>(tile4);
+    __shared__ uint4 ocodes[TQ * 4];      // [q][4 groups x 16 B]
+    __shared__ uint32_t oscales[TQ];      // [q][4 B]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t p0 = (int64_t)blockIdx.x * kTrP, q0 = (int64_t)blockIdx.y * TQ;
-    constexpr int kVec = 16 / (int)sizeof(T);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int idx = tid + j * 256, row = idx >> 4, cv = idx & 15;
-        uint4 raw = make_uint4(0, 0, 0, 0);
-        if (p0 + row < P && q0 + cv * kVec < Q)
-            raw = *reinterpret_cast<const uint4*>(x + (p0 + row) * Q + q0 + cv * kVec);
-        tile4[idx] = raw;
-    }
-    __syncthreads();
     const int64_t pbase = p0 + wave * 32;       // this wave's group along p
     const int64_t qa = q0 + lane * GPL;         // this lane's first column
     const bool active = pbase < P && qa < Q;    // P % 32 == 0 and Q % 8 == 0: all of a lane's groups or none
-    GroupCodes res[GPL];
     if (active) {
         float v[GPL][32];
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(x + pbase * Q + qa);
+        const int64_t row_dw = Q * (int64_t)sizeof(T) / 4;
 #pragma unroll
         for (int i = 0; i < 32; ++i) {
-            const uint32_t w = tile[(wave * 32 + i) * 64 + lane];
+            const uint32_t w = src[i * row_dw];
             if constexpr (sizeof(T) == 2) {
                 v[0][i] = u2f(w << 16);
                 v[1][i] = u2f(w & 0xffff0000u);
@@ -329,20 +324,12 @@ __global__ __launch_bounds__(256) void quantize_transposed_g32_kernel(const T* _
 #pragma unroll
         for (int gq = 0; gq < GPL; ++gq) {
             const int64_t gi = (qa + gq) * (P / 32) + pbase / 32;
+            GroupCodes res;
             rotate_group(v[gq], c, sign_word);
-            quantize_group_regs<MODE>(v[gq], seed, gi, res[gq]);
-            if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res[gq]);
-        }
-    }
-    __syncthreads();  // every wave is done reading the input tile: reuse it as the output stage
-    // stage: codes [TQ][4 groups x 16 B], then scales [TQ][4 B]
-    uint4* ocodes = tile4;
-    uint8_t* oscales = reinterpret_cast<uint8_t*>(tile4 + TQ * 4);
-    if (active) {
-#pragma unroll
-        for (int gq = 0; gq < GPL; ++gq) {
-            ocodes[(lane * GPL + gq) * 4 + wave] = make_uint4(res[gq].w[0], res[gq].w[1], res[gq].w[2], res[gq].w[3]);
-            oscales[(lane * GPL + gq) * 4 + wave] = (uint8_t)res[gq].scale_byte;
+            quantize_group_regs<MODE, false>(v[gq], seed, gi, res);
+            if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res);
+            ocodes[(lane * GPL + gq) * 4 + wave] = make_uint4(res.w[0], res.w[1], res.w[2], res.w[3]);
+            reinterpret_cast<uint8_t*>(oscales)[(lane * GPL + gq) * 4 + wave] = (uint8_t)res.scale_byte;
         }
     }
     __syncthreads();
@@ -353,7 +340,7 @@ __global__ __launch_bounds__(256) void quantize_transposed_g32_kernel(const T* _
             *reinterpret_cast<uint4*>(codes + (q0 + ql) * code_pitch + p0 / 2 + part * 16) = ocodes[idx];
     }
     if (tid < TQ && q0 + tid < Q) {
-        const uint32_t sw = reinterpret_cast<const uint32_t*>(oscales)[tid];
+        const uint32_t sw = oscales[tid];
         uint8_t* dst = scales + (q0 + tid) * scale_pitch + p0 / 32;
         if (p0 + kTrP <= P) {
             *reinterpret_cast<uint32_t*>(dst) = sw;
@@ -365,10 +352,12 @@ __global__ __launch_bounds__(256) void quantize_transposed_g32_kernel(const T* _
 }
 
 // ---- packed MXFP4 in, transposed + rotated + re-quantized out --------------------------------------------
-// in: codes [R, C/2], scales [R, C/32]; out: the [C, R] tensor quantized along R.  Tile = 128 r x 256 c
-// (rows of 128 code bytes + 8 scale bytes).  Wave w owns r-group w; a lane handles one byte column = two
-// adjacent c, 32 rows deep; the hardware FP4 de-quantizing convert turns each byte into two floats.
-constexpr int kRqR = 128, kRqC = 256;
+// in: codes [R, C/2], scales [R, C/32]; out: the [C, R] tensor quantized along R.  A workgroup owns 128
+// columns (64 code bytes per row) by 128 rows; wave w owns r-group w; a lane handles one byte column = two
+// adjacent c, 32 rows deep, read straight from global memory (one contiguous 64-byte row segment per wave
+// load, plus the row's E8M0 byte of the lane's column group).  The hardware FP4 de-quantizing convert turns
+// each byte into two floats.  Outputs leave through LDS as in the transposed quantizer.
+constexpr int kRqR = 128, kRqC = 128;
 
 template <int VAL_DTYPE, int MODE>
 __global__ __launch_bounds__(256) void requantize_transposed_g32_kernel(const uint8_t* __restrict__ codes_in,
@@ -379,53 +368,27 @@ __global__ __launch_bounds__(256) void requantize_transposed_g32_kernel(const ui
                                                                         uint8_t* __restrict__ scales,
                                                                         void* __restrict__ dequant) {
     using T = typename std::conditional<VAL_DTYPE == BF16, uint16_t, float>::type;
-    __shared__ uint4 ctile4[kRqR * 8];   // 128 rows x 128 bytes of codes; later the output stage (16 KiB)
-    __shared__ uint2 stile2[kRqR];       // 8 scale bytes per row
-    const uint8_t* ctile = reinterpret_cast<const uint8_t*>(ctile4);
-    const uint8_t* stile = reinterpret_cast<const uint8_t*>(stile2);
+    __shared__ uint4 ocodes[kRqC * 4];
+    __shared__ uint32_t oscales[kRqC];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t r0 = (int64_t)blockIdx.x * kRqR, c0 = (int64_t)blockIdx.y * kRqC;
     const int64_t in_code_pitch = C / 2, in_scale_pitch = C / 32;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int idx = tid + j * 256, row = idx >> 3, cv = idx & 7;
-        uint4 raw = make_uint4(0, 0, 0, 0);
-        if (r0 + row < R && c0 + cv * 32 < C)
-            raw = *reinterpret_cast<const uint4*>(codes_in + (r0 + row) * in_code_pitch + c0 / 2 + cv * 16);
-        ctile4[idx] = raw;
-    }
-    if (tid < kRqR) {
-        uint2 s = make_uint2(0, 0);
-        if (r0 + tid < R) {
-            const uint8_t* sp = scales_in + (r0 + tid) * in_scale_pitch + c0 / 32;
-            if (c0 + kRqC <= C && (in_scale_pitch & 7) == 0) {
-                s = *reinterpret_cast<const uint2*>(sp);
-            } else {
-                uint32_t lo = 0, hi = 0;
-                for (int b = 0; b < 8; ++b)
-                    if (c0 + b * 32 < C) (b < 4 ? lo : hi) |= (uint32_t)sp[b] << (8 * (b & 3));
-                s = make_uint2(lo, hi);
-            }
-        }
-        stile2[tid] = s;
-    }
-    __syncthreads();
     const int64_t rbase = r0 + wave * 32;
-    GroupCodes res[2][2];  // [pass][column of the pair]
-    bool active[2];
-#pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-        const int bcol = pass * 64 + lane;           // byte column within the tile: c = c0 + 2*bcol, +1
-        const int64_t ca = c0 + 2 * bcol;
-        active[pass] = rbase < R && ca < C;          // C % 32 == 0: both columns of the pair or none
-        if (!active[pass]) continue;
+    const int64_t ca = c0 + 2 * lane;            // this lane's column pair
+    const bool active = rbase < R && ca < C;     // C % 32 == 0: both columns of the pair or none
+    if (active) {
         float v[2][32];
+        const uint8_t* cp = codes_in + rbase * in_code_pitch + ca / 2;
+        const uint8_t* sp = scales_in + rbase * in_scale_pitch + ca / 32;
+        uint32_t byte[32], sbyte[32];
 #pragma unroll
         for (int i = 0; i < 32; ++i) {
-            const int row = wave * 32 + i;
-            const uint32_t byte = ctile[row * 128 + bcol];
-            const uint32_t sbyte = stile[row * 8 + (bcol >> 4)];
-            const v2f pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(byte, u2f(sbyte << 23), 0);
+            byte[i] = cp[i * in_code_pitch];
+            sbyte[i] = sp[i * in_scale_pitch];
+        }
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const v2f pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(byte[i], u2f(sbyte[i] << 23), 0);
             float a = pr.x, b = pr.y;
             if (post != 1.0f) {  // absmax-coded input: value = code * 2^k * post, held in val_dtype
                 a *= post;
@@ -441,44 +404,23 @@ __global__ __launch_bounds__(256) void requantize_transposed_g32_kernel(const ui
 #pragma unroll
         for (int gq = 0; gq < 2; ++gq) {
             const int64_t gi = (ca + gq) * (R / 32) + rbase / 32;
+            GroupCodes res;
             rotate_group(v[gq], c, sign_word);
-            quantize_group_regs<MODE>(v[gq], seed, gi, res[pass][gq]);
-            if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res[pass][gq]);
-        }
-    }
-    __syncthreads();
-    // output stage: codes [256 c][4 groups x 16 B] = 16 KiB over the code tile, scales [256 c][4 B] over ... a
-    // second pass: the scale tile is only 1 KiB, so scales are staged after the codes have been written out
-    uint4* ocodes = ctile4;
-#pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-        if (!active[pass]) continue;
-#pragma unroll
-        for (int gq = 0; gq < 2; ++gq) {
-            const int cl = 2 * (pass * 64 + lane) + gq;
-            const GroupCodes& g = res[pass][gq];
-            ocodes[cl * 4 + wave] = make_uint4(g.w[0], g.w[1], g.w[2], g.w[3]);
+            quantize_group_regs<MODE, false>(v[gq], seed, gi, res);
+            if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res);
+            ocodes[(lane * 2 + gq) * 4 + wave] = make_uint4(res.w[0], res.w[1], res.w[2], res.w[3]);
+            reinterpret_cast<uint8_t*>(oscales)[(lane * 2 + gq) * 4 + wave] = (uint8_t)res.scale_byte;
         }
     }
     __syncthreads();
     const int64_t code_pitch = R / 2, scale_pitch = R / 32;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int idx = tid + j * 256, cl = idx >> 2, part = idx & 3;
+    for (int idx = tid; idx < kRqC * 4; idx += 256) {
+        const int cl = idx >> 2, part = idx & 3;
         if (c0 + cl < C && r0 + part * 32 < R)
             *reinterpret_cast<uint4*>(codes + (c0 + cl) * code_pitch + r0 / 2 + part * 16) = ocodes[idx];
     }
-    __syncthreads();
-    uint8_t* oscales = reinterpret_cast<uint8_t*>(ctile4);
-#pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-        if (!active[pass]) continue;
-#pragma unroll
-        for (int gq = 0; gq < 2; ++gq) oscales[(2 * (pass * 64 + lane) + gq) * 4 + wave] = (uint8_t)res[pass][gq].scale_byte;
-    }
-    __syncthreads();
-    if (c0 + tid < C) {
-        const uint32_t sw = reinterpret_cast<const uint32_t*>(oscales)[tid];
+    if (tid < kRqC && c0 + tid < C) {
+        const uint32_t sw = oscales[tid];
         uint8_t* dst = scales + (c0 + tid) * scale_pitch + r0 / 32;
         if (r0 + kRqR <= R) {
             *reinterpret_cast<uint32_t*>(dst) = sw;
@@ -523,8 +465,13 @@ hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t n, uint32_t 
                                   hipStream_t stream) {
     GroupOut out{reinterpret_cast<uint4*>(codes), scales, reinterpret_cast<uint32_t*>(maskbits), dequant};
     const float c = hadamard_scale(32, dtype);
-    if (dtype == BF16) launch_rowmajor_g32<uint16_t>(mode, x, n, c, sign_word, seed, out, stream);
-    else launch_rowmajor_g32<float>(mode, x, n, c, sign_word, seed, out, stream);
+    if (maskbits) {
+        if (dtype == BF16) launch_rowmajor_g32<uint16_t, true>(mode, x, n, c, sign_word, seed, out, stream);
+        else launch_rowmajor_g32<float, true>(mode, x, n, c, sign_word, seed, out, stream);
+    } else {
+        if (dtype == BF16) launch_rowmajor_g32<uint16_t, false>(mode, x, n, c, sign_word, seed, out, stream);
+        else launch_rowmajor_g32<float, false>(mode, x, n, c, sign_word, seed, out, stream);
+    }
     return hipGetLastError();
 }
 

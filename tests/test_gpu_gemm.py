@@ -72,3 +72,45 @@ def test_gemm_one_hot_operand_selects_single_products(oracle, K):
     B = oracle.dequantize(bc, bs)
     want = np.stack([B[:, k] for k in ks], axis=0)
     assert np.array_equal(got.cpu().numpy(), want)
+
+
+def _torch_dequant(codes, scales):
+    """E2M1/E8M0 unpacking in plain torch ops (float64), checked against the oracle in the test below."""
+    lut = torch.tensor([0, .5, 1, 1.5, 2, 3, 4, 6, -0.0, -.5, -1, -1.5, -2, -3, -4, -6], dtype=torch.float64, device=codes.device)
+    lo, hi = (codes & 15).long(), (codes >> 4).long()
+    v = torch.stack([lut[lo], lut[hi]], dim=-1).reshape(codes.shape[0], -1)
+    s = torch.exp2(scales.to(torch.float64) - 127.0).repeat_interleave(32, dim=1)
+    return v * s
+
+
+# Shapes the 256x256-tile kernels serve: a single tile, fewer tiles than CUs, more tiles than CUs (each
+# workgroup walks several tiles, with an odd and an even number of scale blocks per tile), and K that is a
+# multiple of 128 but not of 512 (per-step scale loads).
+@pytest.mark.parametrize("M,N,K_", [(256, 256, 512), (512, 768, 1024), (4352, 4352, 512), (4608, 4352, 1024),
+                                    (768, 512, 1536), (512, 256, 640), (4352, 4608, 384), (8192, 4096, 2048)])
+@pytest.mark.parametrize("exact", [True, False])
+def test_gemm_tile_kernels(oracle, K, M, N, K_, exact):
+    print(f"case gemm tiles {M}x{N}x{K_} exact={exact}", flush=True)
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(M * 7 + N * 3 + K_)
+    ac = torch.randint(0, 256, (M, K_ // 2), generator=g, dtype=torch.uint8).to(dev)
+    bc = torch.randint(0, 256, (N, K_ // 2), generator=g, dtype=torch.uint8).to(dev)
+    if exact:  # equal scales: every product is a multiple of 1/4 and every partial sum is exact in fp32
+        as_ = torch.full((M, K_ // 32), 127, dtype=torch.uint8, device=dev)
+        bs = torch.full((N, K_ // 32), 125, dtype=torch.uint8, device=dev)
+    else:
+        as_ = torch.randint(118, 132, (M, K_ // 32), generator=g, dtype=torch.uint8).to(dev)
+        bs = torch.randint(120, 136, (N, K_ // 32), generator=g, dtype=torch.uint8).to(dev)
+    A, B = _torch_dequant(ac, as_), _torch_dequant(bc, bs)
+    # the unpacking helper itself, on a corner of the operands
+    assert np.array_equal(A[:64].cpu().numpy(), oracle.dequantize(ac[:64].cpu().numpy(), as_[:64].cpu().numpy()).astype(np.float64))
+    want = A @ B.T
+    got32 = K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha=1.0, out_dtype=torch.float32)
+    got16 = K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha=1.0, out_dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    if exact:
+        assert torch.equal(got32.double(), want)
+    else:
+        rel = float((got32.double() - want).norm() / want.norm())
+        assert rel <= 1e-5, rel
+    assert torch.equal(got16, got32.to(torch.bfloat16))
