@@ -19,6 +19,10 @@ import torch
 T_TOKENS, IN_F, OUT_F = 8192, 4096, 4096
 PEAK_FP4_TFLOPS = 10100.0   # MI355X dense MXFP4 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+# HBM bytes per launch from profiler byte counters (fetch + write), scaled by what the same counters read for a
+# plain 256 MiB device copy (fetch counter x 2.0 KiB, write counter x 1.0 KiB)
+GEMM_TRAFFIC_BYTES = 174.6e6      # mean of the three GEMMs: 108.4 MiB fetched (operand re-reads that miss L2) + 58.2 MiB written
+QUANTIZE_TRAFFIC_BYTES = 89.2e6   # 64.1 MiB fetched + 21.0 MiB written; algorithmic 89.1e6
 
 
 def make_inputs(device, tokens=T_TOKENS, seed=0):
@@ -60,8 +64,27 @@ def time_kernel(fn, reps=20, warmup=3):
     return start.elapsed_time(stop) / reps
 
 
+COLD_CYCLE_BYTES = 1 << 30  # distinct input bytes walked before a buffer repeats: 4x the 256 MB memory-side cache
+
+
+def time_kernel_cold(make_call, inputs, reps=24, warmup=2):
+    """HBM-cold timing: `inputs` are the tensors one launch reads; the launch is timed over clones of them that
+    together exceed the last-level cache several times, so every launch streams its input from HBM."""
+    nbytes = sum(t.numel() * t.element_size() for t in inputs)
+    n = max(2, min(64, -(-COLD_CYCLE_BYTES // max(nbytes, 1))))
+    sets = [inputs] + [[t.clone() for t in inputs] for _ in range(n - 1)]
+    calls = [make_call(*st) for st in sets]
+    state = {"i": 0}
+
+    def fn():
+        calls[state["i"] % n]()
+        state["i"] += 1
+    return time_kernel(fn, reps=max(reps, n), warmup=warmup)
+
+
 def kernel_breakdown(x, w, dy):
-    """Per-kernel timings of the twelve launches of one step, with algorithmic bytes / flops."""
+    """Per-kernel timings of the eleven launches of one step, with algorithmic bytes / flops.  HBM-bound kernels
+    are timed HBM-cold (see time_kernel_cold) and, for reference, warm on one buffer."""
     from quartet_amd import kernels as K
     T, I, O = x.shape[0], x.shape[1], w.shape[0]
     out = {}
@@ -75,33 +98,63 @@ def kernel_breakdown(x, w, dy):
     gxq = K.gemm_mxfp4_tn(ec, es, wtc, wts, 1.0, torch.bfloat16)
     gwq = K.gemm_mxfp4_tn(etc, ets, xtc, xts, 1.0, torch.bfloat16)
 
-    def hbm(name, elems, bytes_per_elem, fn):
-        ms = time_kernel(fn)
-        out[name] = {"ms": round(ms, 4), "GBps": round(elems * bytes_per_elem / ms / 1e6, 1),
-                     "bytes_per_elem": bytes_per_elem}
+    def hbm(name, elems, bytes_per_elem, make_call, inputs):
+        cold = time_kernel_cold(make_call, inputs)
+        warm = time_kernel(make_call(*inputs))
+        out[name] = {"ms": round(cold, 4), "GBps": round(elems * bytes_per_elem / cold / 1e6, 1),
+                     "bytes_per_elem": bytes_per_elem, "ms_warm": round(warm, 4)}
 
     def mfma(name, m, n, k, fn):
         ms = time_kernel(fn)
         out[name] = {"ms": round(ms, 4), "TFLOPs": round(2.0 * m * n * k / ms / 1e9, 1), "shape": [m, n, k]}
 
-    hbm("quantize_x_quest_rtn_mask", T * I, 2.65625, lambda: K.quantize_mxfp4(x, 32, None, K.QM_QUEST_RTN, want_mask=True))
-    hbm("quantize_w_quest_rtn_mask", O * I, 2.65625, lambda: K.quantize_mxfp4(w, 32, None, K.QM_QUEST_RTN, want_mask=True))
+    hbm("quantize_x_quest_rtn_mask", T * I, 2.65625,
+        lambda a: (lambda: K.quantize_mxfp4(a, 32, None, K.QM_QUEST_RTN, want_mask=True)), [x])
+    hbm("quantize_w_quest_rtn_mask", O * I, 2.65625,
+        lambda a: (lambda: K.quantize_mxfp4(a, 32, None, K.QM_QUEST_RTN, want_mask=True)), [w])
     mfma("gemm_fwd", T, O, I, lambda: K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.bfloat16))
-    hbm("quantize_e_absmax_sr", T * O, 2.53125, lambda: K.quantize_mxfp4(dy, 32, signs, K.QM_ABSMAX_SR, seed=1))
+    hbm("quantize_e_absmax_sr", T * O, 2.53125,
+        lambda a: (lambda: K.quantize_mxfp4(a, 32, signs, K.QM_ABSMAX_SR, seed=1)), [dy])
     hbm("quantize_et_absmax_sr_transposed", T * O, 2.53125,
-        lambda: K.quantize_mxfp4(dy, 32, signs, K.QM_ABSMAX_SR, transposed_in=True, seed=2))
+        lambda a: (lambda: K.quantize_mxfp4(a, 32, signs, K.QM_ABSMAX_SR, transposed_in=True, seed=2)), [dy])
     hbm("requantize_wt", O * I, 1.0625,
-        lambda: K.requantize_transposed_mxfp4(wc, ws, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=3))
+        lambda c, sc: (lambda: K.requantize_transposed_mxfp4(c, sc, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=3)),
+        [wc, ws])
     hbm("requantize_xt", T * I, 1.0625,
-        lambda: K.requantize_transposed_mxfp4(xc, xs, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=4))
+        lambda c, sc: (lambda: K.requantize_transposed_mxfp4(c, sc, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=4)),
+        [xc, xs])
     mfma("gemm_dgrad", T, I, O, lambda: K.gemm_mxfp4_tn(ec, es, wtc, wts, 1.0, torch.bfloat16))
     mfma("gemm_wgrad", O, I, T, lambda: K.gemm_mxfp4_tn(etc, ets, xtc, xts, 1.0, torch.bfloat16))
-    hbm("hadamard_bwd_x", T * I, 4.125, lambda: K.masked_hadamard_bwd(gxq, 32, torch.bfloat16, None, xm))
-    hbm("hadamard_bwd_w", O * I, 4.125, lambda: K.masked_hadamard_bwd(gwq, 32, torch.bfloat16, None, wm))
+    hbm("hadamard_bwd_x", T * I, 4.125,
+        lambda g, m: (lambda: K.masked_hadamard_bwd(g, 32, torch.bfloat16, None, m)), [gxq, xm])
+    hbm("hadamard_bwd_w", O * I, 4.125,
+        lambda g, m: (lambda: K.masked_hadamard_bwd(g, 32, torch.bfloat16, None, m)), [gwq, wm])
     return out
 
 
-def cpu_baseline(sample_tokens=2048):
+def quantizer_sweep(device):
+    """Quantizer-only throughput (HBM-cold) on [rows x 4096] bf16 with 0.1 % entries at +-1e3, for the three
+    production modes and Hadamard blocks 32/64/128."""
+    from quartet_amd import kernels as K
+    res = []
+    for rows in (4096, 16384, 65536):
+        g = torch.Generator().manual_seed(rows)
+        x = torch.randn(rows, 4096, generator=g)
+        spike = torch.rand(rows, 4096, generator=g) < 1e-3
+        sgn = torch.where(torch.rand(rows, 4096, generator=g) < 0.5, -1e3, 1e3)
+        x = torch.where(spike, sgn, x).to(torch.bfloat16).to(device)
+        for hd in (32, 64, 128):
+            for name, mode, mask, bpe in (("quest_rtn_mask", K.QM_QUEST_RTN, True, 2.65625),
+                                          ("absmax_rtn", K.QM_ABSMAX_RTN, False, 2.53125),
+                                          ("absmax_sr", K.QM_ABSMAX_SR, False, 2.53125)):
+                ms = time_kernel_cold(lambda a: (lambda: K.quantize_mxfp4(a, hd, None, mode, want_mask=mask, seed=7)), [x],
+                                      reps=8, warmup=1)
+                res.append({"rows": rows, "hd": hd, "mode": name, "ms": round(ms, 4),
+                            "GBps": round(rows * 4096 * bpe / ms / 1e6, 1)})
+    return res
+
+
+def cpu_baseline(sample_tokens=T_TOKENS):
     """The CPU restatement of the same pseudo-quantized linear (oracle quantizers + fp32 BLAS matmuls on
     de-quantized operands, i.e. the op sequence the reference runs) on a row sample of the workload."""
     import numpy as np
@@ -134,7 +187,7 @@ def cpu_baseline(sample_tokens=2048):
     assert y.shape[0] == sample_tokens and gx.shape == (sample_tokens, IN_F) and gw.shape == (OUT_F, IN_F)
     flops = 6.0 * sample_tokens * IN_F * OUT_F
     return {"value": round(flops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"one fwd+bwd on the first {sample_tokens} of {T_TOKENS} tokens (same I={IN_F}, O={OUT_F}); "
+            "sample": f"one fwd+bwd on {sample_tokens} of {T_TOKENS} tokens (same I={IN_F}, O={OUT_F}); "
                       f"CPU oracle quantizers + fp32 BLAS matmuls on de-quantized operands, {dt:.2f} s"}
 
 
@@ -145,6 +198,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (a known-traffic kernel for scaling profiler byte counters)")
+    ap.add_argument("--quantizer-sweep", action="store_true",
+                    help="also time the quantizer alone on [rows x 4096] for rows 4096/16384/65536, three modes, hd 32/64/128")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)")
@@ -165,6 +222,12 @@ def main():
         x.grad = None
         layer.weight.grad = None
 
+    if args.calibration_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=device).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -188,17 +251,22 @@ def main():
         x.requires_grad_(False)
         kb = kernel_breakdown(x.detach(), w, dy)
         result["kernels"] = kb
-        g = kb["gemm_fwd"]
-        gemm_ms = g["ms"]
-        result["roofline"] = {"bound": "mfma", "kernel": "gemm_mxfp4_tn (fwd 8192x4096x4096)",
-                              "achieved": g["TFLOPs"], "peak": PEAK_FP4_TFLOPS, "unit": "TFLOP/s",
-                              "frac": round(g["TFLOPs"] / PEAK_FP4_TFLOPS, 4), "traffic": None,
-                              "avg_launch_ms": gemm_ms}
+        # the three GEMMs of a step (fwd, dgrad, wgrad) run the same kernel on the same flop count: the roofline
+        # entry is their mean, which is what a profiler's per-kernel average over the run reports
+        gemms = [kb[k] for k in ("gemm_fwd", "gemm_dgrad", "gemm_wgrad")]
+        gemm_ms = sum(g["ms"] for g in gemms) / 3.0
+        gemm_tf = 2.0 * T_TOKENS * IN_F * OUT_F / gemm_ms / 1e9
+        result["roofline"] = {"bound": "mfma", "kernel": "gemm_mxfp4_tn_big4_kernel (8192x4096x4096, 8192x4096x4096, 4096x4096x8192)",
+                              "achieved": round(gemm_tf, 1), "peak": PEAK_FP4_TFLOPS, "unit": "TFLOP/s",
+                              "frac": round(gemm_tf / PEAK_FP4_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
+                              "avg_launch_ms": round(gemm_ms, 4)}
         qk = kb["quantize_x_quest_rtn_mask"]
         result["roofline_quantize"] = {"bound": "hbm", "kernel": "quantize_rowmajor (quest RTN + mask, 8192x4096 bf16)",
                                        "achieved": qk["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                       "frac": round(qk["GBps"] / PEAK_HBM_GBS, 4), "traffic": None,
+                                       "frac": round(qk["GBps"] / PEAK_HBM_GBS, 4), "traffic": QUANTIZE_TRAFFIC_BYTES,
                                        "avg_launch_ms": qk["ms"]}
+    if args.quantizer_sweep:
+        result["quantizer_sweep"] = quantizer_sweep(device)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))

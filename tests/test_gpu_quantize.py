@@ -99,6 +99,71 @@ def test_requantize_transposed_bit_exact(oracle, K, hd, val_dtype):
         assert np.array_equal(a, b)
 
 
+# The group-layout kernels serve Hadamard block 32 with round-to-nearest or the in-kernel Philox stream; these
+# shapes meet their alignment rules (physical P % 128 == 0 for transposed input, R % 128 == 0 for the
+# re-quantizer) with ragged and multi-tile extents in the other direction.
+@pytest.mark.parametrize("mode", ["absmax_sr", "absmax_rtn", "quest_rtn", "quest_sr"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("P,Q", [(128, 32), (256, 200), (384, 320)])
+def test_transposed_group_layout_bit_exact(oracle, K, mode, dtype, P, Q):
+    print(f"case transposed-g32 mode={mode} dtype={dtype} P={P} Q={Q}", flush=True)
+    x = make_input(P, Q, dtype, seed=P + Q, zero_rows=1)
+    x[0:32, 5] = 0  # logical row 5 starts with an all-zero MX group
+    g = torch.Generator().manual_seed(12)
+    signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
+    dev = torch.device("cuda:0")
+    seed = 0x0BAD_5EED_0000_0001 + P
+    codes, scales, _, deq = K.quantize_mxfp4(x.to(dev), 32, sign_int(signs), MODES[mode], True, None, seed,
+                                             want_mask=False, want_dequant=True)
+    torch.cuda.synchronize()
+    ref = oracle.quantize(to_oracle(x), 32, signs=signs.numpy(), mode=MODES[mode], transposed_in=True, u=None,
+                          seed=seed, want_mask=False, want_dequant=True)
+    assert np.array_equal(to_oracle(scales), ref["scales"])
+    assert np.array_equal(to_oracle(codes), ref["codes"])
+    a, b = to_oracle(deq), ref["dequant"]
+    if a.dtype == np.float32:
+        a, b = a.view(np.uint32), b.view(np.uint32)
+    assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("mode", ["absmax_sr", "absmax_rtn"])
+@pytest.mark.parametrize("val_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("R,C", [(128, 32), (256, 160), (384, 512)])
+def test_requantize_group_layout_bit_exact(oracle, K, mode, val_dtype, R, C):
+    print(f"case requant-g32 mode={mode} val_dtype={val_dtype} R={R} C={C}", flush=True)
+    dev = torch.device("cuda:0")
+    x = make_input(R, C, torch.bfloat16, seed=R + C, zero_rows=1)
+    q = oracle.quantize(to_oracle(x), 32, mode=oracle.QUEST_RTN)
+    g = torch.Generator().manual_seed(13)
+    signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
+    vd = oracle.BF16 if val_dtype == torch.bfloat16 else oracle.F32
+    seed = 0x7777_0000_1234 + C
+    for post in (1.0, float(oracle.FOUR_THIRDS)):
+        ref = oracle.requantize_transposed(q["codes"], q["scales"], post=post, val_dtype=vd, hd=32, signs=signs.numpy(),
+                                           mode=MODES[mode], u=None, seed=seed, want_dequant=True)
+        co, so, dq = K.requantize_transposed_mxfp4(torch.from_numpy(q["codes"]).to(dev),
+                                                   torch.from_numpy(q["scales"]).to(dev), post, val_dtype, 32,
+                                                   sign_int(signs), MODES[mode], None, seed, want_dequant=True)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_oracle(so), ref["scales"])
+        assert np.array_equal(to_oracle(co), ref["codes"])
+        a, b = to_oracle(dq), ref["dequant"]
+        if a.dtype == np.float32:
+            a, b = a.view(np.uint32), b.view(np.uint32)
+        assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rowmajor_group_layout_seeded(oracle, K, mode, dtype):
+    print(f"case rowmajor-g32 mode={mode} dtype={dtype}", flush=True)
+    # 33 rows x 2080 columns: the element count is not a multiple of the kernel's per-block share
+    x = make_input(33, 2080, dtype, seed=21, zero_rows=1)
+    g = torch.Generator().manual_seed(14)
+    signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
+    _check(oracle, K, x, 32, MODES[mode], signs, False, None, 0xFEED_F00D_CAFE, f"rowmajor-g32/{mode}/{dtype}")
+
+
 def test_order_independent_integer_fixture(oracle, K):
     # x = S @ g with small integers and hd = 64: every partial sum is exact, so the expected
     # rotated values (8*g) and hence codes/scales do not depend on any summation order.
