@@ -191,6 +191,52 @@ def cpu_baseline(sample_tokens=T_TOKENS):
                       f"CPU oracle quantizers + fp32 BLAS matmuls on de-quantized operands, {dt:.2f} s"}
 
 
+def llama_step(args, device):
+    """Whole-model step of a Llama configuration with every block linear on the Quartet path: bf16 autocast around
+    forward and backward, cross-entropy on random ids, AdamW (fp32 state) for the ~800 M configuration."""
+    from quartet_amd import llama as L
+    torch.manual_seed(0)
+    over = L.unquantized() if args.unquantized else {}
+    if args.workload == "llama30m":
+        cfg, batch, seq, opt_step = L.llama_30m(**over), 64, 512, False
+    else:
+        cfg, batch, seq, opt_step = L.llama_800m(**over), 16, 2048, True
+    model = L.Llama(cfg).to(device)
+    opt = torch.optim.AdamW(model.parameters(), lr=1e-4, fused=True) if opt_step else None
+    g = torch.Generator().manual_seed(1)
+    idx = torch.randint(0, cfg.vocab_size, (batch, seq), generator=g).to(device)
+    tgt = torch.randint(0, cfg.vocab_size, (batch, seq), generator=g).to(device)
+
+    def step():
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            loss = model(idx, targets=tgt)["loss"]
+            loss.backward()
+        if opt is not None:
+            opt.step()
+        model.zero_grad(set_to_none=True)
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    lin = sum(m.weight.numel() for _, m in model.block_linears())
+    tokens = batch * seq
+    flops = 6.0 * tokens * lin
+    return {"metric": "Quartet linear fwd+bwd TFLOPS (MXFP4 MFMA) + Hadamard/quantize HBM GB/s",
+            "value": round(flops / (ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16" if args.unquantized else "mxfp4", "data": "synthetic",
+            "config": {"workload": f"{args.workload}{' (unquantized bf16 linears)' if args.unquantized else ''} whole-model step ({cfg.n_layer} layers, d {cfg.n_embd}, {batch}x{seq} tokens, "
+                                   f"{'fwd+bwd+AdamW' if opt_step else 'fwd+bwd'}); value counts the block linears' 6*tokens*params "
+                                   f"flops only ({flops / 1e12:.2f} TFLOP) over the whole step time"},
+            "tokens_per_s": round(tokens / (ms * 1e-3), 1), "final_loss": round(float(loss.detach()), 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -198,6 +244,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--workload", default="linear", choices=["linear", "llama30m", "llama800m"],
+                    help="linear (default): the isolated 8192x4096x4096 layer the metric is quoted on; llama30m / llama800m: "
+                         "whole-model fwd+bwd(+AdamW) step of the 30 M / ~800 M Llama configurations, reported in the same unit "
+                         "over the block linears' flops")
+    ap.add_argument("--unquantized", action="store_true",
+                    help="with a llama workload: identity quantizers and the plain scheme (the bf16 model, for context)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a known-traffic kernel for scaling profiler byte counters)")
     ap.add_argument("--quantizer-sweep", action="store_true",
@@ -209,6 +261,9 @@ def main():
         sys.exit("bench.py needs a GPU: the quantized-linear path has no CPU fallback")
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     device = torch.device("cuda:0")
+    if args.workload != "linear":
+        print(json.dumps(llama_step(args, device)))
+        return
     x, w, dy = make_inputs(device)
     layer = build_layer(device)
     with torch.no_grad():
