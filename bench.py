@@ -88,15 +88,16 @@ def kernel_breakdown(x, w, dy):
     from quartet_amd import kernels as K
     T, I, O = x.shape[0], x.shape[1], w.shape[0]
     out = {}
-    xc, xs, xm, _ = K.quantize_mxfp4(x, 32, None, K.QM_QUEST_RTN, want_mask=True)
-    wc, ws, wm, _ = K.quantize_mxfp4(w, 32, None, K.QM_QUEST_RTN, want_mask=True)
+    tl = True  # tiled code bytes, as the layer uses for these extents
+    xc, xs, xm, _ = K.quantize_mxfp4(x, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)
+    wc, ws, wm, _ = K.quantize_mxfp4(w, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)
     signs = 0x5A5AA5A5
-    ec, es, _, _ = K.quantize_mxfp4(dy, 32, signs, K.QM_ABSMAX_SR, seed=1)
-    etc, ets, _, _ = K.quantize_mxfp4(dy, 32, signs, K.QM_ABSMAX_SR, transposed_in=True, seed=2)
-    wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=3)
-    xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=4)
-    gxq = K.gemm_mxfp4_tn(ec, es, wtc, wts, 1.0, torch.bfloat16)
-    gwq = K.gemm_mxfp4_tn(etc, ets, xtc, xts, 1.0, torch.bfloat16)
+    ec, es, _, _ = K.quantize_mxfp4(dy, 32, signs, K.QM_ABSMAX_SR, seed=1, tiled=tl)
+    etc, ets, _, _ = K.quantize_mxfp4(dy, 32, signs, K.QM_ABSMAX_SR, transposed_in=True, seed=2, tiled=tl)
+    wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=3, tiled_in=tl, tiled_out=tl)
+    xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=4, tiled_in=tl, tiled_out=tl)
+    gxq = K.gemm_mxfp4_tn(ec, es, wtc, wts, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl)
+    gwq = K.gemm_mxfp4_tn(etc, ets, xtc, xts, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl)
 
     def hbm(name, elems, bytes_per_elem, make_call, inputs):
         cold = time_kernel_cold(make_call, inputs)
@@ -109,22 +110,24 @@ def kernel_breakdown(x, w, dy):
         out[name] = {"ms": round(ms, 4), "TFLOPs": round(2.0 * m * n * k / ms / 1e9, 1), "shape": [m, n, k]}
 
     hbm("quantize_x_quest_rtn_mask", T * I, 2.65625,
-        lambda a: (lambda: K.quantize_mxfp4(a, 32, None, K.QM_QUEST_RTN, want_mask=True)), [x])
+        lambda a: (lambda: K.quantize_mxfp4(a, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)), [x])
     hbm("quantize_w_quest_rtn_mask", O * I, 2.65625,
-        lambda a: (lambda: K.quantize_mxfp4(a, 32, None, K.QM_QUEST_RTN, want_mask=True)), [w])
-    mfma("gemm_fwd", T, O, I, lambda: K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.bfloat16))
+        lambda a: (lambda: K.quantize_mxfp4(a, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)), [w])
+    mfma("gemm_fwd", T, O, I, lambda: K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
     hbm("quantize_e_absmax_sr", T * O, 2.53125,
-        lambda a: (lambda: K.quantize_mxfp4(a, 32, signs, K.QM_ABSMAX_SR, seed=1)), [dy])
+        lambda a: (lambda: K.quantize_mxfp4(a, 32, signs, K.QM_ABSMAX_SR, seed=1, tiled=tl)), [dy])
     hbm("quantize_et_absmax_sr_transposed", T * O, 2.53125,
-        lambda a: (lambda: K.quantize_mxfp4(a, 32, signs, K.QM_ABSMAX_SR, transposed_in=True, seed=2)), [dy])
+        lambda a: (lambda: K.quantize_mxfp4(a, 32, signs, K.QM_ABSMAX_SR, transposed_in=True, seed=2, tiled=tl)), [dy])
     hbm("requantize_wt", O * I, 1.0625,
-        lambda c, sc: (lambda: K.requantize_transposed_mxfp4(c, sc, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=3)),
+        lambda c, sc: (lambda: K.requantize_transposed_mxfp4(c, sc, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=3,
+                                                              tiled_in=tl, tiled_out=tl)),
         [wc, ws])
     hbm("requantize_xt", T * I, 1.0625,
-        lambda c, sc: (lambda: K.requantize_transposed_mxfp4(c, sc, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=4)),
+        lambda c, sc: (lambda: K.requantize_transposed_mxfp4(c, sc, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=4,
+                                                              tiled_in=tl, tiled_out=tl)),
         [xc, xs])
-    mfma("gemm_dgrad", T, I, O, lambda: K.gemm_mxfp4_tn(ec, es, wtc, wts, 1.0, torch.bfloat16))
-    mfma("gemm_wgrad", O, I, T, lambda: K.gemm_mxfp4_tn(etc, ets, xtc, xts, 1.0, torch.bfloat16))
+    mfma("gemm_dgrad", T, I, O, lambda: K.gemm_mxfp4_tn(ec, es, wtc, wts, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
+    mfma("gemm_wgrad", O, I, T, lambda: K.gemm_mxfp4_tn(etc, ets, xtc, xts, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
     hbm("hadamard_bwd_x", T * I, 4.125,
         lambda g, m: (lambda: K.masked_hadamard_bwd(g, 32, torch.bfloat16, None, m)), [gxq, xm])
     hbm("hadamard_bwd_w", O * I, 4.125,

@@ -9,6 +9,10 @@
  *     holds the reason, thread-local), > 0 = a hipError_t from the launch;
  *   - packed MXFP4 tensor of logical shape [R, C] (C % 32 == 0):
  *       codes  uint8 [R, C/2]   E2M1, element 2i in the low nibble of byte i, sign in bit 3
+ *                               (QM_LAYOUT_ROWMAJOR); or, for R % 16 == 0 and C % 128 == 0, QM_LAYOUT_TILED:
+ *                               the same bytes as [R/16][C/128][16 rows][64 bytes], so that the 16 rows x 128
+ *                               elements one GEMM wave-load fetches are 1 KiB contiguous.  Scales and mask bits
+ *                               are row-major in both layouts.
  *       scales uint8 [R, C/32]  E8M0 (value 2^(byte-127)), one per 32 consecutive elements
  *       mask   uint8 [R, C/8]   bit i of byte j = clip mask of element 8j+i
  *   - `sign_bits`: HOST pointer to ceil(hd/32) uint32 words, bit j set = rotated column j is
@@ -31,6 +35,9 @@ enum { QM_BF16 = 0, QM_F32 = 1 };
  * (AlbertTsengQuantizer); RTN = ties toward zero, SR = stochastic rounding */
 enum { QM_QUEST_RTN = 0, QM_ABSMAX_RTN = 1, QM_ABSMAX_SR = 2, QM_QUEST_SR = 3 };
 
+/* layout of a packed tensor's code bytes (see above); producers and consumers must agree per tensor */
+enum { QM_LAYOUT_ROWMAJOR = 0, QM_LAYOUT_TILED = 1 };
+
 #define QM_ERR_INVALID (-1)
 #define QM_ERR_UNALIGNED (-2)
 
@@ -51,11 +58,13 @@ const char* qm_last_error(void);
  *                them in-kernel from Philox4x32-10 keyed by (seed, offset)
  *   codes/scales outputs (required); maskbits, dequant optional (NULL to skip); dequant has
  *                x_dtype and logical shape and holds what the reference kernel returns
+ *   codes_layout QM_LAYOUT_TILED needs hadamard_dim 32, rows % 16 == 0, cols % 128 == 0, u == NULL for
+ *                the SR modes and, with transposed_in, maskbits == NULL; rejected otherwise
  */
 int qm_quantize_mxfp4(const void* x, int x_dtype, int64_t rows, int64_t cols, int hadamard_dim,
                       const uint32_t* sign_bits, int mode, int transposed_in, const float* u,
                       uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits,
-                      void* dequant, void* stream);
+                      void* dequant, int codes_layout, void* stream);
 
 /*
  * De-quantize a packed [R, C] tensor, transpose it, rotate and re-quantize along R:
@@ -66,22 +75,26 @@ int qm_quantize_mxfp4(const void* x, int x_dtype, int64_t rows, int64_t cols, in
  *   post       1.0 if the input was quest-coded, fl32(4/3) if absmax-coded
  *   val_dtype  dtype the reference would hold the de-quantized tensor in (selects the rounding
  *              of the Hadamard constant and of the de-quantized values)
+ *   in_layout / out_layout  layouts of codes_in / codes_out; QM_LAYOUT_TILED on either side needs
+ *              hadamard_dim 32, R % 128 == 0, C % 128 == 0 and u == NULL for the SR modes
  */
 int qm_requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R,
                                    int64_t C, float post, int val_dtype, int hadamard_dim,
                                    const uint32_t* sign_bits, int mode, const float* u,
                                    uint64_t seed, uint8_t* codes_out, uint8_t* scales_out,
-                                   void* dequant, void* stream);
+                                   void* dequant, int in_layout, int out_layout, void* stream);
 
 /*
  * C[M, N] = alpha * A[M, K] . B[N, K]^T on packed MXFP4 operands, fp32 accumulation.
  * Replaces F.linear / einsum on de-quantized operands (src/models/quantization/backward.py:62,
  * 71-75, 79-83) and matmul_mxf4_bf16_tn of notebooks/benchmark_mxfp4.ipynb.  K % 32 == 0.
  * alpha carries the per-operand constants of absmax coding (fl32(4/3) each).
+ * a_layout / b_layout: layouts of a_codes / b_codes; QM_LAYOUT_TILED needs M % 256 == 0,
+ * N % 256 == 0 and K % 128 == 0 (the shapes the 256x256-tile kernels serve).
  */
 int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                      const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c,
-                     int c_dtype, void* stream);
+                     int c_dtype, int a_layout, int b_layout, void* stream);
 
 /*
  * out = ((g * mask).view(-1, hd)) @ H^T: the straight-through backward of the forward quantizer,

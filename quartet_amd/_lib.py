@@ -10,6 +10,7 @@ LIB_PATH = os.path.join(_HERE, "libquartet_hip.so")
 
 QM_BF16, QM_F32 = 0, 1
 QM_QUEST_RTN, QM_ABSMAX_RTN, QM_ABSMAX_SR, QM_QUEST_SR = 0, 1, 2, 3
+QM_LAYOUT_ROWMAJOR, QM_LAYOUT_TILED = 0, 1
 
 EXPORTS = (
     "qm_version",
@@ -43,11 +44,11 @@ def lib():
     L.qm_last_error.restype = ctypes.c_char_p
     L.qm_last_error.argtypes = []
     L.qm_quantize_mxfp4.restype = i32
-    L.qm_quantize_mxfp4.argtypes = [vp, i32, i64, i64, i32, vp, i32, i32, vp, u64, vp, vp, vp, vp, vp]
+    L.qm_quantize_mxfp4.argtypes = [vp, i32, i64, i64, i32, vp, i32, i32, vp, u64, vp, vp, vp, vp, i32, vp]
     L.qm_requantize_transposed_mxfp4.restype = i32
-    L.qm_requantize_transposed_mxfp4.argtypes = [vp, vp, i64, i64, f32, i32, i32, vp, i32, vp, u64, vp, vp, vp, vp]
+    L.qm_requantize_transposed_mxfp4.argtypes = [vp, vp, i64, i64, f32, i32, i32, vp, i32, vp, u64, vp, vp, vp, i32, i32, vp]
     L.qm_gemm_mxfp4_tn.restype = i32
-    L.qm_gemm_mxfp4_tn.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, vp]
+    L.qm_gemm_mxfp4_tn.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, i32, vp]
     L.qm_masked_hadamard_bwd.restype = i32
     L.qm_masked_hadamard_bwd.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp, i32, vp]
     L.qm_dequantize_mxfp4.restype = i32

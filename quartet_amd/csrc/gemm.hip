@@ -19,6 +19,7 @@
 // (rows padded from 64 to 80 bytes so the 16-byte fragment reads of 16 consecutive rows hit 64
 // distinct banks), double buffered, one barrier per K step.
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdint.h>
 
 #include "qm_kernels.h"
@@ -272,6 +273,7 @@ struct BigLoadPlan {
     const uint8_t* sa;  // this lane's A scale dword source at K step 0 (+ ks * 4 bytes)
     const uint8_t* sb;
     int64_t row16_bytes;   // 16 rows of codes
+    int kstep_a, kstep_b;  // bytes from one K step to the next in this lane's source: 64 row-major, 1024 tiled
     uint32_t lds_codes;    // wave-uniform LDS byte address of this wave's first A wave-load in stage 0
     uint32_t lds_scales;   // likewise for its A scale wave-load
 };
@@ -295,11 +297,10 @@ __device__ __forceinline__ void load_lds_b32(const uint8_t* gsrc, uint32_t lds_b
 // issue the ten loads of K step ks into ring stage `stage`
 __device__ __forceinline__ void big_issue_loads(const BigLoadPlan& p, int stage, int ks) {
     const uint32_t base = p.lds_codes + stage * kStageBytes;
-    const int kb = ks * kRowBytes;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        load_lds_b128(p.a + j * p.row16_bytes + kb, base + j * 1024);
-        load_lds_b128(p.b + j * p.row16_bytes + kb, base + kBOff + j * 1024);
+        load_lds_b128(p.a + j * p.row16_bytes + ks * p.kstep_a, base + j * 1024);
+        load_lds_b128(p.b + j * p.row16_bytes + ks * p.kstep_b, base + kBOff + j * 1024);
     }
     load_lds_b32(p.sa + ks * 4, p.lds_scales + stage * kStageBytes);
     load_lds_b32(p.sb + ks * 4, p.lds_scales + stage * kStageBytes + (kSBOff - kSAOff));
@@ -329,7 +330,7 @@ __device__ __forceinline__ void big_read_scales(const uint8_t* __restrict__ stag
 // SWAP = false: A rows become result rows.  SWAP = true: B's rows (n) are fed as the MFMA's first operand and
 // A's rows (m) as its second, so a lane ends up with 4 consecutive n of one m (contiguous in row-major C),
 // which the bf16 epilogue packs into 8-byte LDS writes.
-template <int SUB, bool SWAP>
+template <int SUB, bool SWAP, bool ZERO = false>
 __device__ __forceinline__ void big_mfma_sub(const SubFrags& f, const uint32_t (&sca)[4], const uint32_t (&scb)[4],
                                              v16f (&acc)[4][4]) {
 #pragma unroll
@@ -338,10 +339,18 @@ __device__ __forceinline__ void big_mfma_sub(const SubFrags& f, const uint32_t (
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const v8i bv = v8i{(int)f.b[j].x, (int)f.b[j].y, (int)f.b[j].z, (int)f.b[j].w, 0, 0, 0, 0};
+            // ZERO: the tile's first product starts the accumulator from the constant 0 instead of reading it
+            v16f cin;
+            if constexpr (ZERO) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) cin[e] = 0.0f;
+            } else {
+                cin = acc[i][j];
+            }
             if constexpr (SWAP)
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, acc[i][j], 4, 4, SUB, (int)scb[j], SUB, (int)sca[i]);
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, cin, 4, 4, SUB, (int)scb[j], SUB, (int)sca[i]);
             else
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[i][j], 4, 4, SUB, (int)sca[i], SUB, (int)scb[j]);
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, cin, 4, 4, SUB, (int)sca[i], SUB, (int)scb[j]);
         }
     }
 }
@@ -405,7 +414,8 @@ __device__ __forceinline__ void big_epilogue(v16f (&acc)[4][4], float alpha, Out
 template <typename OutT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mxfp4_tn_big_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ b_codes,
-    const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c) {
+    const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c, int a_tiled,
+    int b_tiled) {
     extern __shared__ uint32_t smem[];
     uint8_t* smem_bytes = reinterpret_cast<uint8_t*>(smem);
     const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)smem;
@@ -424,8 +434,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         // codes: wave-load j of wave w fills LDS rows (w*4+j)*16 .. +15; lane l -> row + l/4, slot l%4
         const int row = wave * 64 + (lane >> 2);
         const int cv = (lane & 3) ^ ((row >> 2) & 3);
-        plan.a = a_codes + (m0 + row) * code_pitch + cv * 16;
-        plan.b = b_codes + (n0 + row) * code_pitch + cv * 16;
+        // tiled codes: the wave-load's 16 rows x 64 bytes are one 1 KiB tile; same (row, swizzled slot) pick inside it
+        const int trow = wave * 64;  // first row of this wave's four wave-loads
+        const int tile_off = (lane >> 2) * 64 + cv * 16;
+        plan.a = a_tiled ? a_codes + (m0 + trow) * code_pitch + tile_off : a_codes + (m0 + row) * code_pitch + cv * 16;
+        plan.b = b_tiled ? b_codes + (n0 + trow) * code_pitch + tile_off : b_codes + (n0 + row) * code_pitch + cv * 16;
+        plan.kstep_a = a_tiled ? 1024 : kRowBytes;
+        plan.kstep_b = b_tiled ? 1024 : kRowBytes;
         plan.row16_bytes = (int64_t)16 * code_pitch;
         // scales: LDS dword p = wave*64 + lane holds operand row (p>>7)*128 + (p&3)*32 + ((p>>2)&31)
         const int p = wave * 64 + lane;
@@ -528,7 +543,9 @@ struct Big4Plan {
     const uint8_t* sa;  // uniform: first scale byte of this tile's A panel
     const uint8_t* sb;
     int64_t row16_bytes;    // 16 rows of codes
-    uint32_t lane_codes;    // this lane's byte offset inside a panel for wave-load 0: row wave*64 + lane/4, swizzled 16-byte column
+    uint32_t lane_codes_a;  // this lane's byte offset inside a wave-load's source: row lane/4 + swizzled 16-byte column of a
+    uint32_t lane_codes_b;  //   row-major panel, or the same pick inside the 1 KiB tile of a tiled one
+    int kstep_a, kstep_b;   // bytes from one K step to the next: 64 row-major, 1024 tiled
     uint32_t lane_scales;   // this lane's byte offset inside a panel's scales: row wave*64 + lane
     uint32_t lds_codes;     // wave-uniform LDS address of this wave's first A wave-load in stage 0
     uint32_t lds_scales;    // wave-uniform LDS address of this wave's A scale wave-load in buffer 0
@@ -536,11 +553,10 @@ struct Big4Plan {
 
 __device__ __forceinline__ void big4_issue_codes(const Big4Plan& p, int stage, int ks) {
     const uint32_t base = p.lds_codes + stage * kCodeStageBytes;
-    const int kb = ks * kRowBytes;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        load_lds_b128_s(p.a + j * p.row16_bytes + kb, p.lane_codes, base + j * 1024);
-        load_lds_b128_s(p.b + j * p.row16_bytes + kb, p.lane_codes, base + kBOff + j * 1024);
+        load_lds_b128_s(p.a + j * p.row16_bytes + ks * p.kstep_a, p.lane_codes_a, base + j * 1024);
+        load_lds_b128_s(p.b + j * p.row16_bytes + ks * p.kstep_b, p.lane_codes_b, base + kBOff + j * 1024);
     }
 }
 __device__ __forceinline__ void big4_issue_scales(const Big4Plan& p, int qb, int buf) {
@@ -574,7 +590,7 @@ struct Big4State {
 // One K step of the flat (tile, K step) stream; the step's index in its tile is congruent to Q mod 4, so
 // the ring stage it consumes is Q.  `lks` is the K step (of the tile `plan` points at) whose codes it
 // requests into the stage it has just freed; `par` selects the scale buffer the current block lives in.
-template <int Q, bool SWAP>
+template <int Q, bool SWAP, bool FIRST = false>
 __device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_bytes, int lks, int par, int a_off0,
                                           int a_off1, int b_off0, int b_off1, int a_sc_off, int b_sc_off, int sh,
                                           Big4State& st, v16f (&acc)[4][4]) {
@@ -583,7 +599,7 @@ __device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_by
     const uint32_t sca[4] = {pick<Q>(st.sr.a[0]) >> sh, pick<Q>(st.sr.a[1]) >> sh, pick<Q>(st.sr.a[2]) >> sh, pick<Q>(st.sr.a[3]) >> sh};
     const uint32_t scb[4] = {pick<Q>(st.sr.b[0]) >> sh, pick<Q>(st.sr.b[1]) >> sh, pick<Q>(st.sr.b[2]) >> sh, pick<Q>(st.sr.b[3]) >> sh};
     big_read_sub(cur, a_off1, b_off1, st.f1);
-    big_mfma_sub<0, SWAP>(st.f0, sca, scb, acc);
+    big_mfma_sub<0, SWAP, FIRST>(st.f0, sca, scb, acc);
     QM_SCHED_PAIR(0x100, 8)
     __builtin_amdgcn_sched_barrier(0);
     // loads younger than the codes of the next step: the codes of the two steps after it (16) and, for Q = 1, 2,
@@ -650,7 +666,8 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
 template <typename OutT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mxfp4_tn_big4_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ b_codes,
-    const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c) {
+    const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c, int a_tiled,
+    int b_tiled) {
     extern __shared__ uint32_t smem[];
     uint8_t* smem_bytes = reinterpret_cast<uint8_t*>(smem);
     const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)smem;
@@ -678,7 +695,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     {
         const int prow = lane >> 2;  // the wave's 64-row offset is folded into the uniform part below
         const int pcv = (lane & 3) ^ ((prow >> 2) & 3);
-        plan.lane_codes = (uint32_t)(prow * code_pitch + pcv * 16);
+        const uint32_t rowmajor_off = (uint32_t)(prow * code_pitch + pcv * 16);
+        const uint32_t tiled_off = (uint32_t)(prow * 64 + pcv * 16);  // same (row, swizzled slot) pick inside the 1 KiB tile
+        plan.lane_codes_a = a_tiled ? tiled_off : rowmajor_off;
+        plan.lane_codes_b = b_tiled ? tiled_off : rowmajor_off;
+        plan.kstep_a = a_tiled ? 1024 : kRowBytes;
+        plan.kstep_b = b_tiled ? 1024 : kRowBytes;
         plan.lane_scales = (uint32_t)(lane * groups);
     }
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
@@ -709,16 +731,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     int par = 0;
     for (int t = (int)blockIdx.x; t < total; t += stride) {
         v16f acc[4][4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
         const int64_t m0 = (int64_t)load_tm * kBigM, n0 = (int64_t)load_tn * kBigN;  // the load stream is still in tile t
-        for (int ks = 0; ks < nk; ks += 4) {
-            // where the load stream is: four K steps ahead, rolling over into the next tile; after the last tile
-            // it re-requests the current steps (never consumed), which keeps the outstanding-load counts uniform
+        // One block of four K steps.  The load stream is four K steps ahead and rolls over into the next tile;
+        // after the last tile it re-requests the current steps (never consumed), which keeps the outstanding-load
+        // counts uniform.  FIRST: the tile's first products overwrite the accumulators instead of adding to them.
+        auto block4 = [&](int ks, auto first) {
+            constexpr bool FIRST = decltype(first)::value;
             int lks = ks + 4;
             if (lks == nk) {
                 if (t + stride < total) {
@@ -728,12 +746,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     lks = ks;
                 }
             }
-            big4_step<0, sizeof(OutT) == 2>(plan, smem_bytes, lks, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+            big4_step<0, sizeof(OutT) == 2, FIRST>(plan, smem_bytes, lks, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
             big4_step<1, sizeof(OutT) == 2>(plan, smem_bytes, lks + 1, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
             big4_step<2, sizeof(OutT) == 2>(plan, smem_bytes, lks + 2, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
             big4_step<3, sizeof(OutT) == 2>(plan, smem_bytes, lks + 3, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
             par ^= 1;
-        }
+        };
+        block4(0, std::true_type{});
+        for (int ks = 4; ks < nk; ks += 4) block4(ks, std::false_type{});
         if constexpr (sizeof(OutT) == 2) {
             big4_epilogue_bf16(acc, alpha, reinterpret_cast<uint16_t*>(c), m0, n0, N, wm, wn, wave, lane, smem_bytes);
         } else {
@@ -750,8 +770,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
 template <typename OutT>
 hipError_t launch_big4(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
-                       const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c,
-                       hipStream_t stream) {
+                       const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_tiled,
+                       int b_tiled, hipStream_t stream) {
     auto kern = gemm_mxfp4_tn_big4_kernel<OutT>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kBig4SmemBytes);
     if (e != hipSuccess) return e;
@@ -768,20 +788,20 @@ hipError_t launch_big4(const uint8_t* a_codes, const uint8_t* a_scales, const ui
     if (g > 8) g -= g % 8;
     dim3 grid((unsigned)g), block(256);
     kern<<<grid, block, kBig4SmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
-                                                  reinterpret_cast<OutT*>(c));
+                                                  reinterpret_cast<OutT*>(c), a_tiled, b_tiled);
     return hipGetLastError();
 }
 
 template <typename OutT>
 hipError_t launch_big(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
-                      const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c,
-                      hipStream_t stream) {
+                      const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_tiled,
+                      int b_tiled, hipStream_t stream) {
     auto kern = gemm_mxfp4_tn_big_kernel<OutT>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kBigSmemBytes);
     if (e != hipSuccess) return e;
     dim3 grid((unsigned)((M / kBigM) * (N / kBigN))), block(256);
     kern<<<grid, block, kBigSmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
-                                                 reinterpret_cast<OutT*>(c));
+                                                 reinterpret_cast<OutT*>(c), a_tiled, b_tiled);
     return hipGetLastError();
 }
 
@@ -811,18 +831,25 @@ hipError_t launch_gemm(const uint8_t* a_codes, const uint8_t* a_scales, const ui
 
 }  // namespace
 
+// tiled operands are read by the 256x256-tile kernels only
+bool gemm_supports_tiled(int64_t M, int64_t N, int64_t K) {
+    return M % kBigM == 0 && N % kBigN == 0 && K > 0 && K % kBK == 0 && M < (1 << 30) && N < (1 << 30) && K < (1 << 30);
+}
+
 hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                          const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
-                         hipStream_t stream) {
+                         int a_layout, int b_layout, hipStream_t stream) {
     if (M == 0 || N == 0) return hipSuccess;
-    const bool big_ok = M % kBigM == 0 && N % kBigN == 0 && K > 0 && M < (1 << 30) && N < (1 << 30) && K < (1 << 30);
+    const int at = a_layout == LAYOUT_TILED, bt = b_layout == LAYOUT_TILED;
+    const bool big_ok = gemm_supports_tiled(M, N, K);
+    if ((at || bt) && !big_ok) return hipErrorInvalidValue;
     if (big_ok && K % 512 == 0 && (reinterpret_cast<uintptr_t>(a_scales) & 15) == 0 && (reinterpret_cast<uintptr_t>(b_scales) & 15) == 0) {
-        if (c_dtype == BF16) return launch_big4<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, stream);
-        return launch_big4<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, stream);
+        if (c_dtype == BF16) return launch_big4<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, stream);
+        return launch_big4<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, stream);
     }
-    if (big_ok && K % kBK == 0) {
-        if (c_dtype == BF16) return launch_big<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, stream);
-        return launch_big<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, stream);
+    if (big_ok) {
+        if (c_dtype == BF16) return launch_big<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, stream);
+        return launch_big<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, stream);
     }
     return launch_gemm<128, 128, 64, 64>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, c_dtype, stream);
 }

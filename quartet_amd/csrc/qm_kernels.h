@@ -11,29 +11,44 @@ struct SignBits {
     uint32_t w[4];
 };
 
+// Code-byte layouts of a packed [R, C] tensor.  ROWMAJOR: [R][C/2].  TILED (R % 16 == 0, C % 128 == 0):
+// [R/16][C/128][16 rows][64 bytes] -- the 16 rows x 128 elements one GEMM wave-load fetches are 1 KiB contiguous.
+enum CodeLayout : int { LAYOUT_ROWMAJOR = 0, LAYOUT_TILED = 1 };
+
+// byte offset of the 64-byte piece (row r, column block kb) in the tiled layout
+__host__ __device__ inline int64_t tiled_code_offset(int64_t r, int64_t kb, int64_t kblocks) {
+    return (((r >> 4) * kblocks + kb) << 10) + ((r & 15) << 6);
+}
+
 hipError_t quantize_mxfp4(const void* x, int dtype, int64_t rows, int64_t cols, int hd, const SignBits& sb, int mode,
                           bool transposed_in, const float* u, uint64_t seed, uint8_t* codes, uint8_t* scales,
-                          uint8_t* maskbits, void* dequant, hipStream_t stream);
+                          uint8_t* maskbits, void* dequant, int codes_layout, hipStream_t stream);
+// whether quantize_mxfp4 / requantize_transposed_mxfp4 can emit (read) tiled codes for these arguments
+bool quantize_supports_tiled(int64_t rows, int64_t cols, int hd, int mode, bool transposed_in, const float* u,
+                             const uint8_t* maskbits);
+bool requantize_supports_tiled(int64_t R, int64_t C, int hd, int mode, const float* u);
+bool gemm_supports_tiled(int64_t M, int64_t N, int64_t K);
 
 // hd = 32 fast path (one MX group per lane, hardware FP4 converts); row-major input, RTN or Philox SR
-hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t n, uint32_t sign_word, int mode, uint64_t seed,
-                                  uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
-                                  hipStream_t stream);
+hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t rows, int64_t cols, uint32_t sign_word, int mode,
+                                  uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
+                                  bool tiled, hipStream_t stream);
 
 hipError_t quantize_transposed_hd32(const void* x, int dtype, int64_t P, int64_t Q, uint32_t sign_word, int mode,
-                                    uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant, hipStream_t stream);
+                                    uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant, bool tiled,
+                                    hipStream_t stream);
 hipError_t requantize_transposed_hd32(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C, float post,
                                       int val_dtype, uint32_t sign_word, int mode, uint64_t seed, uint8_t* codes,
-                                      uint8_t* scales, void* dequant, hipStream_t stream);
+                                      uint8_t* scales, void* dequant, bool tiled_in, bool tiled_out, hipStream_t stream);
 
 hipError_t requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C,
                                        float post, int val_dtype, int hd, const SignBits& sb, int mode, const float* u,
                                        uint64_t seed, uint8_t* codes_out, uint8_t* scales_out, void* dequant,
-                                       hipStream_t stream);
+                                       int in_layout, int out_layout, hipStream_t stream);
 
 hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                          const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
-                         hipStream_t stream);
+                         int a_layout, int b_layout, hipStream_t stream);
 
 hipError_t masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t cols, int hd, int scale_dtype,
                                const SignBits& sb, const uint8_t* maskbits, void* out, int out_dtype,

@@ -395,18 +395,33 @@ void dispatch_hd(int hd, F&& f) {
 
 }  // namespace
 
+// The tiled code layout exists on the Hadamard-32 group-layout kernels only.
+bool quantize_supports_tiled(int64_t rows, int64_t cols, int hd, int mode, bool transposed_in, const float* u,
+                             const uint8_t* maskbits) {
+    const bool rtn = (mode == QUEST_RTN || mode == ABSMAX_RTN);
+    if (hd != 32 || !(rtn || u == nullptr) || rows % 16 || cols % 128) return false;
+    return !transposed_in || maskbits == nullptr;
+}
+bool requantize_supports_tiled(int64_t R, int64_t C, int hd, int mode, const float* u) {
+    const bool rtn = (mode == QUEST_RTN || mode == ABSMAX_RTN);
+    return hd == 32 && (rtn || u == nullptr) && R % 128 == 0 && C % 128 == 0;
+}
+
 hipError_t quantize_mxfp4(const void* x, int dtype, int64_t rows, int64_t cols, int hd, const SignBits& sb, int mode,
                           bool transposed_in, const float* u, uint64_t seed, uint8_t* codes, uint8_t* scales,
-                          uint8_t* maskbits, void* dequant, hipStream_t stream) {
+                          uint8_t* maskbits, void* dequant, int codes_layout, hipStream_t stream) {
     if (rows == 0 || cols == 0) return hipSuccess;
     const bool rtn = (mode == QUEST_RTN || mode == ABSMAX_RTN);
+    const bool tiled = codes_layout == LAYOUT_TILED;
+    if (tiled && !quantize_supports_tiled(rows, cols, hd, mode, transposed_in, u, maskbits)) return hipErrorInvalidValue;
     const auto al = [](const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
+    if (tiled && !(al(codes, 16) && al(maskbits, 4) && al(scales, 4))) return hipErrorInvalidValue;
     if (hd == 32 && !transposed_in && (rtn || u == nullptr) && al(codes, 16) && al(maskbits, 4))
-        return quantize_rowmajor_hd32(x, dtype, rows * cols, sb.w[0], mode, seed, codes, scales, maskbits, dequant, stream);
+        return quantize_rowmajor_hd32(x, dtype, rows, cols, sb.w[0], mode, seed, codes, scales, maskbits, dequant, tiled, stream);
     // logical [rows, cols] = physical [P = cols, Q = rows]
     if (hd == 32 && transposed_in && (rtn || u == nullptr) && maskbits == nullptr && al(codes, 16) && al(scales, 4) &&
         cols % 128 == 0)
-        return quantize_transposed_hd32(x, dtype, cols, rows, sb.w[0], mode, seed, codes, scales, dequant, stream);
+        return quantize_transposed_hd32(x, dtype, cols, rows, sb.w[0], mode, seed, codes, scales, dequant, tiled, stream);
     QuantOut out{reinterpret_cast<uint32_t*>(codes), scales, maskbits, dequant};
     const float c = hadamard_scale(hd, dtype);
     dispatch_hd(hd, [&](auto HDc) {
@@ -426,13 +441,16 @@ hipError_t quantize_mxfp4(const void* x, int dtype, int64_t rows, int64_t cols, 
 hipError_t requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C,
                                        float post, int val_dtype, int hd, const SignBits& sb, int mode, const float* u,
                                        uint64_t seed, uint8_t* codes_out, uint8_t* scales_out, void* dequant,
-                                       hipStream_t stream) {
+                                       int in_layout, int out_layout, hipStream_t stream) {
     if (R == 0 || C == 0) return hipSuccess;
     const bool rtn = (mode == QUEST_RTN || mode == ABSMAX_RTN);
+    const bool tiled_in = in_layout == LAYOUT_TILED, tiled_out = out_layout == LAYOUT_TILED;
     const auto al = [](const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
-    if (hd == 32 && (rtn || u == nullptr) && al(codes_out, 16) && al(scales_out, 4) && R % 128 == 0)
+    const bool fast = hd == 32 && (rtn || u == nullptr) && al(codes_out, 16) && al(scales_out, 4) && R % 128 == 0;
+    if ((tiled_in || tiled_out) && !(fast && requantize_supports_tiled(R, C, hd, mode, u))) return hipErrorInvalidValue;
+    if (fast)
         return requantize_transposed_hd32(codes_in, scales_in, R, C, post, val_dtype, sb.w[0], mode, seed, codes_out,
-                                          scales_out, dequant, stream);
+                                          scales_out, dequant, tiled_in, tiled_out, stream);
     QuantOut out{reinterpret_cast<uint32_t*>(codes_out), scales_out, nullptr, dequant};
     const float c = hadamard_scale(hd, val_dtype);
     dispatch_hd(hd, [&](auto HDc) {

@@ -242,14 +242,15 @@ __device__ __forceinline__ void rotate_group(float (&v)[32], float c, uint32_t s
     }
 }
 
-// rotate (hd = 32) + quantize the group in v, write its outputs at group index gi
+// rotate (hd = 32) + quantize the group in v; gi is its logical (row-major) group index, which also keys the
+// random stream; ci is the index of its 16 code bytes in the code buffer (= gi for row-major codes)
 template <typename T, int MODE, bool WANT_MASK>
-__device__ __forceinline__ void finish_group(float (&v)[32], int64_t gi, float c, uint32_t sign_word, uint64_t seed,
-                                             const GroupOut& out) {
+__device__ __forceinline__ void finish_group(float (&v)[32], int64_t gi, int64_t ci, float c, uint32_t sign_word,
+                                             uint64_t seed, const GroupOut& out) {
     rotate_group(v, c, sign_word);
     GroupCodes o;
     quantize_group_regs<MODE, WANT_MASK>(v, seed, gi, o);
-    out.codes[gi] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
+    out.codes[ci] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
     out.scales[gi] = (uint8_t)o.scale_byte;
     if constexpr (WANT_MASK) out.maskbits[gi] = o.keep;
     if (out.dequant) store_dequant<T>(reinterpret_cast<T*>(out.dequant) + gi * 32, o);
@@ -262,15 +263,44 @@ __global__ __launch_bounds__(256) void quantize_rowmajor_g32_kernel(const T* __r
     if (gi >= n_groups) return;
     float v[32];
     load_group<T>(x + gi * 32, v);
-    finish_group<T, MODE, WANT_MASK>(v, gi, c, sign_word, seed, out);
+    finish_group<T, MODE, WANT_MASK>(v, gi, gi, c, sign_word, seed, out);
+}
+
+// Tiled code layout ([rows/16][cols/128][16 rows][64 bytes]): a wave owns one 1 KiB tile = 16 rows x 4 groups, so
+// its codes leave as one contiguous KiB; its input is 16 row segments of 4 groups (256 bytes of bf16) each.
+// blockIdx.x = block of 16 rows, blockIdx.y = run of four 128-column blocks (one per wave).
+template <typename T, int MODE, bool WANT_MASK>
+__global__ __launch_bounds__(256) void quantize_rowmajor_g32_tiled_kernel(const T* __restrict__ x, int64_t cols, float c,
+                                                                          uint32_t sign_word, uint64_t seed,
+                                                                          GroupOut out) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t kblocks = cols / 128;
+    const int64_t kb = (int64_t)blockIdx.y * 4 + wave;
+    if (kb >= kblocks) return;
+    const int64_t r = (int64_t)blockIdx.x * 16 + (lane >> 2);
+    const int64_t gi = r * (cols / 32) + kb * 4 + (lane & 3);
+    const int64_t ci = ((int64_t)blockIdx.x * kblocks + kb) * 64 + lane;
+    float v[32];
+    load_group<T>(x + gi * 32, v);
+    finish_group<T, MODE, WANT_MASK>(v, gi, ci, c, sign_word, seed, out);
 }
 
 template <typename T, bool WANT_MASK>
-void launch_rowmajor_g32(int mode, const void* x, int64_t n, float c, uint32_t sign_word, uint64_t seed,
-                         const GroupOut& out, hipStream_t stream) {
-    const int64_t n_groups = n / 32;
-    dim3 grid((unsigned)((n_groups + 255) / 256)), block(256);
+void launch_rowmajor_g32(int mode, const void* x, int64_t rows, int64_t cols, bool tiled, float c, uint32_t sign_word,
+                         uint64_t seed, const GroupOut& out, hipStream_t stream) {
     const T* xp = reinterpret_cast<const T*>(x);
+    if (tiled) {
+        dim3 grid((unsigned)(rows / 16), (unsigned)((cols / 128 + 3) / 4)), block(256);
+        switch (mode) {
+            case QUEST_RTN: quantize_rowmajor_g32_tiled_kernel<T, QUEST_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, c, sign_word, seed, out); break;
+            case ABSMAX_RTN: quantize_rowmajor_g32_tiled_kernel<T, ABSMAX_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, c, sign_word, seed, out); break;
+            case ABSMAX_SR: quantize_rowmajor_g32_tiled_kernel<T, ABSMAX_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, c, sign_word, seed, out); break;
+            default: quantize_rowmajor_g32_tiled_kernel<T, QUEST_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, c, sign_word, seed, out); break;
+        }
+        return;
+    }
+    const int64_t n_groups = rows * cols / 32;
+    dim3 grid((unsigned)((n_groups + 255) / 256)), block(256);
     switch (mode) {
         case QUEST_RTN: quantize_rowmajor_g32_kernel<T, QUEST_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
         case ABSMAX_RTN: quantize_rowmajor_g32_kernel<T, ABSMAX_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
@@ -297,7 +327,7 @@ __global__ __launch_bounds__(256) void quantize_transposed_g32_kernel(const T* _
                                                                       float c, uint32_t sign_word, uint64_t seed,
                                                                       uint8_t* __restrict__ codes,
                                                                       uint8_t* __restrict__ scales,
-                                                                      void* __restrict__ dequant) {
+                                                                      void* __restrict__ dequant, bool tiled_out) {
     constexpr int TQ = TrTile<T>::kQ;
     constexpr int GPL = TrTile<T>::kGroupsPerLane;
     __shared__ uint4 ocodes[TQ * 4];      // [q][4 groups x 16 B]
@@ -336,8 +366,12 @@ __global__ __launch_bounds__(256) void quantize_transposed_g32_kernel(const T* _
     const int64_t code_pitch = P / 2, scale_pitch = P / 32;
     for (int idx = tid; idx < TQ * 4; idx += 256) {
         const int ql = idx >> 2, part = idx & 3;
-        if (q0 + ql < Q && p0 + part * 32 < P)
-            *reinterpret_cast<uint4*>(codes + (q0 + ql) * code_pitch + p0 / 2 + part * 16) = ocodes[idx];
+        if (q0 + ql < Q && p0 + part * 32 < P) {
+            // tiled: this workgroup's 128 p are one 64-byte column block, so 16 consecutive q rows form one 1 KiB tile
+            const int64_t off = tiled_out ? tiled_code_offset(q0 + ql, p0 / 128, P / 128) + part * 16
+                                          : (q0 + ql) * code_pitch + p0 / 2 + part * 16;
+            *reinterpret_cast<uint4*>(codes + off) = ocodes[idx];
+        }
     }
     if (tid < TQ && q0 + tid < Q) {
         const uint32_t sw = oscales[tid];
@@ -366,7 +400,8 @@ __global__ __launch_bounds__(256) void requantize_transposed_g32_kernel(const ui
                                                                         uint32_t sign_word, uint64_t seed,
                                                                         uint8_t* __restrict__ codes,
                                                                         uint8_t* __restrict__ scales,
-                                                                        void* __restrict__ dequant) {
+                                                                        void* __restrict__ dequant, bool tiled_in,
+                                                                        bool tiled_out) {
     using T = typename std::conditional<VAL_DTYPE == BF16, uint16_t, float>::type;
     __shared__ uint4 ocodes[kRqC * 4];
     __shared__ uint32_t oscales[kRqC];
@@ -378,12 +413,16 @@ __global__ __launch_bounds__(256) void requantize_transposed_g32_kernel(const ui
     const bool active = rbase < R && ca < C;     // C % 32 == 0: both columns of the pair or none
     if (active) {
         float v[2][32];
-        const uint8_t* cp = codes_in + rbase * in_code_pitch + ca / 2;
+        // tiled input: the lane's byte column sits at offset `lane` of the 64-byte rows of column block c0/128
+        const uint8_t* cp = tiled_in ? codes_in + tiled_code_offset(rbase, c0 / 128, C / 128) + lane
+                                     : codes_in + rbase * in_code_pitch + ca / 2;
+        const int64_t row_step = tiled_in ? 64 : in_code_pitch;                            // next row of a 16-row block
+        const int64_t block_step = tiled_in ? (C / 128) * 1024 - 16 * 64 : 0;              // extra hop into the next block
         const uint8_t* sp = scales_in + rbase * in_scale_pitch + ca / 32;
         uint32_t byte[32], sbyte[32];
 #pragma unroll
         for (int i = 0; i < 32; ++i) {
-            byte[i] = cp[i * in_code_pitch];
+            byte[i] = cp[i * row_step + (i >> 4) * block_step];
             sbyte[i] = sp[i * in_scale_pitch];
         }
 #pragma unroll
@@ -416,8 +455,11 @@ __global__ __launch_bounds__(256) void requantize_transposed_g32_kernel(const ui
     const int64_t code_pitch = R / 2, scale_pitch = R / 32;
     for (int idx = tid; idx < kRqC * 4; idx += 256) {
         const int cl = idx >> 2, part = idx & 3;
-        if (c0 + cl < C && r0 + part * 32 < R)
-            *reinterpret_cast<uint4*>(codes + (c0 + cl) * code_pitch + r0 / 2 + part * 16) = ocodes[idx];
+        if (c0 + cl < C && r0 + part * 32 < R) {
+            const int64_t off = tiled_out ? tiled_code_offset(c0 + cl, r0 / 128, R / 128) + part * 16
+                                          : (c0 + cl) * code_pitch + r0 / 2 + part * 16;
+            *reinterpret_cast<uint4*>(codes + off) = ocodes[idx];
+        }
     }
     if (tid < kRqC && c0 + tid < C) {
         const uint32_t sw = oscales[tid];
@@ -433,63 +475,64 @@ __global__ __launch_bounds__(256) void requantize_transposed_g32_kernel(const ui
 
 template <typename T>
 void launch_transposed_g32(int mode, const void* x, int64_t P, int64_t Q, float c, uint32_t sign_word, uint64_t seed,
-                           uint8_t* codes, uint8_t* scales, void* dequant, hipStream_t stream) {
+                           uint8_t* codes, uint8_t* scales, void* dequant, bool tiled, hipStream_t stream) {
     dim3 grid((unsigned)((P + kTrP - 1) / kTrP), (unsigned)((Q + TrTile<T>::kQ - 1) / TrTile<T>::kQ)), block(256);
     const T* xp = reinterpret_cast<const T*>(x);
     switch (mode) {
-        case QUEST_RTN: quantize_transposed_g32_kernel<T, QUEST_RTN><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant); break;
-        case ABSMAX_RTN: quantize_transposed_g32_kernel<T, ABSMAX_RTN><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant); break;
-        case ABSMAX_SR: quantize_transposed_g32_kernel<T, ABSMAX_SR><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant); break;
-        default: quantize_transposed_g32_kernel<T, QUEST_SR><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant); break;
+        case QUEST_RTN: quantize_transposed_g32_kernel<T, QUEST_RTN><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant, tiled); break;
+        case ABSMAX_RTN: quantize_transposed_g32_kernel<T, ABSMAX_RTN><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant, tiled); break;
+        case ABSMAX_SR: quantize_transposed_g32_kernel<T, ABSMAX_SR><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant, tiled); break;
+        default: quantize_transposed_g32_kernel<T, QUEST_SR><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant, tiled); break;
     }
 }
 
 template <int VAL_DTYPE>
 void launch_requant_g32(int mode, const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C, float post,
                         float c, uint32_t sign_word, uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant,
-                        hipStream_t stream) {
+                        bool tiled_in, bool tiled_out, hipStream_t stream) {
     dim3 grid((unsigned)((R + kRqR - 1) / kRqR), (unsigned)((C + kRqC - 1) / kRqC)), block(256);
     switch (mode) {
-        case QUEST_RTN: requantize_transposed_g32_kernel<VAL_DTYPE, QUEST_RTN><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant); break;
-        case ABSMAX_RTN: requantize_transposed_g32_kernel<VAL_DTYPE, ABSMAX_RTN><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant); break;
-        case ABSMAX_SR: requantize_transposed_g32_kernel<VAL_DTYPE, ABSMAX_SR><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant); break;
-        default: requantize_transposed_g32_kernel<VAL_DTYPE, QUEST_SR><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant); break;
+        case QUEST_RTN: requantize_transposed_g32_kernel<VAL_DTYPE, QUEST_RTN><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out); break;
+        case ABSMAX_RTN: requantize_transposed_g32_kernel<VAL_DTYPE, ABSMAX_RTN><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out); break;
+        case ABSMAX_SR: requantize_transposed_g32_kernel<VAL_DTYPE, ABSMAX_SR><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out); break;
+        default: requantize_transposed_g32_kernel<VAL_DTYPE, QUEST_SR><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out); break;
     }
 }
 
 }  // namespace
 
 // hd = 32, row-major input, RTN or Philox-driven SR (explicit uniforms take the generic path)
-hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t n, uint32_t sign_word, int mode, uint64_t seed,
-                                  uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
-                                  hipStream_t stream) {
+hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t rows, int64_t cols, uint32_t sign_word, int mode,
+                                  uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
+                                  bool tiled, hipStream_t stream) {
     GroupOut out{reinterpret_cast<uint4*>(codes), scales, reinterpret_cast<uint32_t*>(maskbits), dequant};
     const float c = hadamard_scale(32, dtype);
     if (maskbits) {
-        if (dtype == BF16) launch_rowmajor_g32<uint16_t, true>(mode, x, n, c, sign_word, seed, out, stream);
-        else launch_rowmajor_g32<float, true>(mode, x, n, c, sign_word, seed, out, stream);
+        if (dtype == BF16) launch_rowmajor_g32<uint16_t, true>(mode, x, rows, cols, tiled, c, sign_word, seed, out, stream);
+        else launch_rowmajor_g32<float, true>(mode, x, rows, cols, tiled, c, sign_word, seed, out, stream);
     } else {
-        if (dtype == BF16) launch_rowmajor_g32<uint16_t, false>(mode, x, n, c, sign_word, seed, out, stream);
-        else launch_rowmajor_g32<float, false>(mode, x, n, c, sign_word, seed, out, stream);
+        if (dtype == BF16) launch_rowmajor_g32<uint16_t, false>(mode, x, rows, cols, tiled, c, sign_word, seed, out, stream);
+        else launch_rowmajor_g32<float, false>(mode, x, rows, cols, tiled, c, sign_word, seed, out, stream);
     }
     return hipGetLastError();
 }
 
 // hd = 32, x is [P, Q] row-major and the output is its transpose quantized along P; no clip mask
 hipError_t quantize_transposed_hd32(const void* x, int dtype, int64_t P, int64_t Q, uint32_t sign_word, int mode,
-                                    uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant, hipStream_t stream) {
+                                    uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant, bool tiled,
+                                    hipStream_t stream) {
     const float c = hadamard_scale(32, dtype);
-    if (dtype == BF16) launch_transposed_g32<uint16_t>(mode, x, P, Q, c, sign_word, seed, codes, scales, dequant, stream);
-    else launch_transposed_g32<float>(mode, x, P, Q, c, sign_word, seed, codes, scales, dequant, stream);
+    if (dtype == BF16) launch_transposed_g32<uint16_t>(mode, x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled, stream);
+    else launch_transposed_g32<float>(mode, x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled, stream);
     return hipGetLastError();
 }
 
 hipError_t requantize_transposed_hd32(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C, float post,
                                       int val_dtype, uint32_t sign_word, int mode, uint64_t seed, uint8_t* codes,
-                                      uint8_t* scales, void* dequant, hipStream_t stream) {
+                                      uint8_t* scales, void* dequant, bool tiled_in, bool tiled_out, hipStream_t stream) {
     const float c = hadamard_scale(32, val_dtype);
-    if (val_dtype == BF16) launch_requant_g32<BF16>(mode, codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, stream);
-    else launch_requant_g32<F32>(mode, codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, stream);
+    if (val_dtype == BF16) launch_requant_g32<BF16>(mode, codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out, stream);
+    else launch_requant_g32<F32>(mode, codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out, stream);
     return hipGetLastError();
 }
 

@@ -5,7 +5,8 @@ import ctypes
 import torch
 
 from . import _lib
-from ._lib import QM_ABSMAX_RTN, QM_ABSMAX_SR, QM_BF16, QM_F32, QM_QUEST_RTN, QM_QUEST_SR  # noqa: F401
+from ._lib import (QM_ABSMAX_RTN, QM_ABSMAX_SR, QM_BF16, QM_F32, QM_LAYOUT_ROWMAJOR, QM_LAYOUT_TILED,  # noqa: F401
+                   QM_QUEST_RTN, QM_QUEST_SR)
 
 FOUR_THIRDS = float(torch.tensor(1.0 / 0.75, dtype=torch.float32))
 
@@ -43,10 +44,27 @@ def sign_words(sign_bits):
     return (ctypes.c_uint32 * 4)(*[(sign_bits >> (32 * i)) & 0xFFFFFFFF for i in range(4)])
 
 
+def tile_codes(codes):
+    """Row-major code bytes [R, C/2] -> the tiled layout [R/16][C/128][16][64], returned with the same shape."""
+    R, B = codes.shape
+    return codes.view(R // 16, 16, B // 64, 64).permute(0, 2, 1, 3).contiguous().view(R, B)
+
+
+def untile_codes(codes):
+    """Inverse of tile_codes: tiled code bytes (held as an [R, C/2] tensor) -> row-major [R, C/2]."""
+    R, B = codes.shape
+    return codes.view(R // 16, B // 64, 16, 64).permute(0, 2, 1, 3).contiguous().view(R, B)
+
+
+def _layout(tiled):
+    return QM_LAYOUT_TILED if tiled else QM_LAYOUT_ROWMAJOR
+
+
 def quantize_mxfp4(x, hadamard_dim=32, sign_bits=None, mode=QM_QUEST_RTN, transposed_in=False, u=None, seed=0,
-                   want_mask=False, want_dequant=False):
+                   want_mask=False, want_dequant=False, tiled=False):
     """x: 2-D contiguous tensor.  Returns (codes [R,C/2] u8, scales [R,C/32] u8, maskbits [R,C/8] u8 | None,
-    dequant [R,C] like x | None) for the logical [R,C] tensor (x, or x.T when transposed_in)."""
+    dequant [R,C] like x | None) for the logical [R,C] tensor (x, or x.T when transposed_in).  With `tiled` the
+    code bytes come in the tiled layout (see tile_codes); scales and mask stay row-major."""
     _require_cuda(x, u)
     assert x.dim() == 2 and x.is_contiguous()
     rows, cols = (x.shape[1], x.shape[0]) if transposed_in else x.shape
@@ -59,13 +77,13 @@ def quantize_mxfp4(x, hadamard_dim=32, sign_bits=None, mode=QM_QUEST_RTN, transp
         assert u.dtype == torch.float32 and u.is_contiguous() and u.numel() == rows * cols
     rc = _lib.lib().qm_quantize_mxfp4(_ptr(x), _dtype_code(x.dtype), rows, cols, hadamard_dim, sign_words(sign_bits),
                                       mode, int(transposed_in), _ptr(u), seed, _ptr(codes), _ptr(scales), _ptr(mask),
-                                      _ptr(deq), _stream())
+                                      _ptr(deq), _layout(tiled), _stream())
     _lib.check(rc, "qm_quantize_mxfp4")
     return codes, scales, mask, deq
 
 
 def requantize_transposed_mxfp4(codes, scales, post=1.0, val_dtype=torch.bfloat16, hadamard_dim=32, sign_bits=None,
-                                mode=QM_ABSMAX_SR, u=None, seed=0, want_dequant=False):
+                                mode=QM_ABSMAX_SR, u=None, seed=0, want_dequant=False, tiled_in=False, tiled_out=False):
     """codes [R,C/2], scales [R,C/32] -> (codes [C,R/2], scales [C,R/32], dequant [C,R] | None)."""
     _require_cuda(codes, scales, u)
     assert codes.is_contiguous() and scales.is_contiguous()
@@ -76,12 +94,13 @@ def requantize_transposed_mxfp4(codes, scales, post=1.0, val_dtype=torch.bfloat1
     deq = torch.empty((C, R), dtype=val_dtype, device=dev) if want_dequant else None
     rc = _lib.lib().qm_requantize_transposed_mxfp4(_ptr(codes), _ptr(scales), R, C, post, _dtype_code(val_dtype),
                                                    hadamard_dim, sign_words(sign_bits), mode, _ptr(u), seed,
-                                                   _ptr(codes_out), _ptr(scales_out), _ptr(deq), _stream())
+                                                   _ptr(codes_out), _ptr(scales_out), _ptr(deq), _layout(tiled_in),
+                                                   _layout(tiled_out), _stream())
     _lib.check(rc, "qm_requantize_transposed_mxfp4")
     return codes_out, scales_out, deq
 
 
-def gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, alpha=1.0, out_dtype=torch.bfloat16):
+def gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, alpha=1.0, out_dtype=torch.bfloat16, a_tiled=False, b_tiled=False):
     """[M,K/2],[M,K/32] x [N,K/2],[N,K/32] -> alpha * A @ B^T as [M,N] of out_dtype."""
     _require_cuda(a_codes, a_scales, b_codes, b_scales)
     M, K = a_codes.shape[0], a_codes.shape[1] * 2
@@ -90,7 +109,7 @@ def gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, alpha=1.0, out_dtype=tor
         raise _lib.QuartetHipError(f"gemm_mxfp4_tn: contraction sizes differ ({K} vs {b_codes.shape[1] * 2})")
     c = torch.empty((M, N), dtype=out_dtype, device=a_codes.device)
     rc = _lib.lib().qm_gemm_mxfp4_tn(_ptr(a_codes), _ptr(a_scales), _ptr(b_codes), _ptr(b_scales), M, N, K, alpha,
-                                     _ptr(c), _dtype_code(out_dtype), _stream())
+                                     _ptr(c), _dtype_code(out_dtype), _layout(a_tiled), _layout(b_tiled), _stream())
     _lib.check(rc, "qm_gemm_mxfp4_tn")
     return c
 

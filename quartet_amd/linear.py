@@ -30,11 +30,16 @@ class QuartetLinearFn(torch.autograd.Function):
         x2 = x.reshape(-1, in_features).contiguous()
         w2 = weight.contiguous()
         out_dtype = torch.bfloat16 if _autocast_bf16() else x.dtype
-        xc, xs, xm, _ = K.quantize_mxfp4(x2, a_q.hadamard_dim, a_q.sign_bits, K.QM_QUEST_RTN, want_mask=True)
-        wc, ws, wm, _ = K.quantize_mxfp4(w2, w_q.hadamard_dim, w_q.sign_bits, K.QM_QUEST_RTN, want_mask=True)
-        y = K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, out_dtype)
+        # Tiled code bytes (16 rows x 128 elements contiguous) when every operand of the three products qualifies:
+        # all three extents multiples of 256 and Hadamard block 32 throughout; row-major codes otherwise.
+        tiled = (x2.shape[0] % 256 == 0 and in_features % 256 == 0 and weight.shape[0] % 256 == 0 and
+                 a_q.hadamard_dim == 32 and w_q.hadamard_dim == 32 and g_q.hadamard_dim == 32)
+        xc, xs, xm, _ = K.quantize_mxfp4(x2, a_q.hadamard_dim, a_q.sign_bits, K.QM_QUEST_RTN, want_mask=True, tiled=tiled)
+        wc, ws, wm, _ = K.quantize_mxfp4(w2, w_q.hadamard_dim, w_q.sign_bits, K.QM_QUEST_RTN, want_mask=True, tiled=tiled)
+        y = K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, out_dtype, a_tiled=tiled, b_tiled=tiled)
         ctx.save_for_backward(xc, xs, xm, wc, ws, wm)
         ctx.g_q = g_q
+        ctx.tiled = tiled
         ctx.fwd = (a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits)
         ctx.x_shape, ctx.x_dtype, ctx.w_dtype = x.shape, x.dtype, weight.dtype
         return y.view(*x.shape[:-1], weight.shape[0])
@@ -53,13 +58,16 @@ class QuartetLinearFn(torch.autograd.Function):
         mid_dtype = torch.bfloat16 if low else e2.dtype
         alpha = K.FOUR_THIRDS * K.FOUR_THIRDS  # both operands are absmax-coded: value = code * 2^k * 4/3
 
-        ec, es, _, _ = K.quantize_mxfp4(e2, hd, signs, mode, seed=seed())
-        wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, ctx.w_dtype, hd, signs, mode, seed=seed())
-        gxq = K.gemm_mxfp4_tn(ec, es, wtc, wts, alpha, mid_dtype)
+        t = ctx.tiled
+        ec, es, _, _ = K.quantize_mxfp4(e2, hd, signs, mode, seed=seed(), tiled=t)
+        wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, ctx.w_dtype, hd, signs, mode, seed=seed(),
+                                                    tiled_in=t, tiled_out=t)
+        gxq = K.gemm_mxfp4_tn(ec, es, wtc, wts, alpha, mid_dtype, a_tiled=t, b_tiled=t)
 
-        etc, ets, _, _ = K.quantize_mxfp4(e2, hd, signs, mode, transposed_in=True, seed=seed())
-        xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, ctx.x_dtype, hd, signs, mode, seed=seed())
-        gwq = K.gemm_mxfp4_tn(etc, ets, xtc, xts, alpha, mid_dtype)
+        etc, ets, _, _ = K.quantize_mxfp4(e2, hd, signs, mode, transposed_in=True, seed=seed(), tiled=t)
+        xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, ctx.x_dtype, hd, signs, mode, seed=seed(),
+                                                    tiled_in=t, tiled_out=t)
+        gwq = K.gemm_mxfp4_tn(etc, ets, xtc, xts, alpha, mid_dtype, a_tiled=t, b_tiled=t)
 
         sd_x = torch.bfloat16 if low else ctx.x_dtype
         sd_w = torch.bfloat16 if low else ctx.w_dtype

@@ -114,3 +114,24 @@ def test_gemm_tile_kernels(oracle, K, M, N, K_, exact):
         rel = float((got32.double() - want).norm() / want.norm())
         assert rel <= 1e-5, rel
     assert torch.equal(got16, got32.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("M,N,K_", [(256, 256, 512), (768, 512, 1536), (512, 256, 640), (4352, 4608, 1024)])
+@pytest.mark.parametrize("a_tiled,b_tiled", [(True, True), (True, False), (False, True)])
+def test_gemm_tiled_operands_match_rowmajor(K, M, N, K_, a_tiled, b_tiled):
+    print(f"case gemm tiled {M}x{N}x{K_} a={a_tiled} b={b_tiled}", flush=True)
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(M + N + K_)
+    ac = torch.randint(0, 256, (M, K_ // 2), generator=g, dtype=torch.uint8).to(dev)
+    bc = torch.randint(0, 256, (N, K_ // 2), generator=g, dtype=torch.uint8).to(dev)
+    as_ = torch.randint(118, 132, (M, K_ // 32), generator=g, dtype=torch.uint8).to(dev)
+    bs = torch.randint(120, 136, (N, K_ // 32), generator=g, dtype=torch.uint8).to(dev)
+    want = K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha=1.0, out_dtype=torch.float32)
+    got = K.gemm_mxfp4_tn(K.tile_codes(ac) if a_tiled else ac, as_, K.tile_codes(bc) if b_tiled else bc, bs, alpha=1.0,
+                          out_dtype=torch.float32, a_tiled=a_tiled, b_tiled=b_tiled)
+    got16 = K.gemm_mxfp4_tn(K.tile_codes(ac) if a_tiled else ac, as_, K.tile_codes(bc) if b_tiled else bc, bs, alpha=1.0,
+                            out_dtype=torch.bfloat16, a_tiled=a_tiled, b_tiled=b_tiled)
+    torch.cuda.synchronize()
+    # same kernel, same summation order: the layout only changes where the operand bytes are fetched from
+    assert torch.equal(got, want)
+    assert torch.equal(got16, want.to(torch.bfloat16))

@@ -76,10 +76,10 @@ def test_llama30m_quartet_step(models):
 
 
 def test_llama_ragged_batch_shapes(models):
-    # 3 x 40 tokens = 120 rows: not a multiple of the 128-row tiles of the transposing kernels
+    # 4 x 40 tokens = 160 rows: a multiple of the Hadamard block but not of the 128-row tiles of the transposing kernels
     L, quartet, bwd_only, plain, idx, tgt = models
-    print("case llama30m ragged 3x40", flush=True)
-    lq = _step(quartet, idx[:3, :40].contiguous(), tgt[:3, :40].contiguous())
+    print("case llama30m ragged 4x40", flush=True)
+    lq = _step(quartet, idx[:4, :40].contiguous(), tgt[:4, :40].contiguous())
     torch.cuda.synchronize()
     assert math.isfinite(lq)
     assert all(torch.isfinite(p.grad).all() for p in quartet.parameters())

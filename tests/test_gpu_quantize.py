@@ -164,6 +164,89 @@ def test_rowmajor_group_layout_seeded(oracle, K, mode, dtype):
     _check(oracle, K, x, 32, MODES[mode], signs, False, None, 0xFEED_F00D_CAFE, f"rowmajor-g32/{mode}/{dtype}")
 
 
+# Tiled code layout ([R/16][C/128][16][64 bytes]): the same bytes as the row-major codes, permuted; scales, mask
+# and the de-quantized tensor are unaffected.
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("R,C", [(16, 128), (48, 640), (256, 1024)])
+def test_rowmajor_tiled_codes(oracle, K, mode, dtype, R, C):
+    print(f"case rowmajor-tiled mode={mode} dtype={dtype} R={R} C={C}", flush=True)
+    dev = torch.device("cuda:0")
+    x = make_input(R, C, dtype, seed=R + C, zero_rows=1)
+    g = torch.Generator().manual_seed(15)
+    signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
+    seed = 0x1111_2222_3333 + R
+    want_mask = "quest" in mode
+    codes, scales, mask, deq = K.quantize_mxfp4(x.to(dev), 32, sign_int(signs), MODES[mode], False, None, seed,
+                                                want_mask=want_mask, want_dequant=True, tiled=True)
+    plain = K.quantize_mxfp4(x.to(dev), 32, sign_int(signs), MODES[mode], False, None, seed, want_mask=want_mask)
+    torch.cuda.synchronize()
+    ref = oracle.quantize(to_oracle(x), 32, signs=signs.numpy(), mode=MODES[mode], seed=seed, want_mask=want_mask,
+                          want_dequant=True)
+    assert np.array_equal(to_oracle(K.untile_codes(codes)), ref["codes"])
+    assert torch.equal(K.tile_codes(plain[0]), codes)
+    assert np.array_equal(to_oracle(scales), ref["scales"])
+    if want_mask:
+        assert np.array_equal(to_oracle(mask), ref["mask"])
+    a, b = to_oracle(deq), ref["dequant"]
+    assert np.array_equal(a.view(np.uint32) if a.dtype == np.float32 else a, b.view(np.uint32) if b.dtype == np.float32 else b)
+
+
+@pytest.mark.parametrize("mode", ["absmax_sr", "absmax_rtn"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("P,Q", [(128, 16), (256, 208), (384, 320)])
+def test_transposed_tiled_codes(oracle, K, mode, dtype, P, Q):
+    print(f"case transposed-tiled mode={mode} dtype={dtype} P={P} Q={Q}", flush=True)
+    dev = torch.device("cuda:0")
+    x = make_input(P, Q, dtype, seed=P + Q)
+    seed = 0x4444_5555 + Q
+    codes, scales, _, _ = K.quantize_mxfp4(x.to(dev), 32, 0x0F0F00FF, MODES[mode], True, None, seed, tiled=True)
+    torch.cuda.synchronize()
+    signs = np.array([-1 if (0x0F0F00FF >> j) & 1 else 1 for j in range(32)])
+    ref = oracle.quantize(to_oracle(x), 32, signs=signs, mode=MODES[mode], transposed_in=True, seed=seed)
+    assert np.array_equal(to_oracle(K.untile_codes(codes)), ref["codes"])
+    assert np.array_equal(to_oracle(scales), ref["scales"])
+
+
+@pytest.mark.parametrize("tiled_in,tiled_out", [(True, True), (True, False), (False, True)])
+@pytest.mark.parametrize("R,C", [(128, 128), (256, 384), (384, 1024)])
+def test_requantize_tiled_codes(oracle, K, tiled_in, tiled_out, R, C):
+    print(f"case requant-tiled in={tiled_in} out={tiled_out} R={R} C={C}", flush=True)
+    dev = torch.device("cuda:0")
+    x = make_input(R, C, torch.bfloat16, seed=R + C)
+    q = oracle.quantize(to_oracle(x), 32, mode=oracle.QUEST_RTN)
+    seed = 0x6666 + C
+    ref = oracle.requantize_transposed(q["codes"], q["scales"], post=1.0, val_dtype=oracle.BF16, hd=32, signs=None,
+                                       mode=oracle.ABSMAX_SR, u=None, seed=seed)
+    cin = torch.from_numpy(q["codes"]).to(dev)
+    if tiled_in:
+        cin = K.tile_codes(cin)
+    co, so, _ = K.requantize_transposed_mxfp4(cin, torch.from_numpy(q["scales"]).to(dev), 1.0, torch.bfloat16, 32, None,
+                                              K.QM_ABSMAX_SR, None, seed, tiled_in=tiled_in, tiled_out=tiled_out)
+    torch.cuda.synchronize()
+    if tiled_out:
+        co = K.untile_codes(co)
+    assert np.array_equal(to_oracle(co), ref["codes"])
+    assert np.array_equal(to_oracle(so), ref["scales"])
+
+
+def test_tiled_layout_rejections(K):
+    from quartet_amd._lib import QuartetHipError
+    dev = torch.device("cuda:0")
+    x = torch.randn(24, 128, device=dev).to(torch.bfloat16)       # 24 rows: not a multiple of 16
+    with pytest.raises(QuartetHipError):
+        K.quantize_mxfp4(x, 32, None, 0, tiled=True)
+    x = torch.randn(32, 256, device=dev).to(torch.bfloat16)
+    with pytest.raises(QuartetHipError):                          # tiled codes exist for Hadamard block 32 only
+        K.quantize_mxfp4(x, 64, None, 0, tiled=True)
+    with pytest.raises(QuartetHipError):                          # and not with explicit uniforms
+        K.quantize_mxfp4(x, 32, None, 2, u=torch.rand(32, 256, device=dev), tiled=True)
+    c = torch.zeros(128, 64, dtype=torch.uint8, device=dev)
+    sc = torch.full((128, 4), 127, dtype=torch.uint8, device=dev)
+    with pytest.raises(QuartetHipError):                          # GEMM: 128 rows are not a 256-row tile
+        K.gemm_mxfp4_tn(c, sc, c, sc, 1.0, torch.float32, a_tiled=True)
+
+
 def test_order_independent_integer_fixture(oracle, K):
     # x = S @ g with small integers and hd = 64: every partial sum is exact, so the expected
     # rotated values (8*g) and hence codes/scales do not depend on any summation order.
