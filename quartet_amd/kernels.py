@@ -114,12 +114,15 @@ def gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, alpha=1.0, out_dtype=tor
     return c
 
 
-def masked_hadamard_bwd(g, hadamard_dim=32, scale_dtype=torch.bfloat16, sign_bits=None, maskbits=None, out_dtype=None):
-    """g [R,C] -> ((g*mask).view(-1,hd) @ H^T) as [R,C] of out_dtype (default g.dtype)."""
+def masked_hadamard_bwd(g, hadamard_dim=32, scale_dtype=torch.bfloat16, sign_bits=None, maskbits=None, out_dtype=None,
+                        out=None):
+    """g [R,C] -> ((g*mask).view(-1,hd) @ H^T) as [R,C] of out_dtype (default g.dtype); `out` may be pre-allocated."""
     _require_cuda(g, maskbits)
     assert g.dim() == 2 and g.is_contiguous()
     out_dtype = g.dtype if out_dtype is None else out_dtype
-    out = torch.empty(g.shape, dtype=out_dtype, device=g.device)
+    if out is None:
+        out = torch.empty(g.shape, dtype=out_dtype, device=g.device)
+    assert out.shape == g.shape and out.dtype == out_dtype and out.is_contiguous()
     rc = _lib.lib().qm_masked_hadamard_bwd(_ptr(g), _dtype_code(g.dtype), g.shape[0], g.shape[1], hadamard_dim,
                                            _dtype_code(scale_dtype), sign_words(sign_bits), _ptr(maskbits), _ptr(out),
                                            _dtype_code(out_dtype), _stream())

@@ -59,18 +59,21 @@ class QuartetLinearFn(torch.autograd.Function):
         alpha = K.FOUR_THIRDS * K.FOUR_THIRDS  # both operands are absmax-coded: value = code * 2^k * 4/3
 
         t = ctx.tiled
-        ec, es, _, _ = K.quantize_mxfp4(e2, hd, signs, mode, seed=seed(), tiled=t)
-        wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, ctx.w_dtype, hd, signs, mode, seed=seed(),
+        sd_x = torch.bfloat16 if low else ctx.x_dtype
+        sd_w = torch.bfloat16 if low else ctx.w_dtype
+        seeds = [seed() for _ in range(4)]  # drawn in the order e, W^T, e^T, x^T whatever order the kernels run in
+        ec, es, _, _ = K.quantize_mxfp4(e2, hd, signs, mode, seed=seeds[0], tiled=t)
+        wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, ctx.w_dtype, hd, signs, mode, seed=seeds[1],
                                                     tiled_in=t, tiled_out=t)
         gxq = K.gemm_mxfp4_tn(ec, es, wtc, wts, alpha, mid_dtype, a_tiled=t, b_tiled=t)
 
-        etc, ets, _, _ = K.quantize_mxfp4(e2, hd, signs, mode, transposed_in=True, seed=seed(), tiled=t)
-        xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, ctx.x_dtype, hd, signs, mode, seed=seed(),
+        etc, ets, _, _ = K.quantize_mxfp4(e2, hd, signs, mode, transposed_in=True, seed=seeds[2], tiled=t)
+        xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, ctx.x_dtype, hd, signs, mode, seed=seeds[3],
                                                     tiled_in=t, tiled_out=t)
         gwq = K.gemm_mxfp4_tn(etc, ets, xtc, xts, alpha, mid_dtype, a_tiled=t, b_tiled=t)
 
-        sd_x = torch.bfloat16 if low else ctx.x_dtype
-        sd_w = torch.bfloat16 if low else ctx.w_dtype
+        # (Running the bandwidth-bound inverse rotation of gxq on a second stream next to the two ALU-bound quantizers
+        # above was measured slower than this single-stream order: the cross-stream joins cost more than they hide.)
         gx = K.masked_hadamard_bwd(gxq, a_hd, sd_x, a_signs, xm, mid_dtype).to(ctx.x_dtype)
         gw = K.masked_hadamard_bwd(gwq, w_hd, sd_w, w_signs, wm, mid_dtype).to(ctx.w_dtype)
         return gx.view(ctx.x_shape), gw, None, None, None
