@@ -34,6 +34,9 @@ hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t rows, int64_
                                   uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
                                   bool tiled, hipStream_t stream);
 
+hipError_t quantize_rowmajor_wide(const void* x, int dtype, int64_t n, int hd, const SignBits& sb, int mode, uint64_t seed,
+                                  uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant, hipStream_t stream);
+
 hipError_t quantize_transposed_hd32(const void* x, int dtype, int64_t P, int64_t Q, uint32_t sign_word, int mode,
                                     uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant, bool tiled,
                                     hipStream_t stream);

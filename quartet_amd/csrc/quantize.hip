@@ -418,6 +418,8 @@ hipError_t quantize_mxfp4(const void* x, int dtype, int64_t rows, int64_t cols, 
     if (tiled && !(al(codes, 16) && al(maskbits, 4) && al(scales, 4))) return hipErrorInvalidValue;
     if (hd == 32 && !transposed_in && (rtn || u == nullptr) && al(codes, 16) && al(maskbits, 4))
         return quantize_rowmajor_hd32(x, dtype, rows, cols, sb.w[0], mode, seed, codes, scales, maskbits, dequant, tiled, stream);
+    if ((hd == 64 || hd == 128) && !transposed_in && (rtn || u == nullptr) && al(codes, 16) && al(maskbits, 4))
+        return quantize_rowmajor_wide(x, dtype, rows * cols, hd, sb, mode, seed, codes, scales, maskbits, dequant, stream);
     // logical [rows, cols] = physical [P = cols, Q = rows]
     if (hd == 32 && transposed_in && (rtn || u == nullptr) && maskbits == nullptr && al(codes, 16) && al(scales, 4) &&
         cols % 128 == 0)

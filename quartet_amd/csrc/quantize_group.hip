@@ -309,6 +309,63 @@ void launch_rowmajor_g32(int mode, const void* x, int64_t rows, int64_t cols, bo
     }
 }
 
+// ---- Hadamard blocks 64 and 128, row-major ---------------------------------------------------------------
+// Same one-group-per-lane layout; a Hadamard chunk is HD/32 consecutive lanes (a lane pair or a quad).  The
+// five in-register stages are followed by the stride-32 (and stride-64) stages across the lanes of the chunk:
+// the lower lane of a butterfly gets a + b, the upper one a - b = partner + (-own), one sign flip and one
+// DPP-fed add per element.  The column sign word differs per lane of the chunk.
+template <int CTRL>
+__device__ __forceinline__ void cross_lane_stage(float (&v)[32], bool upper) {
+    const uint32_t flip = upper ? 0x80000000u : 0u;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        const float partner = u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(v[i]), CTRL, 0xf, 0xf, false));
+        v[i] = partner + u2f(f2u(v[i]) ^ flip);
+    }
+}
+
+template <typename T, int MODE, bool WANT_MASK, int HD>
+__global__ __launch_bounds__(256) void quantize_rowmajor_wide_kernel(const T* __restrict__ x, int64_t n_groups, float c,
+                                                                     SignBits sb, uint64_t seed, GroupOut out) {
+    static_assert(HD == 64 || HD == 128, "lane pairs or quads");
+    const int64_t gi = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (gi >= n_groups) return;  // n_groups is a multiple of HD/32: the lanes of a chunk leave together
+    float v[32];
+    load_group<T>(x + gi * 32, v);
+    butterfly32(v);
+    const int part = (int)threadIdx.x & (HD / 32 - 1);
+    cross_lane_stage<0xB1>(v, (part & 1) != 0);                           // quad_perm [1,0,3,2]: stride 32
+    if constexpr (HD == 128) cross_lane_stage<0x4E>(v, (part & 2) != 0);  // quad_perm [2,3,0,1]: stride 64
+    uint32_t sw = sb.w[0];
+    if (part == 1) sw = sb.w[1];
+    if constexpr (HD == 128) {
+        if (part == 2) sw = sb.w[2];
+        if (part == 3) sw = sb.w[3];
+    }
+#pragma unroll
+    for (int j = 0; j < 32; ++j) v[j] = u2f(f2u(v[j] * c) ^ ((sw << (31 - j)) & 0x80000000u));
+    GroupCodes o;
+    quantize_group_regs<MODE, WANT_MASK>(v, seed, gi, o);
+    out.codes[gi] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
+    out.scales[gi] = (uint8_t)o.scale_byte;
+    if constexpr (WANT_MASK) out.maskbits[gi] = o.keep;
+    if (out.dequant) store_dequant<T>(reinterpret_cast<T*>(out.dequant) + gi * 32, o);
+}
+
+template <typename T, bool WANT_MASK, int HD>
+void launch_rowmajor_wide(int mode, const void* x, int64_t n, float c, const SignBits& sb, uint64_t seed,
+                          const GroupOut& out, hipStream_t stream) {
+    const T* xp = reinterpret_cast<const T*>(x);
+    const int64_t n_groups = n / 32;
+    dim3 grid((unsigned)((n_groups + 255) / 256)), block(256);
+    switch (mode) {
+        case QUEST_RTN: quantize_rowmajor_wide_kernel<T, QUEST_RTN, WANT_MASK, HD><<<grid, block, 0, stream>>>(xp, n_groups, c, sb, seed, out); break;
+        case ABSMAX_RTN: quantize_rowmajor_wide_kernel<T, ABSMAX_RTN, WANT_MASK, HD><<<grid, block, 0, stream>>>(xp, n_groups, c, sb, seed, out); break;
+        case ABSMAX_SR: quantize_rowmajor_wide_kernel<T, ABSMAX_SR, WANT_MASK, HD><<<grid, block, 0, stream>>>(xp, n_groups, c, sb, seed, out); break;
+        default: quantize_rowmajor_wide_kernel<T, QUEST_SR, WANT_MASK, HD><<<grid, block, 0, stream>>>(xp, n_groups, c, sb, seed, out); break;
+    }
+}
+
 // ---- transposed input: x is [P, Q] row-major, output is the [Q, P] tensor quantized along P ----------
 // A workgroup owns a strip of 256 bytes of columns (128 bf16 / 64 fp32) by 128 rows; wave w owns p-group w.
 // A lane reads its column (bf16: two adjacent columns per 32-bit load) at 32 successive rows straight from
@@ -513,6 +570,29 @@ hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t rows, int64_
     } else {
         if (dtype == BF16) launch_rowmajor_g32<uint16_t, false>(mode, x, rows, cols, tiled, c, sign_word, seed, out, stream);
         else launch_rowmajor_g32<float, false>(mode, x, rows, cols, tiled, c, sign_word, seed, out, stream);
+    }
+    return hipGetLastError();
+}
+
+// hd = 64 or 128, row-major input, RTN or Philox-driven SR, row-major codes
+hipError_t quantize_rowmajor_wide(const void* x, int dtype, int64_t n, int hd, const SignBits& sb, int mode, uint64_t seed,
+                                  uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant, hipStream_t stream) {
+    GroupOut out{reinterpret_cast<uint4*>(codes), scales, reinterpret_cast<uint32_t*>(maskbits), dequant};
+    const float c = hadamard_scale(hd, dtype);
+    const auto go = [&](auto tag, auto mask, auto hdc) {
+        using T = decltype(tag);
+        launch_rowmajor_wide<T, decltype(mask)::value, decltype(hdc)::value>(mode, x, n, c, sb, seed, out, stream);
+    };
+    const auto by_hd = [&](auto tag, auto mask) {
+        if (hd == 64) go(tag, mask, std::integral_constant<int, 64>{});
+        else go(tag, mask, std::integral_constant<int, 128>{});
+    };
+    if (maskbits) {
+        if (dtype == BF16) by_hd(uint16_t{}, std::true_type{});
+        else by_hd(float{}, std::true_type{});
+    } else {
+        if (dtype == BF16) by_hd(uint16_t{}, std::false_type{});
+        else by_hd(float{}, std::false_type{});
     }
     return hipGetLastError();
 }

@@ -155,13 +155,14 @@ def test_requantize_group_layout_bit_exact(oracle, K, mode, val_dtype, R, C):
 
 @pytest.mark.parametrize("mode", list(MODES))
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-def test_rowmajor_group_layout_seeded(oracle, K, mode, dtype):
-    print(f"case rowmajor-g32 mode={mode} dtype={dtype}", flush=True)
-    # 33 rows x 2080 columns: the element count is not a multiple of the kernel's per-block share
-    x = make_input(33, 2080, dtype, seed=21, zero_rows=1)
-    g = torch.Generator().manual_seed(14)
-    signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
-    _check(oracle, K, x, 32, MODES[mode], signs, False, None, 0xFEED_F00D_CAFE, f"rowmajor-g32/{mode}/{dtype}")
+@pytest.mark.parametrize("hd", [32, 64, 128])
+def test_rowmajor_group_layout_seeded(oracle, K, mode, dtype, hd):
+    print(f"case rowmajor-group mode={mode} dtype={dtype} hd={hd}", flush=True)
+    # 33 rows x 2176 columns: the element count is not a multiple of the kernel's per-block share
+    x = make_input(33, 2176, dtype, seed=21 + hd, zero_rows=1)
+    g = torch.Generator().manual_seed(14 + hd)
+    signs = torch.randint(0, 2, (hd,), generator=g) * 2 - 1
+    _check(oracle, K, x, hd, MODES[mode], signs, False, None, 0xFEED_F00D_CAFE + hd, f"rowmajor-group/{mode}/{dtype}/{hd}")
 
 
 # Tiled code layout ([R/16][C/128][16][64 bytes]): the same bytes as the row-major codes, permuted; scales, mask
