@@ -24,6 +24,7 @@
 #ifndef QUARTET_HIP_H
 #define QUARTET_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -109,6 +110,35 @@ int qm_masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t col
 /* out[r, c] = e2m1(code) * post * 2^(scale-127); the tensor the reference's pseudo-quantizer returns */
 int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, int64_t C,
                         float post, void* out, int out_dtype, void* stream);
+
+/*
+ * Whole-layer entry points: one call issues every launch of a Quartet linear's forward or backward pass (the
+ * per-kernel entry points above, in order), so the host pays one foreign call instead of three / eight.
+ *
+ * qm_linear_forward = QuestMXFP4QuantizerFn.forward on x and W (quantizers/mxfp4.py:129-140) followed by
+ * QEQWtt_QEtQXttFn.forward (src/models/quantization/backward.py:59-62):
+ *   x [T, I], w [O, I] -> y [T, O] = Q(x) Q(w)^T; `saved` (qm_linear_saved_bytes(T, I, O) bytes, 256-byte
+ *   aligned, caller-owned) receives the packed operands and clip-mask bits the backward pass needs.
+ * qm_linear_backward = QEQWtt_QEtQXttFn.backward (backward.py:64-85) with the straight-through backward of both
+ * forward quantizers (mxfp4.py:143-146) applied: e [T, O] -> gx [T, I], gw [O, I], both of mid_dtype.
+ *   g_mode            QM_ABSMAX_SR or QM_ABSMAX_RTN (AlbertTsengQuantizer stochastic or not)
+ *   seeds             HOST pointer to four seeds, for the quantizations of e, Q(w)^T, e^T, Q(x)^T in that order
+ *   x_val_dtype, w_val_dtype   dtypes the reference would hold the de-quantized x and w in
+ *   x_scale_dtype, w_scale_dtype  dtypes whose rounding of hd^-1/2 the forward quantizers' matrices carry in backward
+ *   workspace         qm_linear_backward_workspace_bytes(T, I, O, mid_dtype) bytes of scratch, 256-byte aligned
+ * codes_layout applies to every packed tensor inside; QM_LAYOUT_TILED needs T, I, O multiples of 256 and all
+ * Hadamard blocks 32.  T, I, O must be multiples of 32 for the backward pass.
+ */
+size_t qm_linear_saved_bytes(int64_t T, int64_t I, int64_t O);
+size_t qm_linear_backward_workspace_bytes(int64_t T, int64_t I, int64_t O, int mid_dtype);
+int qm_linear_forward(const void* x, int x_dtype, const void* w, int w_dtype, int64_t T, int64_t I, int64_t O,
+                      int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, void* saved,
+                      size_t saved_bytes, void* y, int y_dtype, int codes_layout, void* stream);
+int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t O, const void* saved, int hd_x,
+                       const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, int hd_g,
+                       const uint32_t* signs_g, int g_mode, const uint64_t* seeds, int x_val_dtype,
+                       int w_val_dtype, int mid_dtype, int x_scale_dtype, int w_scale_dtype, void* workspace,
+                       size_t workspace_bytes, void* gx, void* gw, int codes_layout, void* stream);
 
 #ifdef __cplusplus
 }

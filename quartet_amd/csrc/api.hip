@@ -144,4 +144,122 @@ int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, 
                     "qm_dequantize_mxfp4");
 }
 
+
+// ---- whole-layer entry points: one call issues every launch of the forward / backward pass -------------------
+
+namespace {
+size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
+size_t esize(int dtype) { return dtype == QM_BF16 ? 2 : 4; }
+
+struct SavedLayout {
+    size_t xc, xs, xm, wc, ws, wm, total;
+};
+SavedLayout saved_layout(int64_t T, int64_t I, int64_t O) {
+    SavedLayout l;
+    size_t o = 0;
+    l.xc = o; o += up256((size_t)T * I / 2);
+    l.xs = o; o += up256((size_t)T * I / 32);
+    l.xm = o; o += up256((size_t)T * I / 8);
+    l.wc = o; o += up256((size_t)O * I / 2);
+    l.ws = o; o += up256((size_t)O * I / 32);
+    l.wm = o; o += up256((size_t)O * I / 8);
+    l.total = o;
+    return l;
+}
+struct WorkLayout {
+    size_t ec, es, wtc, wts, gxq, etc, ets, xtc, xts, gwq, total;
+};
+WorkLayout work_layout(int64_t T, int64_t I, int64_t O, int mid_dtype) {
+    WorkLayout l;
+    size_t o = 0;
+    l.ec = o; o += up256((size_t)T * O / 2);
+    l.es = o; o += up256((size_t)T * O / 32);
+    l.wtc = o; o += up256((size_t)I * O / 2);
+    l.wts = o; o += up256((size_t)I * O / 32);
+    l.gxq = o; o += up256((size_t)T * I * esize(mid_dtype));
+    l.etc = o; o += up256((size_t)O * T / 2);
+    l.ets = o; o += up256((size_t)O * T / 32);
+    l.xtc = o; o += up256((size_t)I * T / 2);
+    l.xts = o; o += up256((size_t)I * T / 32);
+    l.gwq = o; o += up256((size_t)O * I * esize(mid_dtype));
+    l.total = o;
+    return l;
+}
+}  // namespace
+
+size_t qm_linear_saved_bytes(int64_t T, int64_t I, int64_t O) {
+    if (T < 0 || I < 0 || O < 0 || I % 32) return 0;
+    return saved_layout(T, I, O).total;
+}
+
+size_t qm_linear_backward_workspace_bytes(int64_t T, int64_t I, int64_t O, int mid_dtype) {
+    if (T < 0 || I < 0 || O < 0 || I % 32 || O % 32 || T % 32 || !valid_dtype(mid_dtype)) return 0;
+    return work_layout(T, I, O, mid_dtype).total;
+}
+
+int qm_linear_forward(const void* x, int x_dtype, const void* w, int w_dtype, int64_t T, int64_t I, int64_t O, int hd_x,
+                      const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, void* saved, size_t saved_bytes, void* y,
+                      int y_dtype, int codes_layout, void* stream) {
+    if (T < 0 || I < 0 || O < 0) return fail(QM_ERR_INVALID, "qm_linear_forward: negative extent");
+    if (T == 0 || O == 0 || I == 0) return 0;
+    if (I % 32) return fail(QM_ERR_INVALID, "qm_linear_forward: in_features %lld not a multiple of 32", (long long)I);
+    const SavedLayout l = saved_layout(T, I, O);
+    if (!saved || saved_bytes < l.total || !aligned(saved, 256))
+        return fail(QM_ERR_INVALID, "qm_linear_forward: saved buffer needs %zu bytes, 256-byte aligned", l.total);
+    uint8_t* s = static_cast<uint8_t*>(saved);
+    int rc = qm_quantize_mxfp4(x, x_dtype, T, I, hd_x, signs_x, QM_QUEST_RTN, 0, nullptr, 0, s + l.xc, s + l.xs, s + l.xm, nullptr,
+                               codes_layout, stream);
+    if (rc) return rc;
+    rc = qm_quantize_mxfp4(w, w_dtype, O, I, hd_w, signs_w, QM_QUEST_RTN, 0, nullptr, 0, s + l.wc, s + l.ws, s + l.wm, nullptr,
+                           codes_layout, stream);
+    if (rc) return rc;
+    return qm_gemm_mxfp4_tn(s + l.xc, s + l.xs, s + l.wc, s + l.ws, T, O, I, 1.0f, y, y_dtype, codes_layout, codes_layout, stream);
+}
+
+int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t O, const void* saved, int hd_x,
+                       const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, int hd_g, const uint32_t* signs_g,
+                       int g_mode, const uint64_t* seeds, int x_val_dtype, int w_val_dtype, int mid_dtype, int x_scale_dtype,
+                       int w_scale_dtype, void* workspace, size_t workspace_bytes, void* gx, void* gw, int codes_layout,
+                       void* stream) {
+    if (T < 0 || I < 0 || O < 0) return fail(QM_ERR_INVALID, "qm_linear_backward: negative extent");
+    if (T == 0 || O == 0 || I == 0) return 0;
+    if (g_mode != QM_ABSMAX_RTN && g_mode != QM_ABSMAX_SR)
+        return fail(QM_ERR_INVALID, "qm_linear_backward: gradient mode must be QM_ABSMAX_RTN or QM_ABSMAX_SR");
+    if (!valid_dtype(mid_dtype)) return fail(QM_ERR_INVALID, "qm_linear_backward: mid_dtype %d", mid_dtype);
+    if (I % 32 || O % 32 || T % 32)
+        return fail(QM_ERR_INVALID, "qm_linear_backward: tokens, in_features and out_features must be multiples of 32 (T=%lld I=%lld O=%lld)",
+                    (long long)T, (long long)I, (long long)O);
+    if (!seeds || !saved || !aligned(saved, 256)) return fail(QM_ERR_INVALID, "qm_linear_backward: null seeds or saved buffer");
+    const SavedLayout sl = saved_layout(T, I, O);
+    const WorkLayout wl = work_layout(T, I, O, mid_dtype);
+    if (!workspace || workspace_bytes < wl.total || !aligned(workspace, 256))
+        return fail(QM_ERR_INVALID, "qm_linear_backward: workspace needs %zu bytes, 256-byte aligned", wl.total);
+    const uint8_t* s = static_cast<const uint8_t*>(saved);
+    uint8_t* k = static_cast<uint8_t*>(workspace);
+    // value = code * 2^k * fl32(4/3) on both operands of the two gradient products
+    const float d = (float)(1.0 / 0.75);
+    const float alpha = d * d;
+    int rc = qm_quantize_mxfp4(e, e_dtype, T, O, hd_g, signs_g, g_mode, 0, nullptr, seeds[0], k + wl.ec, k + wl.es, nullptr, nullptr,
+                               codes_layout, stream);
+    if (rc) return rc;
+    rc = qm_requantize_transposed_mxfp4(s + sl.wc, s + sl.ws, O, I, 1.0f, w_val_dtype, hd_g, signs_g, g_mode, nullptr, seeds[1],
+                                        k + wl.wtc, k + wl.wts, nullptr, codes_layout, codes_layout, stream);
+    if (rc) return rc;
+    rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, k + wl.gxq, mid_dtype, codes_layout,
+                          codes_layout, stream);
+    if (rc) return rc;
+    rc = qm_quantize_mxfp4(e, e_dtype, O, T, hd_g, signs_g, g_mode, 1, nullptr, seeds[2], k + wl.etc, k + wl.ets, nullptr, nullptr,
+                           codes_layout, stream);
+    if (rc) return rc;
+    rc = qm_requantize_transposed_mxfp4(s + sl.xc, s + sl.xs, T, I, 1.0f, x_val_dtype, hd_g, signs_g, g_mode, nullptr, seeds[3],
+                                        k + wl.xtc, k + wl.xts, nullptr, codes_layout, codes_layout, stream);
+    if (rc) return rc;
+    rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, k + wl.gwq, mid_dtype, codes_layout,
+                          codes_layout, stream);
+    if (rc) return rc;
+    rc = qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, s + sl.xm, gx, mid_dtype, stream);
+    if (rc) return rc;
+    return qm_masked_hadamard_bwd(k + wl.gwq, mid_dtype, O, I, hd_w, w_scale_dtype, signs_w, s + sl.wm, gw, mid_dtype, stream);
+}
+
 }  // extern "C"

@@ -34,49 +34,34 @@ class QuartetLinearFn(torch.autograd.Function):
         # all three extents multiples of 256 and Hadamard block 32 throughout; row-major codes otherwise.
         tiled = (x2.shape[0] % 256 == 0 and in_features % 256 == 0 and weight.shape[0] % 256 == 0 and
                  a_q.hadamard_dim == 32 and w_q.hadamard_dim == 32 and g_q.hadamard_dim == 32)
-        xc, xs, xm, _ = K.quantize_mxfp4(x2, a_q.hadamard_dim, a_q.sign_bits, K.QM_QUEST_RTN, want_mask=True, tiled=tiled)
-        wc, ws, wm, _ = K.quantize_mxfp4(w2, w_q.hadamard_dim, w_q.sign_bits, K.QM_QUEST_RTN, want_mask=True, tiled=tiled)
-        y = K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, out_dtype, a_tiled=tiled, b_tiled=tiled)
-        ctx.save_for_backward(xc, xs, xm, wc, ws, wm)
+        y, saved = K.linear_forward(x2, w2, a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits, out_dtype, tiled)
+        ctx.save_for_backward(saved)
         ctx.g_q = g_q
         ctx.tiled = tiled
         ctx.fwd = (a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits)
+        ctx.dims = (x2.shape[0], in_features, weight.shape[0])
         ctx.x_shape, ctx.x_dtype, ctx.w_dtype = x.shape, x.dtype, weight.dtype
         return y.view(*x.shape[:-1], weight.shape[0])
 
     @staticmethod
     def backward(ctx, e):
-        xc, xs, xm, wc, ws, wm = ctx.saved_tensors
+        (saved,) = ctx.saved_tensors
         g_q = ctx.g_q
         a_hd, a_signs, w_hd, w_signs = ctx.fwd
+        T, I, O = ctx.dims
         g_q.re_randomize()
         hd, signs = g_q.hadamard_dim, g_q.sign_bits
         mode = K.QM_ABSMAX_SR if g_q.stochastic else K.QM_ABSMAX_RTN
-        seed = (lambda: _fresh_seed()) if g_q.stochastic else (lambda: 0)
+        # one host-side draw per stochastic quantization, in the order e, W^T, e^T, x^T
+        seeds = [_fresh_seed() if g_q.stochastic else 0 for _ in range(4)]
         e2 = e.reshape(-1, e.shape[-1]).contiguous()
         low = _autocast_bf16() or e2.dtype == torch.bfloat16
         mid_dtype = torch.bfloat16 if low else e2.dtype
-        alpha = K.FOUR_THIRDS * K.FOUR_THIRDS  # both operands are absmax-coded: value = code * 2^k * 4/3
-
-        t = ctx.tiled
         sd_x = torch.bfloat16 if low else ctx.x_dtype
         sd_w = torch.bfloat16 if low else ctx.w_dtype
-        seeds = [seed() for _ in range(4)]  # drawn in the order e, W^T, e^T, x^T whatever order the kernels run in
-        ec, es, _, _ = K.quantize_mxfp4(e2, hd, signs, mode, seed=seeds[0], tiled=t)
-        wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, ctx.w_dtype, hd, signs, mode, seed=seeds[1],
-                                                    tiled_in=t, tiled_out=t)
-        gxq = K.gemm_mxfp4_tn(ec, es, wtc, wts, alpha, mid_dtype, a_tiled=t, b_tiled=t)
-
-        etc, ets, _, _ = K.quantize_mxfp4(e2, hd, signs, mode, transposed_in=True, seed=seeds[2], tiled=t)
-        xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, ctx.x_dtype, hd, signs, mode, seed=seeds[3],
-                                                    tiled_in=t, tiled_out=t)
-        gwq = K.gemm_mxfp4_tn(etc, ets, xtc, xts, alpha, mid_dtype, a_tiled=t, b_tiled=t)
-
-        # (Running the bandwidth-bound inverse rotation of gxq on a second stream next to the two ALU-bound quantizers
-        # above was measured slower than this single-stream order: the cross-stream joins cost more than they hide.)
-        gx = K.masked_hadamard_bwd(gxq, a_hd, sd_x, a_signs, xm, mid_dtype).to(ctx.x_dtype)
-        gw = K.masked_hadamard_bwd(gwq, w_hd, sd_w, w_signs, wm, mid_dtype).to(ctx.w_dtype)
-        return gx.view(ctx.x_shape), gw, None, None, None
+        gx, gw = K.linear_backward(e2, saved, T, I, O, a_hd, a_signs, w_hd, w_signs, hd, signs, mode, seeds, ctx.x_dtype,
+                                   ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled)
+        return gx.to(ctx.x_dtype).view(ctx.x_shape), gw.to(ctx.w_dtype), None, None, None
 
 
 class QuantizedLinear(nn.Linear):
