@@ -90,12 +90,17 @@ int qm_requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scale
  * Replaces F.linear / einsum on de-quantized operands (src/models/quantization/backward.py:62,
  * 71-75, 79-83) and matmul_mxf4_bf16_tn of notebooks/benchmark_mxfp4.ipynb.  K % 32 == 0.
  * alpha carries the per-operand constants of absmax coding (fl32(4/3) each).
- * a_layout / b_layout: layouts of a_codes / b_codes; QM_LAYOUT_TILED needs M % 256 == 0,
- * N % 256 == 0 and K % 128 == 0 (the shapes the 256x256-tile kernels serve).
+ * a_layout / b_layout: layouts of a_codes / b_codes; QM_LAYOUT_TILED needs M and N multiples of 64 and
+ * at least 256, and K % 128 == 0 (the shapes the 256x256-tile kernels serve).
+ * workspace: optional scratch (NULL, 0 for none).  With qm_gemm_workspace_bytes(M, N, K) > 0 bytes of it, 16-byte
+ * aligned, a product with few output tiles and a long K is cut into K ranges whose fp32 partial sums are added in
+ * a fixed order (results are reproducible, but differ in rounding from the unsplit product).
  */
+size_t qm_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                      const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c,
-                     int c_dtype, int a_layout, int b_layout, void* stream);
+                     int c_dtype, int a_layout, int b_layout, void* workspace, size_t workspace_bytes,
+                     void* stream);
 
 /*
  * out = ((g * mask).view(-1, hd)) @ H^T: the straight-through backward of the forward quantizer,
@@ -126,8 +131,8 @@ int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, 
  *   x_val_dtype, w_val_dtype   dtypes the reference would hold the de-quantized x and w in
  *   x_scale_dtype, w_scale_dtype  dtypes whose rounding of hd^-1/2 the forward quantizers' matrices carry in backward
  *   workspace         qm_linear_backward_workspace_bytes(T, I, O, mid_dtype) bytes of scratch, 256-byte aligned
- * codes_layout applies to every packed tensor inside; QM_LAYOUT_TILED needs T, I, O multiples of 256 and all
- * Hadamard blocks 32.  T, I, O must be multiples of 32 for the backward pass.
+ * codes_layout applies to every packed tensor inside; QM_LAYOUT_TILED needs T, I, O multiples of 128 and at
+ * least 256, and all Hadamard blocks 32.  T, I, O must be multiples of 32 for the backward pass.
  */
 size_t qm_linear_saved_bytes(int64_t T, int64_t I, int64_t O);
 size_t qm_linear_backward_workspace_bytes(int64_t T, int64_t I, int64_t O, int mid_dtype);

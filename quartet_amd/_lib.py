@@ -20,6 +20,7 @@ EXPORTS = (
     "qm_gemm_mxfp4_tn",
     "qm_masked_hadamard_bwd",
     "qm_dequantize_mxfp4",
+    "qm_gemm_workspace_bytes",
     "qm_linear_saved_bytes",
     "qm_linear_backward_workspace_bytes",
     "qm_linear_forward",
@@ -52,7 +53,9 @@ def lib():
     L.qm_requantize_transposed_mxfp4.restype = i32
     L.qm_requantize_transposed_mxfp4.argtypes = [vp, vp, i64, i64, f32, i32, i32, vp, i32, vp, u64, vp, vp, vp, i32, i32, vp]
     L.qm_gemm_mxfp4_tn.restype = i32
-    L.qm_gemm_mxfp4_tn.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, i32, vp]
+    L.qm_gemm_mxfp4_tn.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, i32, vp, ctypes.c_size_t, vp]
+    L.qm_gemm_workspace_bytes.restype = ctypes.c_size_t
+    L.qm_gemm_workspace_bytes.argtypes = [i64, i64, i64]
     L.qm_masked_hadamard_bwd.restype = i32
     L.qm_masked_hadamard_bwd.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp, i32, vp]
     L.qm_dequantize_mxfp4.restype = i32

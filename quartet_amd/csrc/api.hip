@@ -100,7 +100,7 @@ int qm_requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scale
 
 int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
                      int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype, int a_layout, int b_layout,
-                     void* stream) {
+                     void* workspace, size_t workspace_bytes, void* stream) {
     if (!valid_layout(a_layout) || !valid_layout(b_layout))
         return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn: unknown layout %d / %d", a_layout, b_layout);
     if (!valid_dtype(c_dtype)) return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn: c_dtype %d", c_dtype);
@@ -110,11 +110,16 @@ int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint
     if (!aligned(a_codes, 16) || !aligned(b_codes, 16) || !aligned(a_scales, 4) || !aligned(b_scales, 4) || !aligned(c, 4))
         return fail(QM_ERR_UNALIGNED, "qm_gemm_mxfp4_tn: codes need 16-byte, scales and c 4-byte alignment");
     if ((a_layout == QM_LAYOUT_TILED || b_layout == QM_LAYOUT_TILED) && !qm::gemm_supports_tiled(M, N, K))
-        return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn: tiled operands need M %% 256 == 0, N %% 256 == 0, K %% 128 == 0 (M=%lld N=%lld K=%lld)",
+        return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn: tiled operands need M, N multiples of 64 and >= 256, K %% 128 == 0 (M=%lld N=%lld K=%lld)",
                     (long long)M, (long long)N, (long long)K);
     return from_hip(qm::gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, c_dtype, a_layout, b_layout,
-                                      reinterpret_cast<hipStream_t>(stream)),
+                                      workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream)),
                     "qm_gemm_mxfp4_tn");
+}
+
+size_t qm_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || K % 32) return 0;
+    return qm::gemm_workspace_bytes(M, N, K);
 }
 
 int qm_masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t cols, int hadamard_dim, int scale_dtype,
@@ -167,7 +172,7 @@ SavedLayout saved_layout(int64_t T, int64_t I, int64_t O) {
     return l;
 }
 struct WorkLayout {
-    size_t ec, es, wtc, wts, gxq, etc, ets, xtc, xts, gwq, total;
+    size_t ec, es, wtc, wts, gxq, etc, ets, xtc, xts, gwq, gemm_ws, gemm_ws_bytes, total;
 };
 WorkLayout work_layout(int64_t T, int64_t I, int64_t O, int mid_dtype) {
     WorkLayout l;
@@ -182,6 +187,9 @@ WorkLayout work_layout(int64_t T, int64_t I, int64_t O, int mid_dtype) {
     l.xtc = o; o += up256((size_t)I * T / 2);
     l.xts = o; o += up256((size_t)I * T / 32);
     l.gwq = o; o += up256((size_t)O * I * esize(mid_dtype));
+    const size_t g1 = qm::gemm_workspace_bytes(T, I, O), g2 = qm::gemm_workspace_bytes(O, I, T);
+    l.gemm_ws_bytes = g1 > g2 ? g1 : g2;  // split-K scratch, shared by the two products (they run one after the other)
+    l.gemm_ws = o; o += up256(l.gemm_ws_bytes);
     l.total = o;
     return l;
 }
@@ -213,7 +221,8 @@ int qm_linear_forward(const void* x, int x_dtype, const void* w, int w_dtype, in
     rc = qm_quantize_mxfp4(w, w_dtype, O, I, hd_w, signs_w, QM_QUEST_RTN, 0, nullptr, 0, s + l.wc, s + l.ws, s + l.wm, nullptr,
                            codes_layout, stream);
     if (rc) return rc;
-    return qm_gemm_mxfp4_tn(s + l.xc, s + l.xs, s + l.wc, s + l.ws, T, O, I, 1.0f, y, y_dtype, codes_layout, codes_layout, stream);
+    return qm_gemm_mxfp4_tn(s + l.xc, s + l.xs, s + l.wc, s + l.ws, T, O, I, 1.0f, y, y_dtype, codes_layout, codes_layout, nullptr, 0,
+                            stream);
 }
 
 int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t O, const void* saved, int hd_x,
@@ -245,8 +254,9 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
     rc = qm_requantize_transposed_mxfp4(s + sl.wc, s + sl.ws, O, I, 1.0f, w_val_dtype, hd_g, signs_g, g_mode, nullptr, seeds[1],
                                         k + wl.wtc, k + wl.wts, nullptr, codes_layout, codes_layout, stream);
     if (rc) return rc;
+    void* gws = wl.gemm_ws_bytes ? k + wl.gemm_ws : nullptr;
     rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, k + wl.gxq, mid_dtype, codes_layout,
-                          codes_layout, stream);
+                          codes_layout, gws, wl.gemm_ws_bytes, stream);
     if (rc) return rc;
     rc = qm_quantize_mxfp4(e, e_dtype, O, T, hd_g, signs_g, g_mode, 1, nullptr, seeds[2], k + wl.etc, k + wl.ets, nullptr, nullptr,
                            codes_layout, stream);
@@ -255,7 +265,7 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                                         k + wl.xtc, k + wl.xts, nullptr, codes_layout, codes_layout, stream);
     if (rc) return rc;
     rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, k + wl.gwq, mid_dtype, codes_layout,
-                          codes_layout, stream);
+                          codes_layout, gws, wl.gemm_ws_bytes, stream);
     if (rc) return rc;
     rc = qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, s + sl.xm, gx, mid_dtype, stream);
     if (rc) return rc;

@@ -361,16 +361,21 @@ __device__ __forceinline__ void big_mfma_sub(const SubFrags& f, const uint32_t (
 // rows spread over the banks), then writes it out as 16-byte pieces, four full 256-byte row segments per
 // instruction.  The LDS used is the operand ring, free once every wave has passed the final barrier.
 constexpr int kEpiPitch = 272;
+// rows_valid / cols_valid: how many of the wave's 128 rows / columns lie inside the matrix (multiples of 64, may be
+// <= 0 for a wave that hangs over the edge of M or N entirely); everything beyond is computed on clamped operand
+// rows and dropped here.
 template <typename OutT>
 __device__ __forceinline__ void big_epilogue(v16f (&acc)[4][4], float alpha, OutT* __restrict__ c, int64_t m0, int64_t n0,
-                                             int64_t N, int wm, int wn, int wave, int lane, uint8_t* smem_bytes) {
+                                             int64_t N, int wm, int wn, int wave, int lane, uint8_t* smem_bytes,
+                                             int rows_valid, int cols_valid) {
     const int lrow = lane & 31, half = lane >> 5;
     if constexpr (sizeof(OutT) == 4) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                store_tile<OutT>(acc[i][j], alpha, c, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
+                if (i * 32 < rows_valid && j * 32 < cols_valid)
+                    store_tile<OutT>(acc[i][j], alpha, c, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
     } else {
         uint8_t* region = smem_bytes + wave * (128 * kEpiPitch);
 #pragma unroll
@@ -393,7 +398,7 @@ __device__ __forceinline__ void big_epilogue(v16f (&acc)[4][4], float alpha, Out
         for (int r4 = 0; r4 < 32; ++r4) {
             const int row = r4 * 4 + rsub;
             const uint4 v = *reinterpret_cast<const uint4*>(region + row * kEpiPitch + chunk * 16);
-            *reinterpret_cast<uint4*>(cbase + (int64_t)row * N * 2) = v;
+            if (r4 * 4 < rows_valid && chunk * 8 < cols_valid) *reinterpret_cast<uint4*>(cbase + (int64_t)row * N * 2) = v;
         }
     }
 }
@@ -424,7 +429,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int wm = wave >> 1, wn = wave & 1;
     const int lrow = lane & 31, half = lane >> 5;
     int tm, tn;
-    tile_of_block((int)blockIdx.x, M / kBigM, N / kBigN, tm, tn);
+    tile_of_block((int)blockIdx.x, (M + kBigM - 1) / kBigM, (N + kBigN - 1) / kBigN, tm, tn);
     const int64_t m0 = (int64_t)tm * kBigM, n0 = (int64_t)tn * kBigN;
     const int code_pitch = K / 2, groups = K / 32;
     const int nk = K / kBK;
@@ -437,16 +442,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         // tiled codes: the wave-load's 16 rows x 64 bytes are one 1 KiB tile; same (row, swizzled slot) pick inside it
         const int trow = wave * 64;  // first row of this wave's four wave-loads
         const int tile_off = (lane >> 2) * 64 + cv * 16;
-        plan.a = a_tiled ? a_codes + (m0 + trow) * code_pitch + tile_off : a_codes + (m0 + row) * code_pitch + cv * 16;
-        plan.b = b_tiled ? b_codes + (n0 + trow) * code_pitch + tile_off : b_codes + (n0 + row) * code_pitch + cv * 16;
+        // M and N are multiples of 64: a wave's 64-row share of a panel is inside the matrix or outside it as a whole;
+        // an outside share reads the matrix's last 64 rows instead (its products are dropped by the epilogue)
+        const int64_t ma = m0 + trow < M ? m0 + trow : (int64_t)M - 64;
+        const int64_t nb = n0 + trow < N ? n0 + trow : (int64_t)N - 64;
+        plan.a = a_tiled ? a_codes + ma * code_pitch + tile_off : a_codes + (ma + (lane >> 2)) * code_pitch + cv * 16;
+        plan.b = b_tiled ? b_codes + nb * code_pitch + tile_off : b_codes + (nb + (lane >> 2)) * code_pitch + cv * 16;
         plan.kstep_a = a_tiled ? 1024 : kRowBytes;
         plan.kstep_b = b_tiled ? 1024 : kRowBytes;
         plan.row16_bytes = (int64_t)16 * code_pitch;
         // scales: LDS dword p = wave*64 + lane holds operand row (p>>7)*128 + (p&3)*32 + ((p>>2)&31)
         const int p = wave * 64 + lane;
         const int srow = (p >> 7) * 128 + (p & 3) * 32 + ((p >> 2) & 31);
-        plan.sa = a_scales + (m0 + srow) * groups;
-        plan.sb = b_scales + (n0 + srow) * groups;
+        plan.sa = a_scales + (m0 + srow < M ? m0 + srow : (int64_t)M - 1) * groups;
+        plan.sb = b_scales + (n0 + srow < N ? n0 + srow : (int64_t)N - 1) * groups;
         plan.lds_codes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + wave * 4096));
         plan.lds_scales = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + kSAOff + wave * 256));
     }
@@ -522,7 +531,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
 
     __syncthreads();  // every wave has finished reading the operand ring: it becomes the epilogue stage
-    big_epilogue<OutT>(acc, alpha, c, m0, n0, N, wm, wn, wave, lane, smem_bytes);
+    big_epilogue<OutT>(acc, alpha, c, m0, n0, N, wm, wn, wave, lane, smem_bytes, (int)(M - m0) - wm * 128,
+                       (int)(N - n0) - wn * 128);
 }
 
 // ---- variant for K % 512 == 0: scales travel in blocks of four K steps -----------------------------
@@ -622,7 +632,7 @@ __device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_by
 // all banks.
 __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alpha, uint16_t* __restrict__ c, int64_t m0,
                                                    int64_t n0, int64_t N, int wm, int wn, int wave, int lane_in,
-                                                   uint8_t* smem_bytes) {
+                                                   uint8_t* smem_bytes, int rows_valid, int cols_valid) {
     // The opaque copy keeps the address arithmetic below inside the (rarely executed) epilogue instead of being
     // hoisted out of the K loop, where it would hold dozens of registers across the MFMA schedule.
     int lane = lane_in;
@@ -639,6 +649,7 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
         for (int jp = 0; jp < 2; ++jp) {
+            if (i * 32 >= rows_valid || jp * 64 >= cols_valid) continue;  // uniform: this pass lies outside the matrix
 #pragma unroll
             for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
@@ -667,7 +678,7 @@ template <typename OutT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mxfp4_tn_big4_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ b_codes,
     const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c, int a_tiled,
-    int b_tiled) {
+    int b_tiled, int splits) {
     extern __shared__ uint32_t smem[];
     uint8_t* smem_bytes = reinterpret_cast<uint8_t*>(smem);
     const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)smem;
@@ -675,9 +686,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int lrow = lane & 31, half = lane >> 5;
-    const int tiles_m = M / kBigM, tiles_n = N / kBigN, total = tiles_m * tiles_n;
+    const int tiles_m = (M + kBigM - 1) / kBigM, tiles_n = (N + kBigN - 1) / kBigN, total = tiles_m * tiles_n;
     const int code_pitch = K / 2, groups = K / 32;
-    const int nk = K / kBK;  // a multiple of 4
+    // Split K: a work item is (tile, K range); with splits > 1 (fp32 instantiation only) item (t, s) covers K steps
+    // [s * nk, (s + 1) * nk) and stores its partial sums, unscaled, into slab s of c = [splits][M][N].
+    const int nk = K / kBK / splits;  // K steps per work item, a multiple of 4
+    const int total_items = total * splits;
     const int stride = (int)gridDim.x;
 
     const int swz = (lrow >> 2) & 3;
@@ -704,14 +718,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         plan.lane_scales = (uint32_t)(lane * groups);
     }
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    int load_tm, load_tn;  // tile the load stream is in
-    auto plan_tile = [&](int t) {
+    int load_tm, load_tn, load_split;  // work item the load stream is in
+    auto plan_tile = [&](int item) {
+        const int t = item / splits;
+        load_split = item - t * splits;
         tile_of_block(t, tiles_m, tiles_n, load_tm, load_tn);
-        const int64_t m0 = (int64_t)load_tm * kBigM + wave_u * 64, n0 = (int64_t)load_tn * kBigN + wave_u * 64;
-        plan.a = a_codes + m0 * code_pitch;
-        plan.b = b_codes + n0 * code_pitch;
-        plan.sa = a_scales + m0 * groups;
-        plan.sb = b_scales + n0 * groups;
+        // M and N are multiples of 64: a wave's 64-row share of a panel is inside the matrix or outside it as a whole;
+        // an outside share reads the matrix's last 64 rows instead (its products are dropped by the epilogue)
+        int64_t m0 = (int64_t)load_tm * kBigM + wave_u * 64, n0 = (int64_t)load_tn * kBigN + wave_u * 64;
+        m0 = m0 < M ? m0 : (int64_t)M - 64;
+        n0 = n0 < N ? n0 : (int64_t)N - 64;
+        const int64_t k0 = (int64_t)load_split * nk;  // first K step of the item
+        plan.a = a_codes + m0 * code_pitch + k0 * plan.kstep_a;
+        plan.b = b_codes + n0 * code_pitch + k0 * plan.kstep_b;
+        plan.sa = a_scales + m0 * groups + k0 * 4;
+        plan.sb = b_scales + n0 * groups + k0 * 4;
     };
 
     plan_tile((int)blockIdx.x);
@@ -729,9 +750,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     big_read_sub(smem_bytes, a_off0, b_off0, st.f0);
 
     int par = 0;
-    for (int t = (int)blockIdx.x; t < total; t += stride) {
+    for (int t = (int)blockIdx.x; t < total_items; t += stride) {
         v16f acc[4][4];
-        const int64_t m0 = (int64_t)load_tm * kBigM, n0 = (int64_t)load_tn * kBigN;  // the load stream is still in tile t
+        const int64_t m0 = (int64_t)load_tm * kBigM, n0 = (int64_t)load_tn * kBigN;  // the load stream is still in item t
+        const int cur_split = load_split;
+        const int rows_valid = (int)(M - m0) - wm * 128, cols_valid = (int)(N - n0) - wn * 128;
         // One block of four K steps.  The load stream is four K steps ahead and rolls over into the next tile;
         // after the last tile it re-requests the current steps (never consumed), which keeps the outstanding-load
         // counts uniform.  FIRST: the tile's first products overwrite the accumulators instead of adding to them.
@@ -739,7 +762,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             constexpr bool FIRST = decltype(first)::value;
             int lks = ks + 4;
             if (lks == nk) {
-                if (t + stride < total) {
+                if (t + stride < total_items) {
                     plan_tile(t + stride);
                     lks = 0;
                 } else {
@@ -755,40 +778,88 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         block4(0, std::true_type{});
         for (int ks = 4; ks < nk; ks += 4) block4(ks, std::false_type{});
         if constexpr (sizeof(OutT) == 2) {
-            big4_epilogue_bf16(acc, alpha, reinterpret_cast<uint16_t*>(c), m0, n0, N, wm, wn, wave, lane, smem_bytes);
+            big4_epilogue_bf16(acc, alpha, reinterpret_cast<uint16_t*>(c), m0, n0, N, wm, wn, wave, lane, smem_bytes,
+                               rows_valid, cols_valid);
         } else {
+            OutT* dst = splits > 1 ? c + (int64_t)cur_split * M * N : c;
+            const float a_eff = splits > 1 ? 1.0f : alpha;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    store_tile<OutT>(acc[i][j], alpha, c, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
+                    if (i * 32 < rows_valid && j * 32 < cols_valid)
+                        store_tile<OutT>(acc[i][j], a_eff, dst, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
         }
     }
     // direct-to-LDS loads must not outlive the workgroup's LDS allocation
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
 }
 
+// c[i] = alpha * (p[0][i] + p[1][i] + ... ) in slab order: the fixed order makes split-K results reproducible
+template <typename OutT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int splits, int64_t mn,
+                                                            float alpha, OutT* __restrict__ c) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= mn) return;  // mn is a multiple of 4 (N % 64 == 0)
+    float4 acc = *reinterpret_cast<const float4*>(partial + i);
+    for (int s = 1; s < splits; ++s) {
+        const float4 v = *reinterpret_cast<const float4*>(partial + (int64_t)s * mn + i);
+        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    }
+    acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
+    if constexpr (sizeof(OutT) == 4) {
+        *reinterpret_cast<float4*>(c + i) = acc;
+    } else {
+        const uint32_t lo = (uint32_t)f32_to_bf16(acc.x) | ((uint32_t)f32_to_bf16(acc.y) << 16);
+        const uint32_t hi = (uint32_t)f32_to_bf16(acc.z) | ((uint32_t)f32_to_bf16(acc.w) << 16);
+        *reinterpret_cast<uint2*>(c + i) = make_uint2(lo, hi);
+    }
+}
+
+int device_cus() {
+    static int cached = 0;  // one GPU model per process
+    if (cached > 0) return cached;
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+        n > 0)
+        return cached = n;
+    return 256;
+}
+
+// How many K ranges to cut a GEMM into so that its (tile, range) items fill the CUs: the divisor s of K/512 that
+// minimises rounds(s) * steps(s) plus a per-item overhead, each range keeping at least eight K steps.  1 = no split.
+int choose_splits(int64_t M, int64_t N, int64_t K, int cus) {
+    const int64_t tiles = ((M + kBigM - 1) / kBigM) * ((N + kBigN - 1) / kBigN);
+    const int64_t nblk = K / 512;
+    if (tiles * 4 >= cus * 3 || nblk < 4) return 1;
+    int best = 1;
+    double best_cost = 1e30;
+    for (int sp = 1; sp <= nblk && sp <= 64; ++sp) {
+        if (nblk % sp || (nblk / sp) * 4 < 8) continue;
+        const int64_t rounds = (tiles * sp + cus - 1) / cus;
+        const double cost = (double)rounds * ((double)(nblk / sp) * 4 + 6.0) + (sp > 1 ? 4.0 + 0.5 * sp : 0.0);
+        if (cost < best_cost - 1e-9) {
+            best_cost = cost;
+            best = sp;
+        }
+    }
+    return best;
+}
+
 template <typename OutT>
 hipError_t launch_big4(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                        const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_tiled,
-                       int b_tiled, hipStream_t stream) {
+                       int b_tiled, int splits, int cus, hipStream_t stream) {
     auto kern = gemm_mxfp4_tn_big4_kernel<OutT>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kBig4SmemBytes);
     if (e != hipSuccess) return e;
-    const int64_t tiles = (M / kBigM) * (N / kBigN);
-    int cus = 256;
-    {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-    }
-    // one workgroup per CU, and a grid that is a multiple of 8 so that tile t and t + grid land on the same XCD
-    int64_t g = tiles < cus ? tiles : cus;
+    const int64_t items = ((M + kBigM - 1) / kBigM) * ((N + kBigN - 1) / kBigN) * splits;
+    // one workgroup per CU, and a grid that is a multiple of 8 so that item t and t + grid land on the same XCD
+    int64_t g = items < cus ? items : cus;
     if (g > 8) g -= g % 8;
     dim3 grid((unsigned)g), block(256);
     kern<<<grid, block, kBig4SmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
-                                                  reinterpret_cast<OutT*>(c), a_tiled, b_tiled);
+                                                  reinterpret_cast<OutT*>(c), a_tiled, b_tiled, splits);
     return hipGetLastError();
 }
 
@@ -799,7 +870,7 @@ hipError_t launch_big(const uint8_t* a_codes, const uint8_t* a_scales, const uin
     auto kern = gemm_mxfp4_tn_big_kernel<OutT>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kBigSmemBytes);
     if (e != hipSuccess) return e;
-    dim3 grid((unsigned)((M / kBigM) * (N / kBigN))), block(256);
+    dim3 grid((unsigned)(((M + kBigM - 1) / kBigM) * ((N + kBigN - 1) / kBigN))), block(256);
     kern<<<grid, block, kBigSmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
                                                  reinterpret_cast<OutT*>(c), a_tiled, b_tiled);
     return hipGetLastError();
@@ -831,21 +902,45 @@ hipError_t launch_gemm(const uint8_t* a_codes, const uint8_t* a_scales, const ui
 
 }  // namespace
 
-// tiled operands are read by the 256x256-tile kernels only
+// Shapes the 256x256-tile kernels serve (they also read tiled operands): extents multiples of 64 and at least one
+// full tile wide, K a multiple of 128; tiles hanging over the edge of M or N compute on clamped rows and store nothing there.
 bool gemm_supports_tiled(int64_t M, int64_t N, int64_t K) {
-    return M % kBigM == 0 && N % kBigN == 0 && K > 0 && K % kBK == 0 && M < (1 << 30) && N < (1 << 30) && K < (1 << 30);
+    return M % 64 == 0 && N % 64 == 0 && M >= kBigM && N >= kBigN && K > 0 && K % kBK == 0 && M < (1 << 30) && N < (1 << 30) &&
+           K < (1 << 30);
+}
+
+// bytes of scratch with which gemm_mxfp4_tn cuts this shape into K ranges (0: it would not)
+size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (!gemm_supports_tiled(M, N, K) || K % 512) return 0;
+    const int sp = choose_splits(M, N, K, device_cus());
+    return sp > 1 ? (size_t)sp * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 
 hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                          const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
-                         int a_layout, int b_layout, hipStream_t stream) {
+                         int a_layout, int b_layout, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     if (M == 0 || N == 0) return hipSuccess;
     const int at = a_layout == LAYOUT_TILED, bt = b_layout == LAYOUT_TILED;
     const bool big_ok = gemm_supports_tiled(M, N, K);
     if ((at || bt) && !big_ok) return hipErrorInvalidValue;
     if (big_ok && K % 512 == 0 && (reinterpret_cast<uintptr_t>(a_scales) & 15) == 0 && (reinterpret_cast<uintptr_t>(b_scales) & 15) == 0) {
-        if (c_dtype == BF16) return launch_big4<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, stream);
-        return launch_big4<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, stream);
+        const int cus = device_cus();
+        int sp = workspace ? choose_splits(M, N, K, cus) : 1;
+        if (sp > 1 && ((size_t)sp * M * N * sizeof(float) > workspace_bytes || (reinterpret_cast<uintptr_t>(workspace) & 15))) sp = 1;
+        if (sp > 1) {
+            // partial sums per K range in fp32 (plain accumulator layout), then one ordered reduction
+            hipError_t e = launch_big4<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, 1.0f, workspace, at, bt, sp, cus, stream);
+            if (e != hipSuccess) return e;
+            const int64_t mn = M * N;
+            dim3 grid((unsigned)((mn / 4 + 255) / 256)), block(256);
+            if (c_dtype == BF16)
+                splitk_reduce_kernel<uint16_t><<<grid, block, 0, stream>>>(static_cast<const float*>(workspace), sp, mn, alpha, static_cast<uint16_t*>(c));
+            else
+                splitk_reduce_kernel<float><<<grid, block, 0, stream>>>(static_cast<const float*>(workspace), sp, mn, alpha, static_cast<float*>(c));
+            return hipGetLastError();
+        }
+        if (c_dtype == BF16) return launch_big4<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, 1, cus, stream);
+        return launch_big4<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, 1, cus, stream);
     }
     if (big_ok) {
         if (c_dtype == BF16) return launch_big<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, stream);

@@ -51,7 +51,8 @@ hipError_t requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* s
 
 hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                          const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
-                         int a_layout, int b_layout, hipStream_t stream);
+                         int a_layout, int b_layout, void* workspace, size_t workspace_bytes, hipStream_t stream);
+size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 hipError_t masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t cols, int hd, int scale_dtype,
                                const SignBits& sb, const uint8_t* maskbits, void* out, int out_dtype,

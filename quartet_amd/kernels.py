@@ -100,16 +100,21 @@ def requantize_transposed_mxfp4(codes, scales, post=1.0, val_dtype=torch.bfloat1
     return codes_out, scales_out, deq
 
 
-def gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, alpha=1.0, out_dtype=torch.bfloat16, a_tiled=False, b_tiled=False):
-    """[M,K/2],[M,K/32] x [N,K/2],[N,K/32] -> alpha * A @ B^T as [M,N] of out_dtype."""
+def gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, alpha=1.0, out_dtype=torch.bfloat16, a_tiled=False, b_tiled=False,
+                  split_k=True):
+    """[M,K/2],[M,K/32] x [N,K/2],[N,K/32] -> alpha * A @ B^T as [M,N] of out_dtype.  With `split_k` the library
+    may cut a long-K, few-tile product into K ranges (scratch is allocated here when it asks for it)."""
     _require_cuda(a_codes, a_scales, b_codes, b_scales)
     M, K = a_codes.shape[0], a_codes.shape[1] * 2
     N = b_codes.shape[0]
     if b_codes.shape[1] * 2 != K:
         raise _lib.QuartetHipError(f"gemm_mxfp4_tn: contraction sizes differ ({K} vs {b_codes.shape[1] * 2})")
     c = torch.empty((M, N), dtype=out_dtype, device=a_codes.device)
+    ws_bytes = _lib.lib().qm_gemm_workspace_bytes(M, N, K) if split_k else 0
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a_codes.device) if ws_bytes else None
     rc = _lib.lib().qm_gemm_mxfp4_tn(_ptr(a_codes), _ptr(a_scales), _ptr(b_codes), _ptr(b_scales), M, N, K, alpha,
-                                     _ptr(c), _dtype_code(out_dtype), _layout(a_tiled), _layout(b_tiled), _stream())
+                                     _ptr(c), _dtype_code(out_dtype), _layout(a_tiled), _layout(b_tiled), _ptr(ws), ws_bytes,
+                                     _stream())
     _lib.check(rc, "qm_gemm_mxfp4_tn")
     return c
 

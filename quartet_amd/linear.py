@@ -31,8 +31,8 @@ class QuartetLinearFn(torch.autograd.Function):
         w2 = weight.contiguous()
         out_dtype = torch.bfloat16 if _autocast_bf16() else x.dtype
         # Tiled code bytes (16 rows x 128 elements contiguous) when every operand of the three products qualifies:
-        # all three extents multiples of 256 and Hadamard block 32 throughout; row-major codes otherwise.
-        tiled = (x2.shape[0] % 256 == 0 and in_features % 256 == 0 and weight.shape[0] % 256 == 0 and
+        # all three extents multiples of 128 and at least 256, Hadamard block 32 throughout; row-major codes otherwise.
+        tiled = (all(d % 128 == 0 and d >= 256 for d in (x2.shape[0], in_features, weight.shape[0])) and
                  a_q.hadamard_dim == 32 and w_q.hadamard_dim == 32 and g_q.hadamard_dim == 32)
         y, saved = K.linear_forward(x2, w2, a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits, out_dtype, tiled)
         ctx.save_for_backward(saved)

@@ -87,7 +87,12 @@ def _torch_dequant(codes, scales):
 # workgroup walks several tiles, with an odd and an even number of scale blocks per tile), and K that is a
 # multiple of 128 but not of 512 (per-step scale loads).
 @pytest.mark.parametrize("M,N,K_", [(256, 256, 512), (512, 768, 1024), (4352, 4352, 512), (4608, 4352, 1024),
-                                    (768, 512, 1536), (512, 256, 640), (4352, 4608, 384), (8192, 4096, 2048)])
+                                    (768, 512, 1536), (512, 256, 640), (4352, 4608, 384), (8192, 4096, 2048),
+                                    # tiles hanging over the edge of M and/or N (extents multiples of 64, not of 256)
+                                    (320, 256, 512), (256, 448, 640), (640, 1920, 640), (1728, 640, 1024), (4416, 4160, 512),
+                                    (320, 320, 128),
+                                    # few output tiles, long K: cut into K ranges (split-K) when scratch is offered
+                                    (512, 256, 8192), (320, 640, 16384), (1920, 640, 4096)])
 @pytest.mark.parametrize("exact", [True, False])
 def test_gemm_tile_kernels(oracle, K, M, N, K_, exact):
     print(f"case gemm tiles {M}x{N}x{K_} exact={exact}", flush=True)
@@ -116,7 +121,8 @@ def test_gemm_tile_kernels(oracle, K, M, N, K_, exact):
     assert torch.equal(got16, got32.to(torch.bfloat16))
 
 
-@pytest.mark.parametrize("M,N,K_", [(256, 256, 512), (768, 512, 1536), (512, 256, 640), (4352, 4608, 1024)])
+@pytest.mark.parametrize("M,N,K_", [(256, 256, 512), (768, 512, 1536), (512, 256, 640), (4352, 4608, 1024), (640, 1920, 640),
+                                    (1728, 448, 1024)])
 @pytest.mark.parametrize("a_tiled,b_tiled", [(True, True), (True, False), (False, True)])
 def test_gemm_tiled_operands_match_rowmajor(K, M, N, K_, a_tiled, b_tiled):
     print(f"case gemm tiled {M}x{N}x{K_} a={a_tiled} b={b_tiled}", flush=True)
@@ -135,3 +141,25 @@ def test_gemm_tiled_operands_match_rowmajor(K, M, N, K_, a_tiled, b_tiled):
     # same kernel, same summation order: the layout only changes where the operand bytes are fetched from
     assert torch.equal(got, want)
     assert torch.equal(got16, want.to(torch.bfloat16))
+
+
+def test_split_k_is_offered_and_reproducible(K):
+    from quartet_amd import _lib
+    L = _lib.lib()
+    assert L.qm_gemm_workspace_bytes(512, 256, 8192) > 0          # 2 tiles, 64 K steps
+    assert L.qm_gemm_workspace_bytes(8192, 4096, 4096) == 0       # 512 tiles fill the chip
+    assert L.qm_gemm_workspace_bytes(512, 256, 640) == 0          # K not a multiple of 512
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(5)
+    M, N, K_ = 512, 256, 8192
+    ac = torch.randint(0, 256, (M, K_ // 2), generator=g, dtype=torch.uint8).to(dev)
+    bc = torch.randint(0, 256, (N, K_ // 2), generator=g, dtype=torch.uint8).to(dev)
+    as_ = torch.randint(118, 132, (M, K_ // 32), generator=g, dtype=torch.uint8).to(dev)
+    bs = torch.randint(120, 136, (N, K_ // 32), generator=g, dtype=torch.uint8).to(dev)
+    a = K.gemm_mxfp4_tn(ac, as_, bc, bs, 1.5, torch.float32)
+    b = K.gemm_mxfp4_tn(ac, as_, bc, bs, 1.5, torch.float32)
+    plain = K.gemm_mxfp4_tn(ac, as_, bc, bs, 1.5, torch.float32, split_k=False)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)  # fixed reduction order
+    rel = float((a.double() - plain.double()).norm() / plain.double().norm())
+    assert rel < 1e-6, rel

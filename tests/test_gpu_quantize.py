@@ -244,7 +244,7 @@ def test_tiled_layout_rejections(K):
         K.quantize_mxfp4(x, 32, None, 2, u=torch.rand(32, 256, device=dev), tiled=True)
     c = torch.zeros(128, 64, dtype=torch.uint8, device=dev)
     sc = torch.full((128, 4), 127, dtype=torch.uint8, device=dev)
-    with pytest.raises(QuartetHipError):                          # GEMM: 128 rows are not a 256-row tile
+    with pytest.raises(QuartetHipError):                          # GEMM: 128 rows are less than one 256-row tile
         K.gemm_mxfp4_tn(c, sc, c, sc, 1.0, torch.float32, a_tiled=True)
 
 
