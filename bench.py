@@ -21,8 +21,8 @@ PEAK_FP4_TFLOPS = 10100.0   # MI355X dense MXFP4 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch from profiler byte counters (fetch + write), scaled by what the same counters read for a
 # plain 256 MiB device copy (fetch counter x 2.0 KiB, write counter x 1.0 KiB)
-GEMM_TRAFFIC_BYTES = 174.6e6      # mean of the three GEMMs: 108.4 MiB fetched (operand re-reads that miss L2) + 58.2 MiB written
-QUANTIZE_TRAFFIC_BYTES = 89.2e6   # 64.1 MiB fetched + 21.0 MiB written; algorithmic 89.1e6
+GEMM_TRAFFIC_BYTES = 173.9e6      # mean of the three GEMMs: 108.7 MiB fetched (operand re-reads that miss L2) + 57.1 MiB written
+QUANTIZE_TRAFFIC_BYTES = 89.8e6   # 64.1 MiB fetched + 21.5 MiB written; algorithmic 89.1e6
 
 
 def make_inputs(device, tokens=T_TOKENS, seed=0):
