@@ -266,23 +266,37 @@ __global__ __launch_bounds__(256) void quantize_rowmajor_g32_kernel(const T* __r
     finish_group<T, MODE, WANT_MASK>(v, gi, gi, c, sign_word, seed, out);
 }
 
-// Tiled code layout ([rows/16][cols/128][16 rows][64 bytes]): a wave owns one 1 KiB tile = 16 rows x 4 groups, so
-// its codes leave as one contiguous KiB; its input is 16 row segments of 4 groups (256 bytes of bf16) each.
-// blockIdx.x = block of 16 rows, blockIdx.y = run of four 128-column blocks (one per wave).
+// Tiled code layout ([rows/16][cols/128][16 rows][64 bytes]).  Workgroup b owns block b / chunks of 16 rows and run
+// b % chunks of 512 columns (four code tiles); wave w owns rows 4w..4w+3 of the block, lane l its row l / 16 and
+// group l % 16 of the run: the wave reads four contiguous KiB (bf16) and writes, per tile, four rows' 64-byte pieces
+// = 256 contiguous bytes.  The four scale bytes of four adjacent groups are gathered into one dword store.
 template <typename T, int MODE, bool WANT_MASK>
-__global__ __launch_bounds__(256) void quantize_rowmajor_g32_tiled_kernel(const T* __restrict__ x, int64_t cols, float c,
-                                                                          uint32_t sign_word, uint64_t seed,
+__global__ __launch_bounds__(256) void quantize_rowmajor_g32_tiled_kernel(const T* __restrict__ x, int64_t cols, int chunks,
+                                                                          float c, uint32_t sign_word, uint64_t seed,
                                                                           GroupOut out) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t kblocks = cols / 128;
-    const int64_t kb = (int64_t)blockIdx.y * 4 + wave;
-    if (kb >= kblocks) return;
-    const int64_t r = (int64_t)blockIdx.x * 16 + (lane >> 2);
-    const int64_t gi = r * (cols / 32) + kb * 4 + (lane & 3);
-    const int64_t ci = ((int64_t)blockIdx.x * kblocks + kb) * 64 + lane;
+    const int groups = (int)(cols / 32);  // per row
+    const unsigned rb = blockIdx.x / (unsigned)chunks;
+    const int g = (int)(blockIdx.x - rb * chunks) * 16 + (lane & 15);  // group within the row
+    if (g >= groups) return;  // cols % 128 == 0: quads of lanes leave together, the gather below sees full quads
+    const int rin = wave * 4 + (lane >> 4);  // row within the block
+    // uniform 64-bit block bases + small per-lane offsets
+    const int64_t gi = (int64_t)rb * 16 * groups + (rin * groups + g);
+    const int64_t ci = (int64_t)rb * 16 * groups + ((g >> 2) * 64 + rin * 4 + (g & 3));
     float v[32];
     load_group<T>(x + gi * 32, v);
-    finish_group<T, MODE, WANT_MASK>(v, gi, ci, c, sign_word, seed, out);
+    rotate_group(v, c, sign_word);
+    GroupCodes o;
+    quantize_group_regs<MODE, WANT_MASK>(v, seed, gi, o);
+    out.codes[ci] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
+    // quad_perm broadcasts of lanes 1, 2, 3 of each quad
+    const uint32_t s1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0x55, 0xf, 0xf, false);
+    const uint32_t s2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0xAA, 0xf, 0xf, false);
+    const uint32_t s3 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0xFF, 0xf, 0xf, false);
+    if ((lane & 3) == 0)
+        *reinterpret_cast<uint32_t*>(out.scales + gi) = o.scale_byte | (s1 << 8) | (s2 << 16) | (s3 << 24);
+    if constexpr (WANT_MASK) out.maskbits[gi] = o.keep;
+    if (out.dequant) store_dequant<T>(reinterpret_cast<T*>(out.dequant) + gi * 32, o);
 }
 
 template <typename T, bool WANT_MASK>
@@ -290,12 +304,13 @@ void launch_rowmajor_g32(int mode, const void* x, int64_t rows, int64_t cols, bo
                          uint64_t seed, const GroupOut& out, hipStream_t stream) {
     const T* xp = reinterpret_cast<const T*>(x);
     if (tiled) {
-        dim3 grid((unsigned)(rows / 16), (unsigned)((cols / 128 + 3) / 4)), block(256);
+        const int chunks = (int)((cols / 128 + 3) / 4);
+        dim3 grid((unsigned)((rows / 16) * chunks)), block(256);
         switch (mode) {
-            case QUEST_RTN: quantize_rowmajor_g32_tiled_kernel<T, QUEST_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, c, sign_word, seed, out); break;
-            case ABSMAX_RTN: quantize_rowmajor_g32_tiled_kernel<T, ABSMAX_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, c, sign_word, seed, out); break;
-            case ABSMAX_SR: quantize_rowmajor_g32_tiled_kernel<T, ABSMAX_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, c, sign_word, seed, out); break;
-            default: quantize_rowmajor_g32_tiled_kernel<T, QUEST_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, c, sign_word, seed, out); break;
+            case QUEST_RTN: quantize_rowmajor_g32_tiled_kernel<T, QUEST_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, chunks, c, sign_word, seed, out); break;
+            case ABSMAX_RTN: quantize_rowmajor_g32_tiled_kernel<T, ABSMAX_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, chunks, c, sign_word, seed, out); break;
+            case ABSMAX_SR: quantize_rowmajor_g32_tiled_kernel<T, ABSMAX_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, chunks, c, sign_word, seed, out); break;
+            default: quantize_rowmajor_g32_tiled_kernel<T, QUEST_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, chunks, c, sign_word, seed, out); break;
         }
         return;
     }
