@@ -1,4 +1,4 @@
-// MXFP4 x MXFP4 "TN" GEMM on gfx950's block-scaled FP4 MFMA (K2).
+// MXFP4 x MXFP4 "TN" GEMM on gfx950's block-scaled FP4 MFMA.
 //
 //   C[m, n] = alpha * sum_k A[m, k] * B[n, k]
 //
@@ -14,10 +14,15 @@
 // in the two successive MFMAs; both operands use the same assignment, which is all the
 // instruction needs.
 //
-// Tiling: workgroup = 4 waves, macro tile BM x BN, each wave owns a WM x WN block of 32x32 MFMA
-// tiles with fp32 accumulators in registers.  Operands are staged global -> registers -> LDS
-// (rows padded from 64 to 80 bytes so the 16-byte fragment reads of 16 consecutive rows hit 64
-// distinct banks), double buffered, one barrier per K step.
+// Three kernels, picked by shape in gemm_mxfp4_tn() at the end of the file:
+//   gemm_mxfp4_tn_big4_kernel  M, N multiples of 64 and >= 256, K % 512 == 0.  Persistent, 256x256 macro tile,
+//                              4 waves x 128x128, operands global -> LDS directly into a 4-stage ring, scales in
+//                              blocks of four K steps, row-major or tiled code bytes, optional split-K.
+//   gemm_mxfp4_tn_big_kernel   same tile for other K % 128 == 0: one workgroup per tile, scales per K step.
+//   gemm_mxfp4_tn_kernel       any M, N and K % 32 == 0: 128x128 macro tile, 4 waves x 64x64, operands staged
+//                              global -> registers -> LDS (rows padded from 64 to 80 bytes so the 16-byte fragment
+//                              reads of 16 consecutive rows hit 64 distinct banks), double buffered.
+// All keep fp32 accumulators in registers, use one barrier per K step and apply alpha in the epilogue.
 #include <hip/hip_runtime.h>
 #include <type_traits>
 #include <stdint.h>

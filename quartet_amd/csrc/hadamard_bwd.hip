@@ -1,4 +1,4 @@
-// Straight-through backward of the forward quantizer (K3) and the MXFP4 de-quantizer.
+// Straight-through backward of the forward quantizer and the MXFP4 de-quantizer.
 //
 // masked_hadamard_bwd replaces src/models/quantization/quantizers/mxfp4.py:143-146
 //     grad_in = ((grad_out * mask).view(-1, hd)) @ H^T,   H = c * S * diag(signs)

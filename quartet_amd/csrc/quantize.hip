@@ -1,4 +1,4 @@
-// Fused block-Hadamard rotation + MXFP4 quantizer for gfx950 (K1 family).
+// Fused block-Hadamard rotation + MXFP4 quantizer for gfx950.
 //
 // Replaces the reference's Triton kernel src/models/quantization/quantizers/mxfp4_triton.py:19-174
 // and, for the transposed / re-quantizing variants, the .T.contiguous() copies followed by that

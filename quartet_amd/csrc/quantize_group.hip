@@ -1,4 +1,5 @@
-// Fast path of the fused block-Hadamard + MXFP4 quantizer for Hadamard block 32 (K1, "group layout").
+// Fast path of the fused block-Hadamard + MXFP4 quantizer ("group layout"): Hadamard block 32 for row-major,
+// transposed and packed (re-quantize) input; Hadamard blocks 64 and 128 for row-major input.
 //
 // Same arithmetic as quantize.hip (the reference kernel
 // src/models/quantization/quantizers/mxfp4_triton.py:19-174), different work decomposition: one lane

@@ -1,4 +1,4 @@
-"""GPU parity of the MXFP4 x MXFP4 GEMM (K2) against the oracle's fp64 matmul of the de-quantized
+"""GPU parity of the MXFP4 x MXFP4 GEMM against the oracle's fp64 matmul of the de-quantized
 operands: relative Frobenius error <= 1e-3 (the tolerance the target states); bit-exact in the
 special cases where every partial sum is exactly representable."""
 import numpy as np

@@ -1,4 +1,4 @@
-"""GPU parity of the K1 quantizer family against the CPU oracle: FP4 codes, E8M0 scales, clip-mask
+"""GPU parity of the quantizer family against the CPU oracle: FP4 codes, E8M0 scales, clip-mask
 bits and the de-quantized tensor must be bit-exact (integer/byte work), through the C ABI."""
 import numpy as np
 import pytest
