@@ -1,23 +1,46 @@
-"""Backward schemes: which GEMM operands of a linear layer's backward are quantized.
-Same classes, registry keys and operand orientation as the reference's
-src/models/quantization/backward.py; these generic schemes run on the pseudo-quantized
-(de-quantized) tensors the quantizer modules return, with library GEMMs.  The production
-combination is short-circuited to the packed-FP4 path in quartet_amd.linear."""
-import math
+"""Backward schemes: which operands of a linear layer's two gradient products are quantized.
 
-import torch
+Registry keys, class names and operand orientation follow the reference's
+src/models/quantization/backward.py; these generic schemes work on the pseudo-quantized (de-quantized)
+tensors the quantizer modules return and use library GEMMs.  The production combination never gets here:
+``quartet_amd.linear`` routes it to the packed-FP4 path.
+
+For y = x W^T with upstream gradient e (tokens flattened to rows):
+
+    scheme key                  grad_x                   grad_W                     sign re-randomisation
+    EW_EtX                      e W                      e^T x                      -
+    Q(E)W_Q(Et)X                Q(e) W                   Q(e^T) x                   -
+    Q(E)Q(Wt)t_Q(Et)Q(Xt)t      Q(e) Q(W^T)^T            Q(e^T) Q(x^T)^T            once, before the four Q(.)
+
+Every Q(.) quantizes along its tensor's last axis, which is the contraction axis of the product it feeds,
+hence the explicit transposes."""
 import torch.nn as nn
 import torch.nn.functional as F
 from torch.autograd import Function
 
 
-class EW_EtX_Scheme(nn.Module):
-    def __init__(self):
-        super().__init__()
-        self.g_quantizer = None
+def _save_and_multiply(ctx, x, w, g_quantizer):
+    ctx.save_for_backward(x, w)
+    ctx.g_quantizer = g_quantizer
+    return F.linear(x, w, None)
 
-    def forward(self, x, w):
-        return F.linear(x, w, None)
+
+def _gradients(ctx, e, quantize_saved):
+    """The two gradient products with the gradient quantizer applied to e (always) and, when
+    ``quantize_saved``, to the saved operands as well."""
+    x, w = ctx.saved_tensors
+    q = ctx.g_quantizer
+    out_features, in_features = w.shape
+    x_rows = x.reshape(-1, in_features)
+    e_rows = e.reshape(-1, out_features)
+    if quantize_saved:
+        q.re_randomize()
+        grad_x = q(e) @ q(w.T.contiguous()).T
+        grad_w = q(e_rows.T.contiguous()) @ q(x_rows.T.contiguous()).T
+    else:
+        grad_x = q(e) @ w
+        grad_w = q(e_rows.T.contiguous()) @ x_rows
+    return grad_x, grad_w, None
 
 
 class QEW_QEtXFn(Function):
@@ -25,48 +48,46 @@ class QEW_QEtXFn(Function):
 
     @staticmethod
     def forward(ctx, x, w, g_quantizer):
-        ctx.save_for_backward(x, w)
-        ctx.g_quantizer = g_quantizer
-        return F.linear(x, w, None)
+        return _save_and_multiply(ctx, x, w, g_quantizer)
 
     @staticmethod
     def backward(ctx, e):
-        x, w = ctx.saved_tensors
-        grad_x = F.linear(ctx.g_quantizer(e), w.T, None)
-        tokens = math.prod(x.shape[:-1])
-        grad_w = torch.einsum("ib,bj->ij", ctx.g_quantizer(e.reshape(tokens, -1).T.contiguous()),
-                              x.reshape(tokens, -1))
-        return grad_x, grad_w, None
-
-
-class QEW_QEtX_Scheme(EW_EtX_Scheme):
-    def forward(self, x, w):
-        return QEW_QEtXFn.apply(x, w, self.g_quantizer)
+        return _gradients(ctx, e, quantize_saved=False)
 
 
 class QEQWtt_QEtQXttFn(Function):
-    """backward.py:57-85: all four backward GEMM operands quantized along their contraction axis."""
+    """backward.py:57-85: all four operands of the gradient products are quantized."""
 
     @staticmethod
     def forward(ctx, x, w, g_quantizer):
-        ctx.save_for_backward(x, w)
-        ctx.g_quantizer = g_quantizer
-        return F.linear(x, w, None)
+        return _save_and_multiply(ctx, x, w, g_quantizer)
 
     @staticmethod
     def backward(ctx, e):
-        x, w = ctx.saved_tensors
-        ctx.g_quantizer.re_randomize()
-        grad_x = F.linear(ctx.g_quantizer(e), ctx.g_quantizer(w.T.contiguous()), None)
-        tokens = math.prod(x.shape[:-1])
-        grad_w = torch.einsum("ib,jb->ij", ctx.g_quantizer(e.reshape(tokens, -1).T.contiguous()),
-                              ctx.g_quantizer(x.reshape(tokens, -1).T.contiguous()))
-        return grad_x, grad_w, None
+        return _gradients(ctx, e, quantize_saved=True)
+
+
+class EW_EtX_Scheme(nn.Module):
+    """No quantization in backward; ``g_quantizer`` is attached by QuantizedLinear and unused here."""
+
+    fn = None
+
+    def __init__(self):
+        super().__init__()
+        self.g_quantizer = None
+
+    def forward(self, x, w):
+        if self.fn is None:
+            return F.linear(x, w, None)
+        return self.fn.apply(x, w, self.g_quantizer)
+
+
+class QEW_QEtX_Scheme(EW_EtX_Scheme):
+    fn = QEW_QEtXFn
 
 
 class QEQWtt_QEtQXtt_Scheme(QEW_QEtX_Scheme):
-    def forward(self, x, w):
-        return QEQWtt_QEtQXttFn.apply(x, w, self.g_quantizer)
+    fn = QEQWtt_QEtQXttFn
 
 
 BACKWARD_SCHEMES = {

@@ -1,6 +1,6 @@
 """Quantizer registry: the names the reference's CLI and model constructors use
 (src/models/quantization/quantizers/__init__.py:59-100) for the MXFP4 path."""
-from .base import OPTIMAL_GAUSSIAN_SCALES, BaseQuantizer, NoQuantizer
+from .base import BaseQuantizer, NoQuantizer
 from .mxfp4 import (AlbertTsengQuantizer, AlignedAlbertTsengQuantizer, QuestMXFP4Quantizer,
                     mxfp4_forward_kernel_wrapper)
 
@@ -11,6 +11,6 @@ QUANTIZER_CLASSES = {
     "AlignedAlbertTsengQuantizer": AlignedAlbertTsengQuantizer,
 }
 
-__all__ = ["BaseQuantizer", "NoQuantizer", "OPTIMAL_GAUSSIAN_SCALES", "QuestMXFP4Quantizer",
+__all__ = ["BaseQuantizer", "NoQuantizer", "QuestMXFP4Quantizer",
            "AlbertTsengQuantizer", "AlignedAlbertTsengQuantizer", "mxfp4_forward_kernel_wrapper",
            "QUANTIZER_CLASSES"]

@@ -1,36 +1,35 @@
-"""Quantizer base classes (API of the reference's src/models/quantization/quantizers/base.py:6-37)."""
+"""Quantizer interface shared by every quantizer module (the contract of the reference's
+src/models/quantization/quantizers/base.py:6-24): calling the module returns the pseudo-quantized tensor,
+``re_randomize()`` draws a fresh random rotation where the quantizer has one, and ``bits`` / ``n_levels``
+describe the grid."""
 import torch.nn as nn
 
 
 class BaseQuantizer(nn.Module):
+    """Abstract quantizer: subclasses implement ``forward(x)``; a quantizer without randomness inherits the
+    no-op ``re_randomize``."""
+
     def __init__(self, bits=4):
         super().__init__()
         self.bits = bits
-        self.n_levels = 2 ** bits
+
+    @property
+    def n_levels(self):
+        return 2 ** self.bits
 
     def forward(self, x):
-        raise NotImplementedError
+        raise NotImplementedError(f"{type(self).__name__} does not implement forward()")
 
     def re_randomize(self):
-        pass
+        return None
 
 
 class NoQuantizer(BaseQuantizer):
-    def __init__(self, **kwargs):
-        super().__init__(16)
+    """Identity: the tensor passes through untouched (reported as a 16-bit grid).  Accepts and ignores any
+    keyword arguments so that registry-driven constructors can pass a kwargs dict."""
+
+    def __init__(self, **_ignored):
+        super().__init__(bits=16)
 
     def forward(self, x):
         return x
-
-
-OPTIMAL_GAUSSIAN_SCALES = {
-    1: 0.7978845587140913,
-    1.585: 1.2240089519030855,
-    2: 1.4935346200015913,
-    3: 2.051068354131873,
-    4: 2.513930578568423,
-    5: 2.9160938834961225,
-    6: 3.276597282593217,
-    7: 3.6010497188221655,
-    8: 3.884938678807525,
-}
