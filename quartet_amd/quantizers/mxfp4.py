@@ -41,7 +41,7 @@ def _as_2d(x, hd):
 
 
 def _autocast_bf16():
-    return torch.is_autocast_enabled() and torch.get_autocast_gpu_dtype() == torch.bfloat16
+    return torch.is_autocast_enabled() and torch.get_autocast_dtype("cuda") == torch.bfloat16
 
 
 @torch.compiler.disable()
