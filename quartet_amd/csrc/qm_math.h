@@ -57,12 +57,20 @@ QM_HD float scale_pow2(float x, int e) {
 
 // IEEE round-to-nearest g / fl32(4/3) without a hardware divide: fl32(3/4) is the correctly
 // rounded reciprocal of 0x3FAAAAAB, so one residual correction gives the correctly rounded
-// quotient (checked over every fp32 bit pattern on the host).
+// quotient for |g| >= 2^-104 (checked over every fp32 bit pattern on the host; below that the
+// residual loses bits to underflow, the result keeps g's sign and stays non-zero).
 QM_HD float div_four_thirds(float g) {
     float q0 = g * 0.75f;
     float r = __builtin_fmaf(-q0, kFourThirds, g);
     return __builtin_fmaf(r, 0.75f, q0);
 }
+
+// The same quotient in two operations for |g| >= 2^-100 (and for zeros up to the sign of zero): fl32(4/3) is exactly
+// (4/3)(1 + 2^-25), so 1/fl32(4/3) = 3/4 - 3/2 * 2^-26 + O(2^-50) and one fma over the rounded low part is correctly
+// rounded (checked over every fp32 bit pattern on the host; below 2^-100 the low part loses bits to underflow, the
+// result keeps g's sign and stays non-zero).
+constexpr float kInvFourThirdsLo = -0x1.8p-26f;
+QM_HD float div_four_thirds_fast(float g) { return __builtin_fmaf(g, 0.75f, g * kInvFourThirdsLo); }
 
 // RTN onto the E2M1 magnitudes {0,.5,1,1.5,2,3,4,6}: strict '>' against the seven midpoints,
 // i.e. ties go toward zero and anything above 5 saturates at 6 (mxfp4_triton.py:131-159).

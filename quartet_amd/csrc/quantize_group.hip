@@ -127,15 +127,42 @@ __device__ __forceinline__ void quantize_group_regs(const float (&g)[32], uint64
         o.deq_scale = scale_pow2(kFourThirds, k);
         // |t| < 6 with t = RN(g 2^-k / d): evaluated on the quotient h = RN(g / d) against 6 * 2^k
         thr_bits = f2u(6.0f * hw_scale);
+        // t = RN(RN(g 2^-k) / d) by definition.  For a group whose maximum is at least 2^-60 this is RN(g / d) scaled by
+        // 2^-k inside the convert: the two-operation quotient is exact for |g| >= 2^-100, and a smaller element lies
+        // below 2^-38 of the scale, so its code is a zero whose sign is the element's own whatever the quotient's last
+        // bit.  A group with a smaller non-zero maximum (where g / d would lose bits to underflow) follows the
+        // definition literally, with a true division, and hands the convert an already scaled value.
+        if (__builtin_expect(a < 0x1p-60f && !all_zero, 0)) {
 #pragma unroll
-        for (int i = 0; i < 32; ++i) t[i] = div_four_thirds(g[i]);
+            for (int i = 0; i < 32; ++i) t[i] = scale_pow2(g[i], -k) / kFourThirds;
+            hw_scale = 1.0f;
+            thr_bits = f2u(6.0f);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 32; ++i) t[i] = div_four_thirds_fast(g[i]);
+        }
     }
     o.keep = 0u;
     if constexpr (WANT_MASK) {
         // clip mask, most significant element first so that element 0 lands in bit 0
+        // one compare into the carry flag and one add-with-carry (keep = 2 keep + flag) per element, sixteen
+        // elements per statement (the operand limit of an asm statement)
         uint32_t keep = 0u;
-#pragma unroll
-        for (int i = 31; i >= 0; --i) keep = (keep << 1) | (((f2u(t[i]) & 0x7fffffffu) < thr_bits) ? 1u : 0u);
+        const float thr = u2f(thr_bits);
+#define QM_KEEP_BIT(N) "v_cmp_lt_f32_e64 vcc, |%" #N "|, %17\n\tv_addc_co_u32_e32 %0, vcc, %0, %0, vcc\n\t"
+#define QM_KEEP_16(B)                                                                                               \
+    asm(QM_KEEP_BIT(16) QM_KEEP_BIT(15) QM_KEEP_BIT(14) QM_KEEP_BIT(13) QM_KEEP_BIT(12) QM_KEEP_BIT(11) QM_KEEP_BIT(10) \
+        QM_KEEP_BIT(9) QM_KEEP_BIT(8) QM_KEEP_BIT(7) QM_KEEP_BIT(6) QM_KEEP_BIT(5) QM_KEEP_BIT(4) QM_KEEP_BIT(3)        \
+        QM_KEEP_BIT(2) QM_KEEP_BIT(1)                                                                                   \
+        : "+v"(keep)                                                                                                    \
+        : "v"(t[(B)]), "v"(t[(B) + 1]), "v"(t[(B) + 2]), "v"(t[(B) + 3]), "v"(t[(B) + 4]), "v"(t[(B) + 5]),             \
+          "v"(t[(B) + 6]), "v"(t[(B) + 7]), "v"(t[(B) + 8]), "v"(t[(B) + 9]), "v"(t[(B) + 10]), "v"(t[(B) + 11]),       \
+          "v"(t[(B) + 12]), "v"(t[(B) + 13]), "v"(t[(B) + 14]), "v"(t[(B) + 15]), "v"(thr)                              \
+        : "vcc")
+        QM_KEEP_16(16);
+        QM_KEEP_16(0);
+#undef QM_KEEP_16
+#undef QM_KEEP_BIT
         o.keep = all_zero ? 0u : keep;
     }
 
@@ -238,7 +265,7 @@ __device__ __forceinline__ void rotate_group(float (&v)[32], float c, uint32_t s
     butterfly32(v);
 #pragma unroll
     for (int j = 0; j < 32; ++j) {
-        const float cj = ((sign_word >> j) & 1u) ? -c : c;
+        const float cj = u2f(f2u(c) ^ (((sign_word >> j) & 1u) << 31));  // wave-uniform: stays in scalar registers
         v[j] = v[j] * cj;
     }
 }

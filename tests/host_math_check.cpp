@@ -1,0 +1,118 @@
+// Host build of the kernels' scalar arithmetic (quartet_amd/csrc/qm_math.h) checked against IEEE-754 arithmetic of the
+// host compiler.  Built and run by tests/test_host_math.py; prints one line per failed property and exits non-zero.
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "qm_math.h"
+
+using namespace qm;
+
+static int failures = 0;
+static void fail(const char* what, uint32_t bits) {
+    if (failures++ < 20) std::printf("FAIL %s at 0x%08x\n", what, bits);
+}
+
+static void check_division(uint32_t b) {
+    const float g = u2f(b);
+    if (std::isnan(g) || std::isinf(g)) return;
+    volatile float d = kFourThirds;
+    const float want = g / d;  // correctly rounded by the host
+    const uint32_t mag = b & 0x7fffffffu;
+    if (mag >= (23u << 23)) {  // |g| >= 2^-104
+        if (f2u(div_four_thirds(g)) != f2u(want)) fail("div_four_thirds", b);
+    } else if (mag != 0) {
+        const float got = div_four_thirds(g);
+        if (got == 0.0f || std::signbit(got) != std::signbit(g)) fail("div_four_thirds sign", b);
+    }
+    if (mag >= (27u << 23)) {  // |g| >= 2^-100
+        if (f2u(div_four_thirds_fast(g)) != f2u(want)) fail("div_four_thirds_fast", b);
+    } else if (mag != 0) {
+        // below the exact range the fast form may be off in the last bits but never changes sign or becomes zero
+        const float got = div_four_thirds_fast(g);
+        if (got == 0.0f || std::signbit(got) != std::signbit(g)) fail("div_four_thirds_fast sign", b);
+    }
+    // with the signed-zero rule applied (adding -2^-149) the two forms agree for zeros as well
+    if (mag == 0 && f2u(div_four_thirds_fast(g) + u2f(0x80000001u)) != f2u(want + u2f(0x80000001u))) fail("zero rule", b);
+}
+
+int main() {
+    // every 1021st bit pattern (all exponents, both signs), plus every mantissa of a few binades
+    for (uint64_t b = 0; b < (1ull << 32); b += 1021) check_division((uint32_t)b);
+    const uint32_t binades[] = {0, 1, 22, 23, 24, 26, 27, 28, 100, 126, 127, 128, 200, 253, 254};
+    for (uint32_t e : binades)
+        for (uint32_t m = 0; m < (1u << 23); ++m) {
+            check_division((e << 23) | m);
+            check_division(0x80000000u | (e << 23) | m);
+        }
+
+    // bf16 round trip and round-to-nearest-even
+    for (uint32_t h = 0; h < 65536; ++h) {
+        const float f = bf16_to_f32((uint16_t)h);
+        if (std::isnan(f)) continue;
+        if (f32_to_bf16(f) != h) fail("bf16 round trip", h);
+        const uint32_t base = h << 16;
+        if ((h & 0x7f80u) == 0x7f80u || ((h + 1) & 0x7f80u) == 0x7f80u) continue;
+        // just below / at / just above the midpoint to the next bf16 value
+        if (f32_to_bf16(u2f(base + 0x7fffu)) != h) fail("bf16 below midpoint", h);
+        if (f32_to_bf16(u2f(base + 0x8001u)) != h + 1) fail("bf16 above midpoint", h);
+        if (f32_to_bf16(u2f(base + 0x8000u)) != ((h & 1u) ? h + 1 : h)) fail("bf16 tie to even", h);
+    }
+
+    // E2M1 grid, strict-threshold rounding, stochastic brackets
+    const float grid[8] = {0.f, .5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f};
+    for (int m = 0; m < 8; ++m) {
+        if (e2m1_value(m) != grid[m]) fail("e2m1_value", (uint32_t)m);
+        if (rtn_code(grid[m]) != m) fail("rtn grid point", (uint32_t)m);
+        if (m < 7) {
+            const float mid = 0.5f * (grid[m] + grid[m + 1]);
+            if (rtn_code(mid) != m) fail("rtn tie goes down", (uint32_t)m);
+            if (rtn_code(std::nextafter(mid, 10.f)) != m + 1) fail("rtn above tie goes up", (uint32_t)m);
+            // up with probability p: up iff u < p, never at p = 0, always at p = 1 given u < 1
+            const float a = grid[m] + 0.25f * (grid[m + 1] - grid[m]);
+            if (sr_code(a, 0.2499f) != m + 1 || sr_code(a, 0.25f) != m) fail("sr threshold", (uint32_t)m);
+            if (sr_code(grid[m + 1], 0.999f) != m + 1) fail("sr upper end", (uint32_t)m);
+        }
+    }
+    if (rtn_code(1e9f) != 7 || sr_code(7.5f, 0.f) != 7) fail("saturation", 0);
+
+    // the uniform of a random byte turns "u < p" into the integer comparison floor(p 2^22) > r8 2^14 + 2^13
+    for (uint32_t r8 = 0; r8 < 256; ++r8) {
+        const float u = uniform_from_r8(r8);
+        const uint32_t R = r8 * 16384u + 8192u;
+        for (int d = -2; d <= 2; ++d) {
+            const uint32_t k = R + (uint32_t)d;  // p = k 2^-22, exact in fp32
+            const float p = (float)k * (1.0f / 4194304.0f);
+            if ((u < p) != (k > R)) fail("uniform_from_r8", r8);
+            const float p_half = ((float)k + 0.5f) * (1.0f / 4194304.0f);  // p with bits below 2^-22
+            if ((u < p_half) != (k > R)) fail("uniform_from_r8 (sub-grid p)", r8);
+        }
+    }
+
+    // Philox4x32-10 known-answer vectors (Random123)
+    {
+        const Philox4 a = philox4x32_10(0, 0, 0, 0, 0, 0);
+        const uint32_t wa[4] = {0x6627e8d5u, 0xe169c58du, 0xbc57ac4cu, 0x9b00dbd8u};
+        const Philox4 b = philox4x32_10(0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu);
+        const uint32_t wb[4] = {0x408f276du, 0x41c83b0eu, 0xa20bc7c6u, 0x6d5451fdu};
+        for (int i = 0; i < 4; ++i) {
+            if (a.w[i] != wa[i]) fail("philox zeros", (uint32_t)i);
+            if (b.w[i] != wb[i]) fail("philox ones", (uint32_t)i);
+        }
+    }
+
+    // powers of two and the Hadamard constants
+    for (int e = -149; e <= 127; ++e)
+        if (pow2i(e) != std::ldexp(1.0f, e)) fail("pow2i", (uint32_t)(e + 149));
+    if (hadamard_scale(32, BF16) != 0.1767578125f || hadamard_scale(64, BF16) != 0.125f ||
+        hadamard_scale(128, BF16) != 0.08837890625f || hadamard_scale(32, F32) != (float)std::sqrt(1.0 / 32.0))
+        fail("hadamard_scale", 0);
+
+    if (failures) {
+        std::printf("%d failures\n", failures);
+        return 1;
+    }
+    std::printf("ok\n");
+    return 0;
+}

@@ -165,6 +165,24 @@ def test_rowmajor_group_layout_seeded(oracle, K, mode, dtype, hd):
     _check(oracle, K, x, hd, MODES[mode], signs, False, None, 0xFEED_F00D_CAFE + hd, f"rowmajor-group/{mode}/{dtype}/{hd}")
 
 
+@pytest.mark.parametrize("mode", ["absmax_rtn", "absmax_sr"])
+@pytest.mark.parametrize("transposed", [False, True])
+def test_tiny_magnitudes_follow_the_definition(oracle, K, mode, transposed):
+    """Groups whose maximum lies far below the normal range (down into the denormals) and tiny elements inside
+    ordinary groups: the quotient by fl32(4/3) is computed from the scaled value, as the definition says."""
+    print(f"case tiny magnitudes mode={mode} transposed={transposed}", flush=True)
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(128, 256, generator=g)
+    exps = torch.tensor([0, -20, -50, -59, -60, -61, -70, -90, -100, -104, -110, -120, -124, -126, -130, -140])
+    x = x * torch.pow(2.0, exps.repeat_interleave(8).double())[:, None].float()   # row r scaled by 2^exps[r // 8]
+    x[::8, ::5] *= 2.0 ** -40                                                       # much smaller elements inside each group
+    x[3, :32] = torch.tensor([2.0 ** -149, -(2.0 ** -149), 2.0 ** -148, 0.0] * 8)   # smallest denormals and zero
+    if transposed:
+        x = x.t().contiguous()
+    signs = torch.randint(0, 2, (32,), generator=g) * 2 - 1
+    _check(oracle, K, x, 32, MODES[mode], signs, transposed, None, 0xBEEF + int(transposed), f"tiny/{mode}/{transposed}")
+
+
 # Tiled code layout ([R/16][C/128][16][64 bytes]): the same bytes as the row-major codes, permuted; scales, mask
 # and the de-quantized tensor are unaffected.
 @pytest.mark.parametrize("mode", list(MODES))
