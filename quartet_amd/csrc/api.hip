@@ -193,6 +193,12 @@ WorkLayout work_layout(int64_t T, int64_t I, int64_t O, int mid_dtype) {
     l.total = o;
     return l;
 }
+// The whole-layer calls issue independent launches two to a grid when all of them run on the Hadamard-32 kernels with
+// tiled codes (which needs every extent to be a multiple of 128).
+bool pair_launches(int codes_layout, int64_t T, int64_t I, int64_t O, int hd_a, int hd_b, int hd_c) {
+    return codes_layout == QM_LAYOUT_TILED && hd_a == 32 && hd_b == 32 && hd_c == 32 && T % 128 == 0 && I % 128 == 0 &&
+           O % 128 == 0;
+}
 }  // namespace
 
 size_t qm_linear_saved_bytes(int64_t T, int64_t I, int64_t O) {
@@ -215,12 +221,22 @@ int qm_linear_forward(const void* x, int x_dtype, const void* w, int w_dtype, in
     if (!saved || saved_bytes < l.total || !aligned(saved, 256))
         return fail(QM_ERR_INVALID, "qm_linear_forward: saved buffer needs %zu bytes, 256-byte aligned", l.total);
     uint8_t* s = static_cast<uint8_t*>(saved);
-    int rc = qm_quantize_mxfp4(x, x_dtype, T, I, hd_x, signs_x, QM_QUEST_RTN, 0, nullptr, 0, s + l.xc, s + l.xs, s + l.xm, nullptr,
+    int rc;
+    if (pair_launches(codes_layout, T, I, O, hd_x, hd_w, 32) && x && w && y && valid_dtype(x_dtype) && valid_dtype(w_dtype) &&
+        aligned(x, 16) && aligned(w, 16)) {
+        // both forward quantizers in one grid
+        const qm::RowmajorArgs ax{x, x_dtype, T, I, signs_x ? signs_x[0] : 0u, s + l.xc, s + l.xs, s + l.xm};
+        const qm::RowmajorArgs aw{w, w_dtype, O, I, signs_w ? signs_w[0] : 0u, s + l.wc, s + l.ws, s + l.wm};
+        rc = from_hip(qm::quantize_rowmajor_hd32_tiled_pair(ax, aw, reinterpret_cast<hipStream_t>(stream)), "qm_linear_forward");
+        if (rc) return rc;
+    } else {
+        rc = qm_quantize_mxfp4(x, x_dtype, T, I, hd_x, signs_x, QM_QUEST_RTN, 0, nullptr, 0, s + l.xc, s + l.xs, s + l.xm, nullptr,
                                codes_layout, stream);
-    if (rc) return rc;
-    rc = qm_quantize_mxfp4(w, w_dtype, O, I, hd_w, signs_w, QM_QUEST_RTN, 0, nullptr, 0, s + l.wc, s + l.ws, s + l.wm, nullptr,
-                           codes_layout, stream);
-    if (rc) return rc;
+        if (rc) return rc;
+        rc = qm_quantize_mxfp4(w, w_dtype, O, I, hd_w, signs_w, QM_QUEST_RTN, 0, nullptr, 0, s + l.wc, s + l.ws, s + l.wm, nullptr,
+                               codes_layout, stream);
+        if (rc) return rc;
+    }
     return qm_gemm_mxfp4_tn(s + l.xc, s + l.xs, s + l.wc, s + l.ws, T, O, I, 1.0f, y, y_dtype, codes_layout, codes_layout, nullptr, 0,
                             stream);
 }
@@ -248,13 +264,38 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
     // value = code * 2^k * fl32(4/3) on both operands of the two gradient products
     const float d = (float)(1.0 / 0.75);
     const float alpha = d * d;
-    int rc = qm_quantize_mxfp4(e, e_dtype, T, O, hd_g, signs_g, g_mode, 0, nullptr, seeds[0], k + wl.ec, k + wl.es, nullptr, nullptr,
-                               codes_layout, stream);
+    void* gws = wl.gemm_ws_bytes ? k + wl.gemm_ws : nullptr;
+    hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+    int rc;
+    if (pair_launches(codes_layout, T, I, O, hd_x, hd_w, hd_g) && e && gx && gw && valid_dtype(e_dtype) && aligned(e, 16) &&
+        aligned(gx, 16) && aligned(gw, 16) && valid_dtype(x_val_dtype) && valid_dtype(w_val_dtype) &&
+        valid_dtype(x_scale_dtype) && valid_dtype(w_scale_dtype)) {
+        // seven launches: Q(e) with Q(e^T), Q(Q(W)^T) with Q(Q(x)^T), the two products, the two inverse rotations
+        const uint32_t sg = signs_g ? signs_g[0] : 0u;
+        rc = from_hip(qm::quantize_both_orientations_hd32_tiled(e, e_dtype, T, O, sg, g_mode, seeds[0], seeds[2], k + wl.ec, k + wl.es,
+                                                                k + wl.etc, k + wl.ets, hs), "qm_linear_backward");
+        if (rc) return rc;
+        const qm::RequantArgs rw{s + sl.wc, s + sl.ws, O, I, w_val_dtype, seeds[1], k + wl.wtc, k + wl.wts};
+        const qm::RequantArgs rx{s + sl.xc, s + sl.xs, T, I, x_val_dtype, seeds[3], k + wl.xtc, k + wl.xts};
+        rc = from_hip(qm::requantize_transposed_hd32_tiled_pair(rx, rw, sg, g_mode, hs), "qm_linear_backward");
+        if (rc) return rc;
+        rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, k + wl.gxq, mid_dtype, codes_layout,
+                              codes_layout, gws, wl.gemm_ws_bytes, stream);
+        if (rc) return rc;
+        rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, k + wl.gwq, mid_dtype, codes_layout,
+                              codes_layout, gws, wl.gemm_ws_bytes, stream);
+        if (rc) return rc;
+        return from_hip(qm::masked_hadamard_bwd_hd32_pair(k + wl.gxq, T * I, x_scale_dtype,
+                                                          signs_x ? signs_x[0] : 0u, s + sl.xm, gx, k + wl.gwq, O * I,
+                                                          w_scale_dtype, signs_w ? signs_w[0] : 0u,
+                                                          s + sl.wm, gw, mid_dtype, hs), "qm_linear_backward");
+    }
+    rc = qm_quantize_mxfp4(e, e_dtype, T, O, hd_g, signs_g, g_mode, 0, nullptr, seeds[0], k + wl.ec, k + wl.es, nullptr, nullptr,
+                           codes_layout, stream);
     if (rc) return rc;
     rc = qm_requantize_transposed_mxfp4(s + sl.wc, s + sl.ws, O, I, 1.0f, w_val_dtype, hd_g, signs_g, g_mode, nullptr, seeds[1],
                                         k + wl.wtc, k + wl.wts, nullptr, codes_layout, codes_layout, stream);
     if (rc) return rc;
-    void* gws = wl.gemm_ws_bytes ? k + wl.gemm_ws : nullptr;
     rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, k + wl.gxq, mid_dtype, codes_layout,
                           codes_layout, gws, wl.gemm_ws_bytes, stream);
     if (rc) return rc;

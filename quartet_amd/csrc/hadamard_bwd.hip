@@ -39,61 +39,83 @@ __device__ __forceinline__ void cross_lane_stage(float (&v)[8], int lane_in_chun
     }
 }
 
+// The work of one launch with its block count; two independent jobs can share a grid (see job_pair_kernel).
 template <typename TIn, typename TOut, int HD>
-__global__ __launch_bounds__(256) void masked_hadamard_bwd_kernel(const TIn* __restrict__ g, int64_t n_octets,
-                                                                  float c, SignBits sb,
-                                                                  const uint8_t* __restrict__ maskbits,
-                                                                  TOut* __restrict__ out) {
-    const int64_t octet = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (octet >= n_octets) return;
-    const int lic = (int)(octet & (HD / 8 - 1));
-    float v[8];
-    if constexpr (sizeof(TIn) == 2) {
-        uint4 raw = *reinterpret_cast<const uint4*>(g + octet * 8);
-        uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+struct HadamardBwdJob {
+    const TIn* g;
+    int64_t n_octets;
+    float c;
+    SignBits sb;
+    const uint8_t* maskbits;
+    TOut* out;
+    unsigned blocks;
+
+    HadamardBwdJob(const void* g_, int64_t n, float c_, const SignBits& sb_, const uint8_t* maskbits_, void* out_)
+        : g(reinterpret_cast<const TIn*>(g_)), n_octets(n / 8), c(c_), sb(sb_), maskbits(maskbits_),
+          out(reinterpret_cast<TOut*>(out_)), blocks((unsigned)((n / 8 + 255) / 256)) {}
+
+    __device__ __forceinline__ void run(unsigned bid) const {
+        const int64_t octet = (int64_t)bid * 256 + threadIdx.x;
+        if (octet >= n_octets) return;
+        const int lic = (int)(octet & (HD / 8 - 1));
+        float v[8];
+        if constexpr (sizeof(TIn) == 2) {
+            uint4 raw = *reinterpret_cast<const uint4*>(g + octet * 8);
+            uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            v[2 * i] = u2f(w[i] << 16);
-            v[2 * i + 1] = u2f(w[i] & 0xffff0000u);
+            for (int i = 0; i < 4; ++i) {
+                v[2 * i] = u2f(w[i] << 16);
+                v[2 * i + 1] = u2f(w[i] & 0xffff0000u);
+            }
+        } else {
+            float4 a = *reinterpret_cast<const float4*>(g + octet * 8);
+            float4 b = *reinterpret_cast<const float4*>(g + octet * 8 + 4);
+            v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+            v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
         }
-    } else {
-        float4 a = *reinterpret_cast<const float4*>(g + octet * 8);
-        float4 b = *reinterpret_cast<const float4*>(g + octet * 8 + 4);
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-    }
-    const uint32_t keep = maskbits ? (uint32_t)maskbits[octet] : 0xffu;
-    const int j0 = lic * 8;
-    const uint32_t sign8 = (sb.w[j0 >> 5] >> (j0 & 31)) & 0xffu;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        float x = v[i] * (float)((keep >> i) & 1u);  // g * mask, as the reference multiplies
-        v[i] = ((sign8 >> i) & 1u) ? -x : x;
-    }
-#pragma unroll
-    for (int h = 1; h < 8; h <<= 1) {
+        const uint32_t keep = maskbits ? (uint32_t)maskbits[octet] : 0xffu;
+        const int j0 = lic * 8;
+        const uint32_t sign8 = (sb.w[j0 >> 5] >> (j0 & 31)) & 0xffu;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            if (i & h) continue;
-            float a = v[i], b = v[i + h];
-            v[i] = a + b;
-            v[i + h] = a - b;
+            float x = v[i] * (float)((keep >> i) & 1u);  // g * mask, as the reference multiplies
+            v[i] = ((sign8 >> i) & 1u) ? -x : x;
+        }
+#pragma unroll
+        for (int h = 1; h < 8; h <<= 1) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (i & h) continue;
+                float a = v[i], b = v[i + h];
+                v[i] = a + b;
+                v[i + h] = a - b;
+            }
+        }
+        cross_lane_stage<1>(v, lic);
+        cross_lane_stage<2>(v, lic);
+        if constexpr (HD >= 64) cross_lane_stage<4>(v, lic);
+        if constexpr (HD >= 128) cross_lane_stage<8>(v, lic);
+        if constexpr (sizeof(TOut) == 2) {
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                w[i] = (uint32_t)f32_to_bf16(v[2 * i] * c) | ((uint32_t)f32_to_bf16(v[2 * i + 1] * c) << 16);
+            *reinterpret_cast<uint4*>(out + octet * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+        } else {
+            *reinterpret_cast<float4*>(out + octet * 8) = make_float4(v[0] * c, v[1] * c, v[2] * c, v[3] * c);
+            *reinterpret_cast<float4*>(out + octet * 8 + 4) = make_float4(v[4] * c, v[5] * c, v[6] * c, v[7] * c);
         }
     }
-    cross_lane_stage<1>(v, lic);
-    cross_lane_stage<2>(v, lic);
-    if constexpr (HD >= 64) cross_lane_stage<4>(v, lic);
-    if constexpr (HD >= 128) cross_lane_stage<8>(v, lic);
-    if constexpr (sizeof(TOut) == 2) {
-        uint32_t w[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            w[i] = (uint32_t)f32_to_bf16(v[2 * i] * c) | ((uint32_t)f32_to_bf16(v[2 * i + 1] * c) << 16);
-        *reinterpret_cast<uint4*>(out + octet * 8) = make_uint4(w[0], w[1], w[2], w[3]);
-    } else {
-        *reinterpret_cast<float4*>(out + octet * 8) = make_float4(v[0] * c, v[1] * c, v[2] * c, v[3] * c);
-        *reinterpret_cast<float4*>(out + octet * 8 + 4) = make_float4(v[4] * c, v[5] * c, v[6] * c, v[7] * c);
-    }
+};
+
+template <class A>
+__global__ __launch_bounds__(256) void job_kernel(A a) {
+    a.run(blockIdx.x);
+}
+template <class A, class B>
+__global__ __launch_bounds__(256) void job_pair_kernel(A a, B b) {
+    if (blockIdx.x < a.blocks) a.run(blockIdx.x);
+    else b.run(blockIdx.x - a.blocks);
 }
 
 template <typename TOut>
@@ -125,13 +147,10 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t* __restr
 template <typename TIn, typename TOut>
 void launch_bwd(int hd, const void* g, int64_t n, float c, const SignBits& sb, const uint8_t* maskbits, void* out,
                 hipStream_t stream) {
-    const int64_t n_octets = n / 8;
-    dim3 grid((unsigned)((n_octets + 255) / 256)), block(256);
-    const TIn* gp = reinterpret_cast<const TIn*>(g);
-    TOut* op = reinterpret_cast<TOut*>(out);
-    if (hd == 32) masked_hadamard_bwd_kernel<TIn, TOut, 32><<<grid, block, 0, stream>>>(gp, n_octets, c, sb, maskbits, op);
-    else if (hd == 64) masked_hadamard_bwd_kernel<TIn, TOut, 64><<<grid, block, 0, stream>>>(gp, n_octets, c, sb, maskbits, op);
-    else masked_hadamard_bwd_kernel<TIn, TOut, 128><<<grid, block, 0, stream>>>(gp, n_octets, c, sb, maskbits, op);
+    const auto go = [&](auto job) { job_kernel<<<dim3(job.blocks), dim3(256), 0, stream>>>(job); };
+    if (hd == 32) go(HadamardBwdJob<TIn, TOut, 32>(g, n, c, sb, maskbits, out));
+    else if (hd == 64) go(HadamardBwdJob<TIn, TOut, 64>(g, n, c, sb, maskbits, out));
+    else go(HadamardBwdJob<TIn, TOut, 128>(g, n, c, sb, maskbits, out));
 }
 
 }  // namespace
@@ -146,6 +165,24 @@ hipError_t masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t
     else if (g_dtype == BF16) launch_bwd<uint16_t, float>(hd, g, n, c, sb, maskbits, out, stream);
     else if (out_dtype == BF16) launch_bwd<float, uint16_t>(hd, g, n, c, sb, maskbits, out, stream);
     else launch_bwd<float, float>(hd, g, n, c, sb, maskbits, out, stream);
+    return hipGetLastError();
+}
+
+// two independent masked inverse rotations (Hadamard block 32, same element type in and out) in one grid
+hipError_t masked_hadamard_bwd_hd32_pair(const void* ga, int64_t na, int scale_dtype_a, uint32_t sign_a, const uint8_t* mask_a, void* out_a,
+                                         const void* gb, int64_t nb, int scale_dtype_b, uint32_t sign_b, const uint8_t* mask_b, void* out_b,
+                                         int dtype, hipStream_t stream) {
+    const SignBits sa{{sign_a, 0, 0, 0}}, sb{{sign_b, 0, 0, 0}};
+    const float ca = hadamard_scale(32, scale_dtype_a), cb = hadamard_scale(32, scale_dtype_b);
+    if (dtype == BF16) {
+        using J = HadamardBwdJob<uint16_t, uint16_t, 32>;
+        const J a(ga, na, ca, sa, mask_a, out_a), b(gb, nb, cb, sb, mask_b, out_b);
+        job_pair_kernel<<<dim3(a.blocks + b.blocks), dim3(256), 0, stream>>>(a, b);
+    } else {
+        using J = HadamardBwdJob<float, float, 32>;
+        const J a(ga, na, ca, sa, mask_a, out_a), b(gb, nb, cb, sb, mask_b, out_b);
+        job_pair_kernel<<<dim3(a.blocks + b.blocks), dim3(256), 0, stream>>>(a, b);
+    }
     return hipGetLastError();
 }
 

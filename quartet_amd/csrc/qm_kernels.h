@@ -44,6 +44,36 @@ hipError_t requantize_transposed_hd32(const uint8_t* codes_in, const uint8_t* sc
                                       int val_dtype, uint32_t sign_word, int mode, uint64_t seed, uint8_t* codes,
                                       uint8_t* scales, void* dequant, bool tiled_in, bool tiled_out, hipStream_t stream);
 
+// Pairs of independent quantizer launches issued as one grid (Hadamard block 32, tiled codes in and out).
+struct RowmajorArgs {
+    const void* x;
+    int dtype;
+    int64_t rows, cols;
+    uint32_t sign_word;
+    uint8_t* codes;
+    uint8_t* scales;
+    uint8_t* maskbits;
+};
+struct RequantArgs {
+    const uint8_t* codes_in;
+    const uint8_t* scales_in;
+    int64_t R, C;
+    int val_dtype;
+    uint64_t seed;
+    uint8_t* codes;
+    uint8_t* scales;
+};
+hipError_t quantize_rowmajor_hd32_tiled_pair(const RowmajorArgs& a, const RowmajorArgs& b, hipStream_t stream);
+hipError_t quantize_both_orientations_hd32_tiled(const void* e, int dtype, int64_t T, int64_t O, uint32_t sign_word, int mode,
+                                                 uint64_t seed_rows, uint64_t seed_transposed, uint8_t* codes_rows,
+                                                 uint8_t* scales_rows, uint8_t* codes_transposed, uint8_t* scales_transposed,
+                                                 hipStream_t stream);
+hipError_t requantize_transposed_hd32_tiled_pair(const RequantArgs& a, const RequantArgs& b, uint32_t sign_word, int mode,
+                                                 hipStream_t stream);
+hipError_t masked_hadamard_bwd_hd32_pair(const void* ga, int64_t na, int scale_dtype_a, uint32_t sign_a, const uint8_t* mask_a, void* out_a,
+                                         const void* gb, int64_t nb, int scale_dtype_b, uint32_t sign_b, const uint8_t* mask_b, void* out_b,
+                                         int dtype, hipStream_t stream);
+
 hipError_t requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C,
                                        float post, int val_dtype, int hd, const SignBits& sb, int mode, const float* u,
                                        uint64_t seed, uint8_t* codes_out, uint8_t* scales_out, void* dequant,

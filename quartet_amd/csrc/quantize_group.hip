@@ -294,51 +294,77 @@ __global__ __launch_bounds__(256) void quantize_rowmajor_g32_kernel(const T* __r
     finish_group<T, MODE, WANT_MASK>(v, gi, gi, c, sign_word, seed, out);
 }
 
+// A job is the work of one kernel launch with its block count; job kernels run one job, or two independent jobs
+// one after the other in a single grid (the second job's blocks fill the machine while the first one drains, and
+// the pause between two dependent launches is paid once).
+template <class A>
+__global__ __launch_bounds__(256) void job_kernel(A a) {
+    a.run(blockIdx.x);
+}
+template <class A, class B>
+__global__ __launch_bounds__(256) void job_pair_kernel(A a, B b) {
+    if (blockIdx.x < a.blocks) a.run(blockIdx.x);
+    else b.run(blockIdx.x - a.blocks);
+}
+
 // Tiled code layout ([rows/16][cols/128][16 rows][64 bytes]).  Workgroup b owns block b / chunks of 16 rows and run
 // b % chunks of 512 columns (four code tiles); wave w owns rows 4w..4w+3 of the block, lane l its row l / 16 and
 // group l % 16 of the run: the wave reads four contiguous KiB (bf16) and writes, per tile, four rows' 64-byte pieces
 // = 256 contiguous bytes.  The four scale bytes of four adjacent groups are gathered into one dword store.
 template <typename T, int MODE, bool WANT_MASK>
-__global__ __launch_bounds__(256) void quantize_rowmajor_g32_tiled_kernel(const T* __restrict__ x, int64_t cols, int chunks,
-                                                                          float c, uint32_t sign_word, uint64_t seed,
-                                                                          GroupOut out) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int groups = (int)(cols / 32);  // per row
-    const unsigned rb = blockIdx.x / (unsigned)chunks;
-    const int g = (int)(blockIdx.x - rb * chunks) * 16 + (lane & 15);  // group within the row
-    if (g >= groups) return;  // cols % 128 == 0: quads of lanes leave together, the gather below sees full quads
-    const int rin = wave * 4 + (lane >> 4);  // row within the block
-    // uniform 64-bit block bases + small per-lane offsets
-    const int64_t gi = (int64_t)rb * 16 * groups + (rin * groups + g);
-    const int64_t ci = (int64_t)rb * 16 * groups + ((g >> 2) * 64 + rin * 4 + (g & 3));
-    float v[32];
-    load_group<T>(x + gi * 32, v);
-    rotate_group(v, c, sign_word);
-    GroupCodes o;
-    quantize_group_regs<MODE, WANT_MASK>(v, seed, gi, o);
-    out.codes[ci] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
-    // quad_perm broadcasts of lanes 1, 2, 3 of each quad
-    const uint32_t s1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0x55, 0xf, 0xf, false);
-    const uint32_t s2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0xAA, 0xf, 0xf, false);
-    const uint32_t s3 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0xFF, 0xf, 0xf, false);
-    if ((lane & 3) == 0)
-        *reinterpret_cast<uint32_t*>(out.scales + gi) = o.scale_byte | (s1 << 8) | (s2 << 16) | (s3 << 24);
-    if constexpr (WANT_MASK) out.maskbits[gi] = o.keep;
-    if (out.dequant) store_dequant<T>(reinterpret_cast<T*>(out.dequant) + gi * 32, o);
-}
+struct RowmajorTiledJob {
+    const T* x;
+    int64_t cols;
+    int chunks;
+    float c;
+    uint32_t sign_word;
+    uint64_t seed;
+    GroupOut out;
+    unsigned blocks;
+
+    RowmajorTiledJob(const void* x_, int64_t rows, int64_t cols_, float c_, uint32_t sign_word_, uint64_t seed_,
+                     const GroupOut& out_)
+        : x(reinterpret_cast<const T*>(x_)), cols(cols_), chunks((int)((cols_ / 128 + 3) / 4)), c(c_),
+          sign_word(sign_word_), seed(seed_), out(out_), blocks((unsigned)((rows / 16) * ((cols_ / 128 + 3) / 4))) {}
+
+    __device__ __forceinline__ void run(unsigned bid) const {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const int groups = (int)(cols / 32);  // per row
+        const unsigned rb = bid / (unsigned)chunks;
+        const int g = (int)(bid - rb * chunks) * 16 + (lane & 15);  // group within the row
+        if (g >= groups) return;  // cols % 128 == 0: quads of lanes leave together, the gather below sees full quads
+        const int rin = wave * 4 + (lane >> 4);  // row within the block
+        // uniform 64-bit block bases + small per-lane offsets
+        const int64_t gi = (int64_t)rb * 16 * groups + (rin * groups + g);
+        const int64_t ci = (int64_t)rb * 16 * groups + ((g >> 2) * 64 + rin * 4 + (g & 3));
+        float v[32];
+        load_group<T>(x + gi * 32, v);
+        rotate_group(v, c, sign_word);
+        GroupCodes o;
+        quantize_group_regs<MODE, WANT_MASK>(v, seed, gi, o);
+        out.codes[ci] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
+        // quad_perm broadcasts of lanes 1, 2, 3 of each quad
+        const uint32_t s1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0x55, 0xf, 0xf, false);
+        const uint32_t s2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0xAA, 0xf, 0xf, false);
+        const uint32_t s3 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0xFF, 0xf, 0xf, false);
+        if ((lane & 3) == 0)
+            *reinterpret_cast<uint32_t*>(out.scales + gi) = o.scale_byte | (s1 << 8) | (s2 << 16) | (s3 << 24);
+        if constexpr (WANT_MASK) out.maskbits[gi] = o.keep;
+        if (out.dequant) store_dequant<T>(reinterpret_cast<T*>(out.dequant) + gi * 32, o);
+    }
+};
 
 template <typename T, bool WANT_MASK>
 void launch_rowmajor_g32(int mode, const void* x, int64_t rows, int64_t cols, bool tiled, float c, uint32_t sign_word,
                          uint64_t seed, const GroupOut& out, hipStream_t stream) {
     const T* xp = reinterpret_cast<const T*>(x);
     if (tiled) {
-        const int chunks = (int)((cols / 128 + 3) / 4);
-        dim3 grid((unsigned)((rows / 16) * chunks)), block(256);
+        const auto go = [&](auto job) { job_kernel<<<dim3(job.blocks), dim3(256), 0, stream>>>(job); };
         switch (mode) {
-            case QUEST_RTN: quantize_rowmajor_g32_tiled_kernel<T, QUEST_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, chunks, c, sign_word, seed, out); break;
-            case ABSMAX_RTN: quantize_rowmajor_g32_tiled_kernel<T, ABSMAX_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, chunks, c, sign_word, seed, out); break;
-            case ABSMAX_SR: quantize_rowmajor_g32_tiled_kernel<T, ABSMAX_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, chunks, c, sign_word, seed, out); break;
-            default: quantize_rowmajor_g32_tiled_kernel<T, QUEST_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, cols, chunks, c, sign_word, seed, out); break;
+            case QUEST_RTN: go(RowmajorTiledJob<T, QUEST_RTN, WANT_MASK>(x, rows, cols, c, sign_word, seed, out)); break;
+            case ABSMAX_RTN: go(RowmajorTiledJob<T, ABSMAX_RTN, WANT_MASK>(x, rows, cols, c, sign_word, seed, out)); break;
+            case ABSMAX_SR: go(RowmajorTiledJob<T, ABSMAX_SR, WANT_MASK>(x, rows, cols, c, sign_word, seed, out)); break;
+            default: go(RowmajorTiledJob<T, QUEST_SR, WANT_MASK>(x, rows, cols, c, sign_word, seed, out)); break;
         }
         return;
     }
@@ -423,67 +449,83 @@ struct TrTile {
 constexpr int kTrP = 128;
 
 template <typename T, int MODE>
-__global__ __launch_bounds__(256) void quantize_transposed_g32_kernel(const T* __restrict__ x, int64_t P, int64_t Q,
-                                                                      float c, uint32_t sign_word, uint64_t seed,
-                                                                      uint8_t* __restrict__ codes,
-                                                                      uint8_t* __restrict__ scales,
-                                                                      void* __restrict__ dequant, bool tiled_out) {
-    constexpr int TQ = TrTile<T>::kQ;
-    constexpr int GPL = TrTile<T>::kGroupsPerLane;
-    __shared__ uint4 ocodes[TQ * 4];      // [q][4 groups x 16 B]
-    __shared__ uint32_t oscales[TQ];      // [q][4 B]
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t p0 = (int64_t)blockIdx.x * kTrP, q0 = (int64_t)blockIdx.y * TQ;
-    const int64_t pbase = p0 + wave * 32;       // this wave's group along p
-    const int64_t qa = q0 + lane * GPL;         // this lane's first column
-    const bool active = pbase < P && qa < Q;    // P % 32 == 0 and Q % 8 == 0: all of a lane's groups or none
-    if (active) {
-        float v[GPL][32];
-        const uint32_t* src = reinterpret_cast<const uint32_t*>(x + pbase * Q + qa);
-        const int64_t row_dw = Q * (int64_t)sizeof(T) / 4;
+struct TransposedJob {
+    const T* x;
+    int64_t P, Q;
+    float c;
+    uint32_t sign_word;
+    uint64_t seed;
+    uint8_t* codes;
+    uint8_t* scales;
+    void* dequant;
+    bool tiled_out;
+    unsigned grid_p, blocks;
+
+    TransposedJob(const void* x_, int64_t P_, int64_t Q_, float c_, uint32_t sign_word_, uint64_t seed_, uint8_t* codes_,
+                  uint8_t* scales_, void* dequant_, bool tiled_out_)
+        : x(reinterpret_cast<const T*>(x_)), P(P_), Q(Q_), c(c_), sign_word(sign_word_), seed(seed_), codes(codes_),
+          scales(scales_), dequant(dequant_), tiled_out(tiled_out_), grid_p((unsigned)((P_ + kTrP - 1) / kTrP)),
+          blocks((unsigned)(((P_ + kTrP - 1) / kTrP) * ((Q_ + TrTile<T>::kQ - 1) / TrTile<T>::kQ))) {}
+
+    __device__ __forceinline__ void run(unsigned bid) const {
+        constexpr int TQ = TrTile<T>::kQ;
+        constexpr int GPL = TrTile<T>::kGroupsPerLane;
+        __shared__ uint4 ocodes[TQ * 4];      // [q][4 groups x 16 B]
+        __shared__ uint32_t oscales[TQ];      // [q][4 B]
+        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const unsigned bq = bid / grid_p;
+        const int64_t p0 = (int64_t)(bid - bq * grid_p) * kTrP, q0 = (int64_t)bq * TQ;
+        const int64_t pbase = p0 + wave * 32;       // this wave's group along p
+        const int64_t qa = q0 + lane * GPL;         // this lane's first column
+        const bool active = pbase < P && qa < Q;    // P % 32 == 0 and Q % 8 == 0: all of a lane's groups or none
+        if (active) {
+            float v[GPL][32];
+            const uint32_t* src = reinterpret_cast<const uint32_t*>(x + pbase * Q + qa);
+            const int64_t row_dw = Q * (int64_t)sizeof(T) / 4;
 #pragma unroll
-        for (int i = 0; i < 32; ++i) {
-            const uint32_t w = src[i * row_dw];
-            if constexpr (sizeof(T) == 2) {
-                v[0][i] = u2f(w << 16);
-                v[1][i] = u2f(w & 0xffff0000u);
-            } else {
-                v[0][i] = u2f(w);
+            for (int i = 0; i < 32; ++i) {
+                const uint32_t w = src[i * row_dw];
+                if constexpr (sizeof(T) == 2) {
+                    v[0][i] = u2f(w << 16);
+                    v[1][i] = u2f(w & 0xffff0000u);
+                } else {
+                    v[0][i] = u2f(w);
+                }
+            }
+#pragma unroll
+            for (int gq = 0; gq < GPL; ++gq) {
+                const int64_t gi = (qa + gq) * (P / 32) + pbase / 32;
+                GroupCodes res;
+                rotate_group(v[gq], c, sign_word);
+                quantize_group_regs<MODE, false>(v[gq], seed, gi, res);
+                if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res);
+                ocodes[(lane * GPL + gq) * 4 + wave] = make_uint4(res.w[0], res.w[1], res.w[2], res.w[3]);
+                reinterpret_cast<uint8_t*>(oscales)[(lane * GPL + gq) * 4 + wave] = (uint8_t)res.scale_byte;
             }
         }
-#pragma unroll
-        for (int gq = 0; gq < GPL; ++gq) {
-            const int64_t gi = (qa + gq) * (P / 32) + pbase / 32;
-            GroupCodes res;
-            rotate_group(v[gq], c, sign_word);
-            quantize_group_regs<MODE, false>(v[gq], seed, gi, res);
-            if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res);
-            ocodes[(lane * GPL + gq) * 4 + wave] = make_uint4(res.w[0], res.w[1], res.w[2], res.w[3]);
-            reinterpret_cast<uint8_t*>(oscales)[(lane * GPL + gq) * 4 + wave] = (uint8_t)res.scale_byte;
+        __syncthreads();
+        const int64_t code_pitch = P / 2, scale_pitch = P / 32;
+        for (int idx = tid; idx < TQ * 4; idx += 256) {
+            const int ql = idx >> 2, part = idx & 3;
+            if (q0 + ql < Q && p0 + part * 32 < P) {
+                // tiled: this workgroup's 128 p are one 64-byte column block, so 16 consecutive q rows form one 1 KiB tile
+                const int64_t off = tiled_out ? tiled_code_offset(q0 + ql, p0 / 128, P / 128) + part * 16
+                                              : (q0 + ql) * code_pitch + p0 / 2 + part * 16;
+                *reinterpret_cast<uint4*>(codes + off) = ocodes[idx];
+            }
+        }
+        if (tid < TQ && q0 + tid < Q) {
+            const uint32_t sw = oscales[tid];
+            uint8_t* dst = scales + (q0 + tid) * scale_pitch + p0 / 32;
+            if (p0 + kTrP <= P) {
+                *reinterpret_cast<uint32_t*>(dst) = sw;
+            } else {
+                for (int b = 0; b < 4; ++b)
+                    if (p0 + b * 32 < P) dst[b] = (uint8_t)(sw >> (8 * b));
+            }
         }
     }
-    __syncthreads();
-    const int64_t code_pitch = P / 2, scale_pitch = P / 32;
-    for (int idx = tid; idx < TQ * 4; idx += 256) {
-        const int ql = idx >> 2, part = idx & 3;
-        if (q0 + ql < Q && p0 + part * 32 < P) {
-            // tiled: this workgroup's 128 p are one 64-byte column block, so 16 consecutive q rows form one 1 KiB tile
-            const int64_t off = tiled_out ? tiled_code_offset(q0 + ql, p0 / 128, P / 128) + part * 16
-                                          : (q0 + ql) * code_pitch + p0 / 2 + part * 16;
-            *reinterpret_cast<uint4*>(codes + off) = ocodes[idx];
-        }
-    }
-    if (tid < TQ && q0 + tid < Q) {
-        const uint32_t sw = oscales[tid];
-        uint8_t* dst = scales + (q0 + tid) * scale_pitch + p0 / 32;
-        if (p0 + kTrP <= P) {
-            *reinterpret_cast<uint32_t*>(dst) = sw;
-        } else {
-            for (int b = 0; b < 4; ++b)
-                if (p0 + b * 32 < P) dst[b] = (uint8_t)(sw >> (8 * b));
-        }
-    }
-}
+};
 
 // ---- packed MXFP4 in, transposed + rotated + re-quantized out --------------------------------------------
 // in: codes [R, C/2], scales [R, C/32]; out: the [C, R] tensor quantized along R.  A workgroup owns 128
@@ -494,95 +536,118 @@ __global__ __launch_bounds__(256) void quantize_transposed_g32_kernel(const T* _
 constexpr int kRqR = 128, kRqC = 128;
 
 template <int VAL_DTYPE, int MODE>
-__global__ __launch_bounds__(256) void requantize_transposed_g32_kernel(const uint8_t* __restrict__ codes_in,
-                                                                        const uint8_t* __restrict__ scales_in,
-                                                                        int64_t R, int64_t C, float post, float c,
-                                                                        uint32_t sign_word, uint64_t seed,
-                                                                        uint8_t* __restrict__ codes,
-                                                                        uint8_t* __restrict__ scales,
-                                                                        void* __restrict__ dequant, bool tiled_in,
-                                                                        bool tiled_out) {
-    using T = typename std::conditional<VAL_DTYPE == BF16, uint16_t, float>::type;
-    __shared__ uint4 ocodes[kRqC * 4];
-    __shared__ uint32_t oscales[kRqC];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t r0 = (int64_t)blockIdx.x * kRqR, c0 = (int64_t)blockIdx.y * kRqC;
-    const int64_t in_code_pitch = C / 2, in_scale_pitch = C / 32;
-    const int64_t rbase = r0 + wave * 32;
-    const int64_t ca = c0 + 2 * lane;            // this lane's column pair
-    const bool active = rbase < R && ca < C;     // C % 32 == 0: both columns of the pair or none
-    if (active) {
-        float v[2][32];
-        // tiled input: the lane's byte column sits at offset `lane` of the 64-byte rows of column block c0/128
-        const uint8_t* cp = tiled_in ? codes_in + tiled_code_offset(rbase, c0 / 128, C / 128) + lane
-                                     : codes_in + rbase * in_code_pitch + ca / 2;
-        const int64_t row_step = tiled_in ? 64 : in_code_pitch;                            // next row of a 16-row block
-        const int64_t block_step = tiled_in ? (C / 128) * 1024 - 16 * 64 : 0;              // extra hop into the next block
-        const uint8_t* sp = scales_in + rbase * in_scale_pitch + ca / 32;
-        uint32_t byte[32], sbyte[32];
+struct RequantJob {
+    const uint8_t* codes_in;
+    const uint8_t* scales_in;
+    int64_t R, C;
+    float post, c;
+    uint32_t sign_word;
+    uint64_t seed;
+    uint8_t* codes;
+    uint8_t* scales;
+    void* dequant;
+    bool tiled_in, tiled_out;
+    unsigned grid_r, blocks;
+
+    RequantJob(const uint8_t* codes_in_, const uint8_t* scales_in_, int64_t R_, int64_t C_, float post_, float c_,
+               uint32_t sign_word_, uint64_t seed_, uint8_t* codes_, uint8_t* scales_, void* dequant_, bool tiled_in_,
+               bool tiled_out_)
+        : codes_in(codes_in_), scales_in(scales_in_), R(R_), C(C_), post(post_), c(c_), sign_word(sign_word_), seed(seed_),
+          codes(codes_), scales(scales_), dequant(dequant_), tiled_in(tiled_in_), tiled_out(tiled_out_),
+          grid_r((unsigned)((R_ + kRqR - 1) / kRqR)),
+          blocks((unsigned)(((R_ + kRqR - 1) / kRqR) * ((C_ + kRqC - 1) / kRqC))) {}
+
+    __device__ __forceinline__ void run(unsigned bid) const {
+        using T = typename std::conditional<VAL_DTYPE == BF16, uint16_t, float>::type;
+        __shared__ uint4 ocodes[kRqC * 4];
+        __shared__ uint32_t oscales[kRqC];
+        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const unsigned bc = bid / grid_r;
+        const int64_t r0 = (int64_t)(bid - bc * grid_r) * kRqR, c0 = (int64_t)bc * kRqC;
+        const int64_t in_code_pitch = C / 2, in_scale_pitch = C / 32;
+        const int64_t rbase = r0 + wave * 32;
+        const int64_t ca = c0 + 2 * lane;            // this lane's column pair
+        const bool active = rbase < R && ca < C;     // C % 32 == 0: both columns of the pair or none
+        if (active) {
+            float v[2][32];
+            // tiled input: the lane's byte column sits at offset `lane` of the 64-byte rows of column block c0/128
+            const uint8_t* cp = tiled_in ? codes_in + tiled_code_offset(rbase, c0 / 128, C / 128) + lane
+                                         : codes_in + rbase * in_code_pitch + ca / 2;
+            const int64_t row_step = tiled_in ? 64 : in_code_pitch;                            // next row of a 16-row block
+            const int64_t block_step = tiled_in ? (C / 128) * 1024 - 16 * 64 : 0;              // extra hop into the next block
+            const uint8_t* sp = scales_in + rbase * in_scale_pitch + ca / 32;
+            uint32_t byte[32], sbyte[32];
 #pragma unroll
-        for (int i = 0; i < 32; ++i) {
-            byte[i] = cp[i * row_step + (i >> 4) * block_step];
-            sbyte[i] = sp[i * in_scale_pitch];
-        }
-#pragma unroll
-        for (int i = 0; i < 32; ++i) {
-            const v2f pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(byte[i], u2f(sbyte[i] << 23), 0);
-            float a = pr.x, b = pr.y;
-            if (post != 1.0f) {  // absmax-coded input: value = code * 2^k * post, held in val_dtype
-                a *= post;
-                b *= post;
-                if constexpr (VAL_DTYPE == BF16) {
-                    a = bf16_to_f32(f32_to_bf16(a));
-                    b = bf16_to_f32(f32_to_bf16(b));
-                }
+            for (int i = 0; i < 32; ++i) {
+                byte[i] = cp[i * row_step + (i >> 4) * block_step];
+                sbyte[i] = sp[i * in_scale_pitch];
             }
-            v[0][i] = a;
-            v[1][i] = b;
-        }
 #pragma unroll
-        for (int gq = 0; gq < 2; ++gq) {
-            const int64_t gi = (ca + gq) * (R / 32) + rbase / 32;
-            GroupCodes res;
-            rotate_group(v[gq], c, sign_word);
-            quantize_group_regs<MODE, false>(v[gq], seed, gi, res);
-            if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res);
-            ocodes[(lane * 2 + gq) * 4 + wave] = make_uint4(res.w[0], res.w[1], res.w[2], res.w[3]);
-            reinterpret_cast<uint8_t*>(oscales)[(lane * 2 + gq) * 4 + wave] = (uint8_t)res.scale_byte;
+            for (int i = 0; i < 32; ++i) {
+                const v2f pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(byte[i], u2f(sbyte[i] << 23), 0);
+                float a = pr.x, b = pr.y;
+                if (post != 1.0f) {  // absmax-coded input: value = code * 2^k * post, held in val_dtype
+                    a *= post;
+                    b *= post;
+                    if constexpr (VAL_DTYPE == BF16) {
+                        a = bf16_to_f32(f32_to_bf16(a));
+                        b = bf16_to_f32(f32_to_bf16(b));
+                    }
+                }
+                v[0][i] = a;
+                v[1][i] = b;
+            }
+#pragma unroll
+            for (int gq = 0; gq < 2; ++gq) {
+                const int64_t gi = (ca + gq) * (R / 32) + rbase / 32;
+                GroupCodes res;
+                rotate_group(v[gq], c, sign_word);
+                quantize_group_regs<MODE, false>(v[gq], seed, gi, res);
+                if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res);
+                ocodes[(lane * 2 + gq) * 4 + wave] = make_uint4(res.w[0], res.w[1], res.w[2], res.w[3]);
+                reinterpret_cast<uint8_t*>(oscales)[(lane * 2 + gq) * 4 + wave] = (uint8_t)res.scale_byte;
+            }
+        }
+        __syncthreads();
+        const int64_t code_pitch = R / 2, scale_pitch = R / 32;
+        for (int idx = tid; idx < kRqC * 4; idx += 256) {
+            const int cl = idx >> 2, part = idx & 3;
+            if (c0 + cl < C && r0 + part * 32 < R) {
+                const int64_t off = tiled_out ? tiled_code_offset(c0 + cl, r0 / 128, R / 128) + part * 16
+                                              : (c0 + cl) * code_pitch + r0 / 2 + part * 16;
+                *reinterpret_cast<uint4*>(codes + off) = ocodes[idx];
+            }
+        }
+        if (tid < kRqC && c0 + tid < C) {
+            const uint32_t sw = oscales[tid];
+            uint8_t* dst = scales + (c0 + tid) * scale_pitch + r0 / 32;
+            if (r0 + kRqR <= R) {
+                *reinterpret_cast<uint32_t*>(dst) = sw;
+            } else {
+                for (int b = 0; b < 4; ++b)
+                    if (r0 + b * 32 < R) dst[b] = (uint8_t)(sw >> (8 * b));
+            }
         }
     }
-    __syncthreads();
-    const int64_t code_pitch = R / 2, scale_pitch = R / 32;
-    for (int idx = tid; idx < kRqC * 4; idx += 256) {
-        const int cl = idx >> 2, part = idx & 3;
-        if (c0 + cl < C && r0 + part * 32 < R) {
-            const int64_t off = tiled_out ? tiled_code_offset(c0 + cl, r0 / 128, R / 128) + part * 16
-                                          : (c0 + cl) * code_pitch + r0 / 2 + part * 16;
-            *reinterpret_cast<uint4*>(codes + off) = ocodes[idx];
-        }
-    }
-    if (tid < kRqC && c0 + tid < C) {
-        const uint32_t sw = oscales[tid];
-        uint8_t* dst = scales + (c0 + tid) * scale_pitch + r0 / 32;
-        if (r0 + kRqR <= R) {
-            *reinterpret_cast<uint32_t*>(dst) = sw;
-        } else {
-            for (int b = 0; b < 4; ++b)
-                if (r0 + b * 32 < R) dst[b] = (uint8_t)(sw >> (8 * b));
-        }
-    }
+};
+
+template <class Job>
+void launch_job(const Job& job, hipStream_t stream) {
+    job_kernel<<<dim3(job.blocks), dim3(256), 0, stream>>>(job);
+}
+template <class A, class B>
+void launch_job_pair(const A& a, const B& b, hipStream_t stream) {
+    job_pair_kernel<<<dim3(a.blocks + b.blocks), dim3(256), 0, stream>>>(a, b);
 }
 
 template <typename T>
 void launch_transposed_g32(int mode, const void* x, int64_t P, int64_t Q, float c, uint32_t sign_word, uint64_t seed,
                            uint8_t* codes, uint8_t* scales, void* dequant, bool tiled, hipStream_t stream) {
-    dim3 grid((unsigned)((P + kTrP - 1) / kTrP), (unsigned)((Q + TrTile<T>::kQ - 1) / TrTile<T>::kQ)), block(256);
-    const T* xp = reinterpret_cast<const T*>(x);
     switch (mode) {
-        case QUEST_RTN: quantize_transposed_g32_kernel<T, QUEST_RTN><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant, tiled); break;
-        case ABSMAX_RTN: quantize_transposed_g32_kernel<T, ABSMAX_RTN><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant, tiled); break;
-        case ABSMAX_SR: quantize_transposed_g32_kernel<T, ABSMAX_SR><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant, tiled); break;
-        default: quantize_transposed_g32_kernel<T, QUEST_SR><<<grid, block, 0, stream>>>(xp, P, Q, c, sign_word, seed, codes, scales, dequant, tiled); break;
+        case QUEST_RTN: launch_job(TransposedJob<T, QUEST_RTN>(x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled), stream); break;
+        case ABSMAX_RTN: launch_job(TransposedJob<T, ABSMAX_RTN>(x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled), stream); break;
+        case ABSMAX_SR: launch_job(TransposedJob<T, ABSMAX_SR>(x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled), stream); break;
+        default: launch_job(TransposedJob<T, QUEST_SR>(x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled), stream); break;
     }
 }
 
@@ -590,12 +655,11 @@ template <int VAL_DTYPE>
 void launch_requant_g32(int mode, const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C, float post,
                         float c, uint32_t sign_word, uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant,
                         bool tiled_in, bool tiled_out, hipStream_t stream) {
-    dim3 grid((unsigned)((R + kRqR - 1) / kRqR), (unsigned)((C + kRqC - 1) / kRqC)), block(256);
     switch (mode) {
-        case QUEST_RTN: requantize_transposed_g32_kernel<VAL_DTYPE, QUEST_RTN><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out); break;
-        case ABSMAX_RTN: requantize_transposed_g32_kernel<VAL_DTYPE, ABSMAX_RTN><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out); break;
-        case ABSMAX_SR: requantize_transposed_g32_kernel<VAL_DTYPE, ABSMAX_SR><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out); break;
-        default: requantize_transposed_g32_kernel<VAL_DTYPE, QUEST_SR><<<grid, block, 0, stream>>>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out); break;
+        case QUEST_RTN: launch_job(RequantJob<VAL_DTYPE, QUEST_RTN>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out), stream); break;
+        case ABSMAX_RTN: launch_job(RequantJob<VAL_DTYPE, ABSMAX_RTN>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out), stream); break;
+        case ABSMAX_SR: launch_job(RequantJob<VAL_DTYPE, ABSMAX_SR>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out), stream); break;
+        default: launch_job(RequantJob<VAL_DTYPE, QUEST_SR>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out), stream); break;
     }
 }
 
@@ -656,6 +720,73 @@ hipError_t requantize_transposed_hd32(const uint8_t* codes_in, const uint8_t* sc
     const float c = hadamard_scale(32, val_dtype);
     if (val_dtype == BF16) launch_requant_g32<BF16>(mode, codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out, stream);
     else launch_requant_g32<F32>(mode, codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out, stream);
+    return hipGetLastError();
+}
+
+// ---- two independent jobs per launch (the whole-layer entry points) ---------------------------------------------
+
+namespace {
+template <typename F>
+void with_elem_type(int dtype, F&& f) {
+    if (dtype == BF16) f(uint16_t{});
+    else f(float{});
+}
+template <typename F>
+void with_absmax_mode(int mode, F&& f) {
+    if (mode == ABSMAX_SR) f(std::integral_constant<int, ABSMAX_SR>{});
+    else f(std::integral_constant<int, ABSMAX_RTN>{});
+}
+}  // namespace
+
+// forward quantizer (quest RTN + clip mask, tiled codes) of two tensors, e.g. the activations and the weight of a layer
+hipError_t quantize_rowmajor_hd32_tiled_pair(const RowmajorArgs& a, const RowmajorArgs& b, hipStream_t stream) {
+    const GroupOut oa{reinterpret_cast<uint4*>(a.codes), a.scales, reinterpret_cast<uint32_t*>(a.maskbits), nullptr};
+    const GroupOut ob{reinterpret_cast<uint4*>(b.codes), b.scales, reinterpret_cast<uint32_t*>(b.maskbits), nullptr};
+    const float ca = hadamard_scale(32, a.dtype), cb = hadamard_scale(32, b.dtype);
+    with_elem_type(a.dtype, [&](auto ta) {
+        with_elem_type(b.dtype, [&](auto tb) {
+            launch_job_pair(RowmajorTiledJob<decltype(ta), QUEST_RTN, true>(a.x, a.rows, a.cols, ca, a.sign_word, 0, oa),
+                            RowmajorTiledJob<decltype(tb), QUEST_RTN, true>(b.x, b.rows, b.cols, cb, b.sign_word, 0, ob), stream);
+        });
+    });
+    return hipGetLastError();
+}
+
+// absmax quantizer of e [T, O] along its rows and of its transpose along T, tiled codes, one pass of launches
+hipError_t quantize_both_orientations_hd32_tiled(const void* e, int dtype, int64_t T, int64_t O, uint32_t sign_word, int mode,
+                                                 uint64_t seed_rows, uint64_t seed_transposed, uint8_t* codes_rows,
+                                                 uint8_t* scales_rows, uint8_t* codes_transposed, uint8_t* scales_transposed,
+                                                 hipStream_t stream) {
+    const GroupOut orow{reinterpret_cast<uint4*>(codes_rows), scales_rows, nullptr, nullptr};
+    const float c = hadamard_scale(32, dtype);
+    with_elem_type(dtype, [&](auto t) {
+        with_absmax_mode(mode, [&](auto m) {
+            using T_ = decltype(t);
+            constexpr int M = decltype(m)::value;
+            launch_job_pair(TransposedJob<T_, M>(e, T, O, c, sign_word, seed_transposed, codes_transposed, scales_transposed, nullptr, true),
+                            RowmajorTiledJob<T_, M, false>(e, T, O, c, sign_word, seed_rows, orow), stream);
+        });
+    });
+    return hipGetLastError();
+}
+
+// transpose + rotate + re-quantize two packed tensors (tiled codes in and out), e.g. Q(W) and Q(x) of a layer
+hipError_t requantize_transposed_hd32_tiled_pair(const RequantArgs& a, const RequantArgs& b, uint32_t sign_word, int mode,
+                                                 hipStream_t stream) {
+    const float ca = hadamard_scale(32, a.val_dtype), cb = hadamard_scale(32, b.val_dtype);
+    const auto with_val = [](int dt, auto&& f) {
+        if (dt == BF16) f(std::integral_constant<int, BF16>{});
+        else f(std::integral_constant<int, F32>{});
+    };
+    with_val(a.val_dtype, [&](auto va) {
+        with_val(b.val_dtype, [&](auto vb) {
+            with_absmax_mode(mode, [&](auto m) {
+                constexpr int M = decltype(m)::value;
+                launch_job_pair(RequantJob<decltype(va)::value, M>(a.codes_in, a.scales_in, a.R, a.C, 1.0f, ca, sign_word, a.seed, a.codes, a.scales, nullptr, true, true),
+                                RequantJob<decltype(vb)::value, M>(b.codes_in, b.scales_in, b.R, b.C, 1.0f, cb, sign_word, b.seed, b.codes, b.scales, nullptr, true, true), stream);
+            });
+        });
+    });
     return hipGetLastError();
 }
 
