@@ -135,6 +135,11 @@ int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, 
  * least 256, and all Hadamard blocks 32.  T, I, O must be multiples of 32 for the backward pass.
  */
 size_t qm_linear_saved_bytes(int64_t T, int64_t I, int64_t O);
+/* Byte offsets inside `saved` of, in this order: x codes [T, I/2], x scales [T, I/32], x mask bits [T, I/8], w codes
+ * [O, I/2], w scales [O, I/32], w mask bits [O, I/8] -- the tensors notebooks/benchmark_mxfp4.ipynb's CudaGemm keeps
+ * for backward (ctx.save_for_backward in its forward).  `offsets` is a HOST array of six; returns 0, or
+ * QM_ERR_INVALID for extents qm_linear_saved_bytes rejects. */
+int qm_linear_saved_offsets(int64_t T, int64_t I, int64_t O, size_t* offsets);
 size_t qm_linear_backward_workspace_bytes(int64_t T, int64_t I, int64_t O, int mid_dtype);
 int qm_linear_forward(const void* x, int x_dtype, const void* w, int w_dtype, int64_t T, int64_t I, int64_t O,
                       int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, void* saved,

@@ -22,6 +22,7 @@ EXPORTS = (
     "qm_dequantize_mxfp4",
     "qm_gemm_workspace_bytes",
     "qm_linear_saved_bytes",
+    "qm_linear_saved_offsets",
     "qm_linear_backward_workspace_bytes",
     "qm_linear_forward",
     "qm_linear_backward",
@@ -63,6 +64,8 @@ def lib():
     sz = ctypes.c_size_t
     L.qm_linear_saved_bytes.restype = sz
     L.qm_linear_saved_bytes.argtypes = [i64, i64, i64]
+    L.qm_linear_saved_offsets.restype = i32
+    L.qm_linear_saved_offsets.argtypes = [i64, i64, i64, ctypes.POINTER(sz)]
     L.qm_linear_backward_workspace_bytes.restype = sz
     L.qm_linear_backward_workspace_bytes.argtypes = [i64, i64, i64, i32]
     L.qm_linear_forward.restype = i32

@@ -206,6 +206,14 @@ size_t qm_linear_saved_bytes(int64_t T, int64_t I, int64_t O) {
     return saved_layout(T, I, O).total;
 }
 
+int qm_linear_saved_offsets(int64_t T, int64_t I, int64_t O, size_t* offsets) {
+    if (T < 0 || I < 0 || O < 0 || I % 32 || !offsets) return fail(QM_ERR_INVALID, "qm_linear_saved_offsets: bad extents or null array");
+    const SavedLayout l = saved_layout(T, I, O);
+    offsets[0] = l.xc; offsets[1] = l.xs; offsets[2] = l.xm;
+    offsets[3] = l.wc; offsets[4] = l.ws; offsets[5] = l.wm;
+    return 0;
+}
+
 size_t qm_linear_backward_workspace_bytes(int64_t T, int64_t I, int64_t O, int mid_dtype) {
     if (T < 0 || I < 0 || O < 0 || I % 32 || O % 32 || T % 32 || !valid_dtype(mid_dtype)) return 0;
     return work_layout(T, I, O, mid_dtype).total;
