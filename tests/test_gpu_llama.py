@@ -83,3 +83,31 @@ def test_llama_ragged_batch_shapes(models):
     torch.cuda.synchronize()
     assert math.isfinite(lq)
     assert all(torch.isfinite(p.grad).all() for p in quartet.parameters())
+
+
+def test_quartet_model_learns_with_the_training_loop():
+    """A small all-Quartet Llama (every block linear on the packed FP4 path, tiled codes) trained with the
+    reference-style loop -- bf16 autocast around forward and backward, two micro-steps per update, AdamW with
+    decayed linear weights, one-cycle cosine schedule -- must bring the loss well below ln(vocab), and stay close
+    to the bf16 baseline trained on the same batches."""
+    print("case train loop on a small Quartet Llama", flush=True)
+    import math
+    import random
+
+    from quartet_amd.llama import Llama, LlamaConfig, unquantized
+    from quartet_amd.train import TrainConfig, synthetic_batches, train
+    dev = torch.device("cuda:0")
+    shape = dict(vocab_size=256, sequence_length=64, n_layer=2, n_head=2, n_embd=256, multiple_of=128)
+    finals = {}
+    for name, overrides in (("quartet", shape), ("bf16", unquantized(**shape))):
+        torch.manual_seed(0)
+        random.seed(0)
+        model = Llama(LlamaConfig(**overrides)).to(dev)
+        cfg = TrainConfig(iterations=40, warmup_steps=4, lr=3e-3, acc_steps=2)
+        stats = train(model, synthetic_batches(256, 8, 64, dev, seed=1), cfg)   # 512 tokens per micro-step
+        assert all(math.isfinite(v) for v in stats.loss)
+        assert stats.loss[0] == pytest.approx(math.log(256), abs=0.3)
+        finals[name] = sum(stats.loss[-5:]) / 5
+    print(f"final losses {finals}", flush=True)
+    assert finals["quartet"] < math.log(256) - 1.5
+    assert finals["quartet"] < finals["bf16"] + 0.75
