@@ -22,7 +22,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch from profiler byte counters (fetch + write), scaled by what the same counters read for a
 # plain 256 MiB device copy (fetch counter x 2.0 KiB, write counter x 1.0 KiB)
 GEMM_TRAFFIC_BYTES = 173.9e6      # mean of the three GEMMs: 108.7 MiB fetched (operand re-reads that miss L2) + 57.1 MiB written
-QUANTIZE_TRAFFIC_BYTES = 89.8e6   # 64.1 MiB fetched + 21.5 MiB written; algorithmic 89.1e6
+QUANTIZE_TRAFFIC_BYTES = 90.3e6   # two thirds (the X share) of the forward pair launch: 96.1 MiB fetched + 33.0 MiB written; algorithmic 89.1e6
 
 
 def make_inputs(device, tokens=T_TOKENS, seed=0):
