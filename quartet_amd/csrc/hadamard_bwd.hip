@@ -10,6 +10,7 @@
 
 #include <type_traits>
 
+#include "qm_jobs.h"
 #include "qm_kernels.h"
 #include "qm_math.h"
 
@@ -39,7 +40,7 @@ __device__ __forceinline__ void cross_lane_stage(float (&v)[8], int lane_in_chun
     }
 }
 
-// The work of one launch with its block count; two independent jobs can share a grid (see job_pair_kernel).
+// The work of one launch as a job (qm_jobs.h): two independent inverse rotations can share a grid.
 template <typename TIn, typename TOut, int HD>
 struct HadamardBwdJob {
     const TIn* g;
@@ -108,16 +109,6 @@ struct HadamardBwdJob {
     }
 };
 
-template <class A>
-__global__ __launch_bounds__(256) void job_kernel(A a) {
-    a.run(blockIdx.x);
-}
-template <class A, class B>
-__global__ __launch_bounds__(256) void job_pair_kernel(A a, B b) {
-    if (blockIdx.x < a.blocks) a.run(blockIdx.x);
-    else b.run(blockIdx.x - a.blocks);
-}
-
 template <typename TOut>
 __global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t* __restrict__ codes,
                                                          const uint8_t* __restrict__ scales, int64_t n_octets,
@@ -147,7 +138,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t* __restr
 template <typename TIn, typename TOut>
 void launch_bwd(int hd, const void* g, int64_t n, float c, const SignBits& sb, const uint8_t* maskbits, void* out,
                 hipStream_t stream) {
-    const auto go = [&](auto job) { job_kernel<<<dim3(job.blocks), dim3(256), 0, stream>>>(job); };
+    const auto go = [&](auto job) { launch_job(job, stream); };
     if (hd == 32) go(HadamardBwdJob<TIn, TOut, 32>(g, n, c, sb, maskbits, out));
     else if (hd == 64) go(HadamardBwdJob<TIn, TOut, 64>(g, n, c, sb, maskbits, out));
     else go(HadamardBwdJob<TIn, TOut, 128>(g, n, c, sb, maskbits, out));
@@ -176,12 +167,10 @@ hipError_t masked_hadamard_bwd_hd32_pair(const void* ga, int64_t na, int scale_d
     const float ca = hadamard_scale(32, scale_dtype_a), cb = hadamard_scale(32, scale_dtype_b);
     if (dtype == BF16) {
         using J = HadamardBwdJob<uint16_t, uint16_t, 32>;
-        const J a(ga, na, ca, sa, mask_a, out_a), b(gb, nb, cb, sb, mask_b, out_b);
-        job_pair_kernel<<<dim3(a.blocks + b.blocks), dim3(256), 0, stream>>>(a, b);
+        launch_job_pair(J(ga, na, ca, sa, mask_a, out_a), J(gb, nb, cb, sb, mask_b, out_b), stream);
     } else {
         using J = HadamardBwdJob<float, float, 32>;
-        const J a(ga, na, ca, sa, mask_a, out_a), b(gb, nb, cb, sb, mask_b, out_b);
-        job_pair_kernel<<<dim3(a.blocks + b.blocks), dim3(256), 0, stream>>>(a, b);
+        launch_job_pair(J(ga, na, ca, sa, mask_a, out_a), J(gb, nb, cb, sb, mask_b, out_b), stream);
     }
     return hipGetLastError();
 }

@@ -27,6 +27,7 @@
 
 #include <type_traits>
 
+#include "qm_jobs.h"
 #include "qm_kernels.h"
 #include "qm_math.h"
 
@@ -294,19 +295,6 @@ __global__ __launch_bounds__(256) void quantize_rowmajor_g32_kernel(const T* __r
     finish_group<T, MODE, WANT_MASK>(v, gi, gi, c, sign_word, seed, out);
 }
 
-// A job is the work of one kernel launch with its block count; job kernels run one job, or two independent jobs
-// one after the other in a single grid (the second job's blocks fill the machine while the first one drains, and
-// the pause between two dependent launches is paid once).
-template <class A>
-__global__ __launch_bounds__(256) void job_kernel(A a) {
-    a.run(blockIdx.x);
-}
-template <class A, class B>
-__global__ __launch_bounds__(256) void job_pair_kernel(A a, B b) {
-    if (blockIdx.x < a.blocks) a.run(blockIdx.x);
-    else b.run(blockIdx.x - a.blocks);
-}
-
 // Tiled code layout ([rows/16][cols/128][16 rows][64 bytes]).  Workgroup b owns block b / chunks of 16 rows and run
 // b % chunks of 512 columns (four code tiles); wave w owns rows 4w..4w+3 of the block, lane l its row l / 16 and
 // group l % 16 of the run: the wave reads four contiguous KiB (bf16) and writes, per tile, four rows' 64-byte pieces
@@ -359,7 +347,7 @@ void launch_rowmajor_g32(int mode, const void* x, int64_t rows, int64_t cols, bo
                          uint64_t seed, const GroupOut& out, hipStream_t stream) {
     const T* xp = reinterpret_cast<const T*>(x);
     if (tiled) {
-        const auto go = [&](auto job) { job_kernel<<<dim3(job.blocks), dim3(256), 0, stream>>>(job); };
+        const auto go = [&](auto job) { launch_job(job, stream); };
         switch (mode) {
             case QUEST_RTN: go(RowmajorTiledJob<T, QUEST_RTN, WANT_MASK>(x, rows, cols, c, sign_word, seed, out)); break;
             case ABSMAX_RTN: go(RowmajorTiledJob<T, ABSMAX_RTN, WANT_MASK>(x, rows, cols, c, sign_word, seed, out)); break;
@@ -630,15 +618,6 @@ struct RequantJob {
         }
     }
 };
-
-template <class Job>
-void launch_job(const Job& job, hipStream_t stream) {
-    job_kernel<<<dim3(job.blocks), dim3(256), 0, stream>>>(job);
-}
-template <class A, class B>
-void launch_job_pair(const A& a, const B& b, hipStream_t stream) {
-    job_pair_kernel<<<dim3(a.blocks + b.blocks), dim3(256), 0, stream>>>(a, b);
-}
 
 template <typename T>
 void launch_transposed_g32(int mode, const void* x, int64_t P, int64_t Q, float c, uint32_t sign_word, uint64_t seed,

@@ -1,0 +1,85 @@
+"""CPU tests of the C ABI: the shared library loads, exports exactly what include/quartet_hip.h declares, its
+host-only entry points work without a GPU, and argument validation answers with error codes and messages
+(no kernel is launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from quartet_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "quartet_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return set(re.findall(r"^\s*(?:const\s+char\s*\*|int|size_t)\s+(qm_\w+)\s*\(", text, flags=re.M))
+
+
+def test_library_exports_every_declared_function():
+    names = declared_functions()
+    assert len(names) >= 13
+    assert names == set(_lib.EXPORTS), names ^ set(_lib.EXPORTS)
+    L = ctypes.CDLL(_lib.LIB_PATH)
+    for name in names:
+        assert getattr(L, name) is not None
+
+
+def test_host_only_entry_points():
+    L = _lib.lib()
+    assert L.qm_version() == 2
+    T, I, O = 256, 128, 384
+    total = L.qm_linear_saved_bytes(T, I, O)
+    off = (ctypes.c_size_t * 6)()
+    assert L.qm_linear_saved_offsets(T, I, O, off) == 0
+    sizes = [T * I // 2, T * I // 32, T * I // 8, O * I // 2, O * I // 32, O * I // 8]
+    # regions in declaration order, each 256-byte aligned, none overlapping, all inside the buffer
+    assert off[0] == 0
+    for k in range(6):
+        assert off[k] % 256 == 0
+        end = off[k] + sizes[k]
+        assert end <= (off[k + 1] if k < 5 else total)
+    assert L.qm_linear_saved_bytes(T, 100, O) == 0                      # in_features not a multiple of 32
+    assert L.qm_linear_saved_offsets(T, 100, O, off) != 0 and b"qm_linear_saved_offsets" in L.qm_last_error()
+    assert L.qm_linear_saved_offsets(T, I, O, None) != 0
+    assert L.qm_linear_backward_workspace_bytes(T, I, O, _lib.QM_BF16) > 0
+    assert L.qm_linear_backward_workspace_bytes(T, I, 100, _lib.QM_BF16) == 0
+    assert L.qm_linear_backward_workspace_bytes(T, I, O, 7) == 0
+    assert L.qm_gemm_workspace_bytes(256, 256, 100) == 0                # K not a multiple of 32
+
+
+@pytest.mark.parametrize("call,needle", [
+    (lambda L: L.qm_quantize_mxfp4(None, 0, 4, 30, 32, None, 0, 0, None, 0, None, None, None, None, 0, None), b"multiple of hadamard_dim"),
+    (lambda L: L.qm_quantize_mxfp4(None, 5, 4, 32, 32, None, 0, 0, None, 0, None, None, None, None, 0, None), b"x_dtype"),
+    (lambda L: L.qm_quantize_mxfp4(None, 0, 4, 32, 48, None, 0, 0, None, 0, None, None, None, None, 0, None), b"hadamard_dim"),
+    (lambda L: L.qm_quantize_mxfp4(None, 0, 4, 32, 32, None, 9, 0, None, 0, None, None, None, None, 0, None), b"mode"),
+    (lambda L: L.qm_quantize_mxfp4(None, 0, 4, 32, 32, None, 0, 0, None, 0, None, None, None, None, 3, None), b"codes_layout"),
+    (lambda L: L.qm_quantize_mxfp4(None, 0, 4, 32, 32, None, 0, 0, None, 0, None, None, None, None, 0, None), b"non-null"),
+    (lambda L: L.qm_requantize_transposed_mxfp4(None, None, 30, 64, 1.0, 0, 32, None, 2, None, 0, None, None, None, 0, 0, None), b"hadamard_dim"),
+    (lambda L: L.qm_gemm_mxfp4_tn(None, None, None, None, 64, 64, 48, 1.0, None, 0, 0, 0, None, 0, None), b"qm_gemm_mxfp4_tn"),
+    (lambda L: L.qm_masked_hadamard_bwd(None, 0, 4, 40, 32, 0, None, None, None, 0, None), b"multiple of hadamard_dim"),
+    (lambda L: L.qm_dequantize_mxfp4(None, None, 4, 40, 1.0, None, 0, None), b"C % 32"),
+    (lambda L: L.qm_linear_forward(None, 0, None, 0, 64, 40, 64, 32, None, 32, None, None, 0, None, 0, 0, None), b"multiple of 32"),
+    (lambda L: L.qm_linear_forward(None, 0, None, 0, 64, 64, 64, 32, None, 32, None, None, 0, None, 0, 0, None), b"saved buffer"),
+])
+def test_rejected_arguments_report_an_error(call, needle):
+    L = _lib.lib()
+    rc = call(L)
+    assert rc < 0
+    assert needle in L.qm_last_error(), L.qm_last_error()
+
+
+def test_empty_shapes_are_accepted_without_touching_pointers():
+    L = _lib.lib()
+    assert L.qm_quantize_mxfp4(None, 0, 0, 64, 32, None, 0, 0, None, 0, None, None, None, None, 0, None) == 0
+    assert L.qm_gemm_mxfp4_tn(None, None, None, None, 0, 64, 64, 1.0, None, 0, 0, 0, None, 0, None) == 0
+    assert L.qm_linear_forward(None, 0, None, 0, 0, 64, 64, 32, None, 32, None, None, 0, None, 0, 0, None) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libquartet_hip.so"))
+    with pytest.raises(_lib.QuartetHipError, match="no CPU fallback"):
+        _lib.lib()
