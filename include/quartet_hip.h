@@ -54,7 +54,9 @@ const char* qm_last_error(void);
  *   x            input, dtype x_dtype; row-major [rows, cols], or, when transposed_in != 0,
  *                row-major [cols, rows] (the kernel quantizes its transpose: this is
  *                `e.T.contiguous()` + quantize of backward.py:81 in one pass)
- *   hadamard_dim 32, 64 or 128; cols % hadamard_dim == 0
+ *   hadamard_dim 32, 64 or 128; cols % hadamard_dim == 0.  hadamard_dim 1 = the input is already rotated (the dense
+ *                random rotation of rerotate="O32", mxfp4.py:61-64, applied by the caller): groups of 32 are
+ *                quantized as they are; row-major input and codes only, sign_bits == NULL, u == NULL
  *   u            SR modes: device floats in [0,1) indexed by logical flat offset, or NULL to draw
  *                them in-kernel from Philox4x32-10 keyed by (seed, offset)
  *   codes/scales outputs (required); maskbits, dequant optional (NULL to skip); dequant has

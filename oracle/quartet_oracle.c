@@ -290,7 +290,9 @@ int qo_quantize(const void* x, int dtype, int64_t rows, int64_t cols, int hd,
                 const uint32_t* sign_bits, int mode, int transposed_in, const float* u,
                 uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
                 float* rotated) {
-    if (!(hd == 32 || hd == 64 || hd == 128) || cols % hd || rows < 0 || cols < 0) return -1;
+    /* hd == 1: the input is already rotated (a dense rotation applied by the caller, mxfp4.py:61-64): the butterfly
+       has no stage and c = 1 */
+    if (!(hd == 1 || hd == 32 || hd == 64 || hd == 128) || cols % hd || cols % 32 || rows < 0 || cols < 0) return -1;
     if (mode < 0 || mode > 3 || (dtype != QO_BF16 && dtype != QO_F32)) return -1;
     float c = qo_hadamard_scale(hd, dtype);
     int err = 0;

@@ -51,7 +51,12 @@ int qm_quantize_mxfp4(const void* x, int x_dtype, int64_t rows, int64_t cols, in
                       uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant, int codes_layout, void* stream) {
     if (!valid_layout(codes_layout)) return fail(QM_ERR_INVALID, "qm_quantize_mxfp4: unknown codes_layout %d", codes_layout);
     if (!valid_dtype(x_dtype)) return fail(QM_ERR_INVALID, "qm_quantize_mxfp4: x_dtype %d is not QM_BF16/QM_F32", x_dtype);
-    if (!valid_hd(hadamard_dim)) return fail(QM_ERR_INVALID, "qm_quantize_mxfp4: hadamard_dim %d not in {32,64,128}", hadamard_dim);
+    if (!valid_hd(hadamard_dim) && hadamard_dim != 1)
+        return fail(QM_ERR_INVALID, "qm_quantize_mxfp4: hadamard_dim %d not in {1,32,64,128}", hadamard_dim);
+    if (hadamard_dim == 1 && (transposed_in || u || sign_bits || codes_layout != QM_LAYOUT_ROWMAJOR || cols % 32 ||
+                              !aligned(codes, 16) || !aligned(maskbits, 4)))
+        return fail(QM_ERR_INVALID, "qm_quantize_mxfp4: hadamard_dim 1 (input already rotated) needs row-major input and codes, "
+                                    "cols %% 32 == 0, no sign bits, no explicit uniforms, 16-byte aligned codes");
     if (!valid_mode(mode)) return fail(QM_ERR_INVALID, "qm_quantize_mxfp4: unknown mode %d", mode);
     if (rows < 0 || cols < 0) return fail(QM_ERR_INVALID, "qm_quantize_mxfp4: negative shape [%lld, %lld]", (long long)rows, (long long)cols);
     if (cols % hadamard_dim) return fail(QM_ERR_INVALID, "qm_quantize_mxfp4: cols %lld not a multiple of hadamard_dim %d", (long long)cols, hadamard_dim);

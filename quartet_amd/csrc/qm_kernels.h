@@ -32,7 +32,7 @@ bool gemm_supports_tiled(int64_t M, int64_t N, int64_t K);
 // hd = 32 fast path (one MX group per lane, hardware FP4 converts); row-major input, RTN or Philox SR
 hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t rows, int64_t cols, uint32_t sign_word, int mode,
                                   uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
-                                  bool tiled, hipStream_t stream);
+                                  bool tiled, bool rotate, hipStream_t stream);
 
 hipError_t quantize_rowmajor_wide(const void* x, int dtype, int64_t n, int hd, const SignBits& sb, int mode, uint64_t seed,
                                   uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant, hipStream_t stream);

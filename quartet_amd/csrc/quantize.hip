@@ -416,8 +416,13 @@ hipError_t quantize_mxfp4(const void* x, int dtype, int64_t rows, int64_t cols, 
     if (tiled && !quantize_supports_tiled(rows, cols, hd, mode, transposed_in, u, maskbits)) return hipErrorInvalidValue;
     const auto al = [](const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
     if (tiled && !(al(codes, 16) && al(maskbits, 4) && al(scales, 4))) return hipErrorInvalidValue;
+    if (hd == 1) {
+        // already rotated input: groups of 32 pass straight to the quantizer (row-major, RTN or seeded SR only)
+        if (transposed_in || !(rtn || u == nullptr) || tiled || !al(codes, 16) || !al(maskbits, 4)) return hipErrorInvalidValue;
+        return quantize_rowmajor_hd32(x, dtype, rows, cols, 0u, mode, seed, codes, scales, maskbits, dequant, false, false, stream);
+    }
     if (hd == 32 && !transposed_in && (rtn || u == nullptr) && al(codes, 16) && al(maskbits, 4))
-        return quantize_rowmajor_hd32(x, dtype, rows, cols, sb.w[0], mode, seed, codes, scales, maskbits, dequant, tiled, stream);
+        return quantize_rowmajor_hd32(x, dtype, rows, cols, sb.w[0], mode, seed, codes, scales, maskbits, dequant, tiled, true, stream);
     if ((hd == 64 || hd == 128) && !transposed_in && (rtn || u == nullptr) && al(codes, 16) && al(maskbits, 4))
         return quantize_rowmajor_wide(x, dtype, rows * cols, hd, sb, mode, seed, codes, scales, maskbits, dequant, stream);
     // logical [rows, cols] = physical [P = cols, Q = rows]

@@ -262,8 +262,8 @@ struct GroupOut {
 };
 
 // x @ H for one chunk of 32: butterfly, then hd^-1/2 with the column sign folded in (wave-uniform)
-__device__ __forceinline__ void rotate_group(float (&v)[32], float c, uint32_t sign_word) {
-    butterfly32(v);
+__device__ __forceinline__ void rotate_group(float (&v)[32], float c, uint32_t sign_word, bool rotate = true) {
+    if (rotate) butterfly32(v);  // uniform; without it (c = 1, no signs) the group passes through unchanged
 #pragma unroll
     for (int j = 0; j < 32; ++j) {
         const float cj = u2f(f2u(c) ^ (((sign_word >> j) & 1u) << 31));  // wave-uniform: stays in scalar registers
@@ -275,8 +275,8 @@ __device__ __forceinline__ void rotate_group(float (&v)[32], float c, uint32_t s
 // random stream; ci is the index of its 16 code bytes in the code buffer (= gi for row-major codes)
 template <typename T, int MODE, bool WANT_MASK>
 __device__ __forceinline__ void finish_group(float (&v)[32], int64_t gi, int64_t ci, float c, uint32_t sign_word,
-                                             uint64_t seed, const GroupOut& out) {
-    rotate_group(v, c, sign_word);
+                                             uint64_t seed, const GroupOut& out, bool rotate) {
+    rotate_group(v, c, sign_word, rotate);
     GroupCodes o;
     quantize_group_regs<MODE, WANT_MASK>(v, seed, gi, o);
     out.codes[ci] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
@@ -287,12 +287,13 @@ __device__ __forceinline__ void finish_group(float (&v)[32], int64_t gi, int64_t
 
 template <typename T, int MODE, bool WANT_MASK>
 __global__ __launch_bounds__(256) void quantize_rowmajor_g32_kernel(const T* __restrict__ x, int64_t n_groups, float c,
-                                                                    uint32_t sign_word, uint64_t seed, GroupOut out) {
+                                                                    uint32_t sign_word, uint64_t seed, GroupOut out,
+                                                                    int rotate) {
     const int64_t gi = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (gi >= n_groups) return;
     float v[32];
     load_group<T>(x + gi * 32, v);
-    finish_group<T, MODE, WANT_MASK>(v, gi, gi, c, sign_word, seed, out);
+    finish_group<T, MODE, WANT_MASK>(v, gi, gi, c, sign_word, seed, out, rotate != 0);
 }
 
 // Tiled code layout ([rows/16][cols/128][16 rows][64 bytes]).  Workgroup b owns block b / chunks of 16 rows and run
@@ -344,7 +345,7 @@ struct RowmajorTiledJob {
 
 template <typename T, bool WANT_MASK>
 void launch_rowmajor_g32(int mode, const void* x, int64_t rows, int64_t cols, bool tiled, float c, uint32_t sign_word,
-                         uint64_t seed, const GroupOut& out, hipStream_t stream) {
+                         uint64_t seed, const GroupOut& out, bool rotate, hipStream_t stream) {
     const T* xp = reinterpret_cast<const T*>(x);
     if (tiled) {
         const auto go = [&](auto job) { launch_job(job, stream); };
@@ -359,10 +360,10 @@ void launch_rowmajor_g32(int mode, const void* x, int64_t rows, int64_t cols, bo
     const int64_t n_groups = rows * cols / 32;
     dim3 grid((unsigned)((n_groups + 255) / 256)), block(256);
     switch (mode) {
-        case QUEST_RTN: quantize_rowmajor_g32_kernel<T, QUEST_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
-        case ABSMAX_RTN: quantize_rowmajor_g32_kernel<T, ABSMAX_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
-        case ABSMAX_SR: quantize_rowmajor_g32_kernel<T, ABSMAX_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
-        default: quantize_rowmajor_g32_kernel<T, QUEST_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out); break;
+        case QUEST_RTN: quantize_rowmajor_g32_kernel<T, QUEST_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out, (int)rotate); break;
+        case ABSMAX_RTN: quantize_rowmajor_g32_kernel<T, ABSMAX_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out, (int)rotate); break;
+        case ABSMAX_SR: quantize_rowmajor_g32_kernel<T, ABSMAX_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out, (int)rotate); break;
+        default: quantize_rowmajor_g32_kernel<T, QUEST_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, c, sign_word, seed, out, (int)rotate); break;
     }
 }
 
@@ -644,18 +645,20 @@ void launch_requant_g32(int mode, const uint8_t* codes_in, const uint8_t* scales
 
 }  // namespace
 
-// hd = 32, row-major input, RTN or Philox-driven SR (explicit uniforms take the generic path)
+// hd = 32, row-major input, RTN or Philox-driven SR (explicit uniforms take the generic path); rotate = false
+// quantizes groups of 32 as they are (input rotated by the caller)
 hipError_t quantize_rowmajor_hd32(const void* x, int dtype, int64_t rows, int64_t cols, uint32_t sign_word, int mode,
                                   uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
-                                  bool tiled, hipStream_t stream) {
+                                  bool tiled, bool rotate, hipStream_t stream) {
+    if (!rotate && (tiled || sign_word)) return hipErrorInvalidValue;  // pass-through groups: row-major codes, no signs
     GroupOut out{reinterpret_cast<uint4*>(codes), scales, reinterpret_cast<uint32_t*>(maskbits), dequant};
-    const float c = hadamard_scale(32, dtype);
+    const float c = rotate ? hadamard_scale(32, dtype) : 1.0f;
     if (maskbits) {
-        if (dtype == BF16) launch_rowmajor_g32<uint16_t, true>(mode, x, rows, cols, tiled, c, sign_word, seed, out, stream);
-        else launch_rowmajor_g32<float, true>(mode, x, rows, cols, tiled, c, sign_word, seed, out, stream);
+        if (dtype == BF16) launch_rowmajor_g32<uint16_t, true>(mode, x, rows, cols, tiled, c, sign_word, seed, out, rotate, stream);
+        else launch_rowmajor_g32<float, true>(mode, x, rows, cols, tiled, c, sign_word, seed, out, rotate, stream);
     } else {
-        if (dtype == BF16) launch_rowmajor_g32<uint16_t, false>(mode, x, rows, cols, tiled, c, sign_word, seed, out, stream);
-        else launch_rowmajor_g32<float, false>(mode, x, rows, cols, tiled, c, sign_word, seed, out, stream);
+        if (dtype == BF16) launch_rowmajor_g32<uint16_t, false>(mode, x, rows, cols, tiled, c, sign_word, seed, out, rotate, stream);
+        else launch_rowmajor_g32<float, false>(mode, x, rows, cols, tiled, c, sign_word, seed, out, rotate, stream);
     }
     return hipGetLastError();
 }

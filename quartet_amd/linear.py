@@ -87,7 +87,10 @@ class QuantizedLinear(nn.Linear):
 
     def _is_production_config(self):
         g_q = self.backward_scheme.g_quantizer
-        return (self.use_packed_path
+        # a dense rotation (rerotate="O32") anywhere, now or after the next re_randomize, needs the generic path
+        dense = any(getattr(q_, "is_dense", False) or getattr(q_, "rerotate", None) == "O32"
+                    for q_ in (self.activation_quantizer, self.weight_quantizer, g_q))
+        return (self.use_packed_path and not dense
                 and type(self.activation_quantizer) is QuestMXFP4Quantizer
                 and type(self.weight_quantizer) is QuestMXFP4Quantizer
                 and type(g_q) is AlbertTsengQuantizer

@@ -23,59 +23,29 @@ The rotation argument is the dense ``[hd, hd]`` matrix the reference passes arou
 matrix scaled by ``hd^-1/2`` with negated columns, which is what every quantizer module holds.  Reading its signs
 (and the value of an ``alpha`` tensor) takes one device-to-host copy, remembered for as long as that tensor object lives unmodified.
 """
-import weakref
-
 import torch
 
 from . import kernels as K
-from .quantizers.mxfp4 import _fresh_seed, sylvester_matrix
+from .quantizers.mxfp4 import _fresh_seed, remember_host_value, sylvester_sign_bits
 
 ALPHA_FWD = 1.0
 ALPHA_BWD = K.FOUR_THIRDS * K.FOUR_THIRDS
-
-_host_cache = {}
-_HOST_CACHE_LIMIT = 64
-
-
-def _remember(kind, t, make):
-    """Host-side value derived from tensor `t`, kept while that very tensor object is alive and unmodified (the
-    entry holds a weak reference: an address alone may be handed to another tensor after a free)."""
-    key = (kind, id(t))
-    hit = _host_cache.get(key)
-    if hit is not None and hit[0]() is t and hit[1] == t._version:
-        return hit[2]
-    value = make()
-    if len(_host_cache) >= _HOST_CACHE_LIMIT:
-        _host_cache.clear()
-    _host_cache[key] = (weakref.ref(t), t._version, value)
-    return value
-
 
 def rotation_sign_bits(hadamard_matrix):
     """Bit mask of the negated columns of ``hd^-1/2 * Sylvester * diag(+-1)``; raises for any other matrix."""
     if hadamard_matrix.dim() != 2 or hadamard_matrix.shape[0] != hadamard_matrix.shape[1]:
         raise ValueError(f"rotation must be a square matrix, got shape {tuple(hadamard_matrix.shape)}")
-    hd = hadamard_matrix.shape[0]
-    if hd not in (32, 64, 128):
-        raise ValueError(f"rotation size must be 32, 64 or 128, got {hd}")
-
-    def read():
-        h = hadamard_matrix.detach().to("cpu", torch.float32)
-        bits = 0
-        for j, v in enumerate(h[0].tolist()):
-            if v < 0:
-                bits |= 1 << j
-        c = torch.tensor(hd ** -0.5, dtype=torch.float32).to(hadamard_matrix.dtype).float()
-        want = sylvester_matrix(hd) * c * torch.where(h[0] < 0, -1.0, 1.0)[None, :]
-        if not torch.equal(h, want):
-            raise ValueError("rotation is not a scaled Sylvester Hadamard matrix with negated columns; dense rotations "
-                             "are not supported by the HIP kernels")
-        return bits
-    return _remember("signs", hadamard_matrix, read)
+    if hadamard_matrix.shape[0] not in (32, 64, 128):
+        raise ValueError(f"rotation size must be 32, 64 or 128, got {hadamard_matrix.shape[0]}")
+    bits = sylvester_sign_bits(hadamard_matrix)
+    if bits is None:
+        raise ValueError("rotation is not a scaled Sylvester Hadamard matrix with negated columns; the packed operators "
+                         "do not take dense rotations")
+    return bits
 
 
 def _host_scalar(t):
-    return _remember("scalar", t, lambda: float(t.detach().reshape(-1)[0].item()))
+    return remember_host_value("scalar", t, lambda: float(t.detach().reshape(-1)[0].item()))
 
 
 def _rows(x):

@@ -5,9 +5,13 @@ Differences in representation, not in results:
   * the rotation H = hd^-1/2 * Sylvester * diag(signs) is kept as a sign bit mask; the dense
     ``hadamard_matrix`` attribute is materialised on demand (same values the reference holds);
   * the clip mask saved for backward is bit-packed (1 bit per element);
-  * ``rerotate="O32"`` (dense random rotation) is not built yet and raises.
+  * ``rerotate="O32"`` replaces H by a dense random orthogonal matrix (mxfp4.py:61-64).  The butterfly kernels cannot
+    apply it, so the rotation runs as a library matrix product (fp32 accumulation over the tensor's dtype, which is
+    what the reference's in-kernel ``tl.dot`` does) and the kernel quantizes the rotated groups as they are; a layer
+    whose quantizers hold a dense rotation takes the generic (pseudo-quantized) path.
 """
 import random
+import weakref
 
 import torch
 
@@ -44,26 +48,61 @@ def _autocast_bf16():
     return torch.is_autocast_enabled() and torch.get_autocast_dtype("cuda") == torch.bfloat16
 
 
+_host_cache = {}
+_HOST_CACHE_LIMIT = 64
+
+
+def remember_host_value(kind, t, make):
+    """Host-side value derived from tensor `t` (one device-to-host copy), kept while that very tensor object is alive
+    and unmodified: the entry holds a weak reference, since an address alone may be handed to another tensor after a
+    free."""
+    key = (kind, id(t))
+    hit = _host_cache.get(key)
+    if hit is not None and hit[0]() is t and hit[1] == t._version:
+        return hit[2]
+    value = make()
+    if len(_host_cache) >= _HOST_CACHE_LIMIT:
+        _host_cache.clear()
+    _host_cache[key] = (weakref.ref(t), t._version, value)
+    return value
+
+
+def sylvester_sign_bits(matrix):
+    """Bit mask of the negated columns if `matrix` is ``hd^-1/2 * Sylvester * diag(+-1)`` (hd 32, 64 or 128, the
+    scale rounded to the matrix's dtype), else None: a dense rotation."""
+    if matrix.dim() != 2 or matrix.shape[0] != matrix.shape[1] or matrix.shape[0] not in (32, 64, 128):
+        return None
+    hd = matrix.shape[0]
+
+    def read():
+        h = matrix.detach().to("cpu", torch.float32)
+        c = torch.tensor(hd ** -0.5, dtype=torch.float32).to(matrix.dtype).float()
+        if not torch.equal(h, sylvester_matrix(hd) * c * torch.where(h[0] < 0, -1.0, 1.0)[None, :]):
+            return -1
+        return sum(1 << j for j, v in enumerate(h[0].tolist()) if v < 0)
+    bits = remember_host_value("signs", matrix, read)
+    return None if bits < 0 else bits
+
+
 @torch.compiler.disable()
 def mxfp4_forward_kernel_wrapper(x, hadamard_matrix, return_clip_mask=False, gaussian_scale=3 / 4,
                                  stochastic_round=False, quest=True):
     """Drop-in for mxfp4_triton.py:177-220: returns (pseudo-quantized tensor like x, bool clip mask | None).
-    ``hadamard_matrix`` must be a signed, scaled Sylvester matrix (what the quantizer modules hold)."""
+    A signed, scaled Sylvester matrix (what the quantizer modules hold by default) runs on the butterfly kernels; any
+    other matrix is applied as a dense matrix product and the kernel quantizes the rotated groups as they are."""
     hd = hadamard_matrix.shape[-1]
-    first = hadamard_matrix[0].float()
-    sign_bits = 0
-    for j, v in enumerate(first.tolist()):
-        if v < 0:
-            sign_bits |= 1 << j
     mode = (K.QM_QUEST_SR if stochastic_round else K.QM_QUEST_RTN) if quest else \
         (K.QM_ABSMAX_SR if stochastic_round else K.QM_ABSMAX_RTN)
-    x2 = _as_2d(x, hd)
-    _, _, mask, deq = K.quantize_mxfp4(x2, hd, sign_bits, mode, seed=_fresh_seed() if stochastic_round else 0,
-                                       want_mask=return_clip_mask, want_dequant=True)
-    clip = None
-    if return_clip_mask:
-        shifts = torch.arange(8, device=mask.device, dtype=torch.uint8)
-        clip = ((mask[..., None] >> shifts) & 1).bool().view(x.shape)
+    seed = _fresh_seed() if stochastic_round else 0
+    sign_bits = sylvester_sign_bits(hadamard_matrix)
+    if sign_bits is None:
+        _, _, mask, deq = K.quantize_mxfp4(_rotate_dense(x, hadamard_matrix), 1, None, mode, seed=seed,
+                                           want_mask=return_clip_mask, want_dequant=True)
+        deq = deq.to(x.dtype)
+    else:
+        _, _, mask, deq = K.quantize_mxfp4(_as_2d(x, hd), hd, sign_bits, mode, seed=seed, want_mask=return_clip_mask,
+                                           want_dequant=True)
+    clip = _unpack_mask(mask, x.shape).bool() if return_clip_mask else None
     return deq.view(x.shape), clip
 
 
@@ -77,12 +116,19 @@ class _HadamardQuantizer(BaseQuantizer):
         self.hadamard_dim = hadamard_dim
         self.rerotate = rerotate
         self.sign_bits = 0  # bit j set = column j of H negated
+        self._dense = None  # fp32 [hd, hd] orthogonal matrix once re_randomize("O32") has replaced H
         self._matrix_dtype = torch.float32
         self._matrix_device = torch.device("cpu")
 
     @property
+    def is_dense(self):
+        return self._dense is not None
+
+    @property
     def hadamard_matrix(self):
         hd = self.hadamard_dim
+        if self._dense is not None:
+            return self._dense.to(self._matrix_device).to(self._matrix_dtype)
         signs = torch.tensor([-1.0 if (self.sign_bits >> j) & 1 else 1.0 for j in range(hd)])
         h = sylvester_matrix(hd) * torch.tensor(hd ** -0.5, dtype=torch.float32) * signs[None, :]
         return h.to(self._matrix_device).to(self._matrix_dtype)
@@ -99,11 +145,52 @@ class _HadamardQuantizer(BaseQuantizer):
                 if f == 0:  # randint*2-1 == -1
                     self.sign_bits ^= 1 << j
         elif self.rerotate == "O32":
-            raise NotImplementedError("rerotate='O32' (dense random orthogonal rotation) is not implemented")
+            # H <- U V^T of the SVD of a Gaussian matrix (mxfp4.py:61-64): Haar-distributed up to signs
+            u, _, vh = torch.linalg.svd(torch.randn(self.hadamard_dim, self.hadamard_dim))
+            self._dense = (u @ vh).contiguous()
+            self.sign_bits = 0
         elif self.rerotate is None:
             pass
         else:
             raise ValueError(f"Invalid rerotate value: {self.rerotate}")
+
+
+def _rotate_dense(x, matrix):
+    """x.view(-1, hd) @ matrix with fp32 accumulation and an fp32 result, as rows of x's last dimension."""
+    hd = matrix.shape[0]
+    last = x.shape[-1] if x.dim() > 0 and x.shape[-1] % hd == 0 else hd
+    return (x.reshape(-1, hd).float() @ matrix.to(x.dtype).float()).view(-1, last)
+
+
+def _unpack_mask(maskbits, shape):
+    shifts = torch.arange(8, device=maskbits.device, dtype=torch.uint8)
+    return ((maskbits[..., None] >> shifts) & 1).view(shape)
+
+
+class DenseRotationQuantizerFn(torch.autograd.Function):
+    """Either quantizer with a dense rotation: rotate by a matrix product, quantize the rotated groups of 32 as they
+    are (kernel block size 1), straight-through backward ``(g * mask) @ matrix^T`` (mxfp4.py:30-34,143-146)."""
+
+    @staticmethod
+    def forward(ctx, x, matrix, mode, want_mask, post_scale):
+        xr = _rotate_dense(x, matrix)
+        stochastic = mode in (K.QM_ABSMAX_SR, K.QM_QUEST_SR)
+        _, _, maskbits, deq = K.quantize_mxfp4(xr, 1, None, mode, seed=_fresh_seed() if stochastic else 0,
+                                               want_mask=want_mask, want_dequant=True)
+        if post_scale != 1.0:
+            deq *= post_scale
+        ctx.save_for_backward(matrix, maskbits) if want_mask else ctx.save_for_backward(matrix)
+        ctx.x_shape, ctx.x_dtype, ctx.want_mask = x.shape, x.dtype, want_mask
+        return deq.to(x.dtype).view(x.shape)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        matrix = ctx.saved_tensors[0]
+        g = grad_output
+        if ctx.want_mask:
+            g = g * _unpack_mask(ctx.saved_tensors[1], g.shape).to(g.dtype)
+        out = g.reshape(-1, matrix.shape[0]) @ matrix.to(g.dtype).T
+        return out.view(ctx.x_shape).to(ctx.x_dtype), None, None, None, None
 
 
 class QuestMXFP4QuantizerFn(torch.autograd.Function):
@@ -132,6 +219,8 @@ class QuestMXFP4QuantizerFn(torch.autograd.Function):
 class QuestMXFP4Quantizer(_HadamardQuantizer):
     def forward(self, x):
         self._note_input(x)
+        if self.is_dense:
+            return DenseRotationQuantizerFn.apply(x, self.hadamard_matrix, K.QM_QUEST_RTN, True, 1.0)
         return QuestMXFP4QuantizerFn.apply(x, self.hadamard_dim, self.sign_bits)
 
 
@@ -165,6 +254,9 @@ class AlbertTsengQuantizer(_HadamardQuantizer):
 
     def forward(self, x):
         self._note_input(x)
+        if self.is_dense:
+            mode = K.QM_ABSMAX_SR if self.stochastic else K.QM_ABSMAX_RTN
+            return DenseRotationQuantizerFn.apply(x, self.hadamard_matrix, mode, False, 1.0)
         return AlbertTsengQuantizerFn.apply(x, self.hadamard_dim, self.sign_bits, self.stochastic, 1.0)
 
 
@@ -173,4 +265,6 @@ class AlignedAlbertTsengQuantizer(_HadamardQuantizer):
 
     def forward(self, x):
         self._note_input(x)
+        if self.is_dense:
+            return DenseRotationQuantizerFn.apply(x, self.hadamard_matrix, K.QM_ABSMAX_RTN, False, 1.009276)
         return AlbertTsengQuantizerFn.apply(x, self.hadamard_dim, self.sign_bits, False, 1.009276)

@@ -175,6 +175,71 @@ def test_notebook_error_bands_on_gpu(q):
     wref = w.clone().float().requires_grad_(True)
     yref = torch.nn.functional.linear(x.detach().float(), wref)
     yref.backward(dy.float())
-    err = lambda a, b: float(((a.float() - b.float()) ** 2).sum() / (b.float() ** 2).sum())
+    err = lambda a, b: float(((a.detach().float() - b.detach().float()) ** 2).sum() / (b.detach().float() ** 2).sum())
     assert 2e-2 < err(y, yref) < 6e-2
     assert 6e-2 < err(layer.weight.grad, wref.grad) < 15e-2
+
+
+@pytest.mark.parametrize("cls_name,mode_name,post", [("QuestMXFP4Quantizer", "QUEST_RTN", 1.0),
+                                                     ("AlbertTsengQuantizer", "ABSMAX_SR", 1.0),
+                                                     ("AlignedAlbertTsengQuantizer", "ABSMAX_RTN", 1.009276)])
+def test_dense_rotation_quantizers_against_oracle(oracle, q, cls_name, mode_name, post):
+    """rerotate="O32": the module rotates by a matrix product and the kernel quantizes the rotated groups; on the
+    same rotated tensor the oracle must give the same pseudo-quantized values, and the backward pass is the
+    (masked) product with the transposed matrix."""
+    print(f"case dense rotation {cls_name}", flush=True)
+    import random
+    dev = "cuda:0"
+    torch.manual_seed(11)
+    quant = getattr(q, cls_name)(hadamard_dim=32, rerotate="O32")
+    quant.re_randomize()
+    x = make_input(48, 256, torch.bfloat16, seed=12).to(dev).requires_grad_(True)
+    random.seed(4)
+    y = quant(x)
+    R = quant.hadamard_matrix
+    assert R.dtype == torch.bfloat16 and R.device.type == "cuda"
+    xr = (x.detach().reshape(-1, 32).float() @ R.float()).view(48, 256)
+    random.seed(4)
+    seed = random.getrandbits(63) if "SR" in mode_name else 0
+    want = oracle.quantize(xr.cpu().numpy(), 1, mode=getattr(oracle, mode_name), seed=seed, want_mask=True, want_dequant=True)
+    ref = torch.from_numpy(want["dequant"])
+    if post != 1.0:
+        ref = ref * post
+    assert torch.equal(y.detach().cpu(), ref.to(torch.bfloat16))
+    g = make_input(48, 256, torch.bfloat16, seed=13).to(dev)
+    y.backward(g)
+    gm = g.float()
+    if cls_name == "QuestMXFP4Quantizer":
+        bits = torch.from_numpy(np.unpackbits(want["mask"], axis=1, bitorder="little")).to(dev).float()
+        gm = gm * bits
+    gref = (gm.reshape(-1, 32) @ R.float().T).view(48, 256)
+    assert float((x.grad.float() - gref).norm() / gref.norm()) < 1e-2   # the module's product runs in bf16
+
+
+def test_layer_with_dense_gradient_rotation(q):
+    """The production configuration with rerotate="O32" on the gradient quantizer (generic path): gradients stay as
+    close to the unquantized ones as with sign flips."""
+    print("case layer with O32 gradient rotation", flush=True)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(256, 512, generator=g).to(torch.bfloat16).to("cuda:0")
+    w = torch.randn(128, 512, generator=g).to(torch.bfloat16).to("cuda:0")
+    dy = torch.randn(256, 128, generator=g).to(torch.bfloat16).to("cuda:0")
+    wref = w.clone().float().requires_grad_(True)
+    xref = x.clone().float().requires_grad_(True)
+    torch.nn.functional.linear(xref, wref).backward(dy.float())
+    err = lambda a, b: float(((a.detach().float() - b.detach().float()) ** 2).sum() / (b.detach().float() ** 2).sum())
+    errs = {}
+    for rr in ("signs", "O32"):
+        torch.manual_seed(1)
+        layer = production_layer(q, 512, 128, True, rr, torch.bfloat16)
+        with torch.no_grad():
+            layer.weight.copy_(w)
+        xin = x.clone().requires_grad_(True)
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            y = layer(xin)
+        y.backward(dy)
+        assert layer.backward_scheme.g_quantizer.is_dense == (rr == "O32")
+        errs[rr] = (err(xin.grad, xref.grad), err(layer.weight.grad, wref.grad))
+    print(f"relative squared gradient errors {errs}", flush=True)
+    for k in (0, 1):
+        assert 0.03 < errs["O32"][k] < 0.3 and abs(errs["O32"][k] - errs["signs"][k]) < 0.5 * errs["signs"][k]

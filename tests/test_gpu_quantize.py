@@ -183,6 +183,28 @@ def test_tiny_magnitudes_follow_the_definition(oracle, K, mode, transposed):
     _check(oracle, K, x, 32, MODES[mode], signs, transposed, None, 0xBEEF + int(transposed), f"tiny/{mode}/{transposed}")
 
 
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_already_rotated_input_passes_through(oracle, K, mode, dtype):
+    """hadamard_dim 1: the groups of 32 are quantized as they are (the caller applied a dense rotation)."""
+    print(f"case pass-through mode={mode} dtype={dtype}", flush=True)
+    x = make_input(40, 384, dtype, seed=31, zero_rows=1)
+    _check(oracle, K, x, 1, MODES[mode], None, False, None, 0xABCDEF + MODES[mode], f"pass-through/{mode}/{dtype}")
+
+
+def test_pass_through_rejections(K):
+    from quartet_amd._lib import QuartetHipError
+    dev = torch.device("cuda:0")
+    x = torch.zeros(32, 128, dtype=torch.bfloat16, device=dev)
+    u = torch.rand(32, 128, device=dev)
+    for kwargs in (dict(transposed_in=True), dict(u=u, mode=K.QM_ABSMAX_SR), dict(sign_bits=5), dict(tiled=True)):
+        with pytest.raises(QuartetHipError, match="hadamard_dim 1"):
+            K.quantize_mxfp4(x, 1, **{"sign_bits": None, "mode": K.QM_QUEST_RTN, **kwargs})
+    with pytest.raises(QuartetHipError):
+        K.requantize_transposed_mxfp4(torch.zeros(32, 64, dtype=torch.uint8, device=dev),
+                                      torch.zeros(32, 4, dtype=torch.uint8, device=dev), hadamard_dim=1)
+
+
 # Tiled code layout ([R/16][C/128][16][64 bytes]): the same bytes as the row-major codes, permuted; scales, mask
 # and the de-quantized tensor are unaffected.
 @pytest.mark.parametrize("mode", list(MODES))
