@@ -22,6 +22,9 @@
 //     both zeros into a negative denormal and changes no other value's code.
 // Outputs are one 16-byte code store, one scale byte and one mask dword per lane, all contiguous across
 // lanes; the input is read as 64 (bf16) or 128 (fp32) contiguous bytes per lane.
+// The tiled row-major, transposed and re-quantizing kernels are written as jobs (qm_jobs.h) so that the whole-layer
+// entry points can issue two of them in one grid.  rotate = false (row-major kernel only) skips the butterfly: the
+// caller has already applied a dense rotation.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
