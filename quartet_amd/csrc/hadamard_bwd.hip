@@ -18,6 +18,9 @@ namespace qm {
 
 namespace {
 
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ float dpp_quad_xor1(float v) {
     return u2f((uint32_t)__builtin_amdgcn_mov_dpp((int)f2u(v), 0xB1, 0xF, 0xF, true));
 }
@@ -32,11 +35,12 @@ __device__ __forceinline__ float lane_xor(float v) {
 }
 template <int LANE_MASK>
 __device__ __forceinline__ void cross_lane_stage(float (&v)[8], int lane_in_chunk) {
-    const bool upper = (lane_in_chunk & LANE_MASK) != 0;
+    // lower lane of a butterfly: own + partner; upper lane: partner - own = partner + (-own)
+    const uint32_t flip = (lane_in_chunk & LANE_MASK) ? 0x80000000u : 0u;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        float p = lane_xor<LANE_MASK>(v[i]);
-        v[i] = upper ? (p - v[i]) : (v[i] + p);
+        const float p = lane_xor<LANE_MASK>(v[i]);
+        v[i] = p + u2f(f2u(v[i]) ^ flip);
     }
 }
 
@@ -79,8 +83,10 @@ struct HadamardBwdJob {
         const uint32_t sign8 = (sb.w[j0 >> 5] >> (j0 & 31)) & 0xffu;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            float x = v[i] * (float)((keep >> i) & 1u);  // g * mask, as the reference multiplies
-            v[i] = ((sign8 >> i) & 1u) ? -x : x;
+            // g * mask as the reference multiplies: the factor is the float 1.0 or 0.0 built from the bit
+            const uint32_t all = (uint32_t)__builtin_amdgcn_sbfe((int)keep, i, 1);  // 0 or ~0
+            const float x = v[i] * u2f(all & 0x3f800000u);
+            v[i] = u2f(f2u(x) ^ (((sign8 >> i) & 1u) << 31));
         }
 #pragma unroll
         for (int h = 1; h < 8; h <<= 1) {
@@ -99,8 +105,11 @@ struct HadamardBwdJob {
         if constexpr (sizeof(TOut) == 2) {
             uint32_t w[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                w[i] = (uint32_t)f32_to_bf16(v[2 * i] * c) | ((uint32_t)f32_to_bf16(v[2 * i + 1] * c) << 16);
+            for (int i = 0; i < 4; ++i) {
+                // v_cvt_pk_bf16_f32: round to nearest even, the same rounding as f32_to_bf16
+                const v2bf p = __builtin_convertvector(v2f{v[2 * i] * c, v[2 * i + 1] * c}, v2bf);
+                w[i] = __builtin_bit_cast(uint32_t, p);
+            }
             *reinterpret_cast<uint4*>(out + octet * 8) = make_uint4(w[0], w[1], w[2], w[3]);
         } else {
             *reinterpret_cast<float4*>(out + octet * 8) = make_float4(v[0] * c, v[1] * c, v[2] * c, v[3] * c);
