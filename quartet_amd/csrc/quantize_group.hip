@@ -464,7 +464,8 @@ struct TransposedJob {
         constexpr int GPL = TrTile<T>::kGroupsPerLane;
         __shared__ uint4 ocodes[TQ * 4];      // [q][4 groups x 16 B]
         __shared__ uint32_t oscales[TQ];      // [q][4 B]
-        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const int tid = threadIdx.x, lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // tells the compiler it is wave-uniform
         const unsigned bq = bid / grid_p;
         const int64_t p0 = (int64_t)(bid - bq * grid_p) * kTrP, q0 = (int64_t)bq * TQ;
         const int64_t pbase = p0 + wave * 32;       // this wave's group along p
@@ -472,11 +473,12 @@ struct TransposedJob {
         const bool active = pbase < P && qa < Q;    // P % 32 == 0 and Q % 8 == 0: all of a lane's groups or none
         if (active) {
             float v[GPL][32];
-            const uint32_t* src = reinterpret_cast<const uint32_t*>(x + pbase * Q + qa);
+            // uniform row pointers (scalar unit) + the lane's 32-bit dword offset: no per-lane 64-bit address math
+            const uint32_t* row = reinterpret_cast<const uint32_t*>(x + pbase * Q + q0);
             const int64_t row_dw = Q * (int64_t)sizeof(T) / 4;
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
-                const uint32_t w = src[i * row_dw];
+                const uint32_t w = (row + i * row_dw)[(uint32_t)lane];
                 if constexpr (sizeof(T) == 2) {
                     v[0][i] = u2f(w << 16);
                     v[1][i] = u2f(w & 0xffff0000u);
@@ -553,7 +555,8 @@ struct RequantJob {
         using T = typename std::conditional<VAL_DTYPE == BF16, uint16_t, float>::type;
         __shared__ uint4 ocodes[kRqC * 4];
         __shared__ uint32_t oscales[kRqC];
-        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const int tid = threadIdx.x, lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // tells the compiler it is wave-uniform
         const unsigned bc = bid / grid_r;
         const int64_t r0 = (int64_t)(bid - bc * grid_r) * kRqR, c0 = (int64_t)bc * kRqC;
         const int64_t in_code_pitch = C / 2, in_scale_pitch = C / 32;
@@ -562,17 +565,19 @@ struct RequantJob {
         const bool active = rbase < R && ca < C;     // C % 32 == 0: both columns of the pair or none
         if (active) {
             float v[2][32];
-            // tiled input: the lane's byte column sits at offset `lane` of the 64-byte rows of column block c0/128
-            const uint8_t* cp = tiled_in ? codes_in + tiled_code_offset(rbase, c0 / 128, C / 128) + lane
-                                         : codes_in + rbase * in_code_pitch + ca / 2;
+            // Uniform row pointers (scalar unit) + the lane's 32-bit byte offset: no per-lane 64-bit address math.
+            // Tiled input: the lane's byte column sits at offset `lane` of the 64-byte rows of column block c0/128.
+            const uint8_t* cu = tiled_in ? codes_in + tiled_code_offset(rbase, c0 / 128, C / 128)
+                                         : codes_in + rbase * in_code_pitch + c0 / 2;
             const int64_t row_step = tiled_in ? 64 : in_code_pitch;                            // next row of a 16-row block
             const int64_t block_step = tiled_in ? (C / 128) * 1024 - 16 * 64 : 0;              // extra hop into the next block
-            const uint8_t* sp = scales_in + rbase * in_scale_pitch + ca / 32;
+            const uint8_t* su = scales_in + rbase * in_scale_pitch + c0 / 32;
+            const uint32_t sl = (uint32_t)lane >> 4;  // which of the workgroup's four column groups the lane is in
             uint32_t byte[32], sbyte[32];
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
-                byte[i] = cp[i * row_step + (i >> 4) * block_step];
-                sbyte[i] = sp[i * in_scale_pitch];
+                byte[i] = (cu + i * row_step + (i >> 4) * block_step)[(uint32_t)lane];
+                sbyte[i] = (su + i * in_scale_pitch)[sl];
             }
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
