@@ -122,10 +122,17 @@ int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, 
  * Whole-layer entry points: one call issues every launch of a Quartet linear's forward or backward pass (the
  * per-kernel entry points above, in order), so the host pays one foreign call instead of three / eight.
  *
+ * A packed operand is one caller-owned, 256-byte aligned buffer of qm_packed_operand_bytes(rows, cols) bytes holding,
+ * at the offsets qm_packed_operand_offsets reports, the codes [rows, cols/2], E8M0 scales [rows, cols/32] and
+ * clip-mask bits [rows, cols/8] of a quantized [rows, cols] tensor -- the three tensors per operand that
+ * notebooks/benchmark_mxfp4.ipynb's CudaGemm keeps for backward (ctx.save_for_backward in its forward).
+ *
  * qm_linear_forward = QuestMXFP4QuantizerFn.forward on x and W (quantizers/mxfp4.py:129-140) followed by
  * QEQWtt_QEtQXttFn.forward (src/models/quantization/backward.py:59-62):
- *   x [T, I], w [O, I] -> y [T, O] = Q(x) Q(w)^T; `saved` (qm_linear_saved_bytes(T, I, O) bytes, 256-byte
- *   aligned, caller-owned) receives the packed operands and clip-mask bits the backward pass needs.
+ *   x [T, I], w [O, I] -> y [T, O] = Q(x) Q(w)^T; packed_x ([T, I]) and packed_w ([O, I]) receive the packed
+ *   operands the backward pass needs.  w_is_packed != 0: packed_w already holds Q(w) from an earlier call with the
+ *   same w, signs and layout, and w is not read (W changes only at the optimizer step, src/optim/base.py:188-207,
+ *   so the micro-steps of a gradient accumulation quantize it once).
  * qm_linear_backward = QEQWtt_QEtQXttFn.backward (backward.py:64-85) with the straight-through backward of both
  * forward quantizers (mxfp4.py:143-146) applied: e [T, O] -> gx [T, I], gw [O, I], both of mid_dtype.
  *   g_mode            QM_ABSMAX_SR or QM_ABSMAX_RTN (AlbertTsengQuantizer stochastic or not)
@@ -136,19 +143,17 @@ int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, 
  * codes_layout applies to every packed tensor inside; QM_LAYOUT_TILED needs T, I, O multiples of 128 and at
  * least 256, and all Hadamard blocks 32.  T, I, O must be multiples of 32 for the backward pass.
  */
-size_t qm_linear_saved_bytes(int64_t T, int64_t I, int64_t O);
-/* Byte offsets inside `saved` of, in this order: x codes [T, I/2], x scales [T, I/32], x mask bits [T, I/8], w codes
- * [O, I/2], w scales [O, I/32], w mask bits [O, I/8] -- the tensors notebooks/benchmark_mxfp4.ipynb's CudaGemm keeps
- * for backward (ctx.save_for_backward in its forward).  `offsets` is a HOST array of six; returns 0, or
- * QM_ERR_INVALID for extents qm_linear_saved_bytes rejects. */
-int qm_linear_saved_offsets(int64_t T, int64_t I, int64_t O, size_t* offsets);
+size_t qm_packed_operand_bytes(int64_t rows, int64_t cols);
+/* offsets: HOST array of three (codes, scales, mask bits); returns 0, or QM_ERR_INVALID unless cols % 32 == 0 */
+int qm_packed_operand_offsets(int64_t rows, int64_t cols, size_t* offsets);
 size_t qm_linear_backward_workspace_bytes(int64_t T, int64_t I, int64_t O, int mid_dtype);
 int qm_linear_forward(const void* x, int x_dtype, const void* w, int w_dtype, int64_t T, int64_t I, int64_t O,
-                      int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, void* saved,
-                      size_t saved_bytes, void* y, int y_dtype, int codes_layout, void* stream);
-int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t O, const void* saved, int hd_x,
-                       const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, int hd_g,
-                       const uint32_t* signs_g, int g_mode, const uint64_t* seeds, int x_val_dtype,
+                      int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, void* packed_x,
+                      size_t packed_x_bytes, void* packed_w, size_t packed_w_bytes, int w_is_packed, void* y,
+                      int y_dtype, int codes_layout, void* stream);
+int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t O, const void* packed_x,
+                       const void* packed_w, int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w,
+                       int hd_g, const uint32_t* signs_g, int g_mode, const uint64_t* seeds, int x_val_dtype,
                        int w_val_dtype, int mid_dtype, int x_scale_dtype, int w_scale_dtype, void* workspace,
                        size_t workspace_bytes, void* gx, void* gw, int codes_layout, void* stream);
 

@@ -21,8 +21,8 @@ EXPORTS = (
     "qm_masked_hadamard_bwd",
     "qm_dequantize_mxfp4",
     "qm_gemm_workspace_bytes",
-    "qm_linear_saved_bytes",
-    "qm_linear_saved_offsets",
+    "qm_packed_operand_bytes",
+    "qm_packed_operand_offsets",
     "qm_linear_backward_workspace_bytes",
     "qm_linear_forward",
     "qm_linear_backward",
@@ -62,16 +62,16 @@ def lib():
     L.qm_dequantize_mxfp4.restype = i32
     L.qm_dequantize_mxfp4.argtypes = [vp, vp, i64, i64, f32, vp, i32, vp]
     sz = ctypes.c_size_t
-    L.qm_linear_saved_bytes.restype = sz
-    L.qm_linear_saved_bytes.argtypes = [i64, i64, i64]
-    L.qm_linear_saved_offsets.restype = i32
-    L.qm_linear_saved_offsets.argtypes = [i64, i64, i64, ctypes.POINTER(sz)]
+    L.qm_packed_operand_bytes.restype = sz
+    L.qm_packed_operand_bytes.argtypes = [i64, i64]
+    L.qm_packed_operand_offsets.restype = i32
+    L.qm_packed_operand_offsets.argtypes = [i64, i64, ctypes.POINTER(sz)]
     L.qm_linear_backward_workspace_bytes.restype = sz
     L.qm_linear_backward_workspace_bytes.argtypes = [i64, i64, i64, i32]
     L.qm_linear_forward.restype = i32
-    L.qm_linear_forward.argtypes = [vp, i32, vp, i32, i64, i64, i64, i32, vp, i32, vp, vp, sz, vp, i32, i32, vp]
+    L.qm_linear_forward.argtypes = [vp, i32, vp, i32, i64, i64, i64, i32, vp, i32, vp, vp, sz, vp, sz, i32, vp, i32, i32, vp]
     L.qm_linear_backward.restype = i32
-    L.qm_linear_backward.argtypes = [vp, i32, i64, i64, i64, vp, i32, vp, i32, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32,
+    L.qm_linear_backward.argtypes = [vp, i32, i64, i64, i64, vp, vp, i32, vp, i32, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32,
                                      vp, sz, vp, vp, i32, vp]
     _lib = L
     return L

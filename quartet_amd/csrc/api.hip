@@ -42,7 +42,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 2; }
+int qm_version(void) { return 3; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -161,18 +161,16 @@ namespace {
 size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
 size_t esize(int dtype) { return dtype == QM_BF16 ? 2 : 4; }
 
-struct SavedLayout {
-    size_t xc, xs, xm, wc, ws, wm, total;
+// one packed operand: codes, scales, mask bits, each region 256-byte aligned
+struct PackedLayout {
+    size_t c, s, m, total;
 };
-SavedLayout saved_layout(int64_t T, int64_t I, int64_t O) {
-    SavedLayout l;
+PackedLayout packed_layout(int64_t rows, int64_t cols) {
+    PackedLayout l;
     size_t o = 0;
-    l.xc = o; o += up256((size_t)T * I / 2);
-    l.xs = o; o += up256((size_t)T * I / 32);
-    l.xm = o; o += up256((size_t)T * I / 8);
-    l.wc = o; o += up256((size_t)O * I / 2);
-    l.ws = o; o += up256((size_t)O * I / 32);
-    l.wm = o; o += up256((size_t)O * I / 8);
+    l.c = o; o += up256((size_t)rows * cols / 2);
+    l.s = o; o += up256((size_t)rows * cols / 32);
+    l.m = o; o += up256((size_t)rows * cols / 8);
     l.total = o;
     return l;
 }
@@ -206,16 +204,17 @@ bool pair_launches(int codes_layout, int64_t T, int64_t I, int64_t O, int hd_a, 
 }
 }  // namespace
 
-size_t qm_linear_saved_bytes(int64_t T, int64_t I, int64_t O) {
-    if (T < 0 || I < 0 || O < 0 || I % 32) return 0;
-    return saved_layout(T, I, O).total;
+size_t qm_packed_operand_bytes(int64_t rows, int64_t cols) {
+    if (rows < 0 || cols < 0 || cols % 32) return 0;
+    return packed_layout(rows, cols).total;
 }
 
-int qm_linear_saved_offsets(int64_t T, int64_t I, int64_t O, size_t* offsets) {
-    if (T < 0 || I < 0 || O < 0 || I % 32 || !offsets) return fail(QM_ERR_INVALID, "qm_linear_saved_offsets: bad extents or null array");
-    const SavedLayout l = saved_layout(T, I, O);
-    offsets[0] = l.xc; offsets[1] = l.xs; offsets[2] = l.xm;
-    offsets[3] = l.wc; offsets[4] = l.ws; offsets[5] = l.wm;
+int qm_packed_operand_offsets(int64_t rows, int64_t cols, size_t* offsets) {
+    if (rows < 0 || cols < 0 || cols % 32 || !offsets)
+        return fail(QM_ERR_INVALID, "qm_packed_operand_offsets: need cols %% 32 == 0 and a non-null array (rows=%lld cols=%lld)",
+                    (long long)rows, (long long)cols);
+    const PackedLayout l = packed_layout(rows, cols);
+    offsets[0] = l.c; offsets[1] = l.s; offsets[2] = l.m;
     return 0;
 }
 
@@ -225,37 +224,43 @@ size_t qm_linear_backward_workspace_bytes(int64_t T, int64_t I, int64_t O, int m
 }
 
 int qm_linear_forward(const void* x, int x_dtype, const void* w, int w_dtype, int64_t T, int64_t I, int64_t O, int hd_x,
-                      const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, void* saved, size_t saved_bytes, void* y,
-                      int y_dtype, int codes_layout, void* stream) {
+                      const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, void* packed_x, size_t packed_x_bytes,
+                      void* packed_w, size_t packed_w_bytes, int w_is_packed, void* y, int y_dtype, int codes_layout,
+                      void* stream) {
     if (T < 0 || I < 0 || O < 0) return fail(QM_ERR_INVALID, "qm_linear_forward: negative extent");
     if (T == 0 || O == 0 || I == 0) return 0;
     if (I % 32) return fail(QM_ERR_INVALID, "qm_linear_forward: in_features %lld not a multiple of 32", (long long)I);
-    const SavedLayout l = saved_layout(T, I, O);
-    if (!saved || saved_bytes < l.total || !aligned(saved, 256))
-        return fail(QM_ERR_INVALID, "qm_linear_forward: saved buffer needs %zu bytes, 256-byte aligned", l.total);
-    uint8_t* s = static_cast<uint8_t*>(saved);
+    const PackedLayout lx = packed_layout(T, I), lw = packed_layout(O, I);
+    if (!packed_x || packed_x_bytes < lx.total || !aligned(packed_x, 256) || !packed_w || packed_w_bytes < lw.total ||
+        !aligned(packed_w, 256))
+        return fail(QM_ERR_INVALID, "qm_linear_forward: packed operand buffers need %zu and %zu bytes, 256-byte aligned", lx.total,
+                    lw.total);
+    uint8_t* px = static_cast<uint8_t*>(packed_x);
+    uint8_t* pw = static_cast<uint8_t*>(packed_w);
     int rc;
-    if (pair_launches(codes_layout, T, I, O, hd_x, hd_w, 32) && x && w && y && valid_dtype(x_dtype) && valid_dtype(w_dtype) &&
-        aligned(x, 16) && aligned(w, 16)) {
+    if (!w_is_packed && pair_launches(codes_layout, T, I, O, hd_x, hd_w, 32) && x && w && y && valid_dtype(x_dtype) &&
+        valid_dtype(w_dtype) && aligned(x, 16) && aligned(w, 16)) {
         // both forward quantizers in one grid
-        const qm::RowmajorArgs ax{x, x_dtype, T, I, signs_x ? signs_x[0] : 0u, s + l.xc, s + l.xs, s + l.xm};
-        const qm::RowmajorArgs aw{w, w_dtype, O, I, signs_w ? signs_w[0] : 0u, s + l.wc, s + l.ws, s + l.wm};
+        const qm::RowmajorArgs ax{x, x_dtype, T, I, signs_x ? signs_x[0] : 0u, px + lx.c, px + lx.s, px + lx.m};
+        const qm::RowmajorArgs aw{w, w_dtype, O, I, signs_w ? signs_w[0] : 0u, pw + lw.c, pw + lw.s, pw + lw.m};
         rc = from_hip(qm::quantize_rowmajor_hd32_tiled_pair(ax, aw, reinterpret_cast<hipStream_t>(stream)), "qm_linear_forward");
         if (rc) return rc;
     } else {
-        rc = qm_quantize_mxfp4(x, x_dtype, T, I, hd_x, signs_x, QM_QUEST_RTN, 0, nullptr, 0, s + l.xc, s + l.xs, s + l.xm, nullptr,
+        rc = qm_quantize_mxfp4(x, x_dtype, T, I, hd_x, signs_x, QM_QUEST_RTN, 0, nullptr, 0, px + lx.c, px + lx.s, px + lx.m, nullptr,
                                codes_layout, stream);
         if (rc) return rc;
-        rc = qm_quantize_mxfp4(w, w_dtype, O, I, hd_w, signs_w, QM_QUEST_RTN, 0, nullptr, 0, s + l.wc, s + l.ws, s + l.wm, nullptr,
-                               codes_layout, stream);
-        if (rc) return rc;
+        if (!w_is_packed) {
+            rc = qm_quantize_mxfp4(w, w_dtype, O, I, hd_w, signs_w, QM_QUEST_RTN, 0, nullptr, 0, pw + lw.c, pw + lw.s, pw + lw.m,
+                                   nullptr, codes_layout, stream);
+            if (rc) return rc;
+        }
     }
-    return qm_gemm_mxfp4_tn(s + l.xc, s + l.xs, s + l.wc, s + l.ws, T, O, I, 1.0f, y, y_dtype, codes_layout, codes_layout, nullptr, 0,
-                            stream);
+    return qm_gemm_mxfp4_tn(px + lx.c, px + lx.s, pw + lw.c, pw + lw.s, T, O, I, 1.0f, y, y_dtype, codes_layout, codes_layout, nullptr,
+                            0, stream);
 }
 
-int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t O, const void* saved, int hd_x,
-                       const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, int hd_g, const uint32_t* signs_g,
+int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t O, const void* packed_x, const void* packed_w,
+                       int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, int hd_g, const uint32_t* signs_g,
                        int g_mode, const uint64_t* seeds, int x_val_dtype, int w_val_dtype, int mid_dtype, int x_scale_dtype,
                        int w_scale_dtype, void* workspace, size_t workspace_bytes, void* gx, void* gw, int codes_layout,
                        void* stream) {
@@ -267,12 +272,14 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
     if (I % 32 || O % 32 || T % 32)
         return fail(QM_ERR_INVALID, "qm_linear_backward: tokens, in_features and out_features must be multiples of 32 (T=%lld I=%lld O=%lld)",
                     (long long)T, (long long)I, (long long)O);
-    if (!seeds || !saved || !aligned(saved, 256)) return fail(QM_ERR_INVALID, "qm_linear_backward: null seeds or saved buffer");
-    const SavedLayout sl = saved_layout(T, I, O);
+    if (!seeds || !packed_x || !aligned(packed_x, 256) || !packed_w || !aligned(packed_w, 256))
+        return fail(QM_ERR_INVALID, "qm_linear_backward: null seeds or packed operand buffers");
+    const PackedLayout lx = packed_layout(T, I), lw = packed_layout(O, I);
     const WorkLayout wl = work_layout(T, I, O, mid_dtype);
     if (!workspace || workspace_bytes < wl.total || !aligned(workspace, 256))
         return fail(QM_ERR_INVALID, "qm_linear_backward: workspace needs %zu bytes, 256-byte aligned", wl.total);
-    const uint8_t* s = static_cast<const uint8_t*>(saved);
+    const uint8_t* px = static_cast<const uint8_t*>(packed_x);
+    const uint8_t* pw = static_cast<const uint8_t*>(packed_w);
     uint8_t* k = static_cast<uint8_t*>(workspace);
     // value = code * 2^k * fl32(4/3) on both operands of the two gradient products
     const float d = (float)(1.0 / 0.75);
@@ -288,8 +295,8 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
         rc = from_hip(qm::quantize_both_orientations_hd32_tiled(e, e_dtype, T, O, sg, g_mode, seeds[0], seeds[2], k + wl.ec, k + wl.es,
                                                                 k + wl.etc, k + wl.ets, hs), "qm_linear_backward");
         if (rc) return rc;
-        const qm::RequantArgs rw{s + sl.wc, s + sl.ws, O, I, w_val_dtype, seeds[1], k + wl.wtc, k + wl.wts};
-        const qm::RequantArgs rx{s + sl.xc, s + sl.xs, T, I, x_val_dtype, seeds[3], k + wl.xtc, k + wl.xts};
+        const qm::RequantArgs rw{pw + lw.c, pw + lw.s, O, I, w_val_dtype, seeds[1], k + wl.wtc, k + wl.wts};
+        const qm::RequantArgs rx{px + lx.c, px + lx.s, T, I, x_val_dtype, seeds[3], k + wl.xtc, k + wl.xts};
         rc = from_hip(qm::requantize_transposed_hd32_tiled_pair(rx, rw, sg, g_mode, hs), "qm_linear_backward");
         if (rc) return rc;
         rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, k + wl.gxq, mid_dtype, codes_layout,
@@ -299,14 +306,14 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                               codes_layout, gws, wl.gemm_ws_bytes, stream);
         if (rc) return rc;
         return from_hip(qm::masked_hadamard_bwd_hd32_pair(k + wl.gxq, T * I, x_scale_dtype,
-                                                          signs_x ? signs_x[0] : 0u, s + sl.xm, gx, k + wl.gwq, O * I,
+                                                          signs_x ? signs_x[0] : 0u, px + lx.m, gx, k + wl.gwq, O * I,
                                                           w_scale_dtype, signs_w ? signs_w[0] : 0u,
-                                                          s + sl.wm, gw, mid_dtype, hs), "qm_linear_backward");
+                                                          pw + lw.m, gw, mid_dtype, hs), "qm_linear_backward");
     }
     rc = qm_quantize_mxfp4(e, e_dtype, T, O, hd_g, signs_g, g_mode, 0, nullptr, seeds[0], k + wl.ec, k + wl.es, nullptr, nullptr,
                            codes_layout, stream);
     if (rc) return rc;
-    rc = qm_requantize_transposed_mxfp4(s + sl.wc, s + sl.ws, O, I, 1.0f, w_val_dtype, hd_g, signs_g, g_mode, nullptr, seeds[1],
+    rc = qm_requantize_transposed_mxfp4(pw + lw.c, pw + lw.s, O, I, 1.0f, w_val_dtype, hd_g, signs_g, g_mode, nullptr, seeds[1],
                                         k + wl.wtc, k + wl.wts, nullptr, codes_layout, codes_layout, stream);
     if (rc) return rc;
     rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, k + wl.gxq, mid_dtype, codes_layout,
@@ -315,15 +322,15 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
     rc = qm_quantize_mxfp4(e, e_dtype, O, T, hd_g, signs_g, g_mode, 1, nullptr, seeds[2], k + wl.etc, k + wl.ets, nullptr, nullptr,
                            codes_layout, stream);
     if (rc) return rc;
-    rc = qm_requantize_transposed_mxfp4(s + sl.xc, s + sl.xs, T, I, 1.0f, x_val_dtype, hd_g, signs_g, g_mode, nullptr, seeds[3],
+    rc = qm_requantize_transposed_mxfp4(px + lx.c, px + lx.s, T, I, 1.0f, x_val_dtype, hd_g, signs_g, g_mode, nullptr, seeds[3],
                                         k + wl.xtc, k + wl.xts, nullptr, codes_layout, codes_layout, stream);
     if (rc) return rc;
     rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, k + wl.gwq, mid_dtype, codes_layout,
                           codes_layout, gws, wl.gemm_ws_bytes, stream);
     if (rc) return rc;
-    rc = qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, s + sl.xm, gx, mid_dtype, stream);
+    rc = qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, px + lx.m, gx, mid_dtype, stream);
     if (rc) return rc;
-    return qm_masked_hadamard_bwd(k + wl.gwq, mid_dtype, O, I, hd_w, w_scale_dtype, signs_w, s + sl.wm, gw, mid_dtype, stream);
+    return qm_masked_hadamard_bwd(k + wl.gwq, mid_dtype, O, I, hd_w, w_scale_dtype, signs_w, pw + lw.m, gw, mid_dtype, stream);
 }
 
 }  // extern "C"

@@ -145,28 +145,37 @@ def dequantize_mxfp4(codes, scales, post=1.0, out_dtype=torch.float32):
     return out
 
 
-def linear_forward(x2, w2, hd_x, signs_x, hd_w, signs_w, out_dtype, tiled):
+def packed_operand_buffer(rows, cols, device):
+    """Uninitialised byte buffer for one packed operand (codes, scales, mask bits of a [rows, cols] tensor)."""
+    return torch.empty(_lib.lib().qm_packed_operand_bytes(rows, cols), dtype=torch.uint8, device=device)
+
+
+def linear_forward(x2, w2, hd_x, signs_x, hd_w, signs_w, out_dtype, tiled, packed_w=None):
     """Whole forward pass of a Quartet linear in one foreign call: quantize x [T,I] and w [O,I] (quest RTN + clip
-    mask), y = Q(x) Q(w)^T.  Returns (y [T,O], saved) where `saved` is the byte buffer the backward pass reads."""
-    _require_cuda(x2, w2)
+    mask), y = Q(x) Q(w)^T.  Returns (y [T,O], packed_x, packed_w): the byte buffers the backward pass reads.  A
+    `packed_w` that an earlier call with the same weight, signs and layout returned is reused instead of quantizing
+    the weight again."""
+    _require_cuda(x2, w2, packed_w)
     assert x2.is_contiguous() and w2.is_contiguous()
     T, I = x2.shape
     O = w2.shape[0]
     L = _lib.lib()
-    nbytes = L.qm_linear_saved_bytes(T, I, O)
-    saved = torch.empty(nbytes, dtype=torch.uint8, device=x2.device)
+    packed_x = packed_operand_buffer(T, I, x2.device)
+    reuse = packed_w is not None
+    if not reuse:
+        packed_w = packed_operand_buffer(O, I, x2.device)
     y = torch.empty((T, O), dtype=out_dtype, device=x2.device)
     rc = L.qm_linear_forward(_ptr(x2), _dtype_code(x2.dtype), _ptr(w2), _dtype_code(w2.dtype), T, I, O, hd_x,
-                             sign_words(signs_x), hd_w, sign_words(signs_w), _ptr(saved), nbytes, _ptr(y),
-                             _dtype_code(out_dtype), _layout(tiled), _stream())
+                             sign_words(signs_x), hd_w, sign_words(signs_w), _ptr(packed_x), packed_x.numel(), _ptr(packed_w),
+                             packed_w.numel(), int(reuse), _ptr(y), _dtype_code(out_dtype), _layout(tiled), _stream())
     _lib.check(rc, "qm_linear_forward")
-    return y, saved
+    return y, packed_x, packed_w
 
 
-def linear_backward(e2, saved, T, I, O, hd_x, signs_x, hd_w, signs_w, hd_g, signs_g, mode, seeds, x_val_dtype, w_val_dtype,
-                    mid_dtype, x_scale_dtype, w_scale_dtype, tiled):
+def linear_backward(e2, packed_x, packed_w, T, I, O, hd_x, signs_x, hd_w, signs_w, hd_g, signs_g, mode, seeds, x_val_dtype,
+                    w_val_dtype, mid_dtype, x_scale_dtype, w_scale_dtype, tiled):
     """Whole backward pass in one foreign call: e [T,O] -> (gx [T,I], gw [O,I]) of mid_dtype."""
-    _require_cuda(e2, saved)
+    _require_cuda(e2, packed_x, packed_w)
     assert e2.is_contiguous() and e2.shape == (T, O)
     L = _lib.lib()
     mid = _dtype_code(mid_dtype)
@@ -174,8 +183,8 @@ def linear_backward(e2, saved, T, I, O, hd_x, signs_x, hd_w, signs_w, hd_g, sign
     work = torch.empty(nbytes, dtype=torch.uint8, device=e2.device)
     gx = torch.empty((T, I), dtype=mid_dtype, device=e2.device)
     gw = torch.empty((O, I), dtype=mid_dtype, device=e2.device)
-    rc = L.qm_linear_backward(_ptr(e2), _dtype_code(e2.dtype), T, I, O, _ptr(saved), hd_x, sign_words(signs_x), hd_w,
-                              sign_words(signs_w), hd_g, sign_words(signs_g), mode, (ctypes.c_uint64 * 4)(*seeds),
+    rc = L.qm_linear_backward(_ptr(e2), _dtype_code(e2.dtype), T, I, O, _ptr(packed_x), _ptr(packed_w), hd_x, sign_words(signs_x),
+                              hd_w, sign_words(signs_w), hd_g, sign_words(signs_g), mode, (ctypes.c_uint64 * 4)(*seeds),
                               _dtype_code(x_val_dtype), _dtype_code(w_val_dtype), mid, _dtype_code(x_scale_dtype),
                               _dtype_code(w_scale_dtype), _ptr(work), nbytes, _ptr(gx), _ptr(gw), _layout(tiled), _stream())
     _lib.check(rc, "qm_linear_backward")

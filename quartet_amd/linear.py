@@ -25,7 +25,7 @@ class QuartetLinearFn(torch.autograd.Function):
               B7/B8 masked inverse rotation (straight-through estimators of F1/F2)."""
 
     @staticmethod
-    def forward(ctx, x, weight, a_q, w_q, g_q):
+    def forward(ctx, x, weight, a_q, w_q, g_q, weight_cache):
         in_features = weight.shape[1]
         x2 = x.reshape(-1, in_features).contiguous()
         w2 = weight.contiguous()
@@ -34,8 +34,14 @@ class QuartetLinearFn(torch.autograd.Function):
         # all three extents multiples of 128 and at least 256, Hadamard block 32 throughout; row-major codes otherwise.
         tiled = (all(d % 128 == 0 and d >= 256 for d in (x2.shape[0], in_features, weight.shape[0])) and
                  a_q.hadamard_dim == 32 and w_q.hadamard_dim == 32 and g_q.hadamard_dim == 32)
-        y, saved = K.linear_forward(x2, w2, a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits, out_dtype, tiled)
-        ctx.save_for_backward(saved)
+        # Q(W) of an unchanged weight (the micro-steps of one accumulation) is quantized once and kept by the layer
+        key = (weight.data_ptr(), weight._version, weight.dtype, tuple(weight.shape), w_q.hadamard_dim, w_q.sign_bits, tiled)
+        packed_w = weight_cache.get(key) if weight_cache is not None else None
+        y, packed_x, packed_w = K.linear_forward(x2, w2, a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits,
+                                                 out_dtype, tiled, packed_w)
+        if weight_cache is not None:
+            weight_cache.put(key, packed_w)
+        ctx.save_for_backward(packed_x, packed_w)
         ctx.g_q = g_q
         ctx.tiled = tiled
         ctx.fwd = (a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits)
@@ -45,7 +51,7 @@ class QuartetLinearFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, e):
-        (saved,) = ctx.saved_tensors
+        packed_x, packed_w = ctx.saved_tensors
         g_q = ctx.g_q
         a_hd, a_signs, w_hd, w_signs = ctx.fwd
         T, I, O = ctx.dims
@@ -59,9 +65,48 @@ class QuartetLinearFn(torch.autograd.Function):
         mid_dtype = torch.bfloat16 if low else e2.dtype
         sd_x = torch.bfloat16 if low else ctx.x_dtype
         sd_w = torch.bfloat16 if low else ctx.w_dtype
-        gx, gw = K.linear_backward(e2, saved, T, I, O, a_hd, a_signs, w_hd, w_signs, hd, signs, mode, seeds, ctx.x_dtype,
+        gx, gw = K.linear_backward(e2, packed_x, packed_w, T, I, O, a_hd, a_signs, w_hd, w_signs, hd, signs, mode, seeds, ctx.x_dtype,
                                    ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled)
-        return gx.to(ctx.x_dtype).view(ctx.x_shape), gw.to(ctx.w_dtype), None, None, None
+        return gx.to(ctx.x_dtype).view(ctx.x_shape), gw.to(ctx.w_dtype), None, None, None, None
+
+
+class PackedWeightCache:
+    """The packed Q(W) of a layer's current weight, kept across the micro-steps of one gradient accumulation (the
+    weight changes only at the optimizer step, src/optim/base.py:188-207 of the reference).  One entry, replaced --
+    never overwritten in place, so that a graph built earlier keeps the buffer it saved -- when the weight's storage,
+    version counter, rotation or code layout changes.  An update that bypasses the version counter (``weight.data``
+    arithmetic) is invisible to the key: whoever steps the optimizer calls ``invalidate_packed_weights`` afterwards,
+    as ``quartet_amd.train.train`` does, and the cache is off unless ``enable_packed_weight_cache`` turned it on."""
+
+    def __init__(self):
+        self.key, self.buffer, self.hits, self.misses = None, None, 0, 0
+
+    def get(self, key):
+        if key == self.key:
+            self.hits += 1
+            return self.buffer
+        self.misses += 1
+        return None
+
+    def put(self, key, buffer):
+        self.key, self.buffer = key, buffer
+
+    def clear(self):
+        self.key, self.buffer = None, None
+
+
+def enable_packed_weight_cache(model, enabled=True):
+    """Give every QuantizedLinear of `model` a PackedWeightCache (or remove it)."""
+    for m in model.modules():
+        if isinstance(m, QuantizedLinear):
+            m.packed_weight_cache = PackedWeightCache() if enabled else None
+
+
+def invalidate_packed_weights(model):
+    """Forget every cached Q(W): call after anything that changes the weights (the optimizer step)."""
+    for m in model.modules():
+        if isinstance(m, QuantizedLinear) and m.packed_weight_cache is not None:
+            m.packed_weight_cache.clear()
 
 
 class QuantizedLinear(nn.Linear):
@@ -84,6 +129,7 @@ class QuantizedLinear(nn.Linear):
         self.backward_scheme = backward_scheme
         self.backward_scheme.g_quantizer = gradient_quantizer
         self.use_packed_path = True
+        self.packed_weight_cache = None  # see enable_packed_weight_cache
 
     def _is_production_config(self):
         g_q = self.backward_scheme.g_quantizer
@@ -99,7 +145,7 @@ class QuantizedLinear(nn.Linear):
     def forward(self, x):
         if self._is_production_config():
             return QuartetLinearFn.apply(x, self.weight, self.activation_quantizer, self.weight_quantizer,
-                                         self.backward_scheme.g_quantizer)
+                                         self.backward_scheme.g_quantizer, self.packed_weight_cache)
         xq = self.activation_quantizer(x)
         wq = self.weight_quantizer(self.weight)
         return self.backward_scheme(xq, wq)

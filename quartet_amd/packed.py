@@ -129,22 +129,16 @@ def pack_absmax(x, hadamard_dim=32, sign_bits=0, stochastic=False, seed=0, tiled
                         sign_bits, "absmax")
 
 
-def from_linear_saved(saved, tokens, in_features, out_features, tiled, activation_quantizer, weight_quantizer):
-    """The packed activations and weight inside the byte buffer that ``kernels.linear_forward`` returns
-    (views, no copy): what the layer keeps for its backward pass."""
-    off = (ctypes.c_size_t * 6)()
-    _lib.check(_lib.lib().qm_linear_saved_offsets(tokens, in_features, out_features, off), "qm_linear_saved_offsets")
+def from_operand_buffer(buffer, rows, cols, tiled, quantizer):
+    """The packed tensor inside one of the byte buffers that ``kernels.linear_forward`` returns (views, no copy): what
+    the layer keeps of x or of W for its backward pass.  `quantizer` is the forward quantizer that produced it."""
+    off = (ctypes.c_size_t * 3)()
+    _lib.check(_lib.lib().qm_packed_operand_offsets(rows, cols, off), "qm_packed_operand_offsets")
 
-    def view(start, rows, width):
-        return saved[start:start + rows * width].view(rows, width)
-    layout = "tiled" if tiled else "rowmajor"
-    I = in_features
-    xp = PackedTensor(view(off[0], tokens, I // 2), view(off[1], tokens, I // 32), view(off[2], tokens, I // 8), tokens, I,
-                      layout, activation_quantizer.hadamard_dim, activation_quantizer.sign_bits, "quest")
-    wp = PackedTensor(view(off[3], out_features, I // 2), view(off[4], out_features, I // 32),
-                      view(off[5], out_features, I // 8), out_features, I, layout, weight_quantizer.hadamard_dim,
-                      weight_quantizer.sign_bits, "quest")
-    return xp, wp
+    def view(start, width):
+        return buffer[start:start + rows * width].view(rows, width)
+    return PackedTensor(view(off[0], cols // 2), view(off[1], cols // 32), view(off[2], cols // 8), rows, cols,
+                        "tiled" if tiled else "rowmajor", quantizer.hadamard_dim, quantizer.sign_bits, "quest")
 
 
 def save_packed(path, tensors: Dict[str, PackedTensor], extra_metadata: Optional[Dict[str, str]] = None):

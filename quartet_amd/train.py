@@ -6,7 +6,8 @@ src/models/base.py:313-360 of the reference):
   * every micro-step runs the forward pass *and* ``loss.backward()`` under bf16 autocast (the backward-side
     quantizers rely on it: gradients reach them in bf16 and their rotations run in bf16), with the loss divided by
     the number of accumulation steps;
-  * the weights of a step are constant across its micro-steps: ``opt.step()`` comes after the last of them, preceded
+  * the weights of a step are constant across its micro-steps (so each quantized linear quantizes its weight once per
+    iteration, not once per micro-step): ``opt.step()`` comes after the last of them, preceded
     by gradient-norm clipping (``grad_clip``, 0 disables it) and followed by ``scheduler.step()`` and
     ``zero_grad(set_to_none=True)``;
   * AdamW (or SGD with momentum 0.9) over two parameter groups: weight decay on the weights of every linear layer
@@ -150,6 +151,11 @@ def train(model: nn.Module, get_batch: Callable[[], Tuple[torch.Tensor, torch.Te
                 else lambda: torch.autocast(device_type=device_type, dtype=cfg.dtype))
     stats = TrainStats()
     model.train()
+    if cfg.acc_steps > 1:
+        # Q(W) is the same for every micro-step of an iteration: quantize it once per iteration
+        from .linear import enable_packed_weight_cache
+        enable_packed_weight_cache(model)
+    from .linear import invalidate_packed_weights
     for it in range(cfg.iterations):
         t0 = time.perf_counter()
         total = 0.0
@@ -165,6 +171,7 @@ def train(model: nn.Module, get_batch: Callable[[], Tuple[torch.Tensor, torch.Te
             norm = float(torch.nn.utils.clip_grad_norm_(model.parameters(), cfg.grad_clip))
         stats.lr.append(opt.param_groups[0]["lr"])
         opt.step()
+        invalidate_packed_weights(model)
         if scheduler is not None:
             scheduler.step()
         opt.zero_grad(set_to_none=True)

@@ -29,21 +29,21 @@ def test_library_exports_every_declared_function():
 
 def test_host_only_entry_points():
     L = _lib.lib()
-    assert L.qm_version() == 2
+    assert L.qm_version() == 3
     T, I, O = 256, 128, 384
-    total = L.qm_linear_saved_bytes(T, I, O)
-    off = (ctypes.c_size_t * 6)()
-    assert L.qm_linear_saved_offsets(T, I, O, off) == 0
-    sizes = [T * I // 2, T * I // 32, T * I // 8, O * I // 2, O * I // 32, O * I // 8]
-    # regions in declaration order, each 256-byte aligned, none overlapping, all inside the buffer
-    assert off[0] == 0
-    for k in range(6):
-        assert off[k] % 256 == 0
-        end = off[k] + sizes[k]
-        assert end <= (off[k + 1] if k < 5 else total)
-    assert L.qm_linear_saved_bytes(T, 100, O) == 0                      # in_features not a multiple of 32
-    assert L.qm_linear_saved_offsets(T, 100, O, off) != 0 and b"qm_linear_saved_offsets" in L.qm_last_error()
-    assert L.qm_linear_saved_offsets(T, I, O, None) != 0
+    off = (ctypes.c_size_t * 3)()
+    for rows, cols in ((T, I), (O, I)):
+        total = L.qm_packed_operand_bytes(rows, cols)
+        assert L.qm_packed_operand_offsets(rows, cols, off) == 0
+        sizes = [rows * cols // 2, rows * cols // 32, rows * cols // 8]
+        # codes, scales, mask bits in this order, each 256-byte aligned, none overlapping, all inside the buffer
+        assert off[0] == 0
+        for k in range(3):
+            assert off[k] % 256 == 0
+            assert off[k] + sizes[k] <= (off[k + 1] if k < 2 else total)
+    assert L.qm_packed_operand_bytes(T, 100) == 0                       # cols not a multiple of 32
+    assert L.qm_packed_operand_offsets(T, 100, off) != 0 and b"qm_packed_operand_offsets" in L.qm_last_error()
+    assert L.qm_packed_operand_offsets(T, I, None) != 0
     assert L.qm_linear_backward_workspace_bytes(T, I, O, _lib.QM_BF16) > 0
     assert L.qm_linear_backward_workspace_bytes(T, I, 100, _lib.QM_BF16) == 0
     assert L.qm_linear_backward_workspace_bytes(T, I, O, 7) == 0
@@ -61,8 +61,8 @@ def test_host_only_entry_points():
     (lambda L: L.qm_gemm_mxfp4_tn(None, None, None, None, 64, 64, 48, 1.0, None, 0, 0, 0, None, 0, None), b"qm_gemm_mxfp4_tn"),
     (lambda L: L.qm_masked_hadamard_bwd(None, 0, 4, 40, 32, 0, None, None, None, 0, None), b"multiple of hadamard_dim"),
     (lambda L: L.qm_dequantize_mxfp4(None, None, 4, 40, 1.0, None, 0, None), b"C % 32"),
-    (lambda L: L.qm_linear_forward(None, 0, None, 0, 64, 40, 64, 32, None, 32, None, None, 0, None, 0, 0, None), b"multiple of 32"),
-    (lambda L: L.qm_linear_forward(None, 0, None, 0, 64, 64, 64, 32, None, 32, None, None, 0, None, 0, 0, None), b"saved buffer"),
+    (lambda L: L.qm_linear_forward(None, 0, None, 0, 64, 40, 64, 32, None, 32, None, None, 0, None, 0, 0, None, 0, 0, None), b"multiple of 32"),
+    (lambda L: L.qm_linear_forward(None, 0, None, 0, 64, 64, 64, 32, None, 32, None, None, 0, None, 0, 0, None, 0, 0, None), b"packed operand buffers"),
 ])
 def test_rejected_arguments_report_an_error(call, needle):
     L = _lib.lib()
@@ -75,7 +75,7 @@ def test_empty_shapes_are_accepted_without_touching_pointers():
     L = _lib.lib()
     assert L.qm_quantize_mxfp4(None, 0, 0, 64, 32, None, 0, 0, None, 0, None, None, None, None, 0, None) == 0
     assert L.qm_gemm_mxfp4_tn(None, None, None, None, 0, 64, 64, 1.0, None, 0, 0, 0, None, 0, None) == 0
-    assert L.qm_linear_forward(None, 0, None, 0, 0, 64, 64, 32, None, 32, None, None, 0, None, 0, 0, None) == 0
+    assert L.qm_linear_forward(None, 0, None, 0, 0, 64, 64, 32, None, 32, None, None, 0, None, 0, 0, None, 0, 0, None) == 0
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

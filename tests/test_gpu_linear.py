@@ -243,3 +243,59 @@ def test_layer_with_dense_gradient_rotation(q):
     print(f"relative squared gradient errors {errs}", flush=True)
     for k in (0, 1):
         assert 0.03 < errs["O32"][k] < 0.3 and abs(errs["O32"][k] - errs["signs"][k]) < 0.5 * errs["signs"][k]
+
+
+def test_packed_weight_cache_across_micro_steps(q):
+    """With the cache on, the second micro-step reuses the packed Q(W) of the first: outputs and gradients are
+    bit-identical to a layer that quantizes every time, the buffer saved by an earlier graph survives a weight
+    update, and an update (seen through the version counter, or announced by invalidate) re-quantizes."""
+    torch.manual_seed(5)
+    T, I, O = 256, 256, 384
+    cached = production_layer(q, I, O, False, None, torch.bfloat16)
+    plain = production_layer(q, I, O, False, None, torch.bfloat16)
+    with torch.no_grad():
+        plain.weight.copy_(cached.weight)
+    q.enable_packed_weight_cache(cached)
+    cache = cached.packed_weight_cache
+    assert plain.packed_weight_cache is None and cache.hits == 0
+
+    def step(layer, x, dy):
+        x = x.clone().requires_grad_(True)
+        layer.weight.grad = None
+        y = layer(x)
+        y.backward(dy)
+        return y.detach(), x.grad, layer.weight.grad
+
+    xs = [make_input(T, I, torch.bfloat16, seed=s).to("cuda:0") for s in (1, 2, 3)]
+    dys = [make_input(T, O, torch.bfloat16, seed=10 + s).to("cuda:0") for s in (1, 2, 3)]
+    for k in (0, 1):
+        for got, want in zip(step(cached, xs[k], dys[k]), step(plain, xs[k], dys[k])):
+            assert torch.equal(got, want)
+    assert (cache.misses, cache.hits) == (1, 1)
+    first_buffer = cache.buffer
+
+    # a graph built before the update still owns the old Q(W) when its backward runs after the update
+    x_old = xs[0].clone().requires_grad_(True)
+    y_old = cached(x_old)
+    assert cache.hits == 2
+    with torch.no_grad():
+        cached.weight.mul_(0.5)
+        plain.weight.mul_(0.5)
+    for got, want in zip(step(cached, xs[2], dys[2]), step(plain, xs[2], dys[2])):
+        assert torch.equal(got, want)
+    assert cache.misses == 2 and cache.buffer is not first_buffer
+    y_old.backward(dys[0])
+    with torch.no_grad():
+        plain.weight.mul_(2.0)      # powers of two: exactly the old weight again
+    _, gx_want, _ = step(plain, xs[0], dys[0])
+    assert torch.equal(x_old.grad, gx_want)
+
+    # an update that the version counter does not see has to be announced
+    with torch.no_grad():
+        plain.weight.copy_(cached.weight)
+    cached.weight.data.mul_(2.0)
+    plain.weight.data.mul_(2.0)
+    q.invalidate_packed_weights(cached)
+    for got, want in zip(step(cached, xs[1], dys[1]), step(plain, xs[1], dys[1])):
+        assert torch.equal(got, want)
+    assert cache.misses == 3

@@ -94,6 +94,7 @@ def test_quartet_model_learns_with_the_training_loop():
     import math
     import random
 
+    import quartet_amd
     from quartet_amd.llama import Llama, LlamaConfig, unquantized
     from quartet_amd.train import TrainConfig, synthetic_batches, train
     dev = torch.device("cuda:0")
@@ -108,6 +109,10 @@ def test_quartet_model_learns_with_the_training_loop():
         assert all(math.isfinite(v) for v in stats.loss)
         assert stats.loss[0] == pytest.approx(math.log(256), abs=0.3)
         finals[name] = sum(stats.loss[-5:]) / 5
+        if name == "quartet":
+            # the weight of every quantized linear was quantized once per iteration, not once per micro-step
+            caches = [m.packed_weight_cache for m in model.modules() if isinstance(m, quartet_amd.QuantizedLinear)]
+            assert caches and all((c.misses, c.hits) == (cfg.iterations, cfg.iterations) for c in caches)
     print(f"final losses {finals}", flush=True)
     assert finals["quartet"] < math.log(256) - 1.5
     assert finals["quartet"] < finals["bf16"] + 0.75

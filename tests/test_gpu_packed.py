@@ -47,7 +47,7 @@ def test_pack_save_load_dequantize(oracle, P, tmp_path, tiled):
 
 
 @pytest.mark.parametrize("T,I,O", [(64, 96, 160), (256, 256, 384)])
-def test_views_into_the_saved_buffer(P, T, I, O):
+def test_views_into_the_operand_buffers(P, T, I, O):
     print(f"case saved-buffer views T={T} I={I} O={O}", flush=True)
     import quartet_amd as q
     from quartet_amd import kernels as K
@@ -55,9 +55,10 @@ def test_views_into_the_saved_buffer(P, T, I, O):
     w = make_input(O, I, torch.bfloat16, seed=4, scale=0.02).to(DEV)
     a_q, w_q = q.QuestMXFP4Quantizer(), q.QuestMXFP4Quantizer()
     tiled = all(d % 128 == 0 and d >= 256 for d in (T, I, O))
-    y, saved = K.linear_forward(x, w, 32, 0, 32, 0, torch.bfloat16, tiled)
-    xp, wp = P.from_linear_saved(saved, T, I, O, tiled, a_q, w_q)
-    assert xp.codes.data_ptr() == saved.data_ptr()  # views, not copies
+    y, packed_x, packed_w = K.linear_forward(x, w, 32, 0, 32, 0, torch.bfloat16, tiled)
+    xp = P.from_operand_buffer(packed_x, T, I, tiled, a_q)
+    wp = P.from_operand_buffer(packed_w, O, I, tiled, w_q)
+    assert xp.codes.data_ptr() == packed_x.data_ptr()  # views, not copies
     for got, src in ((xp, x), (wp, w)):
         direct = P.pack_quest(src, 32, 0, tiled=tiled)
         assert torch.equal(got.codes, direct.codes) and torch.equal(got.scales, direct.scales)
