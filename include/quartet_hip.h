@@ -38,6 +38,8 @@ enum { QM_QUEST_RTN = 0, QM_ABSMAX_RTN = 1, QM_ABSMAX_SR = 2, QM_QUEST_SR = 3 };
 
 /* layout of a packed tensor's code bytes (see above); producers and consumers must agree per tensor */
 enum { QM_LAYOUT_ROWMAJOR = 0, QM_LAYOUT_TILED = 1 };
+/* qm_linear_forward: which packed operand buffers already hold their operand on entry */
+enum { QM_W_IS_PACKED = 1, QM_X_IS_PACKED = 2 };
 
 #define QM_ERR_INVALID (-1)
 #define QM_ERR_UNALIGNED (-2)
@@ -130,9 +132,11 @@ int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, 
  * qm_linear_forward = QuestMXFP4QuantizerFn.forward on x and W (quantizers/mxfp4.py:129-140) followed by
  * QEQWtt_QEtQXttFn.forward (src/models/quantization/backward.py:59-62):
  *   x [T, I], w [O, I] -> y [T, O] = Q(x) Q(w)^T; packed_x ([T, I]) and packed_w ([O, I]) receive the packed
- *   operands the backward pass needs.  w_is_packed != 0: packed_w already holds Q(w) from an earlier call with the
- *   same w, signs and layout, and w is not read (W changes only at the optimizer step, src/optim/base.py:188-207,
- *   so the micro-steps of a gradient accumulation quantize it once).
+ *   operands the backward pass needs.  packed_flags & QM_W_IS_PACKED: packed_w already holds Q(w) from an earlier
+ *   call with the same w, signs and layout, and w is not read (W changes only at the optimizer step,
+ *   src/optim/base.py:188-207, so the micro-steps of a gradient accumulation quantize it once).
+ *   packed_flags & QM_X_IS_PACKED: packed_x already holds Q(x), written by one of the fused producers below, and x is
+ *   not read.
  * qm_linear_backward = QEQWtt_QEtQXttFn.backward (backward.py:64-85) with the straight-through backward of both
  * forward quantizers (mxfp4.py:143-146) applied: e [T, O] -> gx [T, I], gw [O, I], both of mid_dtype.
  *   g_mode            QM_ABSMAX_SR or QM_ABSMAX_RTN (AlbertTsengQuantizer stochastic or not)
@@ -149,13 +153,44 @@ int qm_packed_operand_offsets(int64_t rows, int64_t cols, size_t* offsets);
 size_t qm_linear_backward_workspace_bytes(int64_t T, int64_t I, int64_t O, int mid_dtype);
 int qm_linear_forward(const void* x, int x_dtype, const void* w, int w_dtype, int64_t T, int64_t I, int64_t O,
                       int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, void* packed_x,
-                      size_t packed_x_bytes, void* packed_w, size_t packed_w_bytes, int w_is_packed, void* y,
+                      size_t packed_x_bytes, void* packed_w, size_t packed_w_bytes, int packed_flags, void* y,
                       int y_dtype, int codes_layout, void* stream);
 int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t O, const void* packed_x,
                        const void* packed_w, int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w,
                        int hd_g, const uint32_t* signs_g, int g_mode, const uint64_t* seeds, int x_val_dtype,
                        int w_val_dtype, int mid_dtype, int x_scale_dtype, int w_scale_dtype, void* workspace,
                        size_t workspace_bytes, void* gx, void* gw, int codes_layout, void* stream);
+
+/*
+ * Producers fused into the activation quantizer.  The tensor the model would hand to a quantized linear is computed
+ * group by group inside the quantizer kernel and never written; the result is a packed operand buffer (layout as
+ * above) that qm_linear_forward consumes with QM_X_IS_PACKED and qm_linear_backward reads as packed_x.  Hadamard block
+ * 32, QM_QUEST_RTN with clip mask (QuestMXFP4QuantizerFn.forward, quantizers/mxfp4.py:129-140).
+ *
+ * qm_rmsnorm_quantize_mxfp4: RMSNorm.forward (src/models/llama.py:64-75) in front of c_attn / w12 (llama.py:170-171):
+ *   Q((x.float() * rsqrt(mean(x^2, -1) + eps)).type_as(x) * gain), x [rows, cols], gain fp32 [cols]; the product with
+ *   the fp32 gain is fp32, so the quantizer runs as on an fp32 tensor.  factor [rows] fp32 receives
+ *   rsqrt(mean(x^2) + eps) for the backward pass.
+ * qm_swiglu_quantize_mxfp4: the SwiGLU product in front of the MLP's c_proj (llama.py:113-114):
+ *   Q(silu(up) * gate) with h12 [rows, 2 hidden] = (up, gate) the fused w12 output; a bf16 h12 rounds silu and the
+ *   product to bf16 as torch's bf16 ops do, and the quantizer runs as on a tensor of h12's dtype.
+ * qm_rmsnorm_backward: autograd of the RMSNorm line above: gy [rows, cols] (gradient w.r.t. the normalised, scaled
+ *   tensor) -> dx [rows, cols] of x's dtype and dgain fp32 [cols] (summed over rows in a fixed order).  cols <= 8192.
+ *   workspace: qm_rmsnorm_backward_workspace_bytes(rows, cols) bytes, 16-byte aligned.
+ * qm_swiglu_backward: autograd of silu(up) * gate: g [rows, hidden] -> d_h12 [rows, 2 hidden] of h12's dtype.
+ * codes_layout QM_LAYOUT_TILED needs rows % 16 == 0 and cols (hidden) % 128 == 0; cols (hidden) % 32 == 0 always.
+ */
+int qm_rmsnorm_quantize_mxfp4(const void* x, int x_dtype, const float* gain, float eps, int64_t rows, int64_t cols,
+                              const uint32_t* sign_bits, void* packed, size_t packed_bytes, float* factor,
+                              int codes_layout, void* stream);
+int qm_swiglu_quantize_mxfp4(const void* h12, int dtype, int64_t rows, int64_t hidden, const uint32_t* sign_bits,
+                             void* packed, size_t packed_bytes, int codes_layout, void* stream);
+size_t qm_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols);
+int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain,
+                        const float* factor, int64_t rows, int64_t cols, void* dx, float* dgain, void* workspace,
+                        size_t workspace_bytes, void* stream);
+int qm_swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
+                       void* d_h12, void* stream);
 
 #ifdef __cplusplus
 }

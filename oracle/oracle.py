@@ -68,6 +68,14 @@ def lib():
         L.qo_sr_code.argtypes = [f32, f32]
         L.qo_div_four_thirds.restype = f32
         L.qo_div_four_thirds.argtypes = [f32]
+        L.qo_exp.restype = f32
+        L.qo_exp.argtypes = [f32]
+        L.qo_silu.restype = f32
+        L.qo_silu.argtypes = [f32]
+        L.qo_rmsnorm.restype = i32
+        L.qo_rmsnorm.argtypes = [vp, i32, vp, f32, i64, i64, vp, vp]
+        L.qo_swiglu.restype = i32
+        L.qo_swiglu.argtypes = [vp, i32, i64, i64, vp]
         _lib = L
     return _lib
 
@@ -213,6 +221,36 @@ def masked_hadamard_bwd(g, hd=32, scale_dtype=BF16, signs=None, maskbits=None, o
     if rc != 0:
         raise ValueError(f"qo_masked_hadamard_bwd rc={rc}")
     return out
+
+
+def rmsnorm(x, gain, eps):
+    """(normalised * gain as float32 [rows, cols], per-row factor) of src/models/llama.py:64-75 in the canonical order."""
+    x = np.ascontiguousarray(x)
+    rows, cols = x.shape
+    gain = np.ascontiguousarray(gain, dtype=np.float32)
+    out = np.empty((rows, cols), dtype=np.float32)
+    factor = np.empty(rows, dtype=np.float32)
+    rc = lib().qo_rmsnorm(_ptr(x), _dtype_of(x), _ptr(gain), float(eps), rows, cols, _ptr(out), _ptr(factor))
+    assert rc == 0, rc
+    return out, factor
+
+
+def swiglu(h12):
+    """silu(up) * gate of a [rows, 2 * hidden] tensor (up first), in h12's dtype (src/models/llama.py:113-114)."""
+    h12 = np.ascontiguousarray(h12)
+    rows, two = h12.shape
+    out = np.empty((rows, two // 2), dtype=h12.dtype)
+    rc = lib().qo_swiglu(_ptr(h12), _dtype_of(h12), rows, two // 2, _ptr(out))
+    assert rc == 0, rc
+    return out
+
+
+def exp_fixed(z):
+    return np.float32(lib().qo_exp(float(np.float32(z))))
+
+
+def silu(x):
+    return np.float32(lib().qo_silu(float(np.float32(x))))
 
 
 def rtn_code(A):

@@ -441,6 +441,84 @@ int qo_masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t col
     return 0;
 }
 
+/*
+ * Producers in front of the activation quantizer (the callers' side of the path):
+ *   RMSNorm  src/models/llama.py:64-75   (x.float() * rsqrt(mean(x^2) + eps)).type_as(x) * weight
+ *   SwiGLU   src/models/llama.py:113-114 silu(up) * gate, with (up, gate) = split of the fused w12 output
+ * torch's reductions and its device exp are implementation-defined; the canonical choices here:
+ *   - sum of squares of a row: sixteen interleaved partial sums (partial j takes groups j, j+16, j+32, ... of 32
+ *     consecutive elements, each group summed by the pairwise tree, added in ascending order), then the pairwise tree
+ *     over the sixteen partials; mean = sum / cols, factor = 1 / sqrt(mean + eps), IEEE divisions and square root;
+ *   - e^z = 2^n * P(r): n = rint(z * fl32(log2 e)), r = fma(n, -ln2_lo, fma(n, -ln2_hi, z)), P = degree-7 Taylor
+ *     polynomial evaluated by Horner's rule in fmas; silu(x) = x / (1 + e^-x);
+ *   - with a bf16 tensor every torch op rounds its result to bf16: silu, then the product.
+ * Pins: tests compare qo_exp with the C library's double-precision exp (<= 1.5 ulp), qo_silu and qo_rmsnorm with
+ * float64 evaluations of the reference's formulas, and closed forms (constant rows, zeros, saturation).
+ */
+float qo_exp(float z) {
+    if (z != z) return z;
+    if (z > 88.72283935546875f) return INFINITY;
+    if (z < -104.0f) return 0.0f;
+    const float n = rintf(z * 1.44269502162933349609375f);
+    float r = fmaf(n, -0.693145751953125f, z);
+    r = fmaf(n, -1.428606765330187045037746429443359375e-06f, r);
+    float p = 1.0f / 5040.0f;
+    const float coef[7] = {1.0f / 720.0f, 1.0f / 120.0f, 1.0f / 24.0f, 1.0f / 6.0f, 0.5f, 1.0f, 1.0f};
+    for (int i = 0; i < 7; ++i) p = fmaf(p, r, coef[i]);
+    return ldexpf(p, (int)n);
+}
+
+float qo_silu(float x) { return x / (1.0f + qo_exp(-x)); }
+
+/* out [rows, cols] fp32 = what RMSNorm hands to the linear layer; factor [rows] = the per-row 1/sqrt(mean + eps) */
+int qo_rmsnorm(const void* x, int dtype, const float* gain, float eps, int64_t rows, int64_t cols, float* out,
+               float* factor) {
+    if (cols % 32 || rows < 0 || cols <= 0 || (dtype != QO_BF16 && dtype != QO_F32)) return -1;
+    const int64_t groups = cols / 32;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        float partial[16];
+        for (int j = 0; j < 16; ++j) {
+            float acc = 0.0f;
+            for (int64_t g = j; g < groups; g += 16) {
+                float sq[32];
+                for (int i = 0; i < 32; ++i) {
+                    const float v = load_elem(x, dtype, r * cols + g * 32 + i);
+                    sq[i] = v * v;
+                }
+                acc = acc + tree_sum32(sq);
+            }
+            partial[j] = acc;
+        }
+        for (int n = 8; n >= 1; n >>= 1)
+            for (int i = 0; i < n; ++i) partial[i] = partial[2 * i] + partial[2 * i + 1];
+        const float f = 1.0f / sqrtf(partial[0] / (float)cols + eps);
+        if (factor) factor[r] = f;
+        for (int64_t j = 0; j < cols; ++j) {
+            float n = load_elem(x, dtype, r * cols + j) * f;
+            if (dtype == QO_BF16) n = bf16_to_f32(f32_to_bf16(n)); /* .type_as(x) */
+            out[r * cols + j] = n * gain[j];
+        }
+    }
+    return 0;
+}
+
+/* out [rows, hidden] of h12's dtype = silu(h12[:, :hidden]) * h12[:, hidden:] */
+int qo_swiglu(const void* h12, int dtype, int64_t rows, int64_t hidden, void* out) {
+    if (rows < 0 || hidden <= 0 || (dtype != QO_BF16 && dtype != QO_F32)) return -1;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        for (int64_t j = 0; j < hidden; ++j) {
+            const float up = load_elem(h12, dtype, r * 2 * hidden + j);
+            const float gate = load_elem(h12, dtype, r * 2 * hidden + hidden + j);
+            float a = qo_silu(up);
+            if (dtype == QO_BF16) a = bf16_to_f32(f32_to_bf16(a));
+            store_elem(out, dtype, r * hidden + j, a * gate);
+        }
+    }
+    return 0;
+}
+
 /* single-value helpers exported for exhaustive table tests */
 int qo_rtn_code(float A) { return rtn_code(A); }
 int qo_sr_code(float A, float u) { return sr_code(A, u); }

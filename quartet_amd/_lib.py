@@ -26,6 +26,11 @@ EXPORTS = (
     "qm_linear_backward_workspace_bytes",
     "qm_linear_forward",
     "qm_linear_backward",
+    "qm_rmsnorm_quantize_mxfp4",
+    "qm_swiglu_quantize_mxfp4",
+    "qm_rmsnorm_backward_workspace_bytes",
+    "qm_rmsnorm_backward",
+    "qm_swiglu_backward",
 )
 
 _lib = None
@@ -70,6 +75,16 @@ def lib():
     L.qm_linear_backward_workspace_bytes.argtypes = [i64, i64, i64, i32]
     L.qm_linear_forward.restype = i32
     L.qm_linear_forward.argtypes = [vp, i32, vp, i32, i64, i64, i64, i32, vp, i32, vp, vp, sz, vp, sz, i32, vp, i32, i32, vp]
+    L.qm_rmsnorm_quantize_mxfp4.restype = i32
+    L.qm_rmsnorm_quantize_mxfp4.argtypes = [vp, i32, vp, f32, i64, i64, vp, vp, sz, vp, i32, vp]
+    L.qm_swiglu_quantize_mxfp4.restype = i32
+    L.qm_swiglu_quantize_mxfp4.argtypes = [vp, i32, i64, i64, vp, vp, sz, i32, vp]
+    L.qm_rmsnorm_backward_workspace_bytes.restype = sz
+    L.qm_rmsnorm_backward_workspace_bytes.argtypes = [i64, i64]
+    L.qm_rmsnorm_backward.restype = i32
+    L.qm_rmsnorm_backward.argtypes = [vp, i32, vp, i32, vp, vp, i64, i64, vp, vp, vp, sz, vp]
+    L.qm_swiglu_backward.restype = i32
+    L.qm_swiglu_backward.argtypes = [vp, i32, vp, i32, i64, i64, vp, vp]
     L.qm_linear_backward.restype = i32
     L.qm_linear_backward.argtypes = [vp, i32, i64, i64, i64, vp, vp, i32, vp, i32, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32,
                                      vp, sz, vp, vp, i32, vp]

@@ -42,7 +42,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 3; }
+int qm_version(void) { return 4; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -225,7 +225,7 @@ size_t qm_linear_backward_workspace_bytes(int64_t T, int64_t I, int64_t O, int m
 
 int qm_linear_forward(const void* x, int x_dtype, const void* w, int w_dtype, int64_t T, int64_t I, int64_t O, int hd_x,
                       const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, void* packed_x, size_t packed_x_bytes,
-                      void* packed_w, size_t packed_w_bytes, int w_is_packed, void* y, int y_dtype, int codes_layout,
+                      void* packed_w, size_t packed_w_bytes, int packed_flags, void* y, int y_dtype, int codes_layout,
                       void* stream) {
     if (T < 0 || I < 0 || O < 0) return fail(QM_ERR_INVALID, "qm_linear_forward: negative extent");
     if (T == 0 || O == 0 || I == 0) return 0;
@@ -237,8 +237,10 @@ int qm_linear_forward(const void* x, int x_dtype, const void* w, int w_dtype, in
                     lw.total);
     uint8_t* px = static_cast<uint8_t*>(packed_x);
     uint8_t* pw = static_cast<uint8_t*>(packed_w);
-    int rc;
-    if (!w_is_packed && pair_launches(codes_layout, T, I, O, hd_x, hd_w, 32) && x && w && y && valid_dtype(x_dtype) &&
+    if (packed_flags & ~(QM_W_IS_PACKED | QM_X_IS_PACKED)) return fail(QM_ERR_INVALID, "qm_linear_forward: unknown packed_flags %d", packed_flags);
+    const bool w_is_packed = packed_flags & QM_W_IS_PACKED, x_is_packed = packed_flags & QM_X_IS_PACKED;
+    int rc = 0;
+    if (!w_is_packed && !x_is_packed && pair_launches(codes_layout, T, I, O, hd_x, hd_w, 32) && x && w && y && valid_dtype(x_dtype) &&
         valid_dtype(w_dtype) && aligned(x, 16) && aligned(w, 16)) {
         // both forward quantizers in one grid
         const qm::RowmajorArgs ax{x, x_dtype, T, I, signs_x ? signs_x[0] : 0u, px + lx.c, px + lx.s, px + lx.m};
@@ -246,8 +248,9 @@ int qm_linear_forward(const void* x, int x_dtype, const void* w, int w_dtype, in
         rc = from_hip(qm::quantize_rowmajor_hd32_tiled_pair(ax, aw, reinterpret_cast<hipStream_t>(stream)), "qm_linear_forward");
         if (rc) return rc;
     } else {
-        rc = qm_quantize_mxfp4(x, x_dtype, T, I, hd_x, signs_x, QM_QUEST_RTN, 0, nullptr, 0, px + lx.c, px + lx.s, px + lx.m, nullptr,
-                               codes_layout, stream);
+        if (!x_is_packed)
+            rc = qm_quantize_mxfp4(x, x_dtype, T, I, hd_x, signs_x, QM_QUEST_RTN, 0, nullptr, 0, px + lx.c, px + lx.s, px + lx.m,
+                                   nullptr, codes_layout, stream);
         if (rc) return rc;
         if (!w_is_packed) {
             rc = qm_quantize_mxfp4(w, w_dtype, O, I, hd_w, signs_w, QM_QUEST_RTN, 0, nullptr, 0, pw + lw.c, pw + lw.s, pw + lw.m,
@@ -331,6 +334,87 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
     rc = qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, px + lx.m, gx, mid_dtype, stream);
     if (rc) return rc;
     return qm_masked_hadamard_bwd(k + wl.gwq, mid_dtype, O, I, hd_w, w_scale_dtype, signs_w, pw + lw.m, gw, mid_dtype, stream);
+}
+
+int qm_rmsnorm_quantize_mxfp4(const void* x, int x_dtype, const float* gain, float eps, int64_t rows, int64_t cols,
+                              const uint32_t* sign_bits, void* packed, size_t packed_bytes, float* factor, int codes_layout,
+                              void* stream) {
+    if (!valid_layout(codes_layout)) return fail(QM_ERR_INVALID, "qm_rmsnorm_quantize_mxfp4: unknown codes_layout %d", codes_layout);
+    if (!valid_dtype(x_dtype)) return fail(QM_ERR_INVALID, "qm_rmsnorm_quantize_mxfp4: x_dtype %d is not QM_BF16/QM_F32", x_dtype);
+    if (rows < 0 || cols <= 0 || cols % 32)
+        return fail(QM_ERR_INVALID, "qm_rmsnorm_quantize_mxfp4: need rows >= 0 and cols a positive multiple of 32 (got [%lld, %lld])",
+                    (long long)rows, (long long)cols);
+    if (rows == 0) return 0;
+    if (codes_layout == QM_LAYOUT_TILED && (rows % 16 || cols % 128))
+        return fail(QM_ERR_INVALID, "qm_rmsnorm_quantize_mxfp4: tiled codes need rows %% 16 == 0 and cols %% 128 == 0 (rows=%lld cols=%lld)",
+                    (long long)rows, (long long)cols);
+    const PackedLayout l = packed_layout(rows, cols);
+    if (!x || !gain || !factor || !packed || packed_bytes < l.total)
+        return fail(QM_ERR_INVALID, "qm_rmsnorm_quantize_mxfp4: x, gain, factor must be non-null and packed hold %zu bytes", l.total);
+    if (!aligned(x, 16) || !aligned(gain, 16) || !aligned(packed, 256) || !aligned(factor, 4))
+        return fail(QM_ERR_UNALIGNED, "qm_rmsnorm_quantize_mxfp4: x and gain need 16-byte, packed 256-byte alignment");
+    uint8_t* p = static_cast<uint8_t*>(packed);
+    return from_hip(qm::rmsnorm_quantize_hd32(x, x_dtype, gain, eps, rows, cols, sign_bits ? sign_bits[0] : 0u, p + l.c, p + l.s,
+                                              p + l.m, factor, codes_layout == QM_LAYOUT_TILED, reinterpret_cast<hipStream_t>(stream)),
+                    "qm_rmsnorm_quantize_mxfp4");
+}
+
+int qm_swiglu_quantize_mxfp4(const void* h12, int dtype, int64_t rows, int64_t hidden, const uint32_t* sign_bits, void* packed,
+                             size_t packed_bytes, int codes_layout, void* stream) {
+    if (!valid_layout(codes_layout)) return fail(QM_ERR_INVALID, "qm_swiglu_quantize_mxfp4: unknown codes_layout %d", codes_layout);
+    if (!valid_dtype(dtype)) return fail(QM_ERR_INVALID, "qm_swiglu_quantize_mxfp4: dtype %d is not QM_BF16/QM_F32", dtype);
+    if (rows < 0 || hidden <= 0 || hidden % 32)
+        return fail(QM_ERR_INVALID, "qm_swiglu_quantize_mxfp4: need rows >= 0 and hidden a positive multiple of 32 (got [%lld, %lld])",
+                    (long long)rows, (long long)hidden);
+    if (rows == 0) return 0;
+    if (codes_layout == QM_LAYOUT_TILED && (rows % 16 || hidden % 128))
+        return fail(QM_ERR_INVALID, "qm_swiglu_quantize_mxfp4: tiled codes need rows %% 16 == 0 and hidden %% 128 == 0 (rows=%lld hidden=%lld)",
+                    (long long)rows, (long long)hidden);
+    const PackedLayout l = packed_layout(rows, hidden);
+    if (!h12 || !packed || packed_bytes < l.total)
+        return fail(QM_ERR_INVALID, "qm_swiglu_quantize_mxfp4: h12 must be non-null and packed hold %zu bytes", l.total);
+    if (!aligned(h12, 16) || !aligned(packed, 256))
+        return fail(QM_ERR_UNALIGNED, "qm_swiglu_quantize_mxfp4: h12 needs 16-byte, packed 256-byte alignment");
+    uint8_t* p = static_cast<uint8_t*>(packed);
+    return from_hip(qm::swiglu_quantize_hd32(h12, dtype, rows, hidden, sign_bits ? sign_bits[0] : 0u, p + l.c, p + l.s, p + l.m,
+                                             codes_layout == QM_LAYOUT_TILED, reinterpret_cast<hipStream_t>(stream)),
+                    "qm_swiglu_quantize_mxfp4");
+}
+
+size_t qm_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols) {
+    if (rows < 0 || cols <= 0 || cols % 32 || cols > 8192) return 0;
+    return up256(qm::rmsnorm_backward_workspace_bytes(rows, cols));
+}
+
+int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain, const float* factor,
+                        int64_t rows, int64_t cols, void* dx, float* dgain, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!valid_dtype(gy_dtype) || !valid_dtype(x_dtype)) return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: dtypes must be QM_BF16/QM_F32");
+    if (rows < 0 || cols <= 0 || cols % 32 || cols > 8192)
+        return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: need rows >= 0 and cols a multiple of 32 in [32, 8192] (got [%lld, %lld])",
+                    (long long)rows, (long long)cols);
+    if (!dgain) return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: dgain must be non-null");
+    if (rows > 0 && (!gy || !x || !gain || !factor || !dx || !workspace || workspace_bytes < qm::rmsnorm_backward_workspace_bytes(rows, cols)))
+        return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: null tensor, or workspace below %zu bytes", qm_rmsnorm_backward_workspace_bytes(rows, cols));
+    if (!aligned(gy, 8) || !aligned(x, 8) || !aligned(dx, 8) || !aligned(gain, 16) || !aligned(workspace, 16) ||
+        (gy_dtype == QM_F32 && !aligned(gy, 16)) || (x_dtype == QM_F32 && (!aligned(x, 16) || !aligned(dx, 16))))
+        return fail(QM_ERR_UNALIGNED, "qm_rmsnorm_backward: tensors need 16-byte alignment");
+    return from_hip(qm::rmsnorm_backward(gy, gy_dtype, x, x_dtype, gain, factor, rows, cols, dx, dgain, workspace,
+                                         reinterpret_cast<hipStream_t>(stream)),
+                    "qm_rmsnorm_backward");
+}
+
+int qm_swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden, void* d_h12,
+                       void* stream) {
+    if (!valid_dtype(g_dtype) || !valid_dtype(dtype)) return fail(QM_ERR_INVALID, "qm_swiglu_backward: dtypes must be QM_BF16/QM_F32");
+    if (rows < 0 || hidden <= 0 || hidden % 4)
+        return fail(QM_ERR_INVALID, "qm_swiglu_backward: need rows >= 0 and hidden a positive multiple of 4 (got [%lld, %lld])",
+                    (long long)rows, (long long)hidden);
+    if (rows == 0) return 0;
+    if (!g || !h12 || !d_h12) return fail(QM_ERR_INVALID, "qm_swiglu_backward: g, h12 and d_h12 must be non-null");
+    if (!aligned(g, 16) || !aligned(h12, 16) || !aligned(d_h12, 16))
+        return fail(QM_ERR_UNALIGNED, "qm_swiglu_backward: tensors need 16-byte alignment");
+    return from_hip(qm::swiglu_backward(g, g_dtype, h12, dtype, rows, hidden, d_h12, reinterpret_cast<hipStream_t>(stream)),
+                    "qm_swiglu_backward");
 }
 
 }  // extern "C"

@@ -1,0 +1,203 @@
+// Backward passes of the producers that are fused into the forward quantizer: RMSNorm
+// (src/models/llama.py:64-75 of the reference) and the SwiGLU product (llama.py:113-114).  Floating-point kernels:
+// they follow the formulas autograd derives for those lines, not a bit-exact instruction order.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "qm_kernels.h"
+#include "qm_math.h"
+
+namespace qm {
+
+namespace {
+
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+
+template <typename T>
+__device__ __forceinline__ float4 load4(const T* p) {
+    if constexpr (sizeof(T) == 2) {
+        const uint2 raw = *reinterpret_cast<const uint2*>(p);
+        return make_float4(u2f(raw.x << 16), u2f(raw.x & 0xffff0000u), u2f(raw.y << 16), u2f(raw.y & 0xffff0000u));
+    } else {
+        return *reinterpret_cast<const float4*>(p);
+    }
+}
+template <typename T>
+__device__ __forceinline__ void store4(T* p, float4 v) {
+    if constexpr (sizeof(T) == 2) {
+        const uint32_t lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v.x, v.y}, v2bf));
+        const uint32_t hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v.z, v.w}, v2bf));
+        *reinterpret_cast<uint2*>(p) = make_uint2(lo, hi);
+    } else {
+        *reinterpret_cast<float4*>(p) = v;
+    }
+}
+
+constexpr int kRowsPerWave = 16;
+
+// y = x f g with f = (mean(x^2) + eps)^-1/2:
+//   dx_i = f g_i gy_i - x_i f^3 / cols * sum_j gy_j g_j x_j,      dgain_i = sum_rows gy_i x_i f.
+// One wave walks kRowsPerWave rows; lane l owns columns 4 (l + 64 k) .. +3.  The row is read twice (the second time
+// from cache); the gain-gradient sums stay in registers, are added across the workgroup's four waves in wave order
+// through shared memory and leave as one partial row per workgroup.
+template <typename TG, typename TX, int NK>
+__global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const TG* __restrict__ gy, const TX* __restrict__ x,
+                                                          const float* __restrict__ gain, const float* __restrict__ factor,
+                                                          int64_t rows, int cols, TX* __restrict__ dx,
+                                                          float* __restrict__ partial) {
+    extern __shared__ float wave_sums[];  // [cols]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t r0 = ((int64_t)blockIdx.x * 4 + wave) * kRowsPerWave;
+    const int64_t r1 = r0 + kRowsPerWave < rows ? r0 + kRowsPerWave : rows;
+    float4 acc[NK];
+#pragma unroll
+    for (int k = 0; k < NK; ++k) acc[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int64_t r = r0; r < r1; ++r) {
+        const TG* gr = gy + r * cols;
+        const TX* xr = x + r * cols;
+        const float f = factor[r];
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < NK; ++k) {
+            const int col = (k * 64 + lane) * 4;
+            if (col < cols) {
+                const float4 g = load4(gr + col), v = load4(xr + col), w = *reinterpret_cast<const float4*>(gain + col);
+                s += g.x * w.x * v.x + g.y * w.y * v.y + g.z * w.z * v.z + g.w * w.w * v.w;
+                acc[k].x += g.x * v.x * f; acc[k].y += g.y * v.y * f; acc[k].z += g.z * v.z * f; acc[k].w += g.w * v.w * f;
+            }
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
+        const float coef = f * f * f * s / (float)cols;
+#pragma unroll
+        for (int k = 0; k < NK; ++k) {
+            const int col = (k * 64 + lane) * 4;
+            if (col < cols) {
+                const float4 g = load4(gr + col), v = load4(xr + col), w = *reinterpret_cast<const float4*>(gain + col);
+                store4(dx + r * cols + col, make_float4(f * g.x * w.x - v.x * coef, f * g.y * w.y - v.y * coef,
+                                                        f * g.z * w.z - v.z * coef, f * g.w * w.w - v.w * coef));
+            }
+        }
+    }
+    for (int turn = 0; turn < 4; ++turn) {
+        if (wave == turn) {
+#pragma unroll
+            for (int k = 0; k < NK; ++k) {
+                const int col = (k * 64 + lane) * 4;
+                if (col < cols) {
+                    float4* slot = reinterpret_cast<float4*>(wave_sums + col);
+                    float4 t = acc[k];
+                    if (turn) { const float4 p = *slot; t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w; }
+                    if (turn == 3) *reinterpret_cast<float4*>(partial + (int64_t)blockIdx.x * cols + col) = t;
+                    else *slot = t;
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// dgain[c] = sum over the n partial rows, in a fixed order: 16 waves take rows w, w+16, ...; their sums are added in
+// wave order.  One workgroup of 1024 threads per 64 columns.
+__global__ __launch_bounds__(1024) void column_sum_kernel(const float* __restrict__ partial, int n, int cols,
+                                                          float* __restrict__ out) {
+    __shared__ float sums[16][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = blockIdx.x * 64 + lane;
+    float s = 0.0f;
+    if (col < cols)
+        for (int r = wave; r < n; r += 16) s += partial[(int64_t)r * cols + col];
+    sums[wave][lane] = s;
+    __syncthreads();
+    if (wave == 0 && col < cols) {
+        float t = sums[0][lane];
+#pragma unroll
+        for (int w = 1; w < 16; ++w) t += sums[w][lane];
+        out[col] = t;
+    }
+}
+
+// h = silu(up) * gate:  d_gate = g silu(up),  d_up = g gate s (1 + up (1 - s)),  s = 1 / (1 + e^-up).
+// A tensor of bf16 rounds where autograd's bf16 ops would: silu(up), g * gate, and the two results.
+template <typename TG, typename TH>
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const TG* __restrict__ g, const TH* __restrict__ h12,
+                                                         int64_t rows, int64_t hidden, TH* __restrict__ d_h12) {
+    const int64_t quads_per_row = hidden / 4;
+    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (q >= rows * quads_per_row) return;
+    const int64_t row = q / quads_per_row, col = (q - row * quads_per_row) * 4;
+    const float4 gv = load4(g + row * hidden + col);
+    const float4 up = load4(h12 + row * 2 * hidden + col), gate = load4(h12 + row * 2 * hidden + hidden + col);
+    const float G[4] = {gv.x, gv.y, gv.z, gv.w}, U[4] = {up.x, up.y, up.z, up.w}, A[4] = {gate.x, gate.y, gate.z, gate.w};
+    float du[4], da[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float s = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-U[i] * 1.44269504f));
+        float a = U[i] * s, t = G[i] * A[i];
+        if constexpr (sizeof(TH) == 2) {
+            a = bf16_to_f32(f32_to_bf16(a));
+            t = bf16_to_f32(f32_to_bf16(t));
+        }
+        da[i] = G[i] * a;
+        du[i] = t * s * (1.0f + U[i] * (1.0f - s));
+    }
+    store4(d_h12 + row * 2 * hidden + col, make_float4(du[0], du[1], du[2], du[3]));
+    store4(d_h12 + row * 2 * hidden + hidden + col, make_float4(da[0], da[1], da[2], da[3]));
+}
+
+int64_t rmsnorm_bwd_blocks(int64_t rows) { return (rows + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave); }
+
+template <typename TG, typename TX>
+void launch_rmsnorm_bwd(const void* gy, const void* x, const float* gain, const float* factor, int64_t rows, int cols,
+                        void* dx, float* partial, hipStream_t stream) {
+    const dim3 grid((unsigned)rmsnorm_bwd_blocks(rows)), block(256);
+    const size_t lds = (size_t)cols * sizeof(float);
+    const TG* g = reinterpret_cast<const TG*>(gy);
+    const TX* xp = reinterpret_cast<const TX*>(x);
+    TX* dxp = reinterpret_cast<TX*>(dx);
+    if (cols <= 2048) rmsnorm_bwd_kernel<TG, TX, 8><<<grid, block, lds, stream>>>(g, xp, gain, factor, rows, cols, dxp, partial);
+    else rmsnorm_bwd_kernel<TG, TX, 32><<<grid, block, lds, stream>>>(g, xp, gain, factor, rows, cols, dxp, partial);
+}
+
+}  // namespace
+
+size_t rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols) {
+    return (size_t)rmsnorm_bwd_blocks(rows) * (size_t)cols * sizeof(float);
+}
+
+// cols <= 8192, cols % 4 == 0; workspace: rmsnorm_backward_workspace_bytes(rows, cols) bytes, 16-byte aligned
+hipError_t rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain,
+                            const float* factor, int64_t rows, int64_t cols, void* dx, float* dgain, void* workspace,
+                            hipStream_t stream) {
+    if (cols == 0) return hipSuccess;
+    float* partial = reinterpret_cast<float*>(workspace);
+    if (rows == 0) {}  // no rows: the column sums below write zeros
+    else if (gy_dtype == BF16 && x_dtype == BF16) launch_rmsnorm_bwd<uint16_t, uint16_t>(gy, x, gain, factor, rows, (int)cols, dx, partial, stream);
+    else if (gy_dtype == BF16) launch_rmsnorm_bwd<uint16_t, float>(gy, x, gain, factor, rows, (int)cols, dx, partial, stream);
+    else if (x_dtype == BF16) launch_rmsnorm_bwd<float, uint16_t>(gy, x, gain, factor, rows, (int)cols, dx, partial, stream);
+    else launch_rmsnorm_bwd<float, float>(gy, x, gain, factor, rows, (int)cols, dx, partial, stream);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    column_sum_kernel<<<dim3((unsigned)((cols + 63) / 64)), dim3(1024), 0, stream>>>(partial, (int)rmsnorm_bwd_blocks(rows),
+                                                                                    (int)cols, dgain);
+    return hipGetLastError();
+}
+
+// hidden % 4 == 0
+hipError_t swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
+                           void* d_h12, hipStream_t stream) {
+    if (rows == 0 || hidden == 0) return hipSuccess;
+    const dim3 grid((unsigned)((rows * (hidden / 4) + 255) / 256)), block(256);
+    if (g_dtype == BF16 && dtype == BF16)
+        swiglu_bwd_kernel<uint16_t, uint16_t><<<grid, block, 0, stream>>>(reinterpret_cast<const uint16_t*>(g), reinterpret_cast<const uint16_t*>(h12), rows, hidden, reinterpret_cast<uint16_t*>(d_h12));
+    else if (g_dtype == BF16)
+        swiglu_bwd_kernel<uint16_t, float><<<grid, block, 0, stream>>>(reinterpret_cast<const uint16_t*>(g), reinterpret_cast<const float*>(h12), rows, hidden, reinterpret_cast<float*>(d_h12));
+    else if (dtype == BF16)
+        swiglu_bwd_kernel<float, uint16_t><<<grid, block, 0, stream>>>(reinterpret_cast<const float*>(g), reinterpret_cast<const uint16_t*>(h12), rows, hidden, reinterpret_cast<uint16_t*>(d_h12));
+    else
+        swiglu_bwd_kernel<float, float><<<grid, block, 0, stream>>>(reinterpret_cast<const float*>(g), reinterpret_cast<const float*>(h12), rows, hidden, reinterpret_cast<float*>(d_h12));
+    return hipGetLastError();
+}
+
+}  // namespace qm

@@ -74,6 +74,19 @@ hipError_t masked_hadamard_bwd_hd32_pair(const void* ga, int64_t na, int scale_d
                                          const void* gb, int64_t nb, int scale_dtype_b, uint32_t sign_b, const uint8_t* mask_b, void* out_b,
                                          int dtype, hipStream_t stream);
 
+// Producers fused into the forward quantizer (Hadamard block 32, quest RTN, clip mask) and their backward passes
+hipError_t rmsnorm_quantize_hd32(const void* x, int dtype, const float* gain, float eps, int64_t rows, int64_t cols,
+                                 uint32_t sign_word, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, float* factor,
+                                 bool tiled, hipStream_t stream);
+hipError_t swiglu_quantize_hd32(const void* h12, int dtype, int64_t rows, int64_t hidden, uint32_t sign_word,
+                                uint8_t* codes, uint8_t* scales, uint8_t* maskbits, bool tiled, hipStream_t stream);
+size_t rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols);
+hipError_t rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain,
+                            const float* factor, int64_t rows, int64_t cols, void* dx, float* dgain, void* workspace,
+                            hipStream_t stream);
+hipError_t swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
+                           void* d_h12, hipStream_t stream);
+
 hipError_t requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C,
                                        float post, int val_dtype, int hd, const SignBits& sb, int mode, const float* u,
                                        uint64_t seed, uint8_t* codes_out, uint8_t* scales_out, void* dequant,

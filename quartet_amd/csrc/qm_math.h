@@ -106,6 +106,30 @@ QM_HD int sr_code(float A, float u) {
     return lo + (u < p ? 1 : 0);
 }
 
+// ---- SiLU with a fixed instruction sequence ------------------------------------------------------------------
+// e^z from n = rint(z log2 e), r = z - n ln2 (two-constant reduction, fused), the degree-7 Taylor polynomial in r
+// (|r| <= 0.347: truncation error below 2^-27) and an exact scaling by 2^n: the same fmas on the CPU and on the GPU,
+// about one ulp from the exact value.  Above ln(FLT_MAX) the result is +inf; NaN passes through.
+QM_HD float exp_fixed(float z) {
+    if (!(z == z)) return z;
+    if (z > 88.72283935546875f) return u2f(0x7f800000u);
+    if (z < -104.0f) return 0.0f;
+    const float n = __builtin_rintf(z * 1.44269502162933349609375f);
+    float r = __builtin_fmaf(n, -0.693145751953125f, z);
+    r = __builtin_fmaf(n, -1.428606765330187045037746429443359375e-06f, r);
+    float p = 1.0f / 5040.0f;
+    p = __builtin_fmaf(p, r, 1.0f / 720.0f);
+    p = __builtin_fmaf(p, r, 1.0f / 120.0f);
+    p = __builtin_fmaf(p, r, 1.0f / 24.0f);
+    p = __builtin_fmaf(p, r, 1.0f / 6.0f);
+    p = __builtin_fmaf(p, r, 0.5f);
+    p = __builtin_fmaf(p, r, 1.0f);
+    p = __builtin_fmaf(p, r, 1.0f);
+    return scale_pow2(p, (int)n);
+}
+// x / (1 + e^-x), the form torch.nn.functional.silu evaluates (src/models/llama.py:113 of the reference calls it)
+QM_HD float silu_fixed(float x) { return x / (1.0f + exp_fixed(-x)); }
+
 // ---- Philox4x32-10 ----------------------------------------------------------------------
 struct Philox4 {
     uint32_t w[4];

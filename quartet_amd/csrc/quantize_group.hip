@@ -713,6 +713,168 @@ hipError_t requantize_transposed_hd32(const uint8_t* codes_in, const uint8_t* sc
     return hipGetLastError();
 }
 
+// ---- producers fused into the forward quantizer ------------------------------------------------------------------
+// The tensor the model would hand to the quantized linear (RMSNorm output, src/models/llama.py:64-75; SwiGLU product,
+// llama.py:113-114) is computed group by group in registers and never written.  A workgroup owns 16 whole rows:
+// wave w rows 4w..4w+3, the 16 lanes of a row take groups l, l+16, l+32, ... of 32 consecutive elements.
+
+namespace {
+
+typedef __bf16 v2bf16 __attribute__((ext_vector_type(2)));
+// round to bf16 and back (round to nearest even, v_cvt_pk_bf16_f32)
+__device__ __forceinline__ void round_pair_to_bf16(float& a, float& b) {
+    const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{a, b}, v2bf16));
+    a = u2f(w << 16);
+    b = u2f(w & 0xffff0000u);
+}
+
+template <typename T>
+struct RmsNormProducer {
+    static constexpr int kOutDtype = F32;  // bf16-or-fp32 normalised value times the fp32 gain is fp32
+    const T* x;
+    const float* gain;
+    float* factor;  // [rows]: 1 / sqrt(mean(x^2) + eps), kept for the backward pass
+    float eps;
+
+    // sum of squares: per lane its groups in ascending order (each by the pairwise tree), then the butterfly over the
+    // row's 16 lanes, which adds in the order of a pairwise tree and leaves every lane with the same bits
+    __device__ __forceinline__ float prepare(int64_t row, int lane16, int groups, int64_t cols) const {
+        float acc = 0.0f;
+        for (int g = lane16; g < groups; g += 16) {
+            float v[32];
+            load_group<T>(x + row * cols + g * 32, v);
+#pragma unroll
+            for (int i = 0; i < 32; ++i) v[i] = v[i] * v[i];
+            acc = acc + tree_sum32(v);
+        }
+#pragma unroll
+        for (int m = 1; m < 16; m <<= 1) acc = acc + __shfl_xor(acc, m, 64);
+        const float f = 1.0f / __builtin_sqrtf(acc / (float)cols + eps);
+        if (lane16 == 0) factor[row] = f;
+        return f;
+    }
+    __device__ __forceinline__ void load(int64_t row, int g, int64_t cols, float f, float (&v)[32]) const {
+        load_group<T>(x + row * cols + g * 32, v);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) v[i] = v[i] * f;
+        if constexpr (sizeof(T) == 2) {  // .type_as(x)
+#pragma unroll
+            for (int i = 0; i < 32; i += 2) round_pair_to_bf16(v[i], v[i + 1]);
+        }
+        float w[32];
+        load_group<float>(gain + g * 32, w);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) v[i] = v[i] * w[i];
+    }
+};
+
+template <typename T>
+struct SwiGluProducer {
+    static constexpr int kOutDtype = sizeof(T) == 2 ? BF16 : F32;
+    const T* h12;  // [rows, 2 cols]: up, then gate
+
+    __device__ __forceinline__ float prepare(int64_t, int, int, int64_t) const { return 0.0f; }
+    __device__ __forceinline__ void load(int64_t row, int g, int64_t cols, float, float (&v)[32]) const {
+        float gate[32];
+        load_group<T>(h12 + row * 2 * cols + g * 32, v);
+        load_group<T>(h12 + row * 2 * cols + cols + g * 32, gate);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) v[i] = silu_fixed(v[i]);
+        if constexpr (sizeof(T) == 2) {  // a bf16 tensor rounds after each op
+#pragma unroll
+            for (int i = 0; i < 32; i += 2) round_pair_to_bf16(v[i], v[i + 1]);
+        }
+#pragma unroll
+        for (int i = 0; i < 32; ++i) v[i] = v[i] * gate[i];
+        if constexpr (sizeof(T) == 2) {
+#pragma unroll
+            for (int i = 0; i < 32; i += 2) round_pair_to_bf16(v[i], v[i + 1]);
+        }
+    }
+};
+
+// quest RTN + clip mask (the forward quantizer) of rows that a producer computes
+template <typename P, bool TILED>
+struct ProducedRowsJob {
+    P prod;
+    int64_t rows, cols;
+    float c;
+    uint32_t sign_word;
+    GroupOut out;
+    unsigned blocks;
+
+    ProducedRowsJob(const P& prod_, int64_t rows_, int64_t cols_, uint32_t sign_word_, const GroupOut& out_)
+        : prod(prod_), rows(rows_), cols(cols_), c(hadamard_scale(32, P::kOutDtype)), sign_word(sign_word_), out(out_),
+          blocks((unsigned)((rows_ + 15) / 16)) {}
+
+    __device__ __forceinline__ void run(unsigned bid) const {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const int rin = wave * 4 + (lane >> 4), lane16 = lane & 15;
+        const int64_t row = (int64_t)bid * 16 + rin;
+        if (row >= rows) return;  // the 16 lanes of a row leave together
+        const int groups = (int)(cols / 32);
+        const float state = prod.prepare(row, lane16, groups, cols);
+        // TILED: cols % 128 == 0, so the four lanes of a quad run the same number of iterations
+        for (int g = lane16; g < groups; g += 16) {
+            const int64_t gi = row * groups + g;
+            const int64_t ci = TILED ? (int64_t)bid * 16 * groups + ((g >> 2) * 64 + rin * 4 + (g & 3)) : gi;
+            float v[32];
+            prod.load(row, g, cols, state, v);
+            rotate_group(v, c, sign_word);
+            GroupCodes o;
+            quantize_group_regs<QUEST_RTN, true>(v, 0, gi, o);
+            out.codes[ci] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
+            if constexpr (TILED) {
+                const uint32_t s1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0x55, 0xf, 0xf, false);
+                const uint32_t s2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0xAA, 0xf, 0xf, false);
+                const uint32_t s3 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0xFF, 0xf, 0xf, false);
+                if ((lane & 3) == 0)
+                    *reinterpret_cast<uint32_t*>(out.scales + gi) = o.scale_byte | (s1 << 8) | (s2 << 16) | (s3 << 24);
+            } else {
+                out.scales[gi] = (uint8_t)o.scale_byte;
+            }
+            out.maskbits[gi] = o.keep;
+        }
+    }
+};
+
+template <typename P>
+void launch_produced(const P& prod, int64_t rows, int64_t cols, uint32_t sign_word, uint8_t* codes, uint8_t* scales,
+                     uint8_t* maskbits, bool tiled, hipStream_t stream) {
+    const GroupOut out{reinterpret_cast<uint4*>(codes), scales, reinterpret_cast<uint32_t*>(maskbits), nullptr};
+    if (tiled) launch_job(ProducedRowsJob<P, true>(prod, rows, cols, sign_word, out), stream);
+    else launch_job(ProducedRowsJob<P, false>(prod, rows, cols, sign_word, out), stream);
+}
+
+}  // namespace
+
+// Q(rmsnorm(x) * gain): Hadamard block 32, quest RTN, clip mask; factor [rows] receives 1 / sqrt(mean(x^2) + eps)
+hipError_t rmsnorm_quantize_hd32(const void* x, int dtype, const float* gain, float eps, int64_t rows, int64_t cols,
+                                 uint32_t sign_word, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, float* factor,
+                                 bool tiled, hipStream_t stream) {
+    if (rows == 0) return hipSuccess;
+    if (dtype == BF16)
+        launch_produced(RmsNormProducer<uint16_t>{reinterpret_cast<const uint16_t*>(x), gain, factor, eps}, rows, cols,
+                        sign_word, codes, scales, maskbits, tiled, stream);
+    else
+        launch_produced(RmsNormProducer<float>{reinterpret_cast<const float*>(x), gain, factor, eps}, rows, cols, sign_word,
+                        codes, scales, maskbits, tiled, stream);
+    return hipGetLastError();
+}
+
+// Q(silu(up) * gate) of h12 [rows, 2 hidden] = (up, gate): Hadamard block 32, quest RTN, clip mask
+hipError_t swiglu_quantize_hd32(const void* h12, int dtype, int64_t rows, int64_t hidden, uint32_t sign_word,
+                                uint8_t* codes, uint8_t* scales, uint8_t* maskbits, bool tiled, hipStream_t stream) {
+    if (rows == 0) return hipSuccess;
+    if (dtype == BF16)
+        launch_produced(SwiGluProducer<uint16_t>{reinterpret_cast<const uint16_t*>(h12)}, rows, hidden, sign_word, codes,
+                        scales, maskbits, tiled, stream);
+    else
+        launch_produced(SwiGluProducer<float>{reinterpret_cast<const float*>(h12)}, rows, hidden, sign_word, codes, scales,
+                        maskbits, tiled, stream);
+    return hipGetLastError();
+}
+
 // ---- two independent jobs per launch (the whole-layer entry points) ---------------------------------------------
 
 namespace {

@@ -1,0 +1,91 @@
+"""Producers fused into the activation quantizer of a Quartet linear.
+
+In the model the quantized linears sit in (src/models/llama.py of the reference) two of the four linears of a block are
+fed by RMSNorm (``c_attn(ln_1(x))``, ``w12(ln_2(x))``, llama.py:170-171) and one by the SwiGLU product
+(``c_proj(silu(up) * gate)``, llama.py:113-114).  ``rmsnorm_linear`` and ``swiglu_linear`` compute the same results
+without writing the normalised tensor / the product: the quantizer kernel builds each group of 32 values in registers,
+the layer consumes the packed operand, and the backward pass recomputes what it needs from the producer's inputs.
+
+Both fall back to the unfused composition (same mathematics, more memory traffic) when the layer is not in its
+production configuration, uses another Hadamard block than 32, or the tensors are not what the kernels take."""
+import torch
+import torch.nn.functional as F
+
+from . import kernels as K
+from .linear import QuantizedLinear, _backward_packed, _forward_packed, _use_tiled_codes
+from .quantizers.mxfp4 import _autocast_bf16
+
+_KERNEL_DTYPES = (torch.float32, torch.bfloat16)
+
+
+def _layer_is_fusable(layer):
+    return (isinstance(layer, QuantizedLinear) and layer._is_production_config() and layer.weight.is_cuda
+            and layer.activation_quantizer.hadamard_dim == 32 and layer.weight.dtype in _KERNEL_DTYPES)
+
+
+class RMSNormLinearFn(torch.autograd.Function):
+    """y = Q(rmsnorm(x) * gain) Q(W)^T; backward = the layer's quantized backward followed by RMSNorm's."""
+
+    @staticmethod
+    def forward(ctx, x, gain, weight, eps, a_q, w_q, g_q, weight_cache):
+        I = weight.shape[1]
+        x2 = x.reshape(-1, I).contiguous()
+        T, O = x2.shape[0], weight.shape[0]
+        tiled = _use_tiled_codes(T, I, O, a_q, w_q, g_q)
+        packed_x, factor = K.rmsnorm_quantize(x2, gain, eps, a_q.sign_bits, tiled)
+        # the normalised tensor times the fp32 gain is an fp32 tensor: that is the dtype the layer sees
+        out_dtype = torch.bfloat16 if _autocast_bf16() else torch.float32
+        y, packed_x, packed_w = _forward_packed(ctx, None, weight, a_q, w_q, g_q, weight_cache, tiled, out_dtype, torch.float32,
+                                                packed_x, T)
+        ctx.save_for_backward(x2, gain, factor, packed_x, packed_w)
+        ctx.x_shape = x.shape
+        return y.view(*x.shape[:-1], O)
+
+    @staticmethod
+    def backward(ctx, e):
+        x2, gain, factor, packed_x, packed_w = ctx.saved_tensors
+        gy, gw = _backward_packed(ctx, e, packed_x, packed_w)
+        dx, dgain = K.rmsnorm_backward(gy, x2, gain, factor)
+        return dx.view(ctx.x_shape), dgain, gw.to(ctx.w_dtype), None, None, None, None, None
+
+
+class SwiGLULinearFn(torch.autograd.Function):
+    """y = Q(silu(up) * gate) Q(W)^T with h12 = (up, gate); backward = the layer's quantized backward, then SwiGLU's."""
+
+    @staticmethod
+    def forward(ctx, h12, weight, a_q, w_q, g_q, weight_cache):
+        I = weight.shape[1]
+        h2 = h12.reshape(-1, 2 * I).contiguous()
+        T, O = h2.shape[0], weight.shape[0]
+        tiled = _use_tiled_codes(T, I, O, a_q, w_q, g_q)
+        packed_x = K.swiglu_quantize(h2, a_q.sign_bits, tiled)
+        out_dtype = torch.bfloat16 if _autocast_bf16() else h12.dtype
+        y, packed_x, packed_w = _forward_packed(ctx, None, weight, a_q, w_q, g_q, weight_cache, tiled, out_dtype, h12.dtype,
+                                                packed_x, T)
+        ctx.save_for_backward(h2, packed_x, packed_w)
+        ctx.h_shape = h12.shape
+        return y.view(*h12.shape[:-1], O)
+
+    @staticmethod
+    def backward(ctx, e):
+        h2, packed_x, packed_w = ctx.saved_tensors
+        g, gw = _backward_packed(ctx, e, packed_x, packed_w)
+        return K.swiglu_backward(g, h2).view(ctx.h_shape), gw.to(ctx.w_dtype), None, None, None, None
+
+
+def rmsnorm_linear(norm, layer, x):
+    """layer(norm(x)) for an RMSNorm module `norm` (attributes ``weight`` and ``eps``) and a QuantizedLinear."""
+    if (_layer_is_fusable(layer) and x.is_cuda and x.dtype in _KERNEL_DTYPES and norm.weight.dtype == torch.float32
+            and x.shape[-1] <= 8192):
+        return RMSNormLinearFn.apply(x, norm.weight, layer.weight, norm.eps, layer.activation_quantizer, layer.weight_quantizer,
+                                     layer.backward_scheme.g_quantizer, layer.packed_weight_cache)
+    return layer(norm(x))
+
+
+def swiglu_linear(layer, h12):
+    """layer(silu(up) * gate) with (up, gate) the two halves of h12's last dimension."""
+    if _layer_is_fusable(layer) and h12.is_cuda and h12.dtype in _KERNEL_DTYPES:
+        return SwiGLULinearFn.apply(h12, layer.weight, layer.activation_quantizer, layer.weight_quantizer,
+                                    layer.backward_scheme.g_quantizer, layer.packed_weight_cache)
+    up, gate = h12.split(h12.shape[-1] // 2, dim=-1)
+    return layer(F.silu(up) * gate)

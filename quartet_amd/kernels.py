@@ -150,26 +150,88 @@ def packed_operand_buffer(rows, cols, device):
     return torch.empty(_lib.lib().qm_packed_operand_bytes(rows, cols), dtype=torch.uint8, device=device)
 
 
-def linear_forward(x2, w2, hd_x, signs_x, hd_w, signs_w, out_dtype, tiled, packed_w=None):
+QM_W_IS_PACKED, QM_X_IS_PACKED = 1, 2
+
+
+def linear_forward(x2, w2, hd_x, signs_x, hd_w, signs_w, out_dtype, tiled, packed_w=None, packed_x=None, rows=None):
     """Whole forward pass of a Quartet linear in one foreign call: quantize x [T,I] and w [O,I] (quest RTN + clip
     mask), y = Q(x) Q(w)^T.  Returns (y [T,O], packed_x, packed_w): the byte buffers the backward pass reads.  A
     `packed_w` that an earlier call with the same weight, signs and layout returned is reused instead of quantizing
-    the weight again."""
-    _require_cuda(x2, w2, packed_w)
-    assert x2.is_contiguous() and w2.is_contiguous()
-    T, I = x2.shape
-    O = w2.shape[0]
+    the weight again; a `packed_x` written by a fused producer (rmsnorm_quantize, swiglu_quantize) of a [rows, I]
+    tensor replaces x2 (pass None)."""
+    _require_cuda(x2, w2, packed_w, packed_x)
+    assert w2.is_contiguous()
+    O, I = w2.shape
+    if packed_x is None:
+        assert x2.is_contiguous() and x2.shape[1] == I
+        T = x2.shape[0]
+    else:
+        assert x2 is None and rows is not None
+        T = rows
     L = _lib.lib()
-    packed_x = packed_operand_buffer(T, I, x2.device)
-    reuse = packed_w is not None
-    if not reuse:
-        packed_w = packed_operand_buffer(O, I, x2.device)
-    y = torch.empty((T, O), dtype=out_dtype, device=x2.device)
-    rc = L.qm_linear_forward(_ptr(x2), _dtype_code(x2.dtype), _ptr(w2), _dtype_code(w2.dtype), T, I, O, hd_x,
+    flags = (QM_W_IS_PACKED if packed_w is not None else 0) | (QM_X_IS_PACKED if packed_x is not None else 0)
+    if packed_x is None:
+        packed_x = packed_operand_buffer(T, I, w2.device)
+    if packed_w is None:
+        packed_w = packed_operand_buffer(O, I, w2.device)
+    y = torch.empty((T, O), dtype=out_dtype, device=w2.device)
+    rc = L.qm_linear_forward(_ptr(x2), _dtype_code(x2.dtype) if x2 is not None else 0, _ptr(w2), _dtype_code(w2.dtype), T, I, O, hd_x,
                              sign_words(signs_x), hd_w, sign_words(signs_w), _ptr(packed_x), packed_x.numel(), _ptr(packed_w),
-                             packed_w.numel(), int(reuse), _ptr(y), _dtype_code(out_dtype), _layout(tiled), _stream())
+                             packed_w.numel(), flags, _ptr(y), _dtype_code(out_dtype), _layout(tiled), _stream())
     _lib.check(rc, "qm_linear_forward")
     return y, packed_x, packed_w
+
+
+def rmsnorm_quantize(x2, gain, eps, signs, tiled):
+    """Q(rmsnorm(x2) * gain) without writing the normalised tensor: (packed operand buffer, per-row factor fp32)."""
+    _require_cuda(x2, gain)
+    assert x2.is_contiguous() and gain.is_contiguous() and gain.dtype == torch.float32 and gain.shape == (x2.shape[1],)
+    rows, cols = x2.shape
+    packed = packed_operand_buffer(rows, cols, x2.device)
+    factor = torch.empty(rows, dtype=torch.float32, device=x2.device)
+    rc = _lib.lib().qm_rmsnorm_quantize_mxfp4(_ptr(x2), _dtype_code(x2.dtype), _ptr(gain), float(eps), rows, cols, sign_words(signs),
+                                              _ptr(packed), packed.numel(), _ptr(factor), _layout(tiled), _stream())
+    _lib.check(rc, "qm_rmsnorm_quantize_mxfp4")
+    return packed, factor
+
+
+def swiglu_quantize(h12, signs, tiled):
+    """Q(silu(up) * gate) of h12 [rows, 2 hidden] = (up, gate) without writing the product: packed operand buffer."""
+    _require_cuda(h12)
+    assert h12.is_contiguous() and h12.shape[1] % 2 == 0
+    rows, hidden = h12.shape[0], h12.shape[1] // 2
+    packed = packed_operand_buffer(rows, hidden, h12.device)
+    rc = _lib.lib().qm_swiglu_quantize_mxfp4(_ptr(h12), _dtype_code(h12.dtype), rows, hidden, sign_words(signs), _ptr(packed),
+                                             packed.numel(), _layout(tiled), _stream())
+    _lib.check(rc, "qm_swiglu_quantize_mxfp4")
+    return packed
+
+
+def rmsnorm_backward(gy, x2, gain, factor):
+    """gy [rows, cols] (gradient of the normalised, scaled tensor) -> (dx like x2, dgain fp32 [cols])."""
+    _require_cuda(gy, x2, gain, factor)
+    assert gy.is_contiguous() and x2.is_contiguous() and gy.shape == x2.shape
+    rows, cols = x2.shape
+    L = _lib.lib()
+    nbytes = L.qm_rmsnorm_backward_workspace_bytes(rows, cols)
+    work = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=x2.device)
+    dx = torch.empty_like(x2)
+    dgain = torch.empty(cols, dtype=torch.float32, device=x2.device)
+    rc = L.qm_rmsnorm_backward(_ptr(gy), _dtype_code(gy.dtype), _ptr(x2), _dtype_code(x2.dtype), _ptr(gain), _ptr(factor), rows, cols,
+                               _ptr(dx), _ptr(dgain), _ptr(work), nbytes, _stream())
+    _lib.check(rc, "qm_rmsnorm_backward")
+    return dx, dgain
+
+
+def swiglu_backward(g, h12):
+    """g [rows, hidden] (gradient of silu(up) * gate) -> gradient of h12 [rows, 2 hidden], in h12's dtype."""
+    _require_cuda(g, h12)
+    assert g.is_contiguous() and h12.is_contiguous() and h12.shape == (g.shape[0], 2 * g.shape[1])
+    d = torch.empty_like(h12)
+    rc = _lib.lib().qm_swiglu_backward(_ptr(g), _dtype_code(g.dtype), _ptr(h12), _dtype_code(h12.dtype), g.shape[0], g.shape[1],
+                                       _ptr(d), _stream())
+    _lib.check(rc, "qm_swiglu_backward")
+    return d
 
 
 def linear_backward(e2, packed_x, packed_w, T, I, O, hd_x, signs_x, hd_w, signs_w, hd_g, signs_g, mode, seeds, x_val_dtype,

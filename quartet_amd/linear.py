@@ -16,6 +16,51 @@ from .quantizers import QUANTIZER_CLASSES, AlbertTsengQuantizer, NoQuantizer, Qu
 from .quantizers.mxfp4 import _autocast_bf16, _fresh_seed
 
 
+def _use_tiled_codes(T, I, O, a_q, w_q, g_q):
+    """Tiled code bytes (16 rows x 128 elements contiguous) when every operand of the three products qualifies: all
+    three extents multiples of 128 and at least 256, Hadamard block 32 throughout; row-major codes otherwise."""
+    return (all(d % 128 == 0 and d >= 256 for d in (T, I, O)) and
+            a_q.hadamard_dim == 32 and w_q.hadamard_dim == 32 and g_q.hadamard_dim == 32)
+
+
+def _forward_packed(ctx, x2, weight, a_q, w_q, g_q, weight_cache, tiled, out_dtype, x_dtype, packed_x=None, rows=None):
+    """F1 (unless a producer already wrote packed_x), F2 (unless the layer's cache holds Q(W)), F3; records on ctx what
+    the backward pass of the products needs.  Returns (y [T, O], packed_x, packed_w)."""
+    w2 = weight.contiguous()
+    # Q(W) of an unchanged weight (the micro-steps of one accumulation) is quantized once and kept by the layer
+    key = (weight.data_ptr(), weight._version, weight.dtype, tuple(weight.shape), w_q.hadamard_dim, w_q.sign_bits, tiled)
+    packed_w = weight_cache.get(key) if weight_cache is not None else None
+    y, packed_x, packed_w = K.linear_forward(x2, w2, a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits,
+                                             out_dtype, tiled, packed_w, packed_x, rows)
+    if weight_cache is not None:
+        weight_cache.put(key, packed_w)
+    ctx.g_q = g_q
+    ctx.tiled = tiled
+    ctx.fwd = (a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits)
+    ctx.dims = (y.shape[0], weight.shape[1], weight.shape[0])
+    ctx.x_dtype, ctx.w_dtype = x_dtype, weight.dtype
+    return y, packed_x, packed_w
+
+
+def _backward_packed(ctx, e, packed_x, packed_w):
+    """B1-B8: e [.., O] -> (gradient w.r.t. the tensor F1 quantized [T, I], gradient w.r.t. W [O, I])."""
+    g_q = ctx.g_q
+    a_hd, a_signs, w_hd, w_signs = ctx.fwd
+    T, I, O = ctx.dims
+    g_q.re_randomize()
+    hd, signs = g_q.hadamard_dim, g_q.sign_bits
+    mode = K.QM_ABSMAX_SR if g_q.stochastic else K.QM_ABSMAX_RTN
+    # one host-side draw per stochastic quantization, in the order e, W^T, e^T, x^T
+    seeds = [_fresh_seed() if g_q.stochastic else 0 for _ in range(4)]
+    e2 = e.reshape(-1, e.shape[-1]).contiguous()
+    low = _autocast_bf16() or e2.dtype == torch.bfloat16
+    mid_dtype = torch.bfloat16 if low else e2.dtype
+    sd_x = torch.bfloat16 if low else ctx.x_dtype
+    sd_w = torch.bfloat16 if low else ctx.w_dtype
+    return K.linear_backward(e2, packed_x, packed_w, T, I, O, a_hd, a_signs, w_hd, w_signs, hd, signs, mode, seeds, ctx.x_dtype,
+                             ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled)
+
+
 class QuartetLinearFn(torch.autograd.Function):
     """y = Q(x) Q(W)^T with the fully quantized backward of backward.py:57-85, on packed operands.
 
@@ -28,45 +73,17 @@ class QuartetLinearFn(torch.autograd.Function):
     def forward(ctx, x, weight, a_q, w_q, g_q, weight_cache):
         in_features = weight.shape[1]
         x2 = x.reshape(-1, in_features).contiguous()
-        w2 = weight.contiguous()
         out_dtype = torch.bfloat16 if _autocast_bf16() else x.dtype
-        # Tiled code bytes (16 rows x 128 elements contiguous) when every operand of the three products qualifies:
-        # all three extents multiples of 128 and at least 256, Hadamard block 32 throughout; row-major codes otherwise.
-        tiled = (all(d % 128 == 0 and d >= 256 for d in (x2.shape[0], in_features, weight.shape[0])) and
-                 a_q.hadamard_dim == 32 and w_q.hadamard_dim == 32 and g_q.hadamard_dim == 32)
-        # Q(W) of an unchanged weight (the micro-steps of one accumulation) is quantized once and kept by the layer
-        key = (weight.data_ptr(), weight._version, weight.dtype, tuple(weight.shape), w_q.hadamard_dim, w_q.sign_bits, tiled)
-        packed_w = weight_cache.get(key) if weight_cache is not None else None
-        y, packed_x, packed_w = K.linear_forward(x2, w2, a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits,
-                                                 out_dtype, tiled, packed_w)
-        if weight_cache is not None:
-            weight_cache.put(key, packed_w)
+        tiled = _use_tiled_codes(x2.shape[0], in_features, weight.shape[0], a_q, w_q, g_q)
+        y, packed_x, packed_w = _forward_packed(ctx, x2, weight, a_q, w_q, g_q, weight_cache, tiled, out_dtype, x.dtype)
         ctx.save_for_backward(packed_x, packed_w)
-        ctx.g_q = g_q
-        ctx.tiled = tiled
-        ctx.fwd = (a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits)
-        ctx.dims = (x2.shape[0], in_features, weight.shape[0])
-        ctx.x_shape, ctx.x_dtype, ctx.w_dtype = x.shape, x.dtype, weight.dtype
+        ctx.x_shape = x.shape
         return y.view(*x.shape[:-1], weight.shape[0])
 
     @staticmethod
     def backward(ctx, e):
         packed_x, packed_w = ctx.saved_tensors
-        g_q = ctx.g_q
-        a_hd, a_signs, w_hd, w_signs = ctx.fwd
-        T, I, O = ctx.dims
-        g_q.re_randomize()
-        hd, signs = g_q.hadamard_dim, g_q.sign_bits
-        mode = K.QM_ABSMAX_SR if g_q.stochastic else K.QM_ABSMAX_RTN
-        # one host-side draw per stochastic quantization, in the order e, W^T, e^T, x^T
-        seeds = [_fresh_seed() if g_q.stochastic else 0 for _ in range(4)]
-        e2 = e.reshape(-1, e.shape[-1]).contiguous()
-        low = _autocast_bf16() or e2.dtype == torch.bfloat16
-        mid_dtype = torch.bfloat16 if low else e2.dtype
-        sd_x = torch.bfloat16 if low else ctx.x_dtype
-        sd_w = torch.bfloat16 if low else ctx.w_dtype
-        gx, gw = K.linear_backward(e2, packed_x, packed_w, T, I, O, a_hd, a_signs, w_hd, w_signs, hd, signs, mode, seeds, ctx.x_dtype,
-                                   ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled)
+        gx, gw = _backward_packed(ctx, e, packed_x, packed_w)
         return gx.to(ctx.x_dtype).view(ctx.x_shape), gw.to(ctx.w_dtype), None, None, None, None
 
 

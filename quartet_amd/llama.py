@@ -18,6 +18,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .backward import BACKWARD_SCHEMES
+from .fused import rmsnorm_linear, swiglu_linear
 from .linear import QuantizedLinear
 from .quantizers import QUANTIZER_CLASSES
 
@@ -43,6 +44,9 @@ class LlamaConfig:
     g_quant_kwargs: dict = field(default_factory=lambda: {"hadamard_dim": 32, "stochastic": True, "rerotate": "signs"})
     backward_scheme: str = "Q(E)Q(Wt)t_Q(Et)Q(Xt)t"
     backward_scheme_kwargs: dict = field(default_factory=dict)
+    # not in the reference: RMSNorm and the SwiGLU product are computed inside the activation quantizer of the linear
+    # they feed (quartet_amd.fused) instead of being written out; False runs the reference's op-by-op composition
+    fuse_producers: bool = True
 
     @property
     def ffn_dim(self):
@@ -117,7 +121,10 @@ class LlamaMLP(nn.Module):
         self.w12 = _linear(config, config.n_embd, 2 * self.hidden_dim)
         self.c_proj = _linear(config, self.hidden_dim, config.n_embd)
 
-    def forward(self, x):
+    def forward(self, x, norm=None):
+        """`norm`: the block's RMSNorm, applied to x here (fused into w12's quantizer) instead of by the caller."""
+        if norm is not None:
+            return swiglu_linear(self.c_proj, rmsnorm_linear(norm, self.w12, x))
         up, gate = self.w12(x).split(self.hidden_dim, dim=-1)
         return self.c_proj(F.silu(up) * gate)
 
@@ -131,10 +138,11 @@ class LlamaAttention(nn.Module):
         self.resid_dropout = nn.Dropout(config.dropout)
         self.n_head, self.n_embd, self.dropout = config.n_head, config.n_embd, config.dropout
 
-    def forward(self, x, table):
+    def forward(self, x, table, norm=None):
         B, T, C = x.shape
         hs = C // self.n_head
-        q, k, v = self.c_attn(x).split(self.n_embd, dim=2)
+        qkv = self.c_attn(x) if norm is None else rmsnorm_linear(norm, self.c_attn, x)
+        q, k, v = qkv.split(self.n_embd, dim=2)
         q, k = apply_rotary(q.view(B, T, self.n_head, hs), k.view(B, T, self.n_head, hs), table)
         q, k = q.transpose(1, 2), k.transpose(1, 2)
         v = v.view(B, T, self.n_head, hs).transpose(1, 2)
@@ -152,8 +160,12 @@ class LlamaBlock(nn.Module):
         self.attn = LlamaAttention(config)
         self.ln_2 = RMSNorm(config.n_embd, eps=config.rmsnorm_eps)
         self.mlp = LlamaMLP(config)
+        self.fuse_producers = config.fuse_producers
 
     def forward(self, x, table):
+        if self.fuse_producers:
+            x = x + self.attn(x, table, norm=self.ln_1)
+            return x + self.mlp(x, norm=self.ln_2)
         x = x + self.attn(self.ln_1(x), table)
         return x + self.mlp(self.ln_2(x))
 

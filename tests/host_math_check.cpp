@@ -109,6 +109,32 @@ int main() {
         hadamard_scale(128, BF16) != 0.08837890625f || hadamard_scale(32, F32) != (float)std::sqrt(1.0 / 32.0))
         fail("hadamard_scale", 0);
 
+    // e^z with the fixed instruction sequence: within 1.5 ulp of the exact value wherever that is a normal number,
+    // exact at 0, +inf above ln(FLT_MAX), and silu's limits; hashes over every bf16 input let the caller compare
+    // bit for bit with another implementation of the same sequence
+    uint64_t exp_hash = 1469598103934665603ull, silu_hash = 1469598103934665603ull;
+    for (uint32_t h = 0; h < 65536; ++h) {
+        const float z = bf16_to_f32((uint16_t)h);
+        if (std::isnan(z)) continue;
+        const float e = exp_fixed(z);
+        exp_hash = (exp_hash ^ f2u(e)) * 1099511628211ull;
+        silu_hash = (silu_hash ^ f2u(silu_fixed(z))) * 1099511628211ull;
+        const double t = std::exp((double)z);
+        if (t > 3.4028234663852886e38) { if (!(e == INFINITY || e > 3.3e38f)) fail("exp overflow", h); continue; }
+        if (t < 1.1754943508222875e-38) { if (!(e >= 0.0f && e < 1.2e-38f)) fail("exp underflow", h); continue; }
+        const double ulp = std::ldexp(1.0, std::ilogb(t) - 23);
+        if (std::fabs((double)e - t) > 1.5 * ulp) fail("exp accuracy", h);
+    }
+    for (uint32_t i = 0; i < 2000000; ++i) {
+        const float z = -104.0f + 193.0f * (float)i / 2000000.0f;
+        const double t = std::exp((double)z);
+        if (t > 3.4e38 || t < 1.2e-38) continue;
+        if (std::fabs((double)exp_fixed(z) - t) > 1.5 * std::ldexp(1.0, std::ilogb(t) - 23)) fail("exp accuracy (sweep)", i);
+    }
+    if (exp_fixed(0.0f) != 1.0f || exp_fixed(89.0f) != INFINITY || exp_fixed(-200.0f) != 0.0f) fail("exp special values", 0);
+    if (silu_fixed(0.0f) != 0.0f || silu_fixed(100.0f) != 100.0f || f2u(silu_fixed(-200.0f)) != 0x80000000u) fail("silu limits", 0);
+    std::printf("exp_hash=%016llx silu_hash=%016llx\n", (unsigned long long)exp_hash, (unsigned long long)silu_hash);
+
     if (failures) {
         std::printf("%d failures\n", failures);
         return 1;

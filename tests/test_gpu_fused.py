@@ -1,0 +1,231 @@
+"""GPU parity of the producers fused into the activation quantizer (RMSNorm -> F1, SwiGLU -> F1) and of their backward
+kernels: packed operands bit-exact against the oracle, whole layers bit-exact against the unfused layer fed with the
+oracle's producer output, backward passes against float64 autograd of the reference's formulas."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from tests.util import from_oracle_bf16, make_input, sign_int, to_oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def q():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import quartet_amd
+    return quartet_amd
+
+
+def unpack(q, buffer, rows, cols, tiled):
+    """(codes, scales, mask bits) of a packed operand buffer as row-major numpy arrays."""
+    from quartet_amd import packed as P
+    t = P.from_operand_buffer(buffer, rows, cols, tiled, q.QuestMXFP4Quantizer()).to_layout("rowmajor")
+    return t.codes.cpu().numpy(), t.scales.cpu().numpy(), t.maskbits.cpu().numpy()
+
+
+def signs_vector(seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, 2, (32,), generator=g) * 2 - 1
+
+
+def rel(a, b):
+    a, b = a.double(), b.double()
+    return float((a - b).norm() / b.norm())
+
+
+# rows x cols: tiled (several groups per lane, a ragged last chunk of 4 groups), and row-major shapes with rows that do
+# not fill a workgroup and a single group per row
+SHAPES = [(256, 640, True), (512, 1536, True), (64, 4096, True), (100, 96, False), (7, 32, False), (48, 1728, False)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,cols,tiled", SHAPES)
+def test_rmsnorm_quantize_against_oracle(oracle, q, rows, cols, tiled, dtype):
+    print(f"case rmsnorm_quantize rows={rows} cols={cols} tiled={tiled} dtype={dtype}", flush=True)
+    from quartet_amd import kernels as K
+    x = make_input(rows, cols, dtype, seed=rows + cols, scale=3.0, zero_rows=1)
+    gain = (1.0 + 0.2 * torch.randn(cols, generator=torch.Generator().manual_seed(1))).float()
+    signs = signs_vector(cols)
+    eps = 1e-5
+    normed, factor = oracle.rmsnorm(to_oracle(x), gain.numpy(), eps)
+    want = oracle.quantize(normed, 32, signs=signs.numpy(), mode=oracle.QUEST_RTN, want_mask=True)
+    packed, got_factor = K.rmsnorm_quantize(x.to(DEV), gain.to(DEV), eps, sign_int(signs), tiled)
+    assert np.array_equal(got_factor.cpu().numpy().view(np.uint32), factor.view(np.uint32))
+    codes, scales, mask = unpack(q, packed, rows, cols, tiled)
+    assert np.array_equal(scales, want["scales"])
+    assert np.array_equal(codes, want["codes"])
+    assert np.array_equal(mask, want["mask"])
+    # the same packed operand as the stand-alone quantizer produces from the oracle's normalised tensor
+    direct = K.quantize_mxfp4(torch.from_numpy(normed).to(DEV), 32, sign_int(signs), K.QM_QUEST_RTN, want_mask=True, tiled=False)
+    assert np.array_equal(direct[0].cpu().numpy(), codes) and np.array_equal(direct[2].cpu().numpy(), mask)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,hidden,tiled", SHAPES)
+def test_swiglu_quantize_against_oracle(oracle, q, rows, hidden, tiled, dtype):
+    print(f"case swiglu_quantize rows={rows} hidden={hidden} tiled={tiled} dtype={dtype}", flush=True)
+    from quartet_amd import kernels as K
+    h12 = make_input(rows, 2 * hidden, dtype, seed=rows * 3 + hidden, scale=2.0, outlier_frac=1e-3, zero_rows=1)
+    h12[-1, :8] = torch.tensor([-200.0, 200.0, -95.0, 95.0, -88.0, 88.0, 0.0, -0.0]).to(dtype)   # e^-x overflows / vanishes
+    signs = signs_vector(hidden + 1)
+    prod = oracle.swiglu(to_oracle(h12))
+    want = oracle.quantize(prod, 32, signs=signs.numpy(), mode=oracle.QUEST_RTN, want_mask=True)
+    packed = K.swiglu_quantize(h12.to(DEV), sign_int(signs), tiled)
+    codes, scales, mask = unpack(q, packed, rows, hidden, tiled)
+    assert np.array_equal(scales, want["scales"])
+    assert np.array_equal(codes, want["codes"])
+    assert np.array_equal(mask, want["mask"])
+
+
+@pytest.mark.parametrize("gy_dtype,x_dtype", [(torch.bfloat16, torch.float32), (torch.float32, torch.float32),
+                                              (torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("rows,cols", [(256, 640), (1000, 1536), (70, 4096), (3, 32)])
+def test_rmsnorm_backward_against_float64_autograd(q, rows, cols, gy_dtype, x_dtype):
+    print(f"case rmsnorm_backward rows={rows} cols={cols} gy={gy_dtype} x={x_dtype}", flush=True)
+    from quartet_amd import kernels as K
+    x = make_input(rows, cols, x_dtype, seed=rows, scale=2.0, outlier_frac=0)
+    gy = make_input(rows, cols, gy_dtype, seed=rows + 1, scale=1e-2, outlier_frac=0)
+    gain = (1.0 + 0.2 * torch.randn(cols, generator=torch.Generator().manual_seed(2))).float()
+    eps = 1e-5
+    xd = x.double().requires_grad_(True)
+    gd = gain.double().requires_grad_(True)
+    y = xd * torch.rsqrt(xd.pow(2).mean(-1, keepdim=True) + eps) * gd      # llama.py:64-75 in float64
+    y.backward(gy.double())
+    factor = torch.rsqrt(x.double().pow(2).mean(-1) + eps).float()
+    dx, dgain = K.rmsnorm_backward(gy.to(DEV), x.to(DEV), gain.to(DEV), factor.to(DEV))
+    assert dx.dtype == x_dtype and dgain.dtype == torch.float32
+    assert rel(dx.cpu(), xd.grad) < (4e-3 if x_dtype == torch.bfloat16 else 2e-6)
+    assert rel(dgain.cpu(), gd.grad) < 2e-5
+    # reproducible: the column sums are added in a fixed order
+    dx2, dgain2 = K.rmsnorm_backward(gy.to(DEV), x.to(DEV), gain.to(DEV), factor.to(DEV))
+    assert torch.equal(dgain, dgain2) and torch.equal(dx, dx2)
+
+
+@pytest.mark.parametrize("g_dtype,h_dtype", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32),
+                                             (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("rows,hidden", [(256, 1728), (33, 4096), (5, 32)])
+def test_swiglu_backward_against_autograd(q, rows, hidden, g_dtype, h_dtype):
+    print(f"case swiglu_backward rows={rows} hidden={hidden} g={g_dtype} h={h_dtype}", flush=True)
+    from quartet_amd import kernels as K
+    h12 = make_input(rows, 2 * hidden, h_dtype, seed=rows, scale=2.0, outlier_frac=1e-3)
+    g = make_input(rows, hidden, g_dtype, seed=rows + 7, scale=1e-2, outlier_frac=0)
+    hd_ = h12.double().requires_grad_(True)
+    up, gate = hd_.split(hidden, dim=-1)
+    (F.silu(up) * gate).backward(g.double())
+    got = K.swiglu_backward(g.to(DEV), h12.to(DEV))
+    assert got.dtype == h_dtype and got.shape == h12.shape
+    tol = 6e-3 if h_dtype == torch.bfloat16 else 2e-6
+    assert rel(got[:, :hidden].cpu(), hd_.grad[:, :hidden]) < tol
+    assert rel(got[:, hidden:].cpu(), hd_.grad[:, hidden:]) < tol
+    if h_dtype == torch.bfloat16:
+        # element-wise: within two bf16 steps of autograd run op by op in bf16, as the unfused model does
+        hb = h12.clone().to(DEV).requires_grad_(True)
+        ub, gb = hb.split(hidden, dim=-1)
+        (F.silu(ub) * gb).backward(g.to(DEV).to(torch.bfloat16))
+        diff = (got.float() - hb.grad.float()).abs()
+        assert bool((diff <= 2.0 ** -6 * hb.grad.float().abs() + 1e-30).all())
+
+
+def production_layer(q, I, O, dtype):
+    return q.QuantizedLinear(I, O, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(),
+                             activation_quantizer=q.QuestMXFP4Quantizer(),
+                             gradient_quantizer=q.AlbertTsengQuantizer(stochastic=False, rerotate=None),
+                             backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]()).to(DEV, dtype)
+
+
+@pytest.mark.parametrize("autocast", [True, False])
+@pytest.mark.parametrize("T,I,O", [(256, 640, 1920), (96, 160, 224)])
+def test_rmsnorm_linear_matches_the_unfused_layer(oracle, q, T, I, O, autocast):
+    """The fused layer against the same layer called on the oracle's normalised tensor: identical packed operands, so
+    identical outputs and weight gradients; the gradient w.r.t. x against float64 autograd of RMSNorm applied to the
+    unfused layer's input gradient."""
+    print(f"case rmsnorm_linear T={T} I={I} O={O} autocast={autocast}", flush=True)
+    from quartet_amd.fused import rmsnorm_linear
+    from quartet_amd.llama import RMSNorm
+    torch.manual_seed(0)
+    layer = production_layer(q, I, O, torch.float32)
+    norm = RMSNorm(I, eps=1e-5).to(DEV)
+    with torch.no_grad():
+        norm.weight.add_(0.1 * torch.randn(I, device=DEV))
+    x = make_input(2 * (T // 2), I, torch.float32, seed=4, scale=2.0).view(2, T // 2, I).to(DEV)
+    dy = make_input(T, O, torch.bfloat16 if autocast else torch.float32, seed=5, scale=1e-2, outlier_frac=0).view(2, T // 2, O).to(DEV)
+    ctx = (lambda: torch.autocast("cuda", dtype=torch.bfloat16)) if autocast else (lambda: torch.autocast("cuda", enabled=False))
+
+    xf = x.clone().requires_grad_(True)
+    with ctx():
+        y = rmsnorm_linear(norm, layer, xf)
+        y.backward(dy)
+    got = (y.detach(), xf.grad, layer.weight.grad.clone(), norm.weight.grad.clone())
+    layer.weight.grad = None
+    norm.weight.grad = None
+
+    normed, _ = oracle.rmsnorm(x.view(T, I).cpu().numpy(), norm.weight.detach().cpu().numpy(), 1e-5)
+    n = torch.from_numpy(normed).view(2, T // 2, I).to(DEV).requires_grad_(True)
+    with ctx():
+        y_ref = layer(n)
+        y_ref.backward(dy)
+    assert y.dtype == y_ref.dtype and torch.equal(got[0], y_ref.detach())
+    assert torch.equal(got[2], layer.weight.grad)
+    xd = x.double().requires_grad_(True)
+    gd = norm.weight.detach().double().requires_grad_(True)
+    (xd * torch.rsqrt(xd.pow(2).mean(-1, keepdim=True) + 1e-5) * gd).backward(n.grad.double())
+    assert got[1].dtype == torch.float32 and rel(got[1], xd.grad) < 1e-5
+    assert rel(got[3], gd.grad) < 1e-4
+
+
+@pytest.mark.parametrize("autocast", [True, False])
+@pytest.mark.parametrize("T,I,O", [(256, 1792, 640), (64, 96, 160)])
+def test_swiglu_linear_matches_the_unfused_layer(oracle, q, T, I, O, autocast):
+    print(f"case swiglu_linear T={T} hidden={I} O={O} autocast={autocast}", flush=True)
+    from quartet_amd.fused import swiglu_linear
+    torch.manual_seed(0)
+    layer = production_layer(q, I, O, torch.float32)
+    dtype = torch.bfloat16 if autocast else torch.float32    # w12's output dtype under autocast
+    h12 = make_input(T, 2 * I, dtype, seed=6, scale=2.0).to(DEV)
+    dy = make_input(T, O, dtype, seed=7, scale=1e-2, outlier_frac=0).to(DEV)
+    ctx = (lambda: torch.autocast("cuda", dtype=torch.bfloat16)) if autocast else (lambda: torch.autocast("cuda", enabled=False))
+
+    hf = h12.clone().requires_grad_(True)
+    with ctx():
+        y = swiglu_linear(layer, hf)
+        y.backward(dy)
+    got = (y.detach(), hf.grad, layer.weight.grad.clone())
+    layer.weight.grad = None
+
+    prod = oracle.swiglu(to_oracle(h12))
+    p = (from_oracle_bf16(prod) if autocast else torch.from_numpy(prod)).to(DEV).requires_grad_(True)
+    with ctx():
+        y_ref = layer(p)
+        y_ref.backward(dy)
+    assert torch.equal(got[0], y_ref.detach())
+    assert torch.equal(got[2], layer.weight.grad)
+    hd_ = h12.double().requires_grad_(True)
+    up, gate = hd_.split(I, dim=-1)
+    (F.silu(up) * gate).backward(p.grad.double())
+    assert got[1].dtype == dtype and rel(got[1], hd_.grad) < (6e-3 if autocast else 1e-5)
+
+
+def test_fallbacks_keep_the_unfused_composition(q):
+    """A layer that is not in its production configuration (or a Hadamard block other than 32) takes the op-by-op
+    path and gives what layer(norm(x)) / layer(silu(up) * gate) give."""
+    from quartet_amd.fused import rmsnorm_linear, swiglu_linear
+    from quartet_amd.llama import RMSNorm
+    torch.manual_seed(1)
+    plain = q.QuantizedLinear(64, 96, bias=False).to(DEV)            # identity quantizers, plain scheme
+    wide = q.QuantizedLinear(128, 96, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(hadamard_dim=64),
+                             activation_quantizer=q.QuestMXFP4Quantizer(hadamard_dim=64),
+                             gradient_quantizer=q.AlbertTsengQuantizer(hadamard_dim=64, stochastic=False),
+                             backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]()).to(DEV)
+    for layer, I in ((plain, 64), (wide, 128)):
+        norm = RMSNorm(I).to(DEV)
+        x = torch.randn(32, I, device=DEV)
+        assert torch.equal(rmsnorm_linear(norm, layer, x), layer(norm(x)))
+        h12 = torch.randn(32, 2 * I, device=DEV)
+        up, gate = h12.split(I, dim=-1)
+        assert torch.equal(swiglu_linear(layer, h12), layer(F.silu(up) * gate))

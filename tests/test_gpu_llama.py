@@ -85,6 +85,39 @@ def test_llama_ragged_batch_shapes(models):
     assert all(torch.isfinite(p.grad).all() for p in quartet.parameters())
 
 
+def test_fused_producers_agree_with_the_op_by_op_model(models):
+    """RMSNorm and SwiGLU folded into the activation quantizers (the default) against the same model running them as
+    separate torch ops: the two differ only by the last-place differences between torch's rsqrt / exp and the kernels'
+    fixed instruction sequences, which flip a few FP4 codes -- losses agree closely, weight gradients of every linear
+    and of the norms stay aligned."""
+    L, quartet, bwd_only, plain, idx, tgt = models
+    print("case llama30m fused vs op-by-op producers", flush=True)
+    assert quartet.config.fuse_producers
+    g_q = L.llama_30m().g_quant_kwargs
+    det = dict(g_quant_kwargs={**g_q, "stochastic": False, "rerotate": None})   # deterministic backward for the comparison
+    fused = L.Llama(L.llama_30m(**det)).to(idx.device)
+    unfused = L.Llama(L.llama_30m(fuse_producers=False, **det)).to(idx.device)
+    fused.load_state_dict(copy.deepcopy(plain.state_dict()), strict=False)
+    unfused.load_state_dict(copy.deepcopy(plain.state_dict()), strict=False)
+    with torch.no_grad():   # gains away from 1 so that their gradients matter
+        for m in (fused, unfused):
+            torch.manual_seed(3)
+            for blk in m.transformer.h:
+                blk.ln_1.weight.add_(0.1 * torch.randn_like(blk.ln_1.weight))
+                blk.ln_2.weight.add_(0.1 * torch.randn_like(blk.ln_2.weight))
+    lf, lu = _step(fused, idx[:4], tgt[:4]), _step(unfused, idx[:4], tgt[:4])
+    torch.cuda.synchronize()
+    assert abs(lf - lu) < 2e-3, (lf, lu)
+    pf, pu = dict(fused.named_parameters()), dict(unfused.named_parameters())
+    worst = 1.0
+    for name in pf:
+        a, b = pf[name].grad.float().flatten(), pu[name].grad.float().flatten()
+        assert torch.isfinite(a).all(), name
+        worst = min(worst, float(torch.dot(a, b) / (a.norm() * b.norm())))
+    print(f"fused vs op-by-op: losses {lf:.5f} {lu:.5f}, worst gradient cosine {worst:.4f}", flush=True)
+    assert worst > 0.9
+
+
 def test_quartet_model_learns_with_the_training_loop():
     """A small all-Quartet Llama (every block linear on the packed FP4 path, tiled codes) trained with the
     reference-style loop -- bf16 autocast around forward and backward, two micro-steps per update, AdamW with
