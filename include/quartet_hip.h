@@ -192,6 +192,21 @@ int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype
 int qm_swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
                        void* d_h12, void* stream);
 
+/*
+ * Rotary position embedding around the attention that sits between two quantized linears (apply_rotary_emb,
+ * src/models/llama.py:43-61, called at llama.py:141-143 on the split of c_attn's output).
+ * qm_rope_split_qkv: qkv [rows, 3 n_embd] = (q, k, v) -> q, k, v [rows, n_embd] of out_dtype; in every head of q and k
+ *   the pairs (2i, 2i+1) are rotated by the angle of table[r % seq_len, i] = (cos, sin), in fp32 with every product and
+ *   sum rounded (the reference's op-by-op arithmetic); v is copied (converted).  table: fp32 [seq_len, head_dim/2, 2].
+ * qm_rope_merge_qkv_grad: the backward pass: gradients dq, dk, dv [rows, n_embd] of grad_dtype -> d_qkv [rows, 3 n_embd]
+ *   of out_dtype, dq and dk rotated by the negative angle.
+ * head_dim % 8 == 0, n_embd % head_dim == 0.
+ */
+int qm_rope_split_qkv(const void* qkv, int qkv_dtype, int64_t rows, int64_t seq_len, int64_t n_embd, int head_dim,
+                      const float* table, void* q, void* k, void* v, int out_dtype, void* stream);
+int qm_rope_merge_qkv_grad(const void* dq, const void* dk, const void* dv, int grad_dtype, int64_t rows, int64_t seq_len,
+                           int64_t n_embd, int head_dim, const float* table, void* d_qkv, int out_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

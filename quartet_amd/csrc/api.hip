@@ -417,4 +417,41 @@ int qm_swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, i
                     "qm_swiglu_backward");
 }
 
+namespace {
+int check_rope(const char* who, int dtype_a, int dtype_b, int64_t rows, int64_t seq_len, int64_t n_embd, int head_dim) {
+    if (!valid_dtype(dtype_a) || !valid_dtype(dtype_b)) return fail(QM_ERR_INVALID, "%s: dtypes must be QM_BF16/QM_F32", who);
+    if (rows < 0 || seq_len <= 0 || n_embd <= 0 || head_dim <= 0 || head_dim % 8 || n_embd % head_dim || n_embd > (1 << 24) ||
+        seq_len > (1 << 30))
+        return fail(QM_ERR_INVALID, "%s: need rows >= 0, seq_len > 0, head_dim a positive multiple of 8 and n_embd a multiple of "
+                                    "head_dim (rows=%lld seq_len=%lld n_embd=%lld head_dim=%d)",
+                    who, (long long)rows, (long long)seq_len, (long long)n_embd, head_dim);
+    return 0;
+}
+}  // namespace
+
+int qm_rope_split_qkv(const void* qkv, int qkv_dtype, int64_t rows, int64_t seq_len, int64_t n_embd, int head_dim,
+                      const float* table, void* q, void* k, void* v, int out_dtype, void* stream) {
+    if (int rc = check_rope("qm_rope_split_qkv", qkv_dtype, out_dtype, rows, seq_len, n_embd, head_dim)) return rc;
+    if (rows == 0) return 0;
+    if (!qkv || !table || !q || !k || !v) return fail(QM_ERR_INVALID, "qm_rope_split_qkv: qkv, table, q, k, v must be non-null");
+    if (!aligned(qkv, 16) || !aligned(table, 16) || !aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16))
+        return fail(QM_ERR_UNALIGNED, "qm_rope_split_qkv: tensors need 16-byte alignment");
+    return from_hip(qm::rope_split_qkv(qkv, qkv_dtype, rows, (int)seq_len, (int)n_embd, head_dim, table, q, k, v, out_dtype,
+                                       reinterpret_cast<hipStream_t>(stream)),
+                    "qm_rope_split_qkv");
+}
+
+int qm_rope_merge_qkv_grad(const void* dq, const void* dk, const void* dv, int grad_dtype, int64_t rows, int64_t seq_len,
+                           int64_t n_embd, int head_dim, const float* table, void* d_qkv, int out_dtype, void* stream) {
+    if (int rc = check_rope("qm_rope_merge_qkv_grad", grad_dtype, out_dtype, rows, seq_len, n_embd, head_dim)) return rc;
+    if (rows == 0) return 0;
+    if (!dq || !dk || !dv || !table || !d_qkv)
+        return fail(QM_ERR_INVALID, "qm_rope_merge_qkv_grad: dq, dk, dv, table, d_qkv must be non-null");
+    if (!aligned(dq, 16) || !aligned(dk, 16) || !aligned(dv, 16) || !aligned(table, 16) || !aligned(d_qkv, 16))
+        return fail(QM_ERR_UNALIGNED, "qm_rope_merge_qkv_grad: tensors need 16-byte alignment");
+    return from_hip(qm::rope_merge_qkv_grad(dq, dk, dv, grad_dtype, rows, (int)seq_len, (int)n_embd, head_dim, table, d_qkv, out_dtype,
+                                            reinterpret_cast<hipStream_t>(stream)),
+                    "qm_rope_merge_qkv_grad");
+}
+
 }  // extern "C"

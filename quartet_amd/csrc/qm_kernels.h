@@ -87,6 +87,12 @@ hipError_t rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_d
 hipError_t swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
                            void* d_h12, hipStream_t stream);
 
+// Rotary embedding of the fused attention projection: split + rotate, and the merge + inverse rotation of its backward
+hipError_t rope_split_qkv(const void* qkv, int qkv_dtype, int64_t rows, int seq_len, int C, int head_dim, const float* table,
+                          void* q, void* k, void* v, int out_dtype, hipStream_t stream);
+hipError_t rope_merge_qkv_grad(const void* dq, const void* dk, const void* dv, int grad_dtype, int64_t rows, int seq_len, int C,
+                               int head_dim, const float* table, void* d_qkv, int out_dtype, hipStream_t stream);
+
 hipError_t requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C,
                                        float post, int val_dtype, int hd, const SignBits& sb, int mode, const float* u,
                                        uint64_t seed, uint8_t* codes_out, uint8_t* scales_out, void* dequant,

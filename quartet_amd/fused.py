@@ -73,6 +73,46 @@ class SwiGLULinearFn(torch.autograd.Function):
         return K.swiglu_backward(g, h2).view(ctx.h_shape), gw.to(ctx.w_dtype), None, None, None, None
 
 
+class RopeQKVFn(torch.autograd.Function):
+    """(q, k, v) [B, T, heads, head_dim] from the fused projection [B, T, 3C]: q and k rotated (llama.py:43-61), all three
+    in the dtype attention will run in, in one pass; backward merges the three gradients into [B, T, 3C]."""
+
+    @staticmethod
+    def forward(ctx, qkv, table, n_head):
+        B, T, C3 = qkv.shape
+        C = C3 // 3
+        hs = C // n_head
+        # the reference rotates in fp32 and autocast hands attention bf16 copies: one rounding of the fp32 result
+        out_dtype = torch.bfloat16 if _autocast_bf16() else torch.float32
+        q, k, v = K.rope_split_qkv(qkv.reshape(B * T, C3).contiguous(), table, C, hs, T, out_dtype)
+        ctx.save_for_backward(table)
+        ctx.meta = (B, T, C, n_head, hs, qkv.dtype)
+        return q.view(B, T, n_head, hs), k.view(B, T, n_head, hs), v.view(B, T, n_head, hs)
+
+    @staticmethod
+    def backward(ctx, dq, dk, dv):
+        (table,) = ctx.saved_tensors
+        B, T, C, n_head, hs, in_dtype = ctx.meta
+        dt = dq.dtype
+        flat = lambda g: g.to(dt).contiguous().view(B * T, C)
+        d_qkv = K.rope_merge_qkv_grad(flat(dq), flat(dk), flat(dv), table, C, hs, T, in_dtype)
+        return d_qkv.view(B, T, 3 * C), None, None
+
+
+def rope_qkv(qkv, table, n_head):
+    """Split the fused attention projection [B, T, 3C] into q, k, v [B, T, n_head, head_dim] with q and k rotated by the
+    (cos, sin) table [T, head_dim/2, 2]."""
+    C = qkv.shape[-1] // 3
+    hs = C // n_head
+    if qkv.is_cuda and qkv.dtype in _KERNEL_DTYPES and hs % 8 == 0 and table.dtype == torch.float32:
+        return RopeQKVFn.apply(qkv, table.contiguous(), n_head)
+    from .llama import apply_rotary
+    B, T, _ = qkv.shape
+    q, k, v = qkv.split(C, dim=2)
+    q, k = apply_rotary(q.view(B, T, n_head, hs), k.view(B, T, n_head, hs), table)
+    return q, k, v.view(B, T, n_head, hs)
+
+
 def rmsnorm_linear(norm, layer, x):
     """layer(norm(x)) for an RMSNorm module `norm` (attributes ``weight`` and ``eps``) and a QuantizedLinear."""
     if (_layer_is_fusable(layer) and x.is_cuda and x.dtype in _KERNEL_DTYPES and norm.weight.dtype == torch.float32

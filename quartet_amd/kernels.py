@@ -234,6 +234,31 @@ def swiglu_backward(g, h12):
     return d
 
 
+def rope_split_qkv(qkv2, table, n_embd, head_dim, seq_len, out_dtype):
+    """qkv2 [rows, 3 n_embd] -> (q, k, v) [rows, n_embd] of out_dtype, q and k rotated pairwise by table [seq_len, head_dim/2, 2]."""
+    _require_cuda(qkv2, table)
+    assert qkv2.is_contiguous() and table.is_contiguous() and table.dtype == torch.float32
+    assert qkv2.shape[1] == 3 * n_embd and tuple(table.shape) == (seq_len, head_dim // 2, 2)
+    rows = qkv2.shape[0]
+    q, k, v = (torch.empty((rows, n_embd), dtype=out_dtype, device=qkv2.device) for _ in range(3))
+    rc = _lib.lib().qm_rope_split_qkv(_ptr(qkv2), _dtype_code(qkv2.dtype), rows, seq_len, n_embd, head_dim, _ptr(table), _ptr(q),
+                                      _ptr(k), _ptr(v), _dtype_code(out_dtype), _stream())
+    _lib.check(rc, "qm_rope_split_qkv")
+    return q, k, v
+
+
+def rope_merge_qkv_grad(dq, dk, dv, table, n_embd, head_dim, seq_len, out_dtype):
+    """Gradients of rope_split_qkv's outputs, each [rows, n_embd] -> gradient of its input [rows, 3 n_embd] of out_dtype."""
+    _require_cuda(dq, dk, dv, table)
+    assert dq.is_contiguous() and dk.is_contiguous() and dv.is_contiguous() and dq.dtype == dk.dtype == dv.dtype
+    rows = dq.shape[0]
+    d_qkv = torch.empty((rows, 3 * n_embd), dtype=out_dtype, device=dq.device)
+    rc = _lib.lib().qm_rope_merge_qkv_grad(_ptr(dq), _ptr(dk), _ptr(dv), _dtype_code(dq.dtype), rows, seq_len, n_embd, head_dim,
+                                           _ptr(table), _ptr(d_qkv), _dtype_code(out_dtype), _stream())
+    _lib.check(rc, "qm_rope_merge_qkv_grad")
+    return d_qkv
+
+
 def linear_backward(e2, packed_x, packed_w, T, I, O, hd_x, signs_x, hd_w, signs_w, hd_g, signs_g, mode, seeds, x_val_dtype,
                     w_val_dtype, mid_dtype, x_scale_dtype, w_scale_dtype, tiled):
     """Whole backward pass in one foreign call: e [T,O] -> (gx [T,I], gw [O,I]) of mid_dtype."""

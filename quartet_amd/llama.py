@@ -18,7 +18,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .backward import BACKWARD_SCHEMES
-from .fused import rmsnorm_linear, swiglu_linear
+from .fused import rmsnorm_linear, rope_qkv, swiglu_linear
 from .linear import QuantizedLinear
 from .quantizers import QUANTIZER_CLASSES
 
@@ -142,10 +142,13 @@ class LlamaAttention(nn.Module):
         B, T, C = x.shape
         hs = C // self.n_head
         qkv = self.c_attn(x) if norm is None else rmsnorm_linear(norm, self.c_attn, x)
-        q, k, v = qkv.split(self.n_embd, dim=2)
-        q, k = apply_rotary(q.view(B, T, self.n_head, hs), k.view(B, T, self.n_head, hs), table)
-        q, k = q.transpose(1, 2), k.transpose(1, 2)
-        v = v.view(B, T, self.n_head, hs).transpose(1, 2)
+        if norm is not None:   # the fused path: split, rotate and convert in one kernel
+            q, k, v = rope_qkv(qkv, table, self.n_head)
+        else:
+            q, k, v = qkv.split(self.n_embd, dim=2)
+            q, k = apply_rotary(q.view(B, T, self.n_head, hs), k.view(B, T, self.n_head, hs), table)
+            v = v.view(B, T, self.n_head, hs)
+        q, k, v = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
         if not torch.is_autocast_enabled() and v.dtype != q.dtype:
             v = v.to(q.dtype)
         y = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=self.dropout, is_causal=True)

@@ -229,3 +229,35 @@ def test_fallbacks_keep_the_unfused_composition(q):
         h12 = torch.randn(32, 2 * I, device=DEV)
         up, gate = h12.split(I, dim=-1)
         assert torch.equal(swiglu_linear(layer, h12), layer(F.silu(up) * gate))
+
+
+@pytest.mark.parametrize("autocast", [True, False])
+@pytest.mark.parametrize("B,T,n_head,hs", [(2, 64, 5, 128), (3, 40, 2, 32), (1, 16, 3, 8)])
+def test_rope_qkv_matches_the_op_by_op_rotation(q, B, T, n_head, hs, autocast):
+    """Split + rotate + convert in one kernel against the reference's composition (split, fp32 pairwise rotation,
+    autocast's bf16 copies): bit-identical forward and backward -- both evaluate the same fp32 products and sums."""
+    print(f"case rope_qkv B={B} T={T} heads={n_head} head_dim={hs} autocast={autocast}", flush=True)
+    from quartet_amd.fused import rope_qkv
+    from quartet_amd.llama import apply_rotary, rotary_table
+    C = n_head * hs
+    dtype = torch.bfloat16 if autocast else torch.float32
+    table = rotary_table(hs, 2 * T)[:T].to(DEV)
+    qkv = make_input(B * T, 3 * C, dtype, seed=B + T, scale=1.5, outlier_frac=0).view(B, T, 3 * C).to(DEV)
+    grads = [make_input(B * T, C, dtype, seed=10 + i, scale=1e-2, outlier_frac=0).view(B, T, n_head, hs).to(DEV) for i in range(3)]
+
+    a = qkv.clone().requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+        fq, fk, fv = rope_qkv(a, table, n_head)
+    torch.autograd.backward([fq, fk, fv], grads)
+
+    b = qkv.clone().requires_grad_(True)
+    q0, k0, v0 = b.split(C, dim=2)
+    rq, rk = apply_rotary(q0.view(B, T, n_head, hs), k0.view(B, T, n_head, hs), table)
+    rq, rk, rv = rq.to(dtype), rk.to(dtype), v0.view(B, T, n_head, hs)      # what attention receives
+    torch.autograd.backward([rq, rk, rv], grads)
+
+    assert fq.dtype == dtype and fq.shape == (B, T, n_head, hs) and fq.is_contiguous()
+    assert torch.equal(fq, rq) and torch.equal(fk, rk) and torch.equal(fv, rv)
+    assert a.grad.dtype == dtype and torch.equal(a.grad, b.grad)
+    # a rotation: norms of q and k pairs are preserved up to rounding, position 0 is the identity
+    assert torch.equal(fq[:, 0], qkv[:, 0, :C].view(B, n_head, hs))
