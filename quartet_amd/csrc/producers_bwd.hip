@@ -34,67 +34,88 @@ __device__ __forceinline__ void store4(T* p, float4 v) {
     }
 }
 
-constexpr int kRowsPerWave = 16;
+// rows one workgroup walks: at most 1024 workgroups (one resident round on the chip), so at most 1024 partial rows
+inline int rows_per_block(int64_t rows) { return (int)((rows + 1023) / 1024 > 0 ? (rows + 1023) / 1024 : 1); }
 
 // y = x f g with f = (mean(x^2) + eps)^-1/2:
 //   dx_i = f g_i gy_i - x_i f^3 / cols * sum_j gy_j g_j x_j,      dgain_i = sum_rows gy_i x_i f.
-// One wave walks kRowsPerWave rows; lane l owns columns 4 (l + 64 k) .. +3.  The row is read twice (the second time
-// from cache); the gain-gradient sums stay in registers, are added across the workgroup's four waves in wave order
-// through shared memory and leave as one partial row per workgroup.
-template <typename TG, typename TX, int NK>
+// A workgroup walks rpb rows, RB at a time; thread t owns columns 4 (t + 256 k) .. +3 of each, keeps the rows in registers
+// between the reduction and the update, and adds its columns' gain-gradient terms over the rows: one partial row per workgroup.
+template <typename TG, typename TX, int NK, int RB>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const TG* __restrict__ gy, const TX* __restrict__ x,
                                                           const float* __restrict__ gain, const float* __restrict__ factor,
-                                                          int64_t rows, int cols, TX* __restrict__ dx,
+                                                          int64_t rows, int cols, int rpb, TX* __restrict__ dx,
                                                           float* __restrict__ partial) {
-    extern __shared__ float wave_sums[];  // [cols]
+    __shared__ float wave_sums[2][RB][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t r0 = ((int64_t)blockIdx.x * 4 + wave) * kRowsPerWave;
-    const int64_t r1 = r0 + kRowsPerWave < rows ? r0 + kRowsPerWave : rows;
-    float4 acc[NK];
+    const int64_t r0 = (int64_t)blockIdx.x * rpb;
+    const int64_t r1 = r0 + rpb < rows ? r0 + rpb : rows;
+    float4 acc[NK], w[NK];
 #pragma unroll
-    for (int k = 0; k < NK; ++k) acc[k] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int64_t r = r0; r < r1; ++r) {
-        const TG* gr = gy + r * cols;
-        const TX* xr = x + r * cols;
-        const float f = factor[r];
-        float s = 0.0f;
-#pragma unroll
-        for (int k = 0; k < NK; ++k) {
-            const int col = (k * 64 + lane) * 4;
-            if (col < cols) {
-                const float4 g = load4(gr + col), v = load4(xr + col), w = *reinterpret_cast<const float4*>(gain + col);
-                s += g.x * w.x * v.x + g.y * w.y * v.y + g.z * w.z * v.z + g.w * w.w * v.w;
-                acc[k].x += g.x * v.x * f; acc[k].y += g.y * v.y * f; acc[k].z += g.z * v.z * f; acc[k].w += g.w * v.w * f;
-            }
-        }
-#pragma unroll
-        for (int m = 32; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
-        const float coef = f * f * f * s / (float)cols;
-#pragma unroll
-        for (int k = 0; k < NK; ++k) {
-            const int col = (k * 64 + lane) * 4;
-            if (col < cols) {
-                const float4 g = load4(gr + col), v = load4(xr + col), w = *reinterpret_cast<const float4*>(gain + col);
-                store4(dx + r * cols + col, make_float4(f * g.x * w.x - v.x * coef, f * g.y * w.y - v.y * coef,
-                                                        f * g.z * w.z - v.z * coef, f * g.w * w.w - v.w * coef));
-            }
-        }
+    for (int k = 0; k < NK; ++k) {
+        const int col = (k * 256 + (int)threadIdx.x) * 4;
+        acc[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+        w[k] = col < cols ? *reinterpret_cast<const float4*>(gain + col) : acc[k];
     }
-    for (int turn = 0; turn < 4; ++turn) {
-        if (wave == turn) {
+    int parity = 0;
+    for (int64_t rb = r0; rb < r1; rb += RB, parity ^= 1) {  // RB rows in flight at a time
+        float f[RB], s[RB];
+        float4 gk[RB][NK], xk[RB][NK];
+#pragma unroll
+        for (int j = 0; j < RB; ++j) {
+            const int64_t r = rb + j < r1 ? rb + j : r1 - 1;  // a repeated last row is computed and not stored
+            f[j] = factor[r];
 #pragma unroll
             for (int k = 0; k < NK; ++k) {
-                const int col = (k * 64 + lane) * 4;
+                const int col = (k * 256 + (int)threadIdx.x) * 4;
                 if (col < cols) {
-                    float4* slot = reinterpret_cast<float4*>(wave_sums + col);
-                    float4 t = acc[k];
-                    if (turn) { const float4 p = *slot; t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w; }
-                    if (turn == 3) *reinterpret_cast<float4*>(partial + (int64_t)blockIdx.x * cols + col) = t;
-                    else *slot = t;
+                    gk[j][k] = load4(gy + r * cols + col);
+                    xk[j][k] = load4(x + r * cols + col);
                 }
             }
         }
+#pragma unroll
+        for (int j = 0; j < RB; ++j) {
+            s[j] = 0.0f;
+#pragma unroll
+            for (int k = 0; k < NK; ++k) {
+                const int col = (k * 256 + (int)threadIdx.x) * 4;
+                if (col < cols) {
+                    const float4 g = gk[j][k], v = xk[j][k];
+                    s[j] += g.x * w[k].x * v.x + g.y * w[k].y * v.y + g.z * w[k].z * v.z + g.w * w[k].w * v.w;
+                    if (rb + j < r1) {
+                        acc[k].x += g.x * v.x * f[j]; acc[k].y += g.y * v.y * f[j];
+                        acc[k].z += g.z * v.z * f[j]; acc[k].w += g.w * v.w * f[j];
+                    }
+                }
+            }
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1) s[j] += __shfl_xor(s[j], m, 64);
+            // two sets of slots: a wave may start the next rows while another still reads these
+            if (lane == 0) wave_sums[parity][j][wave] = s[j];
+        }
         __syncthreads();
+#pragma unroll
+        for (int j = 0; j < RB; ++j) {
+            if (rb + j >= r1) break;
+            const float* slot = wave_sums[parity][j];
+            const float coef = f[j] * f[j] * f[j] * ((slot[0] + slot[1]) + (slot[2] + slot[3])) / (float)cols;
+#pragma unroll
+            for (int k = 0; k < NK; ++k) {
+                const int col = (k * 256 + (int)threadIdx.x) * 4;
+                if (col < cols) {
+                    const float4 g = gk[j][k], v = xk[j][k];
+                    const float fj = f[j];
+                    store4(dx + (rb + j) * cols + col, make_float4(fj * g.x * w[k].x - v.x * coef, fj * g.y * w[k].y - v.y * coef,
+                                                                   fj * g.z * w[k].z - v.z * coef, fj * g.w * w[k].w - v.w * coef));
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < NK; ++k) {
+        const int col = (k * 256 + (int)threadIdx.x) * 4;
+        if (col < cols) *reinterpret_cast<float4*>(partial + (int64_t)blockIdx.x * cols + col) = acc[k];
     }
 }
 
@@ -106,8 +127,10 @@ __global__ __launch_bounds__(1024) void column_sum_kernel(const float* __restric
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = blockIdx.x * 64 + lane;
     float s = 0.0f;
-    if (col < cols)
+    if (col < cols) {
+#pragma unroll 8
         for (int r = wave; r < n; r += 16) s += partial[(int64_t)r * cols + col];
+    }
     sums[wave][lane] = s;
     __syncthreads();
     if (wave == 0 && col < cols) {
@@ -146,18 +169,19 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const TG* __restrict__ 
     store4(d_h12 + row * 2 * hidden + hidden + col, make_float4(da[0], da[1], da[2], da[3]));
 }
 
-int64_t rmsnorm_bwd_blocks(int64_t rows) { return (rows + 4 * kRowsPerWave - 1) / (4 * kRowsPerWave); }
+int64_t rmsnorm_bwd_blocks(int64_t rows) { return (rows + rows_per_block(rows) - 1) / rows_per_block(rows); }
 
 template <typename TG, typename TX>
 void launch_rmsnorm_bwd(const void* gy, const void* x, const float* gain, const float* factor, int64_t rows, int cols,
                         void* dx, float* partial, hipStream_t stream) {
     const dim3 grid((unsigned)rmsnorm_bwd_blocks(rows)), block(256);
-    const size_t lds = (size_t)cols * sizeof(float);
+    const int rpb = rows_per_block(rows);
     const TG* g = reinterpret_cast<const TG*>(gy);
     const TX* xp = reinterpret_cast<const TX*>(x);
     TX* dxp = reinterpret_cast<TX*>(dx);
-    if (cols <= 2048) rmsnorm_bwd_kernel<TG, TX, 8><<<grid, block, lds, stream>>>(g, xp, gain, factor, rows, cols, dxp, partial);
-    else rmsnorm_bwd_kernel<TG, TX, 32><<<grid, block, lds, stream>>>(g, xp, gain, factor, rows, cols, dxp, partial);
+    if (cols <= 2048) rmsnorm_bwd_kernel<TG, TX, 2, 4><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, dxp, partial);
+    else if (cols <= 4096) rmsnorm_bwd_kernel<TG, TX, 4, 2><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, dxp, partial);
+    else rmsnorm_bwd_kernel<TG, TX, 8, 1><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, dxp, partial);
 }
 
 }  // namespace

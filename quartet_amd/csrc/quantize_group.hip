@@ -715,8 +715,8 @@ hipError_t requantize_transposed_hd32(const uint8_t* codes_in, const uint8_t* sc
 
 // ---- producers fused into the forward quantizer ------------------------------------------------------------------
 // The tensor the model would hand to the quantized linear (RMSNorm output, src/models/llama.py:64-75; SwiGLU product,
-// llama.py:113-114) is computed group by group in registers and never written.  A workgroup owns 16 whole rows:
-// wave w rows 4w..4w+3, the 16 lanes of a row take groups l, l+16, l+32, ... of 32 consecutive elements.
+// llama.py:113-114) is computed group by group in registers and never written.  One wave owns one row: lane l takes
+// groups l, l+64, ... of 32 consecutive elements, so a row of up to 2048 elements is read exactly once.
 
 namespace {
 
@@ -736,25 +736,38 @@ struct RmsNormProducer {
     float* factor;  // [rows]: 1 / sqrt(mean(x^2) + eps), kept for the backward pass
     float eps;
 
-    // sum of squares: per lane its groups in ascending order (each by the pairwise tree), then the butterfly over the
-    // row's 16 lanes, which adds in the order of a pairwise tree and leaves every lane with the same bits
-    __device__ __forceinline__ float prepare(int64_t row, int lane16, int groups, int64_t cols) const {
+    // The row's factor; `first` leaves with the raw elements of the lane's first group (if it has one).
+    // Sum of squares in a fixed order: sixteen interleaved partial sums (partial j adds the sums of groups j, j+16,
+    // j+32, ... in ascending order, each group summed by the pairwise tree), then the pairwise tree over the sixteen.
+    // A lane without a group adds +0, which leaves a sum of squares unchanged.
+    __device__ __forceinline__ float prepare(int64_t row, int lane, int groups, int64_t cols, float (&first)[32]) const {
         float acc = 0.0f;
-        for (int g = lane16; g < groups; g += 16) {
-            float v[32];
-            load_group<T>(x + row * cols + g * 32, v);
+        for (int base = 0; base < groups; base += 64) {
+            const int g = base + lane;
+            float s = 0.0f;
+            if (g < groups) {
+                float v[32];
+                load_group<T>(x + row * cols + g * 32, v);
+                if (base == 0) {
 #pragma unroll
-            for (int i = 0; i < 32; ++i) v[i] = v[i] * v[i];
-            acc = acc + tree_sum32(v);
+                    for (int i = 0; i < 32; ++i) first[i] = v[i];
+                }
+#pragma unroll
+                for (int i = 0; i < 32; ++i) v[i] = v[i] * v[i];
+                s = tree_sum32(v);
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) acc = acc + __shfl(s, (lane & 15) + 16 * k, 64);
         }
 #pragma unroll
         for (int m = 1; m < 16; m <<= 1) acc = acc + __shfl_xor(acc, m, 64);
         const float f = 1.0f / __builtin_sqrtf(acc / (float)cols + eps);
-        if (lane16 == 0) factor[row] = f;
+        if (lane == 0) factor[row] = f;
         return f;
     }
-    __device__ __forceinline__ void load(int64_t row, int g, int64_t cols, float f, float (&v)[32]) const {
-        load_group<T>(x + row * cols + g * 32, v);
+    // v holds the group's raw elements on entry when have_raw
+    __device__ __forceinline__ void load(int64_t row, int g, int64_t cols, float f, bool have_raw, float (&v)[32]) const {
+        if (!have_raw) load_group<T>(x + row * cols + g * 32, v);
 #pragma unroll
         for (int i = 0; i < 32; ++i) v[i] = v[i] * f;
         if constexpr (sizeof(T) == 2) {  // .type_as(x)
@@ -773,8 +786,8 @@ struct SwiGluProducer {
     static constexpr int kOutDtype = sizeof(T) == 2 ? BF16 : F32;
     const T* h12;  // [rows, 2 cols]: up, then gate
 
-    __device__ __forceinline__ float prepare(int64_t, int, int, int64_t) const { return 0.0f; }
-    __device__ __forceinline__ void load(int64_t row, int g, int64_t cols, float, float (&v)[32]) const {
+    __device__ __forceinline__ float prepare(int64_t, int, int, int64_t, float (&)[32]) const { return 0.0f; }
+    __device__ __forceinline__ void load(int64_t row, int g, int64_t cols, float, bool, float (&v)[32]) const {
         float gate[32];
         load_group<T>(h12 + row * 2 * cols + g * 32, v);
         load_group<T>(h12 + row * 2 * cols + cols + g * 32, gate);
@@ -805,21 +818,20 @@ struct ProducedRowsJob {
 
     ProducedRowsJob(const P& prod_, int64_t rows_, int64_t cols_, uint32_t sign_word_, const GroupOut& out_)
         : prod(prod_), rows(rows_), cols(cols_), c(hadamard_scale(32, P::kOutDtype)), sign_word(sign_word_), out(out_),
-          blocks((unsigned)((rows_ + 15) / 16)) {}
+          blocks((unsigned)((rows_ + 3) / 4)) {}
 
     __device__ __forceinline__ void run(unsigned bid) const {
         const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-        const int rin = wave * 4 + (lane >> 4), lane16 = lane & 15;
-        const int64_t row = (int64_t)bid * 16 + rin;
-        if (row >= rows) return;  // the 16 lanes of a row leave together
+        const int64_t row = (int64_t)bid * 4 + wave;
+        if (row >= rows) return;  // a whole wave
         const int groups = (int)(cols / 32);
-        const float state = prod.prepare(row, lane16, groups, cols);
+        float v[32];
+        const float state = prod.prepare(row, lane, groups, cols, v);
         // TILED: cols % 128 == 0, so the four lanes of a quad run the same number of iterations
-        for (int g = lane16; g < groups; g += 16) {
+        for (int g = lane; g < groups; g += 64) {
             const int64_t gi = row * groups + g;
-            const int64_t ci = TILED ? (int64_t)bid * 16 * groups + ((g >> 2) * 64 + rin * 4 + (g & 3)) : gi;
-            float v[32];
-            prod.load(row, g, cols, state, v);
+            const int64_t ci = TILED ? (row >> 4) * 16 * groups + ((g >> 2) * 64 + (int)(row & 15) * 4 + (g & 3)) : gi;
+            prod.load(row, g, cols, state, g == lane, v);
             rotate_group(v, c, sign_word);
             GroupCodes o;
             quantize_group_regs<QUEST_RTN, true>(v, 0, gi, o);
