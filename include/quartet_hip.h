@@ -144,6 +144,9 @@ int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, 
  *   x_val_dtype, w_val_dtype   dtypes the reference would hold the de-quantized x and w in
  *   x_scale_dtype, w_scale_dtype  dtypes whose rounding of hd^-1/2 the forward quantizers' matrices carry in backward
  *   workspace         qm_linear_backward_workspace_bytes(T, I, O, mid_dtype) bytes of scratch, 256-byte aligned
+ *   gx_rotated        != 0: gx receives the gradient w.r.t. the activation quantizer's rotated output (the first
+ *                     product, B3) and its straight-through backward is left to the caller, who folds it into the
+ *                     next kernel (maskbits argument of qm_rmsnorm_backward / qm_swiglu_backward); needs hd_x == 32
  * codes_layout applies to every packed tensor inside; QM_LAYOUT_TILED needs T, I, O multiples of 128 and at
  * least 256, and all Hadamard blocks 32.  T, I, O must be multiples of 32 for the backward pass.
  */
@@ -159,7 +162,7 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                        const void* packed_w, int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w,
                        int hd_g, const uint32_t* signs_g, int g_mode, const uint64_t* seeds, int x_val_dtype,
                        int w_val_dtype, int mid_dtype, int x_scale_dtype, int w_scale_dtype, void* workspace,
-                       size_t workspace_bytes, void* gx, void* gw, int codes_layout, void* stream);
+                       size_t workspace_bytes, void* gx, void* gw, int codes_layout, int gx_rotated, void* stream);
 
 /*
  * Producers fused into the activation quantizer.  The tensor the model would hand to a quantized linear is computed
@@ -178,6 +181,10 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
  *   tensor) -> dx [rows, cols] of x's dtype and dgain fp32 [cols] (summed over rows in a fixed order).  cols <= 8192.
  *   workspace: qm_rmsnorm_backward_workspace_bytes(rows, cols) bytes, 16-byte aligned.
  * qm_swiglu_backward: autograd of silu(up) * gate: g [rows, hidden] -> d_h12 [rows, 2 hidden] of h12's dtype.
+ *   Both backward kernels take the gradient either as it is (maskbits == NULL) or still in the rotated basis of the
+ *   layer's activation quantizer (qm_linear_backward with gx_rotated): then maskbits [rows, cols/8] (the mask region of
+ *   the layer's packed_x), sign_bits and scale_dtype describe that quantizer, and the masked inverse rotation of
+ *   qm_masked_hadamard_bwd (same operations, same bits, rounded to the gradient's dtype) is applied on the fly.
  * codes_layout QM_LAYOUT_TILED needs rows % 16 == 0 and cols (hidden) % 128 == 0; cols (hidden) % 32 == 0 always.
  */
 int qm_rmsnorm_quantize_mxfp4(const void* x, int x_dtype, const float* gain, float eps, int64_t rows, int64_t cols,
@@ -187,10 +194,12 @@ int qm_swiglu_quantize_mxfp4(const void* h12, int dtype, int64_t rows, int64_t h
                              void* packed, size_t packed_bytes, int codes_layout, void* stream);
 size_t qm_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols);
 int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain,
-                        const float* factor, int64_t rows, int64_t cols, void* dx, float* dgain, void* workspace,
+                        const float* factor, int64_t rows, int64_t cols, const uint8_t* maskbits,
+                        const uint32_t* sign_bits, int scale_dtype, void* dx, float* dgain, void* workspace,
                         size_t workspace_bytes, void* stream);
 int qm_swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
-                       void* d_h12, void* stream);
+                       const uint8_t* maskbits, const uint32_t* sign_bits, int scale_dtype, void* d_h12,
+                       void* stream);
 
 /*
  * Rotary position embedding around the attention that sits between two quantized linears (apply_rotary_emb,

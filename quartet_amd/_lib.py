@@ -84,16 +84,16 @@ def lib():
     L.qm_rmsnorm_backward_workspace_bytes.restype = sz
     L.qm_rmsnorm_backward_workspace_bytes.argtypes = [i64, i64]
     L.qm_rmsnorm_backward.restype = i32
-    L.qm_rmsnorm_backward.argtypes = [vp, i32, vp, i32, vp, vp, i64, i64, vp, vp, vp, sz, vp]
+    L.qm_rmsnorm_backward.argtypes = [vp, i32, vp, i32, vp, vp, i64, i64, vp, vp, i32, vp, vp, vp, sz, vp]
     L.qm_swiglu_backward.restype = i32
-    L.qm_swiglu_backward.argtypes = [vp, i32, vp, i32, i64, i64, vp, vp]
+    L.qm_swiglu_backward.argtypes = [vp, i32, vp, i32, i64, i64, vp, vp, i32, vp, vp]
     L.qm_rope_split_qkv.restype = i32
     L.qm_rope_split_qkv.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, vp, vp, i32, vp]
     L.qm_rope_merge_qkv_grad.restype = i32
     L.qm_rope_merge_qkv_grad.argtypes = [vp, vp, vp, i32, i64, i64, i64, i32, vp, vp, i32, vp]
     L.qm_linear_backward.restype = i32
     L.qm_linear_backward.argtypes = [vp, i32, i64, i64, i64, vp, vp, i32, vp, i32, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32,
-                                     vp, sz, vp, vp, i32, vp]
+                                     vp, sz, vp, vp, i32, i32, vp]
     _lib = L
     return L
 

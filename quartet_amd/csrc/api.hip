@@ -42,7 +42,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 4; }
+int qm_version(void) { return 5; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -266,7 +266,7 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                        int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, int hd_g, const uint32_t* signs_g,
                        int g_mode, const uint64_t* seeds, int x_val_dtype, int w_val_dtype, int mid_dtype, int x_scale_dtype,
                        int w_scale_dtype, void* workspace, size_t workspace_bytes, void* gx, void* gw, int codes_layout,
-                       void* stream) {
+                       int gx_rotated, void* stream) {
     if (T < 0 || I < 0 || O < 0) return fail(QM_ERR_INVALID, "qm_linear_backward: negative extent");
     if (T == 0 || O == 0 || I == 0) return 0;
     if (g_mode != QM_ABSMAX_RTN && g_mode != QM_ABSMAX_SR)
@@ -290,6 +290,10 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
     void* gws = wl.gemm_ws_bytes ? k + wl.gemm_ws : nullptr;
     hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
     int rc;
+    // gx_rotated: the caller undoes the activation quantizer's rotation itself (fused into its next kernel); the first
+    // product then lands in gx directly
+    void* gx_product = gx_rotated ? gx : static_cast<void*>(k + wl.gxq);
+    if (gx_rotated && hd_x != 32) return fail(QM_ERR_INVALID, "qm_linear_backward: gx_rotated needs hd_x == 32");
     if (pair_launches(codes_layout, T, I, O, hd_x, hd_w, hd_g) && e && gx && gw && valid_dtype(e_dtype) && aligned(e, 16) &&
         aligned(gx, 16) && aligned(gw, 16) && valid_dtype(x_val_dtype) && valid_dtype(w_val_dtype) &&
         valid_dtype(x_scale_dtype) && valid_dtype(w_scale_dtype)) {
@@ -302,12 +306,14 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
         const qm::RequantArgs rx{px + lx.c, px + lx.s, T, I, x_val_dtype, seeds[3], k + wl.xtc, k + wl.xts};
         rc = from_hip(qm::requantize_transposed_hd32_tiled_pair(rx, rw, sg, g_mode, hs), "qm_linear_backward");
         if (rc) return rc;
-        rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, k + wl.gxq, mid_dtype, codes_layout,
+        rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, gx_product, mid_dtype, codes_layout,
                               codes_layout, gws, wl.gemm_ws_bytes, stream);
         if (rc) return rc;
         rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, k + wl.gwq, mid_dtype, codes_layout,
                               codes_layout, gws, wl.gemm_ws_bytes, stream);
         if (rc) return rc;
+        if (gx_rotated)
+            return qm_masked_hadamard_bwd(k + wl.gwq, mid_dtype, O, I, hd_w, w_scale_dtype, signs_w, pw + lw.m, gw, mid_dtype, stream);
         return from_hip(qm::masked_hadamard_bwd_hd32_pair(k + wl.gxq, T * I, x_scale_dtype,
                                                           signs_x ? signs_x[0] : 0u, px + lx.m, gx, k + wl.gwq, O * I,
                                                           w_scale_dtype, signs_w ? signs_w[0] : 0u,
@@ -319,7 +325,7 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
     rc = qm_requantize_transposed_mxfp4(pw + lw.c, pw + lw.s, O, I, 1.0f, w_val_dtype, hd_g, signs_g, g_mode, nullptr, seeds[1],
                                         k + wl.wtc, k + wl.wts, nullptr, codes_layout, codes_layout, stream);
     if (rc) return rc;
-    rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, k + wl.gxq, mid_dtype, codes_layout,
+    rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, gx_product, mid_dtype, codes_layout,
                           codes_layout, gws, wl.gemm_ws_bytes, stream);
     if (rc) return rc;
     rc = qm_quantize_mxfp4(e, e_dtype, O, T, hd_g, signs_g, g_mode, 1, nullptr, seeds[2], k + wl.etc, k + wl.ets, nullptr, nullptr,
@@ -331,8 +337,10 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
     rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, k + wl.gwq, mid_dtype, codes_layout,
                           codes_layout, gws, wl.gemm_ws_bytes, stream);
     if (rc) return rc;
-    rc = qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, px + lx.m, gx, mid_dtype, stream);
-    if (rc) return rc;
+    if (!gx_rotated) {
+        rc = qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, px + lx.m, gx, mid_dtype, stream);
+        if (rc) return rc;
+    }
     return qm_masked_hadamard_bwd(k + wl.gwq, mid_dtype, O, I, hd_w, w_scale_dtype, signs_w, pw + lw.m, gw, mid_dtype, stream);
 }
 
@@ -387,8 +395,10 @@ size_t qm_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols) {
 }
 
 int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain, const float* factor,
-                        int64_t rows, int64_t cols, void* dx, float* dgain, void* workspace, size_t workspace_bytes, void* stream) {
-    if (!valid_dtype(gy_dtype) || !valid_dtype(x_dtype)) return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: dtypes must be QM_BF16/QM_F32");
+                        int64_t rows, int64_t cols, const uint8_t* maskbits, const uint32_t* sign_bits, int scale_dtype, void* dx,
+                        float* dgain, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!valid_dtype(gy_dtype) || !valid_dtype(x_dtype) || (maskbits && !valid_dtype(scale_dtype)))
+        return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: dtypes must be QM_BF16/QM_F32");
     if (rows < 0 || cols <= 0 || cols % 32 || cols > 8192)
         return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: need rows >= 0 and cols a multiple of 32 in [32, 8192] (got [%lld, %lld])",
                     (long long)rows, (long long)cols);
@@ -398,22 +408,24 @@ int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype
     if (!aligned(gy, 8) || !aligned(x, 8) || !aligned(dx, 8) || !aligned(gain, 16) || !aligned(workspace, 16) ||
         (gy_dtype == QM_F32 && !aligned(gy, 16)) || (x_dtype == QM_F32 && (!aligned(x, 16) || !aligned(dx, 16))))
         return fail(QM_ERR_UNALIGNED, "qm_rmsnorm_backward: tensors need 16-byte alignment");
-    return from_hip(qm::rmsnorm_backward(gy, gy_dtype, x, x_dtype, gain, factor, rows, cols, dx, dgain, workspace,
-                                         reinterpret_cast<hipStream_t>(stream)),
+    return from_hip(qm::rmsnorm_backward(gy, gy_dtype, x, x_dtype, gain, factor, rows, cols, maskbits, sign_bits ? sign_bits[0] : 0u,
+                                         maskbits ? scale_dtype : QM_F32, dx, dgain, workspace, reinterpret_cast<hipStream_t>(stream)),
                     "qm_rmsnorm_backward");
 }
 
-int qm_swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden, void* d_h12,
-                       void* stream) {
-    if (!valid_dtype(g_dtype) || !valid_dtype(dtype)) return fail(QM_ERR_INVALID, "qm_swiglu_backward: dtypes must be QM_BF16/QM_F32");
-    if (rows < 0 || hidden <= 0 || hidden % 4)
-        return fail(QM_ERR_INVALID, "qm_swiglu_backward: need rows >= 0 and hidden a positive multiple of 4 (got [%lld, %lld])",
-                    (long long)rows, (long long)hidden);
+int qm_swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
+                       const uint8_t* maskbits, const uint32_t* sign_bits, int scale_dtype, void* d_h12, void* stream) {
+    if (!valid_dtype(g_dtype) || !valid_dtype(dtype) || (maskbits && !valid_dtype(scale_dtype)))
+        return fail(QM_ERR_INVALID, "qm_swiglu_backward: dtypes must be QM_BF16/QM_F32");
+    if (rows < 0 || hidden <= 0 || hidden % 4 || (maskbits && hidden % 32))
+        return fail(QM_ERR_INVALID, "qm_swiglu_backward: need rows >= 0 and hidden a positive multiple of 4 (of 32 with mask bits) "
+                                    "(got [%lld, %lld])", (long long)rows, (long long)hidden);
     if (rows == 0) return 0;
     if (!g || !h12 || !d_h12) return fail(QM_ERR_INVALID, "qm_swiglu_backward: g, h12 and d_h12 must be non-null");
     if (!aligned(g, 16) || !aligned(h12, 16) || !aligned(d_h12, 16))
         return fail(QM_ERR_UNALIGNED, "qm_swiglu_backward: tensors need 16-byte alignment");
-    return from_hip(qm::swiglu_backward(g, g_dtype, h12, dtype, rows, hidden, d_h12, reinterpret_cast<hipStream_t>(stream)),
+    return from_hip(qm::swiglu_backward(g, g_dtype, h12, dtype, rows, hidden, maskbits, sign_bits ? sign_bits[0] : 0u,
+                                        maskbits ? scale_dtype : QM_F32, d_h12, reinterpret_cast<hipStream_t>(stream)),
                     "qm_swiglu_backward");
 }
 

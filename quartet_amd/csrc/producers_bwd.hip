@@ -34,6 +34,60 @@ __device__ __forceinline__ void store4(T* p, float4 v) {
     }
 }
 
+// The straight-through backward of the forward quantizer (masked inverse rotation, Hadamard block 32,
+// src/models/quantization/quantizers/mxfp4.py:143-146) on four consecutive elements of a lane; the eight lanes that hold
+// a group of 32 cooperate.  The same operations on the same pairs as the stand-alone kernel (mask factor, column sign,
+// ascending butterfly strides, one multiply by c, rounding to the gradient's dtype), hence the same bits.
+struct InverseRotation {
+    const uint8_t* maskbits;  // null: the gradient arrives already rotated back
+    uint32_t sign_word;
+    float c;
+};
+__device__ __forceinline__ float quad_xor1(float v) { return u2f((uint32_t)__builtin_amdgcn_mov_dpp((int)f2u(v), 0xB1, 0xF, 0xF, true)); }
+__device__ __forceinline__ float quad_xor2(float v) { return u2f((uint32_t)__builtin_amdgcn_mov_dpp((int)f2u(v), 0x4E, 0xF, 0xF, true)); }
+template <bool ROUND_BF16>
+__device__ __forceinline__ float4 inverse_rotate_quad(float4 g, const InverseRotation& rot, int64_t elem) {
+    const int q = (int)(elem >> 2) & 7;                                            // the lane's place in its group
+    const uint32_t keep = (uint32_t)rot.maskbits[elem >> 3] >> (elem & 4);         // bit i = element elem + i
+    const uint32_t sign = rot.sign_word >> (q * 4);
+    float v[4] = {g.x, g.y, g.z, g.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float x = v[i] * (((keep >> i) & 1u) ? 1.0f : 0.0f);
+        v[i] = u2f(f2u(x) ^ (((sign >> i) & 1u) << 31));
+    }
+#pragma unroll
+    for (int h = 1; h < 4; h <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (i & h) continue;
+            const float a = v[i], b = v[i + h];
+            v[i] = a + b;
+            v[i + h] = a - b;
+        }
+    }
+#pragma unroll
+    for (int m = 1; m < 8; m <<= 1) {  // lower lane of a butterfly: own + partner; upper lane: partner - own
+        const uint32_t flip = (q & m) ? 0x80000000u : 0u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float p = m == 1 ? quad_xor1(v[i]) : (m == 2 ? quad_xor2(v[i]) : __shfl_xor(v[i], 4, 64));
+            v[i] = p + u2f(f2u(v[i]) ^ flip);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = v[i] * rot.c;
+    if constexpr (ROUND_BF16) {
+#pragma unroll
+        for (int i = 0; i < 4; i += 2) {
+            const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[i], v[i + 1]}, v2bf));
+            v[i] = u2f(w << 16);
+            v[i + 1] = u2f(w & 0xffff0000u);
+        }
+    }
+    return make_float4(v[0], v[1], v[2], v[3]);
+}
+
 // rows one workgroup walks: at most 1024 workgroups (one resident round on the chip), so at most 1024 partial rows
 inline int rows_per_block(int64_t rows) { return (int)((rows + 1023) / 1024 > 0 ? (rows + 1023) / 1024 : 1); }
 
@@ -44,8 +98,8 @@ inline int rows_per_block(int64_t rows) { return (int)((rows + 1023) / 1024 > 0 
 template <typename TG, typename TX, int NK, int RB>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const TG* __restrict__ gy, const TX* __restrict__ x,
                                                           const float* __restrict__ gain, const float* __restrict__ factor,
-                                                          int64_t rows, int cols, int rpb, TX* __restrict__ dx,
-                                                          float* __restrict__ partial) {
+                                                          int64_t rows, int cols, int rpb, InverseRotation rot,
+                                                          TX* __restrict__ dx, float* __restrict__ partial) {
     __shared__ float wave_sums[2][RB][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t r0 = (int64_t)blockIdx.x * rpb;
@@ -68,8 +122,9 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const TG* __restrict__
 #pragma unroll
             for (int k = 0; k < NK; ++k) {
                 const int col = (k * 256 + (int)threadIdx.x) * 4;
-                if (col < cols) {
+                if (col < cols) {  // cols % 32 == 0: the eight lanes of a group of 32 are in or out together
                     gk[j][k] = load4(gy + r * cols + col);
+                    if (rot.maskbits) gk[j][k] = inverse_rotate_quad<sizeof(TG) == 2>(gk[j][k], rot, r * cols + col);
                     xk[j][k] = load4(x + r * cols + col);
                 }
             }
@@ -145,12 +200,14 @@ __global__ __launch_bounds__(1024) void column_sum_kernel(const float* __restric
 // A tensor of bf16 rounds where autograd's bf16 ops would: silu(up), g * gate, and the two results.
 template <typename TG, typename TH>
 __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const TG* __restrict__ g, const TH* __restrict__ h12,
-                                                         int64_t rows, int64_t hidden, TH* __restrict__ d_h12) {
+                                                         int64_t rows, int64_t hidden, InverseRotation rot,
+                                                         TH* __restrict__ d_h12) {
     const int64_t quads_per_row = hidden / 4;
     const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (q >= rows * quads_per_row) return;
     const int64_t row = q / quads_per_row, col = (q - row * quads_per_row) * 4;
-    const float4 gv = load4(g + row * hidden + col);
+    float4 gv = load4(g + row * hidden + col);
+    if (rot.maskbits) gv = inverse_rotate_quad<sizeof(TG) == 2>(gv, rot, row * hidden + col);  // hidden % 32 == 0 then
     const float4 up = load4(h12 + row * 2 * hidden + col), gate = load4(h12 + row * 2 * hidden + hidden + col);
     const float G[4] = {gv.x, gv.y, gv.z, gv.w}, U[4] = {up.x, up.y, up.z, up.w}, A[4] = {gate.x, gate.y, gate.z, gate.w};
     float du[4], da[4];
@@ -173,15 +230,15 @@ int64_t rmsnorm_bwd_blocks(int64_t rows) { return (rows + rows_per_block(rows) -
 
 template <typename TG, typename TX>
 void launch_rmsnorm_bwd(const void* gy, const void* x, const float* gain, const float* factor, int64_t rows, int cols,
-                        void* dx, float* partial, hipStream_t stream) {
+                        const InverseRotation& rot, void* dx, float* partial, hipStream_t stream) {
     const dim3 grid((unsigned)rmsnorm_bwd_blocks(rows)), block(256);
     const int rpb = rows_per_block(rows);
     const TG* g = reinterpret_cast<const TG*>(gy);
     const TX* xp = reinterpret_cast<const TX*>(x);
     TX* dxp = reinterpret_cast<TX*>(dx);
-    if (cols <= 2048) rmsnorm_bwd_kernel<TG, TX, 2, 4><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, dxp, partial);
-    else if (cols <= 4096) rmsnorm_bwd_kernel<TG, TX, 4, 2><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, dxp, partial);
-    else rmsnorm_bwd_kernel<TG, TX, 8, 1><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, dxp, partial);
+    if (cols <= 2048) rmsnorm_bwd_kernel<TG, TX, 2, 4><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, dxp, partial);
+    else if (cols <= 4096) rmsnorm_bwd_kernel<TG, TX, 4, 2><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, dxp, partial);
+    else rmsnorm_bwd_kernel<TG, TX, 8, 1><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, dxp, partial);
 }
 
 }  // namespace
@@ -190,17 +247,19 @@ size_t rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols) {
     return (size_t)rmsnorm_bwd_blocks(rows) * (size_t)cols * sizeof(float);
 }
 
-// cols <= 8192, cols % 4 == 0; workspace: rmsnorm_backward_workspace_bytes(rows, cols) bytes, 16-byte aligned
+// cols <= 8192, cols % 32 == 0; workspace: rmsnorm_backward_workspace_bytes(rows, cols) bytes, 16-byte aligned.
+// maskbits != null: gy is the gradient w.r.t. the quantizer's rotated output and is rotated back on the fly.
 hipError_t rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain,
-                            const float* factor, int64_t rows, int64_t cols, void* dx, float* dgain, void* workspace,
-                            hipStream_t stream) {
+                            const float* factor, int64_t rows, int64_t cols, const uint8_t* maskbits, uint32_t sign_word,
+                            int scale_dtype, void* dx, float* dgain, void* workspace, hipStream_t stream) {
     if (cols == 0) return hipSuccess;
     float* partial = reinterpret_cast<float*>(workspace);
+    const InverseRotation rot{maskbits, sign_word, hadamard_scale(32, scale_dtype)};
     if (rows == 0) {}  // no rows: the column sums below write zeros
-    else if (gy_dtype == BF16 && x_dtype == BF16) launch_rmsnorm_bwd<uint16_t, uint16_t>(gy, x, gain, factor, rows, (int)cols, dx, partial, stream);
-    else if (gy_dtype == BF16) launch_rmsnorm_bwd<uint16_t, float>(gy, x, gain, factor, rows, (int)cols, dx, partial, stream);
-    else if (x_dtype == BF16) launch_rmsnorm_bwd<float, uint16_t>(gy, x, gain, factor, rows, (int)cols, dx, partial, stream);
-    else launch_rmsnorm_bwd<float, float>(gy, x, gain, factor, rows, (int)cols, dx, partial, stream);
+    else if (gy_dtype == BF16 && x_dtype == BF16) launch_rmsnorm_bwd<uint16_t, uint16_t>(gy, x, gain, factor, rows, (int)cols, rot, dx, partial, stream);
+    else if (gy_dtype == BF16) launch_rmsnorm_bwd<uint16_t, float>(gy, x, gain, factor, rows, (int)cols, rot, dx, partial, stream);
+    else if (x_dtype == BF16) launch_rmsnorm_bwd<float, uint16_t>(gy, x, gain, factor, rows, (int)cols, rot, dx, partial, stream);
+    else launch_rmsnorm_bwd<float, float>(gy, x, gain, factor, rows, (int)cols, rot, dx, partial, stream);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
     column_sum_kernel<<<dim3((unsigned)((cols + 63) / 64)), dim3(1024), 0, stream>>>(partial, (int)rmsnorm_bwd_blocks(rows),
@@ -208,19 +267,20 @@ hipError_t rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_d
     return hipGetLastError();
 }
 
-// hidden % 4 == 0
+// hidden % 4 == 0 (% 32 with maskbits); maskbits as for rmsnorm_backward
 hipError_t swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
-                           void* d_h12, hipStream_t stream) {
+                           const uint8_t* maskbits, uint32_t sign_word, int scale_dtype, void* d_h12, hipStream_t stream) {
     if (rows == 0 || hidden == 0) return hipSuccess;
     const dim3 grid((unsigned)((rows * (hidden / 4) + 255) / 256)), block(256);
+    const InverseRotation rot{maskbits, sign_word, hadamard_scale(32, scale_dtype)};
     if (g_dtype == BF16 && dtype == BF16)
-        swiglu_bwd_kernel<uint16_t, uint16_t><<<grid, block, 0, stream>>>(reinterpret_cast<const uint16_t*>(g), reinterpret_cast<const uint16_t*>(h12), rows, hidden, reinterpret_cast<uint16_t*>(d_h12));
+        swiglu_bwd_kernel<uint16_t, uint16_t><<<grid, block, 0, stream>>>(reinterpret_cast<const uint16_t*>(g), reinterpret_cast<const uint16_t*>(h12), rows, hidden, rot, reinterpret_cast<uint16_t*>(d_h12));
     else if (g_dtype == BF16)
-        swiglu_bwd_kernel<uint16_t, float><<<grid, block, 0, stream>>>(reinterpret_cast<const uint16_t*>(g), reinterpret_cast<const float*>(h12), rows, hidden, reinterpret_cast<float*>(d_h12));
+        swiglu_bwd_kernel<uint16_t, float><<<grid, block, 0, stream>>>(reinterpret_cast<const uint16_t*>(g), reinterpret_cast<const float*>(h12), rows, hidden, rot, reinterpret_cast<float*>(d_h12));
     else if (dtype == BF16)
-        swiglu_bwd_kernel<float, uint16_t><<<grid, block, 0, stream>>>(reinterpret_cast<const float*>(g), reinterpret_cast<const uint16_t*>(h12), rows, hidden, reinterpret_cast<uint16_t*>(d_h12));
+        swiglu_bwd_kernel<float, uint16_t><<<grid, block, 0, stream>>>(reinterpret_cast<const float*>(g), reinterpret_cast<const uint16_t*>(h12), rows, hidden, rot, reinterpret_cast<uint16_t*>(d_h12));
     else
-        swiglu_bwd_kernel<float, float><<<grid, block, 0, stream>>>(reinterpret_cast<const float*>(g), reinterpret_cast<const float*>(h12), rows, hidden, reinterpret_cast<float*>(d_h12));
+        swiglu_bwd_kernel<float, float><<<grid, block, 0, stream>>>(reinterpret_cast<const float*>(g), reinterpret_cast<const float*>(h12), rows, hidden, rot, reinterpret_cast<float*>(d_h12));
     return hipGetLastError();
 }
 

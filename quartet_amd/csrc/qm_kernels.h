@@ -82,10 +82,10 @@ hipError_t swiglu_quantize_hd32(const void* h12, int dtype, int64_t rows, int64_
                                 uint8_t* codes, uint8_t* scales, uint8_t* maskbits, bool tiled, hipStream_t stream);
 size_t rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols);
 hipError_t rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain,
-                            const float* factor, int64_t rows, int64_t cols, void* dx, float* dgain, void* workspace,
-                            hipStream_t stream);
+                            const float* factor, int64_t rows, int64_t cols, const uint8_t* maskbits, uint32_t sign_word,
+                            int scale_dtype, void* dx, float* dgain, void* workspace, hipStream_t stream);
 hipError_t swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
-                           void* d_h12, hipStream_t stream);
+                           const uint8_t* maskbits, uint32_t sign_word, int scale_dtype, void* d_h12, hipStream_t stream);
 
 // Rotary embedding of the fused attention projection: split + rotate, and the merge + inverse rotation of its backward
 hipError_t rope_split_qkv(const void* qkv, int qkv_dtype, int64_t rows, int seq_len, int C, int head_dim, const float* table,

@@ -44,8 +44,9 @@ class RMSNormLinearFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, e):
         x2, gain, factor, packed_x, packed_w = ctx.saved_tensors
-        gy, gw = _backward_packed(ctx, e, packed_x, packed_w)
-        dx, dgain = K.rmsnorm_backward(gy, x2, gain, factor)
+        # B7 (the quantizer's straight-through backward) runs inside the RMSNorm backward kernel
+        gy, gw, (maskbits, signs, scale_dtype) = _backward_packed(ctx, e, packed_x, packed_w, gx_rotated=True)
+        dx, dgain = K.rmsnorm_backward(gy, x2, gain, factor, maskbits, signs, scale_dtype)
         return dx.view(ctx.x_shape), dgain, gw.to(ctx.w_dtype), None, None, None, None, None
 
 
@@ -69,8 +70,9 @@ class SwiGLULinearFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, e):
         h2, packed_x, packed_w = ctx.saved_tensors
-        g, gw = _backward_packed(ctx, e, packed_x, packed_w)
-        return K.swiglu_backward(g, h2).view(ctx.h_shape), gw.to(ctx.w_dtype), None, None, None, None
+        g, gw, (maskbits, signs, scale_dtype) = _backward_packed(ctx, e, packed_x, packed_w, gx_rotated=True)
+        d_h12 = K.swiglu_backward(g, h2, maskbits, signs, scale_dtype)
+        return d_h12.view(ctx.h_shape), gw.to(ctx.w_dtype), None, None, None, None
 
 
 class RopeQKVFn(torch.autograd.Function):

@@ -207,9 +207,18 @@ def swiglu_quantize(h12, signs, tiled):
     return packed
 
 
-def rmsnorm_backward(gy, x2, gain, factor):
-    """gy [rows, cols] (gradient of the normalised, scaled tensor) -> (dx like x2, dgain fp32 [cols])."""
-    _require_cuda(gy, x2, gain, factor)
+def packed_mask_bits(packed, rows, cols):
+    """The clip-mask bits [rows, cols/8] inside a packed operand buffer (a view)."""
+    off = (ctypes.c_size_t * 3)()
+    _lib.check(_lib.lib().qm_packed_operand_offsets(rows, cols, off), "qm_packed_operand_offsets")
+    return packed[off[2]: off[2] + rows * cols // 8].view(rows, cols // 8)
+
+
+def rmsnorm_backward(gy, x2, gain, factor, maskbits=None, signs=0, scale_dtype=torch.float32):
+    """gy [rows, cols] (gradient of the normalised, scaled tensor) -> (dx like x2, dgain fp32 [cols]).  With `maskbits`
+    (and the rotation's `signs`, `scale_dtype`), gy is the gradient in the activation quantizer's rotated basis and its
+    straight-through backward is applied first, inside the kernel."""
+    _require_cuda(gy, x2, gain, factor, maskbits)
     assert gy.is_contiguous() and x2.is_contiguous() and gy.shape == x2.shape
     rows, cols = x2.shape
     L = _lib.lib()
@@ -218,18 +227,20 @@ def rmsnorm_backward(gy, x2, gain, factor):
     dx = torch.empty_like(x2)
     dgain = torch.empty(cols, dtype=torch.float32, device=x2.device)
     rc = L.qm_rmsnorm_backward(_ptr(gy), _dtype_code(gy.dtype), _ptr(x2), _dtype_code(x2.dtype), _ptr(gain), _ptr(factor), rows, cols,
-                               _ptr(dx), _ptr(dgain), _ptr(work), nbytes, _stream())
+                               _ptr(maskbits), sign_words(signs), _dtype_code(scale_dtype), _ptr(dx), _ptr(dgain), _ptr(work), nbytes,
+                               _stream())
     _lib.check(rc, "qm_rmsnorm_backward")
     return dx, dgain
 
 
-def swiglu_backward(g, h12):
-    """g [rows, hidden] (gradient of silu(up) * gate) -> gradient of h12 [rows, 2 hidden], in h12's dtype."""
-    _require_cuda(g, h12)
+def swiglu_backward(g, h12, maskbits=None, signs=0, scale_dtype=torch.float32):
+    """g [rows, hidden] (gradient of silu(up) * gate) -> gradient of h12 [rows, 2 hidden], in h12's dtype; `maskbits`
+    as for rmsnorm_backward."""
+    _require_cuda(g, h12, maskbits)
     assert g.is_contiguous() and h12.is_contiguous() and h12.shape == (g.shape[0], 2 * g.shape[1])
     d = torch.empty_like(h12)
     rc = _lib.lib().qm_swiglu_backward(_ptr(g), _dtype_code(g.dtype), _ptr(h12), _dtype_code(h12.dtype), g.shape[0], g.shape[1],
-                                       _ptr(d), _stream())
+                                       _ptr(maskbits), sign_words(signs), _dtype_code(scale_dtype), _ptr(d), _stream())
     _lib.check(rc, "qm_swiglu_backward")
     return d
 
@@ -260,8 +271,10 @@ def rope_merge_qkv_grad(dq, dk, dv, table, n_embd, head_dim, seq_len, out_dtype)
 
 
 def linear_backward(e2, packed_x, packed_w, T, I, O, hd_x, signs_x, hd_w, signs_w, hd_g, signs_g, mode, seeds, x_val_dtype,
-                    w_val_dtype, mid_dtype, x_scale_dtype, w_scale_dtype, tiled):
-    """Whole backward pass in one foreign call: e [T,O] -> (gx [T,I], gw [O,I]) of mid_dtype."""
+                    w_val_dtype, mid_dtype, x_scale_dtype, w_scale_dtype, tiled, gx_rotated=False):
+    """Whole backward pass in one foreign call: e [T,O] -> (gx [T,I], gw [O,I]) of mid_dtype.  With `gx_rotated`, gx is
+    still in the rotated basis of the activation quantizer: its masked inverse rotation is left to the kernel that
+    consumes gx (rmsnorm_backward / swiglu_backward with `maskbits`)."""
     _require_cuda(e2, packed_x, packed_w)
     assert e2.is_contiguous() and e2.shape == (T, O)
     L = _lib.lib()
@@ -273,6 +286,6 @@ def linear_backward(e2, packed_x, packed_w, T, I, O, hd_x, signs_x, hd_w, signs_
     rc = L.qm_linear_backward(_ptr(e2), _dtype_code(e2.dtype), T, I, O, _ptr(packed_x), _ptr(packed_w), hd_x, sign_words(signs_x),
                               hd_w, sign_words(signs_w), hd_g, sign_words(signs_g), mode, (ctypes.c_uint64 * 4)(*seeds),
                               _dtype_code(x_val_dtype), _dtype_code(w_val_dtype), mid, _dtype_code(x_scale_dtype),
-                              _dtype_code(w_scale_dtype), _ptr(work), nbytes, _ptr(gx), _ptr(gw), _layout(tiled), _stream())
+                              _dtype_code(w_scale_dtype), _ptr(work), nbytes, _ptr(gx), _ptr(gw), _layout(tiled), int(gx_rotated), _stream())
     _lib.check(rc, "qm_linear_backward")
     return gx, gw

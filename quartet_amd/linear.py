@@ -42,8 +42,10 @@ def _forward_packed(ctx, x2, weight, a_q, w_q, g_q, weight_cache, tiled, out_dty
     return y, packed_x, packed_w
 
 
-def _backward_packed(ctx, e, packed_x, packed_w):
-    """B1-B8: e [.., O] -> (gradient w.r.t. the tensor F1 quantized [T, I], gradient w.r.t. W [O, I])."""
+def _backward_packed(ctx, e, packed_x, packed_w, gx_rotated=False):
+    """B1-B8: e [.., O] -> (gradient w.r.t. the tensor F1 quantized [T, I], gradient w.r.t. W [O, I]).  With
+    `gx_rotated` B7 is left out: returns (gradient in F1's rotated basis, gradient w.r.t. W, (mask bits, signs, scale
+    dtype) that the consumer's kernel needs to apply B7 itself)."""
     g_q = ctx.g_q
     a_hd, a_signs, w_hd, w_signs = ctx.fwd
     T, I, O = ctx.dims
@@ -57,8 +59,11 @@ def _backward_packed(ctx, e, packed_x, packed_w):
     mid_dtype = torch.bfloat16 if low else e2.dtype
     sd_x = torch.bfloat16 if low else ctx.x_dtype
     sd_w = torch.bfloat16 if low else ctx.w_dtype
-    return K.linear_backward(e2, packed_x, packed_w, T, I, O, a_hd, a_signs, w_hd, w_signs, hd, signs, mode, seeds, ctx.x_dtype,
-                             ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled)
+    gx, gw = K.linear_backward(e2, packed_x, packed_w, T, I, O, a_hd, a_signs, w_hd, w_signs, hd, signs, mode, seeds, ctx.x_dtype,
+                               ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled, gx_rotated)
+    if gx_rotated:
+        return gx, gw, (K.packed_mask_bits(packed_x, T, I), a_signs, sd_x)
+    return gx, gw
 
 
 class QuartetLinearFn(torch.autograd.Function):

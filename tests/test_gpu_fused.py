@@ -261,3 +261,26 @@ def test_rope_qkv_matches_the_op_by_op_rotation(q, B, T, n_head, hs, autocast):
     assert a.grad.dtype == dtype and torch.equal(a.grad, b.grad)
     # a rotation: norms of q and k pairs are preserved up to rounding, position 0 is the identity
     assert torch.equal(fq[:, 0], qkv[:, 0, :C].view(B, n_head, hs))
+
+
+@pytest.mark.parametrize("g_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,cols", [(128, 640), (37, 96), (16, 4096)])
+def test_inverse_rotation_inside_the_backward_kernels(q, rows, cols, g_dtype):
+    """The quantizer's straight-through backward (mask, inverse rotation) applied on the fly by the producers' backward
+    kernels gives the bits of the stand-alone kernel followed by the plain backward kernel."""
+    print(f"case fused inverse rotation rows={rows} cols={cols} g={g_dtype}", flush=True)
+    from quartet_amd import kernels as K
+    g = make_input(rows, cols, g_dtype, seed=rows + cols, scale=1e-2, outlier_frac=0).to(DEV)
+    x = make_input(rows, cols, torch.float32, seed=3, scale=2.0).to(DEV)
+    h12 = make_input(rows, 2 * cols, torch.bfloat16 if g_dtype == torch.bfloat16 else torch.float32, seed=4, scale=2.0).to(DEV)
+    gain = (1.0 + 0.2 * torch.randn(cols, generator=torch.Generator().manual_seed(2))).float().to(DEV)
+    factor = torch.rsqrt(x.double().pow(2).mean(-1) + 1e-5).float()
+    mask = torch.randint(0, 256, (rows, cols // 8), dtype=torch.uint8, generator=torch.Generator().manual_seed(5)).to(DEV)
+    signs = sign_int(signs_vector(11))
+    for scale_dtype in (torch.bfloat16, torch.float32):
+        back = K.masked_hadamard_bwd(g, 32, scale_dtype, signs, mask)
+        assert back.dtype == g_dtype
+        want_dx, want_dg = K.rmsnorm_backward(back, x, gain, factor)
+        got_dx, got_dg = K.rmsnorm_backward(g, x, gain, factor, mask, signs, scale_dtype)
+        assert torch.equal(got_dx, want_dx) and torch.equal(got_dg, want_dg)
+        assert torch.equal(K.swiglu_backward(g, h12, mask, signs, scale_dtype), K.swiglu_backward(back, h12))
