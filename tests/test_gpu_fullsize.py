@@ -183,3 +183,52 @@ def test_linear_step_rows_against_oracle_pipeline(oracle, K, data):
     gx_ref = torch.from_numpy(gx_ref.view(np.int16)).view(torch.bfloat16).float().numpy().astype(np.float64)
     gx = xd.grad[:n].float().cpu().numpy().astype(np.float64)
     assert np.linalg.norm(gx - gx_ref) / np.linalg.norm(gx_ref) < 1e-2  # two bf16 roundings on the way
+
+
+def _signs_from_word(word):
+    return np.array([-1 if (word >> j) & 1 else 1 for j in range(32)])
+
+
+@pytest.mark.parametrize("rows,cols,dtype", [(32768, 1536, torch.float32), (8192, 4096, torch.bfloat16)])
+def test_rmsnorm_quantize_sampled_rows_match_oracle(oracle, K, rows, cols, dtype):
+    """The fused RMSNorm -> quantizer is row-local: sampled rows of a full-size result (the 800 M model's shape, and
+    the benchmark layer's) must equal the oracle's result on those rows, factor included."""
+    print(f"case fullsize rmsnorm_quantize rows={rows} cols={cols} {dtype}", flush=True)
+    from quartet_amd import packed as P
+    import quartet_amd as q
+    dev = torch.device("cuda:0")
+    gd = torch.Generator(device=dev).manual_seed(rows + cols)
+    x = (3.0 * torch.randn(rows, cols, generator=gd, device=dev)).to(dtype)
+    x[torch.rand(rows, cols, generator=gd, device=dev) < 1e-3] = 200.0
+    gain = 1.0 + 0.1 * torch.randn(cols, generator=gd, device=dev)
+    word = 0x6C1B93A5
+    packed, factor = K.rmsnorm_quantize(x, gain, 1e-5, word, True)
+    t = P.from_operand_buffer(packed, rows, cols, True, q.QuestMXFP4Quantizer()).to_layout("rowmajor")
+    idx = torch.randint(0, rows, (96,), generator=torch.Generator().manual_seed(1))
+    idx = torch.cat([idx, torch.tensor([0, rows - 1])])
+    normed, want_factor = oracle.rmsnorm(to_oracle(x[idx.to(dev)]), gain.cpu().numpy(), 1e-5)
+    want = oracle.quantize(normed, 32, signs=_signs_from_word(word), mode=oracle.QUEST_RTN, want_mask=True)
+    assert np.array_equal(factor[idx.to(dev)].cpu().numpy().view(np.uint32), want_factor.view(np.uint32))
+    assert np.array_equal(t.scales[idx.to(dev)].cpu().numpy(), want["scales"])
+    assert np.array_equal(t.codes[idx.to(dev)].cpu().numpy(), want["codes"])
+    assert np.array_equal(t.maskbits[idx.to(dev)].cpu().numpy(), want["mask"])
+
+
+@pytest.mark.parametrize("rows,hidden", [(32768, 4096), (8192, 11008)])
+def test_swiglu_quantize_sampled_rows_match_oracle(oracle, K, rows, hidden):
+    print(f"case fullsize swiglu_quantize rows={rows} hidden={hidden}", flush=True)
+    from quartet_amd import packed as P
+    import quartet_amd as q
+    dev = torch.device("cuda:0")
+    gd = torch.Generator(device=dev).manual_seed(rows + hidden)
+    h12 = (2.0 * torch.randn(rows, 2 * hidden, generator=gd, device=dev)).to(torch.bfloat16)
+    word = 0x1F3D5B79
+    packed = K.swiglu_quantize(h12, word, True)
+    t = P.from_operand_buffer(packed, rows, hidden, True, q.QuestMXFP4Quantizer()).to_layout("rowmajor")
+    idx = torch.randint(0, rows, (64,), generator=torch.Generator().manual_seed(2))
+    idx = torch.cat([idx, torch.tensor([0, rows - 1])])
+    prod = oracle.swiglu(to_oracle(h12[idx.to(dev)]))
+    want = oracle.quantize(prod, 32, signs=_signs_from_word(word), mode=oracle.QUEST_RTN, want_mask=True)
+    assert np.array_equal(t.scales[idx.to(dev)].cpu().numpy(), want["scales"])
+    assert np.array_equal(t.codes[idx.to(dev)].cpu().numpy(), want["codes"])
+    assert np.array_equal(t.maskbits[idx.to(dev)].cpu().numpy(), want["mask"])
