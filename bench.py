@@ -194,6 +194,23 @@ def cpu_baseline(sample_tokens=T_TOKENS):
                       f"CPU oracle quantizers + fp32 BLAS matmuls on de-quantized operands, {dt:.2f} s"}
 
 
+def library_gemm(device, reps=50):
+    """The vendor library's block-scaled FP4 product (hipBLASLt behind torch._scaled_mm) on the forward GEMM's shape and
+    operand formats, for context next to the hand-written kernel: random codes, unit scales."""
+    M, N, K = T_TOKENS, OUT_F, IN_F
+    try:
+        a = torch.randint(0, 256, (M, K // 2), dtype=torch.uint8, device=device).view(torch.float4_e2m1fn_x2)
+        b = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, device=device).view(torch.float4_e2m1fn_x2)
+        sa = torch.full((M, K // 32), 127, dtype=torch.uint8, device=device).view(torch.float8_e8m0fnu)
+        sb = torch.full((N, K // 32), 127, dtype=torch.uint8, device=device).view(torch.float8_e8m0fnu)
+        run = lambda: torch._scaled_mm(a, b.t(), sa, sb, out_dtype=torch.bfloat16)
+        ms = time_kernel(run, reps=reps, warmup=5)
+    except Exception as exc:  # the installed torch / hipBLASLt may not offer this product
+        return {"error": f"{type(exc).__name__}: {str(exc)[:200]}"}
+    return {"what": f"torch._scaled_mm float4_e2m1fn_x2 x float4_e2m1fn_x2, e8m0 scales per 32, {M}x{N}x{K}, bf16 out",
+            "ms": round(ms, 4), "TFLOPs": round(2.0 * M * N * K / ms / 1e9, 1)}
+
+
 def llama_step(args, device):
     """Whole-model step of a Llama configuration with every block linear on the Quartet path: bf16 autocast around
     forward and backward, cross-entropy on random ids, AdamW (fp32 state) for the ~800 M configuration."""
@@ -257,6 +274,8 @@ def main():
                     help="also run one plain 256 MiB device copy (a known-traffic kernel for scaling profiler byte counters)")
     ap.add_argument("--quantizer-sweep", action="store_true",
                     help="also time the quantizer alone on [rows x 4096] for rows 4096/16384/65536, three modes, hd 32/64/128")
+    ap.add_argument("--library-gemm", action="store_true",
+                    help="also time the vendor library's MXFP4 product (torch._scaled_mm) on the forward GEMM's shape, for context")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)")
@@ -325,6 +344,8 @@ def main():
                                        "avg_launch_ms": qk["ms"]}
     if args.quantizer_sweep:
         result["quantizer_sweep"] = quantizer_sweep(device)
+    if args.library_gemm:
+        result["library_gemm"] = library_gemm(device)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
