@@ -154,7 +154,28 @@ def quantizer_sweep(device):
                                       reps=8, warmup=1)
                 res.append({"rows": rows, "hd": hd, "mode": name, "ms": round(ms, 4),
                             "GBps": round(rows * 4096 * bpe / ms / 1e6, 1)})
+    res.append(cpu_quantizer_baseline())
     return res
+
+
+def cpu_quantizer_baseline(rows=4096):
+    """The CPU oracle's quantizer on [rows x 4096] bf16 (quest RTN + mask, Hadamard 32): one thread, and all host threads."""
+    import ctypes
+
+    from oracle import oracle as o
+    from tests.util import to_oracle
+    x = to_oracle(torch.randn(rows, 4096, generator=torch.Generator().manual_seed(0)).to(torch.bfloat16))
+    o.lib()
+    gomp = ctypes.CDLL("libgomp.so.1")
+    out = {"cpu_oracle_quantizer": f"[{rows} x 4096] bf16, quest RTN + mask, hd 32; 2.65625 B/elt"}
+    for label, n in (("one_thread", 1), ("all_threads", min(os.cpu_count() or 1, 16))):
+        gomp.omp_set_num_threads(n)
+        o.quantize(x[:64], 32, mode=o.QUEST_RTN, want_mask=True)
+        t0 = time.perf_counter()
+        o.quantize(x, 32, mode=o.QUEST_RTN, want_mask=True)
+        dt = time.perf_counter() - t0
+        out[label] = {"threads": n, "GBps": round(rows * 4096 * 2.65625 / dt / 1e9, 3)}
+    return out
 
 
 def cpu_baseline(sample_tokens=T_TOKENS):
