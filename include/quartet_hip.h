@@ -138,12 +138,14 @@ int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, 
  *   packed_flags & QM_X_IS_PACKED: packed_x already holds Q(x), written by one of the fused producers below, and x is
  *   not read.
  * qm_linear_backward = QEQWtt_QEtQXttFn.backward (backward.py:64-85) with the straight-through backward of both
- * forward quantizers (mxfp4.py:143-146) applied: e [T, O] -> gx [T, I], gw [O, I], both of mid_dtype.
+ * forward quantizers (mxfp4.py:143-146) applied: e [T, O] -> gx [T, I] of mid_dtype, gw [O, I] of gw_dtype.
  *   g_mode            QM_ABSMAX_SR or QM_ABSMAX_RTN (AlbertTsengQuantizer stochastic or not)
  *   seeds             HOST pointer to four seeds, for the quantizations of e, Q(w)^T, e^T, Q(x)^T in that order
  *   x_val_dtype, w_val_dtype   dtypes the reference would hold the de-quantized x and w in
  *   x_scale_dtype, w_scale_dtype  dtypes whose rounding of hd^-1/2 the forward quantizers' matrices carry in backward
  *   workspace         qm_linear_backward_workspace_bytes(T, I, O, mid_dtype) bytes of scratch, 256-byte aligned
+ *   gw_dtype          dtype of gw: mid_dtype, or QM_F32 with a bf16 mid_dtype -- then gw holds the bf16-rounded values
+ *                     widened to fp32, i.e. what autograd's cast of a bf16 gradient to an fp32 weight's dtype produces
  *   gx_rotated        != 0: gx receives the gradient w.r.t. the activation quantizer's rotated output (the first
  *                     product, B3) and its straight-through backward is left to the caller, who folds it into the
  *                     next kernel (maskbits argument of qm_rmsnorm_backward / qm_swiglu_backward); needs hd_x == 32
@@ -162,7 +164,8 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                        const void* packed_w, int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w,
                        int hd_g, const uint32_t* signs_g, int g_mode, const uint64_t* seeds, int x_val_dtype,
                        int w_val_dtype, int mid_dtype, int x_scale_dtype, int w_scale_dtype, void* workspace,
-                       size_t workspace_bytes, void* gx, void* gw, int codes_layout, int gx_rotated, void* stream);
+                       size_t workspace_bytes, void* gx, void* gw, int gw_dtype, int codes_layout, int gx_rotated,
+                       void* stream);
 
 /*
  * Producers fused into the activation quantizer.  The tensor the model would hand to a quantized linear is computed

@@ -93,7 +93,7 @@ def lib():
     L.qm_rope_merge_qkv_grad.argtypes = [vp, vp, vp, i32, i64, i64, i64, i32, vp, vp, i32, vp]
     L.qm_linear_backward.restype = i32
     L.qm_linear_backward.argtypes = [vp, i32, i64, i64, i64, vp, vp, i32, vp, i32, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32,
-                                     vp, sz, vp, vp, i32, i32, vp]
+                                     vp, sz, vp, vp, i32, i32, i32, vp]
     _lib = L
     return L
 

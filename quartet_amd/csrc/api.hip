@@ -42,7 +42,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 5; }
+int qm_version(void) { return 6; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -138,7 +138,7 @@ int qm_masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t col
     if (!g || !out) return fail(QM_ERR_INVALID, "qm_masked_hadamard_bwd: null tensor");
     if (!aligned(g, 16) || !aligned(out, 16)) return fail(QM_ERR_UNALIGNED, "qm_masked_hadamard_bwd: g and out need 16-byte alignment");
     return from_hip(qm::masked_hadamard_bwd(g, g_dtype, rows, cols, hadamard_dim, scale_dtype,
-                                            make_signs(sign_bits, hadamard_dim), maskbits, out, out_dtype,
+                                            make_signs(sign_bits, hadamard_dim), maskbits, out, out_dtype, false,
                                             reinterpret_cast<hipStream_t>(stream)),
                     "qm_masked_hadamard_bwd");
 }
@@ -265,13 +265,16 @@ int qm_linear_forward(const void* x, int x_dtype, const void* w, int w_dtype, in
 int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t O, const void* packed_x, const void* packed_w,
                        int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, int hd_g, const uint32_t* signs_g,
                        int g_mode, const uint64_t* seeds, int x_val_dtype, int w_val_dtype, int mid_dtype, int x_scale_dtype,
-                       int w_scale_dtype, void* workspace, size_t workspace_bytes, void* gx, void* gw, int codes_layout,
-                       int gx_rotated, void* stream) {
+                       int w_scale_dtype, void* workspace, size_t workspace_bytes, void* gx, void* gw, int gw_dtype,
+                       int codes_layout, int gx_rotated, void* stream) {
     if (T < 0 || I < 0 || O < 0) return fail(QM_ERR_INVALID, "qm_linear_backward: negative extent");
     if (T == 0 || O == 0 || I == 0) return 0;
     if (g_mode != QM_ABSMAX_RTN && g_mode != QM_ABSMAX_SR)
         return fail(QM_ERR_INVALID, "qm_linear_backward: gradient mode must be QM_ABSMAX_RTN or QM_ABSMAX_SR");
     if (!valid_dtype(mid_dtype)) return fail(QM_ERR_INVALID, "qm_linear_backward: mid_dtype %d", mid_dtype);
+    if (gw_dtype != mid_dtype && !(mid_dtype == QM_BF16 && gw_dtype == QM_F32))
+        return fail(QM_ERR_INVALID, "qm_linear_backward: gw_dtype must be mid_dtype, or QM_F32 with a bf16 mid_dtype (got %d, mid %d)",
+                    gw_dtype, mid_dtype);
     if (I % 32 || O % 32 || T % 32)
         return fail(QM_ERR_INVALID, "qm_linear_backward: tokens, in_features and out_features must be multiples of 32 (T=%lld I=%lld O=%lld)",
                     (long long)T, (long long)I, (long long)O);
@@ -293,6 +296,15 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
     // gx_rotated: the caller undoes the activation quantizer's rotation itself (fused into its next kernel); the first
     // product then lands in gx directly
     void* gx_product = gx_rotated ? gx : static_cast<void*>(k + wl.gxq);
+    // B8: gw in gw_dtype; a bf16 result widened to fp32 keeps its bf16 rounding (what converting it afterwards would give)
+    const auto rotate_gw = [&]() -> int {
+        if (gw_dtype == mid_dtype)
+            return qm_masked_hadamard_bwd(k + wl.gwq, mid_dtype, O, I, hd_w, w_scale_dtype, signs_w, pw + lw.m, gw, mid_dtype, stream);
+        if (!valid_hd(hd_w) || I % hd_w || !gw || !aligned(gw, 16) || !valid_dtype(w_scale_dtype))
+            return fail(QM_ERR_INVALID, "qm_linear_backward: bad hd_w, w_scale_dtype or gw");
+        return from_hip(qm::masked_hadamard_bwd(k + wl.gwq, mid_dtype, O, I, hd_w, w_scale_dtype, make_signs(signs_w, hd_w), pw + lw.m, gw,
+                                                gw_dtype, true, hs), "qm_linear_backward");
+    };
     if (gx_rotated && hd_x != 32) return fail(QM_ERR_INVALID, "qm_linear_backward: gx_rotated needs hd_x == 32");
     if (pair_launches(codes_layout, T, I, O, hd_x, hd_w, hd_g) && e && gx && gw && valid_dtype(e_dtype) && aligned(e, 16) &&
         aligned(gx, 16) && aligned(gw, 16) && valid_dtype(x_val_dtype) && valid_dtype(w_val_dtype) &&
@@ -312,12 +324,11 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
         rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, k + wl.gwq, mid_dtype, codes_layout,
                               codes_layout, gws, wl.gemm_ws_bytes, stream);
         if (rc) return rc;
-        if (gx_rotated)
-            return qm_masked_hadamard_bwd(k + wl.gwq, mid_dtype, O, I, hd_w, w_scale_dtype, signs_w, pw + lw.m, gw, mid_dtype, stream);
+        if (gx_rotated) return rotate_gw();
         return from_hip(qm::masked_hadamard_bwd_hd32_pair(k + wl.gxq, T * I, x_scale_dtype,
                                                           signs_x ? signs_x[0] : 0u, px + lx.m, gx, k + wl.gwq, O * I,
                                                           w_scale_dtype, signs_w ? signs_w[0] : 0u,
-                                                          pw + lw.m, gw, mid_dtype, hs), "qm_linear_backward");
+                                                          pw + lw.m, gw, mid_dtype, gw_dtype, hs), "qm_linear_backward");
     }
     rc = qm_quantize_mxfp4(e, e_dtype, T, O, hd_g, signs_g, g_mode, 0, nullptr, seeds[0], k + wl.ec, k + wl.es, nullptr, nullptr,
                            codes_layout, stream);
@@ -341,7 +352,7 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
         rc = qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, px + lx.m, gx, mid_dtype, stream);
         if (rc) return rc;
     }
-    return qm_masked_hadamard_bwd(k + wl.gwq, mid_dtype, O, I, hd_w, w_scale_dtype, signs_w, pw + lw.m, gw, mid_dtype, stream);
+    return rotate_gw();
 }
 
 int qm_rmsnorm_quantize_mxfp4(const void* x, int x_dtype, const float* gain, float eps, int64_t rows, int64_t cols,

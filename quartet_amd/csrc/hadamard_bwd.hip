@@ -45,7 +45,9 @@ __device__ __forceinline__ void cross_lane_stage(float (&v)[8], int lane_in_chun
 }
 
 // The work of one launch as a job (qm_jobs.h): two independent inverse rotations can share a grid.
-template <typename TIn, typename TOut, int HD>
+// ROUND_IN (bf16 in, fp32 out): the result is rounded to bf16 and then widened -- what a bf16 result converted to fp32
+// afterwards holds, without the separate conversion pass.
+template <typename TIn, typename TOut, int HD, bool ROUND_IN = false>
 struct HadamardBwdJob {
     const TIn* g;
     int64_t n_octets;
@@ -112,8 +114,18 @@ struct HadamardBwdJob {
             }
             *reinterpret_cast<uint4*>(out + octet * 8) = make_uint4(w[0], w[1], w[2], w[3]);
         } else {
-            *reinterpret_cast<float4*>(out + octet * 8) = make_float4(v[0] * c, v[1] * c, v[2] * c, v[3] * c);
-            *reinterpret_cast<float4*>(out + octet * 8 + 4) = make_float4(v[4] * c, v[5] * c, v[6] * c, v[7] * c);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = v[i] * c;
+            if constexpr (ROUND_IN) {
+#pragma unroll
+                for (int i = 0; i < 8; i += 2) {
+                    const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[i], v[i + 1]}, v2bf));
+                    v[i] = u2f(w << 16);
+                    v[i + 1] = u2f(w & 0xffff0000u);
+                }
+            }
+            *reinterpret_cast<float4*>(out + octet * 8) = make_float4(v[0], v[1], v[2], v[3]);
+            *reinterpret_cast<float4*>(out + octet * 8 + 4) = make_float4(v[4], v[5], v[6], v[7]);
         }
     }
 };
@@ -144,37 +156,43 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t* __restr
     }
 }
 
-template <typename TIn, typename TOut>
+template <typename TIn, typename TOut, bool ROUND_IN = false>
 void launch_bwd(int hd, const void* g, int64_t n, float c, const SignBits& sb, const uint8_t* maskbits, void* out,
                 hipStream_t stream) {
     const auto go = [&](auto job) { launch_job(job, stream); };
-    if (hd == 32) go(HadamardBwdJob<TIn, TOut, 32>(g, n, c, sb, maskbits, out));
-    else if (hd == 64) go(HadamardBwdJob<TIn, TOut, 64>(g, n, c, sb, maskbits, out));
-    else go(HadamardBwdJob<TIn, TOut, 128>(g, n, c, sb, maskbits, out));
+    if (hd == 32) go(HadamardBwdJob<TIn, TOut, 32, ROUND_IN>(g, n, c, sb, maskbits, out));
+    else if (hd == 64) go(HadamardBwdJob<TIn, TOut, 64, ROUND_IN>(g, n, c, sb, maskbits, out));
+    else go(HadamardBwdJob<TIn, TOut, 128, ROUND_IN>(g, n, c, sb, maskbits, out));
 }
 
 }  // namespace
 
+// round_to_g_dtype: with bf16 g and fp32 out, round the result to bf16 before widening
 hipError_t masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t cols, int hd, int scale_dtype,
                                const SignBits& sb, const uint8_t* maskbits, void* out, int out_dtype,
-                               hipStream_t stream) {
+                               bool round_to_g_dtype, hipStream_t stream) {
     if (rows == 0 || cols == 0) return hipSuccess;
     const float c = hadamard_scale(hd, scale_dtype);
     const int64_t n = rows * cols;
     if (g_dtype == BF16 && out_dtype == BF16) launch_bwd<uint16_t, uint16_t>(hd, g, n, c, sb, maskbits, out, stream);
+    else if (g_dtype == BF16 && round_to_g_dtype) launch_bwd<uint16_t, float, true>(hd, g, n, c, sb, maskbits, out, stream);
     else if (g_dtype == BF16) launch_bwd<uint16_t, float>(hd, g, n, c, sb, maskbits, out, stream);
     else if (out_dtype == BF16) launch_bwd<float, uint16_t>(hd, g, n, c, sb, maskbits, out, stream);
     else launch_bwd<float, float>(hd, g, n, c, sb, maskbits, out, stream);
     return hipGetLastError();
 }
 
-// two independent masked inverse rotations (Hadamard block 32, same element type in and out) in one grid
+// two independent masked inverse rotations (Hadamard block 32, element type `dtype` in; a out in `dtype`, b out in
+// out_dtype_b: `dtype`, or fp32 holding the bf16-rounded result) in one grid
 hipError_t masked_hadamard_bwd_hd32_pair(const void* ga, int64_t na, int scale_dtype_a, uint32_t sign_a, const uint8_t* mask_a, void* out_a,
                                          const void* gb, int64_t nb, int scale_dtype_b, uint32_t sign_b, const uint8_t* mask_b, void* out_b,
-                                         int dtype, hipStream_t stream) {
+                                         int dtype, int out_dtype_b, hipStream_t stream) {
     const SignBits sa{{sign_a, 0, 0, 0}}, sb{{sign_b, 0, 0, 0}};
     const float ca = hadamard_scale(32, scale_dtype_a), cb = hadamard_scale(32, scale_dtype_b);
-    if (dtype == BF16) {
+    if (dtype == BF16 && out_dtype_b == F32) {
+        launch_job_pair(HadamardBwdJob<uint16_t, uint16_t, 32>(ga, na, ca, sa, mask_a, out_a),
+                        HadamardBwdJob<uint16_t, float, 32, true>(gb, nb, cb, sb, mask_b, out_b), stream);
+    } else if (dtype == BF16) {
         using J = HadamardBwdJob<uint16_t, uint16_t, 32>;
         launch_job_pair(J(ga, na, ca, sa, mask_a, out_a), J(gb, nb, cb, sb, mask_b, out_b), stream);
     } else {

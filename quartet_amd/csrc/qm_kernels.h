@@ -72,7 +72,7 @@ hipError_t requantize_transposed_hd32_tiled_pair(const RequantArgs& a, const Req
                                                  hipStream_t stream);
 hipError_t masked_hadamard_bwd_hd32_pair(const void* ga, int64_t na, int scale_dtype_a, uint32_t sign_a, const uint8_t* mask_a, void* out_a,
                                          const void* gb, int64_t nb, int scale_dtype_b, uint32_t sign_b, const uint8_t* mask_b, void* out_b,
-                                         int dtype, hipStream_t stream);
+                                         int dtype, int out_dtype_b, hipStream_t stream);
 
 // Producers fused into the forward quantizer (Hadamard block 32, quest RTN, clip mask) and their backward passes
 hipError_t rmsnorm_quantize_hd32(const void* x, int dtype, const float* gain, float eps, int64_t rows, int64_t cols,
@@ -105,7 +105,7 @@ size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 hipError_t masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t cols, int hd, int scale_dtype,
                                const SignBits& sb, const uint8_t* maskbits, void* out, int out_dtype,
-                               hipStream_t stream);
+                               bool round_to_g_dtype, hipStream_t stream);
 
 hipError_t dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, int64_t C, float post, void* out,
                             int out_dtype, hipStream_t stream);

@@ -60,7 +60,8 @@ def _backward_packed(ctx, e, packed_x, packed_w, gx_rotated=False):
     sd_x = torch.bfloat16 if low else ctx.x_dtype
     sd_w = torch.bfloat16 if low else ctx.w_dtype
     gx, gw = K.linear_backward(e2, packed_x, packed_w, T, I, O, a_hd, a_signs, w_hd, w_signs, hd, signs, mode, seeds, ctx.x_dtype,
-                               ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled, gx_rotated)
+                               ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled, gx_rotated,
+                               ctx.w_dtype if ctx.w_dtype in (torch.float32, torch.bfloat16) else None)
     if gx_rotated:
         return gx, gw, (K.packed_mask_bits(packed_x, T, I), a_signs, sd_x)
     return gx, gw

@@ -299,3 +299,25 @@ def test_packed_weight_cache_across_micro_steps(q):
     for got, want in zip(step(cached, xs[1], dys[1]), step(plain, xs[1], dys[1])):
         assert torch.equal(got, want)
     assert cache.misses == 3
+
+
+@pytest.mark.parametrize("T,I,O", [(256, 256, 384), (64, 96, 160)])
+def test_weight_gradient_widened_in_the_kernel(q, T, I, O):
+    """gw_dtype = float32 with bf16 intermediates: the last kernel of the backward pass writes the bf16-rounded weight
+    gradient as fp32 -- the bits a separate bf16 -> fp32 conversion of the bf16 result holds."""
+    from quartet_amd import kernels as K
+    x = make_input(T, I, torch.bfloat16, seed=1).to("cuda:0")
+    w = make_input(O, I, torch.float32, seed=2, scale=0.02).to("cuda:0")
+    e = make_input(T, O, torch.bfloat16, seed=3, scale=1e-2, outlier_frac=0).to("cuda:0")
+    tiled = all(d % 128 == 0 and d >= 256 for d in (T, I, O))
+    _, px, pw = K.linear_forward(x, w, 32, 0x5A5A5A5A, 32, 0x0F0F1234, torch.bfloat16, tiled)
+    args = (e, px, pw, T, I, O, 32, 0x5A5A5A5A, 32, 0x0F0F1234, 32, 0x13572468, K.QM_ABSMAX_SR, [11, 12, 13, 14],
+            torch.bfloat16, torch.float32, torch.bfloat16, torch.bfloat16, torch.bfloat16, tiled)
+    gx0, gw0 = K.linear_backward(*args)
+    gx1, gw1 = K.linear_backward(*args, gw_dtype=torch.float32)
+    assert gw0.dtype == torch.bfloat16 and gw1.dtype == torch.float32
+    assert torch.equal(gx0, gx1) and torch.equal(gw0.float(), gw1)
+    gx2, gw2 = K.linear_backward(*args, gx_rotated=True, gw_dtype=torch.float32)
+    assert torch.equal(gw2, gw1)
+    mask = K.packed_mask_bits(px, T, I)
+    assert torch.equal(K.masked_hadamard_bwd(gx2, 32, torch.bfloat16, 0x5A5A5A5A, mask), gx0)
