@@ -260,11 +260,13 @@ def llama_step(args, device):
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         loss = step()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / args.steps * 1e3
+    peak_gib = torch.cuda.max_memory_allocated() / 2 ** 30
     lin = sum(m.weight.numel() for _, m in model.block_linears())
     tokens = batch * seq
     flops = 6.0 * tokens * lin
@@ -275,7 +277,8 @@ def llama_step(args, device):
             "config": {"workload": f"{args.workload}{' (unquantized bf16 linears)' if args.unquantized else ''} whole-model step ({cfg.n_layer} layers, d {cfg.n_embd}, {batch}x{seq} tokens, "
                                    f"{'fwd+bwd+AdamW' if opt_step else 'fwd+bwd'}); value counts the block linears' 6*tokens*params "
                                    f"flops only ({flops / 1e12:.2f} TFLOP) over the whole step time"},
-            "tokens_per_s": round(tokens / (ms * 1e-3), 1), "final_loss": round(float(loss.detach()), 4)}
+            "tokens_per_s": round(tokens / (ms * 1e-3), 1), "final_loss": round(float(loss.detach()), 4),
+            "peak_allocated_GiB": round(peak_gib, 2)}
 
 
 def main():
