@@ -284,3 +284,30 @@ def test_inverse_rotation_inside_the_backward_kernels(q, rows, cols, g_dtype):
         got_dx, got_dg = K.rmsnorm_backward(g, x, gain, factor, mask, signs, scale_dtype)
         assert torch.equal(got_dx, want_dx) and torch.equal(got_dg, want_dg)
         assert torch.equal(K.swiglu_backward(g, h12, mask, signs, scale_dtype), K.swiglu_backward(back, h12))
+
+
+def test_producers_on_random_shapes(oracle, q):
+    """Seeded sweep over ragged shapes (rows not a multiple of the 4 rows of a workgroup, one to 130 groups per row, so
+    one, two and three passes of a wave over its row) for both producers, both dtypes and both code layouts."""
+    from quartet_amd import kernels as K
+    rng = np.random.default_rng(7)
+    for case in range(24):
+        groups = int(rng.choice([1, 2, 3, 5, 16, 17, 63, 64, 65, 127, 130]))
+        cols = 32 * groups
+        tiled = bool(groups % 4 == 0 and rng.integers(2))
+        rows = int(rng.integers(1, 12)) * 16 if tiled else int(rng.integers(1, 90))
+        dtype = torch.bfloat16 if rng.integers(2) else torch.float32
+        signs = signs_vector(case)
+        print(f"case sweep {case}: rows={rows} cols={cols} tiled={tiled} {dtype}", flush=True)
+        x = make_input(rows, cols, dtype, seed=case, scale=float(rng.uniform(0.01, 50.0)))
+        gain = (1.0 + 0.3 * torch.randn(cols, generator=torch.Generator().manual_seed(case))).float()
+        normed, factor = oracle.rmsnorm(to_oracle(x), gain.numpy(), 1e-6)
+        want = oracle.quantize(normed, 32, signs=signs.numpy(), mode=oracle.QUEST_RTN, want_mask=True)
+        packed, got_factor = K.rmsnorm_quantize(x.to(DEV), gain.to(DEV), 1e-6, sign_int(signs), tiled)
+        codes, scales, mask = unpack(q, packed, rows, cols, tiled)
+        assert np.array_equal(got_factor.cpu().numpy().view(np.uint32), factor.view(np.uint32))
+        assert np.array_equal(scales, want["scales"]) and np.array_equal(codes, want["codes"]) and np.array_equal(mask, want["mask"])
+        h12 = make_input(rows, 2 * cols, dtype, seed=100 + case, scale=float(rng.uniform(0.1, 8.0)))
+        want = oracle.quantize(oracle.swiglu(to_oracle(h12)), 32, signs=signs.numpy(), mode=oracle.QUEST_RTN, want_mask=True)
+        codes, scales, mask = unpack(q, K.swiglu_quantize(h12.to(DEV), sign_int(signs), tiled), rows, cols, tiled)
+        assert np.array_equal(scales, want["scales"]) and np.array_equal(codes, want["codes"]) and np.array_equal(mask, want["mask"])
