@@ -141,6 +141,22 @@ def from_operand_buffer(buffer, rows, cols, tiled, quantizer):
                         "tiled" if tiled else "rowmajor", quantizer.hadamard_dim, quantizer.sign_bits, "quest")
 
 
+def pack_model_weights(model, tiled=False) -> Dict[str, PackedTensor]:
+    """Quantized weights of every ``QuantizedLinear`` of `model` whose weight quantizer is the forward MXFP4 quantizer,
+    keyed by parameter name (``transformer.h.0.attn.c_attn.weight`` ...): what a layer's forward pass multiplies with,
+    ready for ``save_packed`` -- the quantized checkpoint an inference engine with FP4 GEMMs consumes.  Each tensor is
+    in its layer's rotated basis (``hadamard_dim``, ``sign_bits``): activations must be rotated the same way."""
+    from .linear import QuantizedLinear
+    from .quantizers import QuestMXFP4Quantizer
+    out = {}
+    for name, m in model.named_modules():
+        if isinstance(m, QuantizedLinear) and type(m.weight_quantizer) is QuestMXFP4Quantizer and not m.weight_quantizer.is_dense:
+            w_q = m.weight_quantizer
+            ok = tiled and m.weight.shape[0] % 16 == 0 and m.weight.shape[1] % 128 == 0 and w_q.hadamard_dim == 32
+            out[f"{name}.weight"] = pack_quest(m.weight.detach(), w_q.hadamard_dim, w_q.sign_bits, tiled=ok)
+    return out
+
+
 def save_packed(path, tensors: Dict[str, PackedTensor], extra_metadata: Optional[Dict[str, str]] = None):
     """Write packed tensors to a safetensors file."""
     from safetensors.torch import save_file

@@ -66,3 +66,27 @@ def test_views_into_the_operand_buffers(P, T, I, O):
     # the layer's output is the product of the two de-quantized operands
     ref = xp.dequantize(torch.float32) @ wp.dequantize(torch.float32).T
     assert float((y.float() - ref).norm() / ref.norm()) < 5e-3
+
+
+def test_quantized_checkpoint_of_a_model(P, tmp_path):
+    """pack_model_weights -> file -> load: every block linear's packed weight, and the product of a packed activation
+    with the reloaded packed weight equals the layer's own forward output."""
+    print("case packed model checkpoint", flush=True)
+    import quartet_amd as q
+    from quartet_amd import kernels as K
+    from quartet_amd.llama import Llama, LlamaConfig
+    torch.manual_seed(0)
+    model = Llama(LlamaConfig(vocab_size=128, sequence_length=64, n_layer=2, n_head=2, n_embd=256, multiple_of=128)).to(DEV)
+    packed = P.pack_model_weights(model, tiled=True)
+    assert len(packed) == 8 and all(k.endswith(".weight") for k in packed)
+    P.save_packed(tmp_path / "model.safetensors", packed, {"model": "toy"})
+    back = P.load_packed(tmp_path / "model.safetensors", device=DEV)
+    name, layer = model.block_linears()[0]
+    wp = back[f"{name}.weight"]
+    assert wp.layout == "tiled" and (wp.rows, wp.cols) == tuple(layer.weight.shape)
+    x = make_input(256, layer.weight.shape[1], torch.bfloat16, seed=5).to(DEV)
+    xp = P.pack_quest(x, 32, layer.activation_quantizer.sign_bits, tiled=True)
+    y = K.gemm_mxfp4_tn(xp.codes, xp.scales, wp.codes, wp.scales, 1.0, torch.bfloat16, a_tiled=True, b_tiled=True)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        want = layer(x)
+    assert torch.equal(y, want)
