@@ -256,13 +256,13 @@ constexpr int kBigSmemBytes = kStages * kStageBytes;
 constexpr int kLoadsPerStep = 10;  // VMEM instructions per wave per K step
 
 // Tile order: workgroup ids are dealt round-robin to the 8 XCDs by the hardware; give each XCD a
-// contiguous run of tiles in an order that walks 8-row groups column by column, so the tiles that
+// contiguous run of tiles in an order that walks 4-row groups column by column, so the tiles that
 // share an L2 also share A and B panels.
 __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
     const int total = tiles_m * tiles_n;
     int t = bid;
     if ((total & 7) == 0) t = (bid & 7) * (total >> 3) + (bid >> 3);
-    constexpr int GM = 8;
+    constexpr int GM = 4;
     const int per_group = GM * tiles_n;
     const int group = t / per_group;
     const int first_m = group * GM;
@@ -420,7 +420,8 @@ __device__ __forceinline__ void big_epilogue(v16f (&acc)[4][4], float alpha, Out
 //   phase 1: read sub-step-1 fragments of tile ks | 16 MFMAs on its sub-step-0 fragments (in registers);
 //   wait until this wave's loads of tile ks+1 have landed, barrier (tile ks+1 visible to all, stage ks%4 free);
 //   phase 2: request tile ks+4 into stage ks%4; read scales and sub-step-0 fragments of tile ks+1 |
-//            16 MFMAs on sub-step 1 of tile ks.
+//            16 MFMAs on sub-step 1 of tile ks (in the K % 512 kernel below the requests and reads are dealt out
+//            two each per four MFMAs: a wave that issues its eight requests in one clump stalls behind the others').
 template <typename OutT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mxfp4_tn_big_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ b_codes,
@@ -623,12 +624,34 @@ __device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_by
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (Q == 3) big4_read_scales(smem_bytes + kScaleAreaOff + (par ^ 1) * kScaleBufBytes, a_sc_off, b_sc_off, st.sr);
-    big_read_sub(nxt, a_off0, b_off0, st.f0);
-    big4_issue_codes(plan, Q, lks);
-    if constexpr (Q == 0) big4_issue_scales(plan, lks >> 2, par ^ 1);
-    big_mfma_sub<1, SWAP>(st.f1, sca, scb, acc);
-    QM_SCHED_PAIR(0x100, (Q == 3 ? 16 : 8))
-    __builtin_amdgcn_sched_barrier(0);
+    // one quarter of the step's requests and fragment reads per four MFMAs (same issue order as the clumped form)
+    {
+        const uint32_t base = plan.lds_codes + Q * kCodeStageBytes;
+        if constexpr (Q == 3) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const v8i av = v8i{(int)st.f1.a[i].x, (int)st.f1.a[i].y, (int)st.f1.a[i].z, (int)st.f1.a[i].w, 0, 0, 0, 0};
+            const auto products = [&](int j0, int j1) {
+#pragma unroll
+                for (int j = j0; j < j1; ++j) {
+                    const v8i bv = v8i{(int)st.f1.b[j].x, (int)st.f1.b[j].y, (int)st.f1.b[j].z, (int)st.f1.b[j].w, 0, 0, 0, 0};
+                    if constexpr (SWAP)
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, acc[i][j], 4, 4, 1, (int)scb[j], 1, (int)sca[i]);
+                    else
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[i][j], 4, 4, 1, (int)sca[i], 1, (int)scb[j]);
+                }
+            };
+            st.f0.a[i] = *reinterpret_cast<const uint4*>(nxt + a_off0 + i * 32 * kRowBytes);
+            load_lds_b128_s(plan.a + i * plan.row16_bytes + lks * plan.kstep_a, plan.lane_codes_a, base + i * 1024);
+            st.f0.b[i] = *reinterpret_cast<const uint4*>(nxt + kBOff + b_off0 + i * 32 * kRowBytes);
+            load_lds_b128_s(plan.b + i * plan.row16_bytes + lks * plan.kstep_b, plan.lane_codes_b, base + kBOff + i * 1024);
+            if constexpr (Q == 0) {
+                if (i == 3) big4_issue_scales(plan, lks >> 2, par ^ 1);
+            }
+            products(0, 4);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
 }
 
 // bf16 epilogue (operand roles swapped: a lane's accumulator quads run along n).  Eight passes of 32 rows x 64
