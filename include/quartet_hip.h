@@ -182,7 +182,9 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
  *   product to bf16 as torch's bf16 ops do, and the quantizer runs as on a tensor of h12's dtype.
  * qm_rmsnorm_backward: autograd of the RMSNorm line above: gy [rows, cols] (gradient w.r.t. the normalised, scaled
  *   tensor) -> dx [rows, cols] of x's dtype and dgain fp32 [cols] (summed over rows in a fixed order).  cols <= 8192.
- *   workspace: qm_rmsnorm_backward_workspace_bytes(rows, cols) bytes, 16-byte aligned.
+ *   workspace: qm_rmsnorm_backward_workspace_bytes(rows, cols) bytes, 16-byte aligned.  skip (optional, [rows, cols] of
+ *   x's dtype): the gradient that reaches x past the norm (x + f(norm(x)), llama.py:170-171); dx = skip + the norm's
+ *   gradient, the sum autograd would form in a pass of its own.
  * qm_swiglu_backward: autograd of silu(up) * gate: g [rows, hidden] -> d_h12 [rows, 2 hidden] of h12's dtype.
  *   Both backward kernels take the gradient either as it is (maskbits == NULL) or still in the rotated basis of the
  *   layer's activation quantizer (qm_linear_backward with gx_rotated): then maskbits [rows, cols/8] (the mask region of
@@ -198,8 +200,8 @@ int qm_swiglu_quantize_mxfp4(const void* h12, int dtype, int64_t rows, int64_t h
 size_t qm_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols);
 int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain,
                         const float* factor, int64_t rows, int64_t cols, const uint8_t* maskbits,
-                        const uint32_t* sign_bits, int scale_dtype, void* dx, float* dgain, void* workspace,
-                        size_t workspace_bytes, void* stream);
+                        const uint32_t* sign_bits, int scale_dtype, const void* skip, void* dx, float* dgain,
+                        void* workspace, size_t workspace_bytes, void* stream);
 int qm_swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
                        const uint8_t* maskbits, const uint32_t* sign_bits, int scale_dtype, void* d_h12,
                        void* stream);

@@ -84,7 +84,7 @@ def lib():
     L.qm_rmsnorm_backward_workspace_bytes.restype = sz
     L.qm_rmsnorm_backward_workspace_bytes.argtypes = [i64, i64]
     L.qm_rmsnorm_backward.restype = i32
-    L.qm_rmsnorm_backward.argtypes = [vp, i32, vp, i32, vp, vp, i64, i64, vp, vp, i32, vp, vp, vp, sz, vp]
+    L.qm_rmsnorm_backward.argtypes = [vp, i32, vp, i32, vp, vp, i64, i64, vp, vp, i32, vp, vp, vp, vp, sz, vp]
     L.qm_swiglu_backward.restype = i32
     L.qm_swiglu_backward.argtypes = [vp, i32, vp, i32, i64, i64, vp, vp, i32, vp, vp]
     L.qm_rope_split_qkv.restype = i32

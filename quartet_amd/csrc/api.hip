@@ -42,7 +42,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 6; }
+int qm_version(void) { return 7; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -406,8 +406,8 @@ size_t qm_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols) {
 }
 
 int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain, const float* factor,
-                        int64_t rows, int64_t cols, const uint8_t* maskbits, const uint32_t* sign_bits, int scale_dtype, void* dx,
-                        float* dgain, void* workspace, size_t workspace_bytes, void* stream) {
+                        int64_t rows, int64_t cols, const uint8_t* maskbits, const uint32_t* sign_bits, int scale_dtype,
+                        const void* skip, void* dx, float* dgain, void* workspace, size_t workspace_bytes, void* stream) {
     if (!valid_dtype(gy_dtype) || !valid_dtype(x_dtype) || (maskbits && !valid_dtype(scale_dtype)))
         return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: dtypes must be QM_BF16/QM_F32");
     if (rows < 0 || cols <= 0 || cols % 32 || cols > 8192)
@@ -416,11 +416,12 @@ int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype
     if (!dgain) return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: dgain must be non-null");
     if (rows > 0 && (!gy || !x || !gain || !factor || !dx || !workspace || workspace_bytes < qm::rmsnorm_backward_workspace_bytes(rows, cols)))
         return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: null tensor, or workspace below %zu bytes", qm_rmsnorm_backward_workspace_bytes(rows, cols));
-    if (!aligned(gy, 8) || !aligned(x, 8) || !aligned(dx, 8) || !aligned(gain, 16) || !aligned(workspace, 16) ||
+    if (!aligned(skip, 16) || !aligned(gy, 8) || !aligned(x, 8) || !aligned(dx, 8) || !aligned(gain, 16) || !aligned(workspace, 16) ||
         (gy_dtype == QM_F32 && !aligned(gy, 16)) || (x_dtype == QM_F32 && (!aligned(x, 16) || !aligned(dx, 16))))
         return fail(QM_ERR_UNALIGNED, "qm_rmsnorm_backward: tensors need 16-byte alignment");
     return from_hip(qm::rmsnorm_backward(gy, gy_dtype, x, x_dtype, gain, factor, rows, cols, maskbits, sign_bits ? sign_bits[0] : 0u,
-                                         maskbits ? scale_dtype : QM_F32, dx, dgain, workspace, reinterpret_cast<hipStream_t>(stream)),
+                                         maskbits ? scale_dtype : QM_F32, skip, dx, dgain, workspace,
+                                         reinterpret_cast<hipStream_t>(stream)),
                     "qm_rmsnorm_backward");
 }
 

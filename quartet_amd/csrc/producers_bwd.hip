@@ -99,7 +99,8 @@ template <typename TG, typename TX, int NK, int RB>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const TG* __restrict__ gy, const TX* __restrict__ x,
                                                           const float* __restrict__ gain, const float* __restrict__ factor,
                                                           int64_t rows, int cols, int rpb, InverseRotation rot,
-                                                          TX* __restrict__ dx, float* __restrict__ partial) {
+                                                          const TX* __restrict__ skip, TX* __restrict__ dx,
+                                                          float* __restrict__ partial) {
     __shared__ float wave_sums[2][RB][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t r0 = (int64_t)blockIdx.x * rpb;
@@ -161,8 +162,18 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const TG* __restrict__
                 if (col < cols) {
                     const float4 g = gk[j][k], v = xk[j][k];
                     const float fj = f[j];
-                    store4(dx + (rb + j) * cols + col, make_float4(fj * g.x * w[k].x - v.x * coef, fj * g.y * w[k].y - v.y * coef,
-                                                                   fj * g.z * w[k].z - v.z * coef, fj * g.w * w[k].w - v.w * coef));
+                    float4 d = make_float4(fj * g.x * w[k].x - v.x * coef, fj * g.y * w[k].y - v.y * coef,
+                                           fj * g.z * w[k].z - v.z * coef, fj * g.w * w[k].w - v.w * coef);
+                    if (skip) {  // the gradient that reaches x past the norm (the residual connection), added as autograd would
+                        if constexpr (sizeof(TX) == 2) {  // a bf16 gradient is rounded before the sum, as a stored tensor is
+                            const uint32_t lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{d.x, d.y}, v2bf));
+                            const uint32_t hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{d.z, d.w}, v2bf));
+                            d = make_float4(u2f(lo << 16), u2f(lo & 0xffff0000u), u2f(hi << 16), u2f(hi & 0xffff0000u));
+                        }
+                        const float4 sk = load4(skip + (rb + j) * cols + col);
+                        d = make_float4(d.x + sk.x, d.y + sk.y, d.z + sk.z, d.w + sk.w);
+                    }
+                    store4(dx + (rb + j) * cols + col, d);
                 }
             }
         }
@@ -230,15 +241,16 @@ int64_t rmsnorm_bwd_blocks(int64_t rows) { return (rows + rows_per_block(rows) -
 
 template <typename TG, typename TX>
 void launch_rmsnorm_bwd(const void* gy, const void* x, const float* gain, const float* factor, int64_t rows, int cols,
-                        const InverseRotation& rot, void* dx, float* partial, hipStream_t stream) {
+                        const InverseRotation& rot, const void* skip, void* dx, float* partial, hipStream_t stream) {
     const dim3 grid((unsigned)rmsnorm_bwd_blocks(rows)), block(256);
     const int rpb = rows_per_block(rows);
     const TG* g = reinterpret_cast<const TG*>(gy);
     const TX* xp = reinterpret_cast<const TX*>(x);
     TX* dxp = reinterpret_cast<TX*>(dx);
-    if (cols <= 2048) rmsnorm_bwd_kernel<TG, TX, 2, 4><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, dxp, partial);
-    else if (cols <= 4096) rmsnorm_bwd_kernel<TG, TX, 4, 2><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, dxp, partial);
-    else rmsnorm_bwd_kernel<TG, TX, 8, 1><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, dxp, partial);
+    const TX* sk = reinterpret_cast<const TX*>(skip);
+    if (cols <= 2048) rmsnorm_bwd_kernel<TG, TX, 2, 4><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, sk, dxp, partial);
+    else if (cols <= 4096) rmsnorm_bwd_kernel<TG, TX, 4, 2><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, sk, dxp, partial);
+    else rmsnorm_bwd_kernel<TG, TX, 8, 1><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, sk, dxp, partial);
 }
 
 }  // namespace
@@ -249,17 +261,18 @@ size_t rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols) {
 
 // cols <= 8192, cols % 32 == 0; workspace: rmsnorm_backward_workspace_bytes(rows, cols) bytes, 16-byte aligned.
 // maskbits != null: gy is the gradient w.r.t. the quantizer's rotated output and is rotated back on the fly.
+// skip != null: [rows, cols] of x's dtype, added to dx (the gradient of a residual connection around the norm).
 hipError_t rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain,
                             const float* factor, int64_t rows, int64_t cols, const uint8_t* maskbits, uint32_t sign_word,
-                            int scale_dtype, void* dx, float* dgain, void* workspace, hipStream_t stream) {
+                            int scale_dtype, const void* skip, void* dx, float* dgain, void* workspace, hipStream_t stream) {
     if (cols == 0) return hipSuccess;
     float* partial = reinterpret_cast<float*>(workspace);
     const InverseRotation rot{maskbits, sign_word, hadamard_scale(32, scale_dtype)};
     if (rows == 0) {}  // no rows: the column sums below write zeros
-    else if (gy_dtype == BF16 && x_dtype == BF16) launch_rmsnorm_bwd<uint16_t, uint16_t>(gy, x, gain, factor, rows, (int)cols, rot, dx, partial, stream);
-    else if (gy_dtype == BF16) launch_rmsnorm_bwd<uint16_t, float>(gy, x, gain, factor, rows, (int)cols, rot, dx, partial, stream);
-    else if (x_dtype == BF16) launch_rmsnorm_bwd<float, uint16_t>(gy, x, gain, factor, rows, (int)cols, rot, dx, partial, stream);
-    else launch_rmsnorm_bwd<float, float>(gy, x, gain, factor, rows, (int)cols, rot, dx, partial, stream);
+    else if (gy_dtype == BF16 && x_dtype == BF16) launch_rmsnorm_bwd<uint16_t, uint16_t>(gy, x, gain, factor, rows, (int)cols, rot, skip, dx, partial, stream);
+    else if (gy_dtype == BF16) launch_rmsnorm_bwd<uint16_t, float>(gy, x, gain, factor, rows, (int)cols, rot, skip, dx, partial, stream);
+    else if (x_dtype == BF16) launch_rmsnorm_bwd<float, uint16_t>(gy, x, gain, factor, rows, (int)cols, rot, skip, dx, partial, stream);
+    else launch_rmsnorm_bwd<float, float>(gy, x, gain, factor, rows, (int)cols, rot, skip, dx, partial, stream);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
     column_sum_kernel<<<dim3((unsigned)((cols + 63) / 64)), dim3(1024), 0, stream>>>(partial, (int)rmsnorm_bwd_blocks(rows),

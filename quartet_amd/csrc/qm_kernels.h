@@ -83,7 +83,7 @@ hipError_t swiglu_quantize_hd32(const void* h12, int dtype, int64_t rows, int64_
 size_t rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols);
 hipError_t rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain,
                             const float* factor, int64_t rows, int64_t cols, const uint8_t* maskbits, uint32_t sign_word,
-                            int scale_dtype, void* dx, float* dgain, void* workspace, hipStream_t stream);
+                            int scale_dtype, const void* skip, void* dx, float* dgain, void* workspace, hipStream_t stream);
 hipError_t swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
                            const uint8_t* maskbits, uint32_t sign_word, int scale_dtype, void* d_h12, hipStream_t stream);
 

@@ -24,10 +24,14 @@ def _layer_is_fusable(layer):
 
 
 class RMSNormLinearFn(torch.autograd.Function):
-    """y = Q(rmsnorm(x) * gain) Q(W)^T; backward = the layer's quantized backward followed by RMSNorm's."""
+    """y = Q(rmsnorm(x) * gain) Q(W)^T; backward = the layer's quantized backward followed by RMSNorm's.
+
+    With `pass_input` the function also returns x itself: a block computes ``x + f(norm(x))``, and when the residual sum
+    takes this second output instead of x, both gradients of x (through the norm and past it) arrive here together and
+    the RMSNorm backward kernel adds them, instead of autograd in a pass of its own."""
 
     @staticmethod
-    def forward(ctx, x, gain, weight, eps, a_q, w_q, g_q, weight_cache):
+    def forward(ctx, x, gain, weight, eps, a_q, w_q, g_q, weight_cache, pass_input=False):
         I = weight.shape[1]
         x2 = x.reshape(-1, I).contiguous()
         T, O = x2.shape[0], weight.shape[0]
@@ -39,15 +43,18 @@ class RMSNormLinearFn(torch.autograd.Function):
                                                 packed_x, T)
         ctx.save_for_backward(x2, gain, factor, packed_x, packed_w)
         ctx.x_shape = x.shape
-        return y.view(*x.shape[:-1], O)
+        y = y.view(*x.shape[:-1], O)
+        return (y, x) if pass_input else y
 
     @staticmethod
-    def backward(ctx, e):
+    def backward(ctx, e, skip=None):
         x2, gain, factor, packed_x, packed_w = ctx.saved_tensors
         # B7 (the quantizer's straight-through backward) runs inside the RMSNorm backward kernel
         gy, gw, (maskbits, signs, scale_dtype) = _backward_packed(ctx, e, packed_x, packed_w, gx_rotated=True)
-        dx, dgain = K.rmsnorm_backward(gy, x2, gain, factor, maskbits, signs, scale_dtype)
-        return dx.view(ctx.x_shape), dgain, gw.to(ctx.w_dtype), None, None, None, None, None
+        if skip is not None:
+            skip = skip.reshape(x2.shape).to(x2.dtype).contiguous()
+        dx, dgain = K.rmsnorm_backward(gy, x2, gain, factor, maskbits, signs, scale_dtype, skip)
+        return dx.view(ctx.x_shape), dgain, gw.to(ctx.w_dtype), None, None, None, None, None, None
 
 
 class SwiGLULinearFn(torch.autograd.Function):
@@ -115,13 +122,16 @@ def rope_qkv(qkv, table, n_head):
     return q, k, v.view(B, T, n_head, hs)
 
 
-def rmsnorm_linear(norm, layer, x):
-    """layer(norm(x)) for an RMSNorm module `norm` (attributes ``weight`` and ``eps``) and a QuantizedLinear."""
+def rmsnorm_linear(norm, layer, x, pass_input=False):
+    """layer(norm(x)) for an RMSNorm module `norm` (attributes ``weight`` and ``eps``) and a QuantizedLinear.  With
+    `pass_input` returns (layer(norm(x)), x): use the second value for the residual sum around the norm, so that the sum
+    of x's two gradients happens inside the RMSNorm backward kernel."""
     if (_layer_is_fusable(layer) and x.is_cuda and x.dtype in _KERNEL_DTYPES and norm.weight.dtype == torch.float32
             and x.shape[-1] <= 8192):
         return RMSNormLinearFn.apply(x, norm.weight, layer.weight, norm.eps, layer.activation_quantizer, layer.weight_quantizer,
-                                     layer.backward_scheme.g_quantizer, layer.packed_weight_cache)
-    return layer(norm(x))
+                                     layer.backward_scheme.g_quantizer, layer.packed_weight_cache, pass_input)
+    y = layer(norm(x))
+    return (y, x) if pass_input else y
 
 
 def swiglu_linear(layer, h12):

@@ -214,11 +214,13 @@ def packed_mask_bits(packed, rows, cols):
     return packed[off[2]: off[2] + rows * cols // 8].view(rows, cols // 8)
 
 
-def rmsnorm_backward(gy, x2, gain, factor, maskbits=None, signs=0, scale_dtype=torch.float32):
+def rmsnorm_backward(gy, x2, gain, factor, maskbits=None, signs=0, scale_dtype=torch.float32, skip=None):
     """gy [rows, cols] (gradient of the normalised, scaled tensor) -> (dx like x2, dgain fp32 [cols]).  With `maskbits`
     (and the rotation's `signs`, `scale_dtype`), gy is the gradient in the activation quantizer's rotated basis and its
-    straight-through backward is applied first, inside the kernel."""
-    _require_cuda(gy, x2, gain, factor, maskbits)
+    straight-through backward is applied first, inside the kernel.  `skip` (like x2) is added to dx: the gradient of a
+    residual connection around the norm."""
+    _require_cuda(gy, x2, gain, factor, maskbits, skip)
+    assert skip is None or (skip.is_contiguous() and skip.shape == x2.shape and skip.dtype == x2.dtype)
     assert gy.is_contiguous() and x2.is_contiguous() and gy.shape == x2.shape
     rows, cols = x2.shape
     L = _lib.lib()
@@ -227,8 +229,8 @@ def rmsnorm_backward(gy, x2, gain, factor, maskbits=None, signs=0, scale_dtype=t
     dx = torch.empty_like(x2)
     dgain = torch.empty(cols, dtype=torch.float32, device=x2.device)
     rc = L.qm_rmsnorm_backward(_ptr(gy), _dtype_code(gy.dtype), _ptr(x2), _dtype_code(x2.dtype), _ptr(gain), _ptr(factor), rows, cols,
-                               _ptr(maskbits), sign_words(signs), _dtype_code(scale_dtype), _ptr(dx), _ptr(dgain), _ptr(work), nbytes,
-                               _stream())
+                               _ptr(maskbits), sign_words(signs), _dtype_code(scale_dtype), _ptr(skip), _ptr(dx), _ptr(dgain),
+                               _ptr(work), nbytes, _stream())
     _lib.check(rc, "qm_rmsnorm_backward")
     return dx, dgain
 

@@ -123,8 +123,9 @@ class LlamaMLP(nn.Module):
 
     def forward(self, x, norm=None):
         """`norm`: the block's RMSNorm, applied to x here (fused into w12's quantizer) instead of by the caller."""
-        if norm is not None:
-            return swiglu_linear(self.c_proj, rmsnorm_linear(norm, self.w12, x))
+        if norm is not None:   # returns (mlp output, x for the residual sum)
+            h12, x = rmsnorm_linear(norm, self.w12, x, pass_input=True)
+            return swiglu_linear(self.c_proj, h12), x
         up, gate = self.w12(x).split(self.hidden_dim, dim=-1)
         return self.c_proj(F.silu(up) * gate)
 
@@ -141,7 +142,10 @@ class LlamaAttention(nn.Module):
     def forward(self, x, table, norm=None):
         B, T, C = x.shape
         hs = C // self.n_head
-        qkv = self.c_attn(x) if norm is None else rmsnorm_linear(norm, self.c_attn, x)
+        if norm is None:
+            qkv = self.c_attn(x)
+        else:
+            qkv, x = rmsnorm_linear(norm, self.c_attn, x, pass_input=True)
         if norm is not None:   # the fused path: split, rotate and convert in one kernel
             q, k, v = rope_qkv(qkv, table, self.n_head)
         else:
@@ -153,7 +157,8 @@ class LlamaAttention(nn.Module):
             v = v.to(q.dtype)
         y = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=self.dropout, is_causal=True)
         y = y.transpose(1, 2).contiguous().view(B, T, C)
-        return self.resid_dropout(self.c_proj(y))
+        out = self.resid_dropout(self.c_proj(y))
+        return out if norm is None else (out, x)   # with the fused norm: also x for the residual sum
 
 
 class LlamaBlock(nn.Module):
@@ -167,8 +172,10 @@ class LlamaBlock(nn.Module):
 
     def forward(self, x, table):
         if self.fuse_producers:
-            x = x + self.attn(x, table, norm=self.ln_1)
-            return x + self.mlp(x, norm=self.ln_2)
+            a, x = self.attn(x, table, norm=self.ln_1)
+            x = x + a
+            m, x = self.mlp(x, norm=self.ln_2)
+            return x + m
         x = x + self.attn(self.ln_1(x), table)
         return x + self.mlp(self.ln_2(x))
 

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_function():
 
 def test_host_only_entry_points():
     L = _lib.lib()
-    assert L.qm_version() == 6
+    assert L.qm_version() == 7
     T, I, O = 256, 128, 384
     off = (ctypes.c_size_t * 3)()
     for rows, cols in ((T, I), (O, I)):
@@ -69,8 +69,8 @@ def test_host_only_entry_points():
     (lambda L: L.qm_swiglu_quantize_mxfp4(None, 7, 16, 128, None, None, 0, 0, None), b"dtype"),
     (lambda L: L.qm_swiglu_quantize_mxfp4(None, 0, 16, 100, None, None, 0, 0, None), b"multiple of 32"),
     (lambda L: L.qm_swiglu_quantize_mxfp4(None, 0, 16, 128, None, None, 0, 0, None), b"non-null"),
-    (lambda L: L.qm_rmsnorm_backward(None, 0, None, 0, None, None, 16, 16384, None, None, 0, None, None, None, 0, None), b"[32, 8192]"),
-    (lambda L: L.qm_rmsnorm_backward(None, 0, None, 0, None, None, 16, 128, None, None, 0, None, None, None, 0, None), b"dgain"),
+    (lambda L: L.qm_rmsnorm_backward(None, 0, None, 0, None, None, 16, 16384, None, None, 0, None, None, None, None, 0, None), b"[32, 8192]"),
+    (lambda L: L.qm_rmsnorm_backward(None, 0, None, 0, None, None, 16, 128, None, None, 0, None, None, None, None, 0, None), b"dgain"),
     (lambda L: L.qm_swiglu_backward(None, 0, None, 0, 16, 30, None, None, 0, None, None), b"multiple of 4"),
     (lambda L: L.qm_swiglu_backward(None, 0, None, 0, 16, 32, None, None, 0, None, None), b"non-null"),
 ])

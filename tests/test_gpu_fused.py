@@ -311,3 +311,41 @@ def test_producers_on_random_shapes(oracle, q):
         want = oracle.quantize(oracle.swiglu(to_oracle(h12)), 32, signs=signs.numpy(), mode=oracle.QUEST_RTN, want_mask=True)
         codes, scales, mask = unpack(q, K.swiglu_quantize(h12.to(DEV), sign_int(signs), tiled), rows, cols, tiled)
         assert np.array_equal(scales, want["scales"]) and np.array_equal(codes, want["codes"]) and np.array_equal(mask, want["mask"])
+
+
+def test_residual_gradient_added_inside_the_norm_backward(q):
+    """x + f(norm(x)) with the residual taken from the fused function's second output: the same bits as the plain
+    composition, whose two gradients of x autograd adds in a kernel of its own."""
+    print("case fused residual gradient", flush=True)
+    from quartet_amd import kernels as K
+    from quartet_amd.fused import rmsnorm_linear
+    from quartet_amd.llama import RMSNorm
+    torch.manual_seed(0)
+    T, I, O = 256, 640, 640
+    layer = production_layer(q, I, O, torch.float32)
+    norm = RMSNorm(I, eps=1e-5).to(DEV)
+    x = make_input(T, I, torch.float32, seed=4, scale=2.0).to(DEV)
+    dy = make_input(T, O, torch.float32, seed=5, scale=1e-2, outlier_frac=0).to(DEV)
+    outs = []
+    for pass_input in (False, True):
+        layer.weight.grad = None
+        norm.weight.grad = None
+        xa = x.clone().requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            if pass_input:
+                y, xr = rmsnorm_linear(norm, layer, xa, pass_input=True)
+            else:
+                y, xr = rmsnorm_linear(norm, layer, xa), xa
+            z = xr + y
+        z.backward(dy)
+        outs.append((z.detach(), xa.grad.clone(), layer.weight.grad.clone(), norm.weight.grad.clone()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    # kernel level: skip is added after the norm's own gradient, in x's dtype
+    gy = make_input(T, I, torch.bfloat16, seed=6, scale=1e-2, outlier_frac=0).to(DEV)
+    gain = norm.weight.detach()
+    factor = torch.rsqrt(x.double().pow(2).mean(-1) + 1e-5).float()
+    skip = make_input(T, I, torch.float32, seed=7, scale=1e-2, outlier_frac=0).to(DEV)
+    dx0, dg0 = K.rmsnorm_backward(gy, x, gain, factor)
+    dx1, dg1 = K.rmsnorm_backward(gy, x, gain, factor, skip=skip)
+    assert torch.equal(dx1, dx0 + skip) and torch.equal(dg0, dg1)
