@@ -176,7 +176,9 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
  * qm_rmsnorm_quantize_mxfp4: RMSNorm.forward (src/models/llama.py:64-75) in front of c_attn / w12 (llama.py:170-171):
  *   Q((x.float() * rsqrt(mean(x^2, -1) + eps)).type_as(x) * gain), x [rows, cols], gain fp32 [cols]; the product with
  *   the fp32 gain is fp32, so the quantizer runs as on an fp32 tensor.  factor [rows] fp32 receives
- *   rsqrt(mean(x^2) + eps) for the backward pass.
+ *   rsqrt(mean(x^2) + eps) for the backward pass.  add (optional; x fp32, add of add_dtype): the block's residual sum in
+ *   front of the norm (x + attn(...), x + mlp(...), llama.py:170-171) is formed here: the norm's input is x + add, which
+ *   is also written to x_sum [rows, cols] fp32 for the rest of the model.
  * qm_swiglu_quantize_mxfp4: the SwiGLU product in front of the MLP's c_proj (llama.py:113-114):
  *   Q(silu(up) * gate) with h12 [rows, 2 hidden] = (up, gate) the fused w12 output; a bf16 h12 rounds silu and the
  *   product to bf16 as torch's bf16 ops do, and the quantizer runs as on a tensor of h12's dtype.
@@ -184,7 +186,8 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
  *   tensor) -> dx [rows, cols] of x's dtype and dgain fp32 [cols] (summed over rows in a fixed order).  cols <= 8192.
  *   workspace: qm_rmsnorm_backward_workspace_bytes(rows, cols) bytes, 16-byte aligned.  skip (optional, [rows, cols] of
  *   x's dtype): the gradient that reaches x past the norm (x + f(norm(x)), llama.py:170-171); dx = skip + the norm's
- *   gradient, the sum autograd would form in a pass of its own.
+ *   gradient, the sum autograd would form in a pass of its own.  dx_bf16 (optional): dx rounded to bf16 as well, the
+ *   gradient of a bf16 `add` of qm_rmsnorm_quantize_mxfp4.
  * qm_swiglu_backward: autograd of silu(up) * gate: g [rows, hidden] -> d_h12 [rows, 2 hidden] of h12's dtype.
  *   Both backward kernels take the gradient either as it is (maskbits == NULL) or still in the rotated basis of the
  *   layer's activation quantizer (qm_linear_backward with gx_rotated): then maskbits [rows, cols/8] (the mask region of
@@ -192,16 +195,16 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
  *   qm_masked_hadamard_bwd (same operations, same bits, rounded to the gradient's dtype) is applied on the fly.
  * codes_layout QM_LAYOUT_TILED needs rows % 16 == 0 and cols (hidden) % 128 == 0; cols (hidden) % 32 == 0 always.
  */
-int qm_rmsnorm_quantize_mxfp4(const void* x, int x_dtype, const float* gain, float eps, int64_t rows, int64_t cols,
-                              const uint32_t* sign_bits, void* packed, size_t packed_bytes, float* factor,
-                              int codes_layout, void* stream);
+int qm_rmsnorm_quantize_mxfp4(const void* x, int x_dtype, const void* add, int add_dtype, void* x_sum,
+                              const float* gain, float eps, int64_t rows, int64_t cols, const uint32_t* sign_bits,
+                              void* packed, size_t packed_bytes, float* factor, int codes_layout, void* stream);
 int qm_swiglu_quantize_mxfp4(const void* h12, int dtype, int64_t rows, int64_t hidden, const uint32_t* sign_bits,
                              void* packed, size_t packed_bytes, int codes_layout, void* stream);
 size_t qm_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols);
 int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain,
                         const float* factor, int64_t rows, int64_t cols, const uint8_t* maskbits,
-                        const uint32_t* sign_bits, int scale_dtype, const void* skip, void* dx, float* dgain,
-                        void* workspace, size_t workspace_bytes, void* stream);
+                        const uint32_t* sign_bits, int scale_dtype, const void* skip, void* dx, void* dx_bf16,
+                        float* dgain, void* workspace, size_t workspace_bytes, void* stream);
 int qm_swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
                        const uint8_t* maskbits, const uint32_t* sign_bits, int scale_dtype, void* d_h12,
                        void* stream);

@@ -78,13 +78,13 @@ def lib():
     L.qm_linear_forward.restype = i32
     L.qm_linear_forward.argtypes = [vp, i32, vp, i32, i64, i64, i64, i32, vp, i32, vp, vp, sz, vp, sz, i32, vp, i32, i32, vp]
     L.qm_rmsnorm_quantize_mxfp4.restype = i32
-    L.qm_rmsnorm_quantize_mxfp4.argtypes = [vp, i32, vp, f32, i64, i64, vp, vp, sz, vp, i32, vp]
+    L.qm_rmsnorm_quantize_mxfp4.argtypes = [vp, i32, vp, i32, vp, vp, f32, i64, i64, vp, vp, sz, vp, i32, vp]
     L.qm_swiglu_quantize_mxfp4.restype = i32
     L.qm_swiglu_quantize_mxfp4.argtypes = [vp, i32, i64, i64, vp, vp, sz, i32, vp]
     L.qm_rmsnorm_backward_workspace_bytes.restype = sz
     L.qm_rmsnorm_backward_workspace_bytes.argtypes = [i64, i64]
     L.qm_rmsnorm_backward.restype = i32
-    L.qm_rmsnorm_backward.argtypes = [vp, i32, vp, i32, vp, vp, i64, i64, vp, vp, i32, vp, vp, vp, vp, sz, vp]
+    L.qm_rmsnorm_backward.argtypes = [vp, i32, vp, i32, vp, vp, i64, i64, vp, vp, i32, vp, vp, vp, vp, vp, sz, vp]
     L.qm_swiglu_backward.restype = i32
     L.qm_swiglu_backward.argtypes = [vp, i32, vp, i32, i64, i64, vp, vp, i32, vp, vp]
     L.qm_rope_split_qkv.restype = i32

@@ -42,7 +42,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 7; }
+int qm_version(void) { return 8; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -355,9 +355,9 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
     return rotate_gw();
 }
 
-int qm_rmsnorm_quantize_mxfp4(const void* x, int x_dtype, const float* gain, float eps, int64_t rows, int64_t cols,
-                              const uint32_t* sign_bits, void* packed, size_t packed_bytes, float* factor, int codes_layout,
-                              void* stream) {
+int qm_rmsnorm_quantize_mxfp4(const void* x, int x_dtype, const void* add, int add_dtype, void* x_sum, const float* gain, float eps,
+                              int64_t rows, int64_t cols, const uint32_t* sign_bits, void* packed, size_t packed_bytes,
+                              float* factor, int codes_layout, void* stream) {
     if (!valid_layout(codes_layout)) return fail(QM_ERR_INVALID, "qm_rmsnorm_quantize_mxfp4: unknown codes_layout %d", codes_layout);
     if (!valid_dtype(x_dtype)) return fail(QM_ERR_INVALID, "qm_rmsnorm_quantize_mxfp4: x_dtype %d is not QM_BF16/QM_F32", x_dtype);
     if (rows < 0 || cols <= 0 || cols % 32)
@@ -370,10 +370,12 @@ int qm_rmsnorm_quantize_mxfp4(const void* x, int x_dtype, const float* gain, flo
     const PackedLayout l = packed_layout(rows, cols);
     if (!x || !gain || !factor || !packed || packed_bytes < l.total)
         return fail(QM_ERR_INVALID, "qm_rmsnorm_quantize_mxfp4: x, gain, factor must be non-null and packed hold %zu bytes", l.total);
-    if (!aligned(x, 16) || !aligned(gain, 16) || !aligned(packed, 256) || !aligned(factor, 4))
-        return fail(QM_ERR_UNALIGNED, "qm_rmsnorm_quantize_mxfp4: x and gain need 16-byte, packed 256-byte alignment");
+    if (!aligned(x, 16) || !aligned(gain, 16) || !aligned(packed, 256) || !aligned(factor, 4) || !aligned(add, 16) || !aligned(x_sum, 16))
+        return fail(QM_ERR_UNALIGNED, "qm_rmsnorm_quantize_mxfp4: x, add, x_sum and gain need 16-byte, packed 256-byte alignment");
+    if (add && (x_dtype != QM_F32 || !valid_dtype(add_dtype) || !x_sum))
+        return fail(QM_ERR_INVALID, "qm_rmsnorm_quantize_mxfp4: a residual summand needs an fp32 x, a valid add_dtype and x_sum");
     uint8_t* p = static_cast<uint8_t*>(packed);
-    return from_hip(qm::rmsnorm_quantize_hd32(x, x_dtype, gain, eps, rows, cols, sign_bits ? sign_bits[0] : 0u, p + l.c, p + l.s,
+    return from_hip(qm::rmsnorm_quantize_hd32(x, x_dtype, add, add_dtype, x_sum, gain, eps, rows, cols, sign_bits ? sign_bits[0] : 0u, p + l.c, p + l.s,
                                               p + l.m, factor, codes_layout == QM_LAYOUT_TILED, reinterpret_cast<hipStream_t>(stream)),
                     "qm_rmsnorm_quantize_mxfp4");
 }
@@ -407,7 +409,8 @@ size_t qm_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols) {
 
 int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain, const float* factor,
                         int64_t rows, int64_t cols, const uint8_t* maskbits, const uint32_t* sign_bits, int scale_dtype,
-                        const void* skip, void* dx, float* dgain, void* workspace, size_t workspace_bytes, void* stream) {
+                        const void* skip, void* dx, void* dx_bf16, float* dgain, void* workspace, size_t workspace_bytes,
+                        void* stream) {
     if (!valid_dtype(gy_dtype) || !valid_dtype(x_dtype) || (maskbits && !valid_dtype(scale_dtype)))
         return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: dtypes must be QM_BF16/QM_F32");
     if (rows < 0 || cols <= 0 || cols % 32 || cols > 8192)
@@ -416,11 +419,11 @@ int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype
     if (!dgain) return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: dgain must be non-null");
     if (rows > 0 && (!gy || !x || !gain || !factor || !dx || !workspace || workspace_bytes < qm::rmsnorm_backward_workspace_bytes(rows, cols)))
         return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: null tensor, or workspace below %zu bytes", qm_rmsnorm_backward_workspace_bytes(rows, cols));
-    if (!aligned(skip, 16) || !aligned(gy, 8) || !aligned(x, 8) || !aligned(dx, 8) || !aligned(gain, 16) || !aligned(workspace, 16) ||
+    if (!aligned(skip, 16) || !aligned(dx_bf16, 8) || !aligned(gy, 8) || !aligned(x, 8) || !aligned(dx, 8) || !aligned(gain, 16) || !aligned(workspace, 16) ||
         (gy_dtype == QM_F32 && !aligned(gy, 16)) || (x_dtype == QM_F32 && (!aligned(x, 16) || !aligned(dx, 16))))
         return fail(QM_ERR_UNALIGNED, "qm_rmsnorm_backward: tensors need 16-byte alignment");
     return from_hip(qm::rmsnorm_backward(gy, gy_dtype, x, x_dtype, gain, factor, rows, cols, maskbits, sign_bits ? sign_bits[0] : 0u,
-                                         maskbits ? scale_dtype : QM_F32, skip, dx, dgain, workspace,
+                                         maskbits ? scale_dtype : QM_F32, skip, dx, dx_bf16, dgain, workspace,
                                          reinterpret_cast<hipStream_t>(stream)),
                     "qm_rmsnorm_backward");
 }

@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const TG* __restrict__
                                                           const float* __restrict__ gain, const float* __restrict__ factor,
                                                           int64_t rows, int cols, int rpb, InverseRotation rot,
                                                           const TX* __restrict__ skip, TX* __restrict__ dx,
-                                                          float* __restrict__ partial) {
+                                                          uint16_t* __restrict__ dx_bf16, float* __restrict__ partial) {
     __shared__ float wave_sums[2][RB][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t r0 = (int64_t)blockIdx.x * rpb;
@@ -174,6 +174,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const TG* __restrict__
                         d = make_float4(d.x + sk.x, d.y + sk.y, d.z + sk.z, d.w + sk.w);
                     }
                     store4(dx + (rb + j) * cols + col, d);
+                    if (dx_bf16) store4(dx_bf16 + (rb + j) * cols + col, d);  // the gradient of a bf16 summand of x
                 }
             }
         }
@@ -241,16 +242,17 @@ int64_t rmsnorm_bwd_blocks(int64_t rows) { return (rows + rows_per_block(rows) -
 
 template <typename TG, typename TX>
 void launch_rmsnorm_bwd(const void* gy, const void* x, const float* gain, const float* factor, int64_t rows, int cols,
-                        const InverseRotation& rot, const void* skip, void* dx, float* partial, hipStream_t stream) {
+                        const InverseRotation& rot, const void* skip, void* dx, void* dx_bf16, float* partial,
+                        hipStream_t stream) {
     const dim3 grid((unsigned)rmsnorm_bwd_blocks(rows)), block(256);
     const int rpb = rows_per_block(rows);
     const TG* g = reinterpret_cast<const TG*>(gy);
     const TX* xp = reinterpret_cast<const TX*>(x);
     TX* dxp = reinterpret_cast<TX*>(dx);
     const TX* sk = reinterpret_cast<const TX*>(skip);
-    if (cols <= 2048) rmsnorm_bwd_kernel<TG, TX, 2, 4><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, sk, dxp, partial);
-    else if (cols <= 4096) rmsnorm_bwd_kernel<TG, TX, 4, 2><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, sk, dxp, partial);
-    else rmsnorm_bwd_kernel<TG, TX, 8, 1><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, sk, dxp, partial);
+    if (cols <= 2048) rmsnorm_bwd_kernel<TG, TX, 2, 4><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, sk, dxp, reinterpret_cast<uint16_t*>(dx_bf16), partial);
+    else if (cols <= 4096) rmsnorm_bwd_kernel<TG, TX, 4, 2><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, sk, dxp, reinterpret_cast<uint16_t*>(dx_bf16), partial);
+    else rmsnorm_bwd_kernel<TG, TX, 8, 1><<<grid, block, 0, stream>>>(g, xp, gain, factor, rows, cols, rpb, rot, sk, dxp, reinterpret_cast<uint16_t*>(dx_bf16), partial);
 }
 
 }  // namespace
@@ -262,17 +264,19 @@ size_t rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols) {
 // cols <= 8192, cols % 32 == 0; workspace: rmsnorm_backward_workspace_bytes(rows, cols) bytes, 16-byte aligned.
 // maskbits != null: gy is the gradient w.r.t. the quantizer's rotated output and is rotated back on the fly.
 // skip != null: [rows, cols] of x's dtype, added to dx (the gradient of a residual connection around the norm).
+// dx_bf16 != null: a second copy of dx rounded to bf16 (the gradient of a bf16 tensor that was added into x).
 hipError_t rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain,
                             const float* factor, int64_t rows, int64_t cols, const uint8_t* maskbits, uint32_t sign_word,
-                            int scale_dtype, const void* skip, void* dx, float* dgain, void* workspace, hipStream_t stream) {
+                            int scale_dtype, const void* skip, void* dx, void* dx_bf16, float* dgain, void* workspace,
+                            hipStream_t stream) {
     if (cols == 0) return hipSuccess;
     float* partial = reinterpret_cast<float*>(workspace);
     const InverseRotation rot{maskbits, sign_word, hadamard_scale(32, scale_dtype)};
     if (rows == 0) {}  // no rows: the column sums below write zeros
-    else if (gy_dtype == BF16 && x_dtype == BF16) launch_rmsnorm_bwd<uint16_t, uint16_t>(gy, x, gain, factor, rows, (int)cols, rot, skip, dx, partial, stream);
-    else if (gy_dtype == BF16) launch_rmsnorm_bwd<uint16_t, float>(gy, x, gain, factor, rows, (int)cols, rot, skip, dx, partial, stream);
-    else if (x_dtype == BF16) launch_rmsnorm_bwd<float, uint16_t>(gy, x, gain, factor, rows, (int)cols, rot, skip, dx, partial, stream);
-    else launch_rmsnorm_bwd<float, float>(gy, x, gain, factor, rows, (int)cols, rot, skip, dx, partial, stream);
+    else if (gy_dtype == BF16 && x_dtype == BF16) launch_rmsnorm_bwd<uint16_t, uint16_t>(gy, x, gain, factor, rows, (int)cols, rot, skip, dx, dx_bf16, partial, stream);
+    else if (gy_dtype == BF16) launch_rmsnorm_bwd<uint16_t, float>(gy, x, gain, factor, rows, (int)cols, rot, skip, dx, dx_bf16, partial, stream);
+    else if (x_dtype == BF16) launch_rmsnorm_bwd<float, uint16_t>(gy, x, gain, factor, rows, (int)cols, rot, skip, dx, dx_bf16, partial, stream);
+    else launch_rmsnorm_bwd<float, float>(gy, x, gain, factor, rows, (int)cols, rot, skip, dx, dx_bf16, partial, stream);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
     column_sum_kernel<<<dim3((unsigned)((cols + 63) / 64)), dim3(1024), 0, stream>>>(partial, (int)rmsnorm_bwd_blocks(rows),

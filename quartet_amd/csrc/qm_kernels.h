@@ -75,15 +75,16 @@ hipError_t masked_hadamard_bwd_hd32_pair(const void* ga, int64_t na, int scale_d
                                          int dtype, int out_dtype_b, hipStream_t stream);
 
 // Producers fused into the forward quantizer (Hadamard block 32, quest RTN, clip mask) and their backward passes
-hipError_t rmsnorm_quantize_hd32(const void* x, int dtype, const float* gain, float eps, int64_t rows, int64_t cols,
-                                 uint32_t sign_word, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, float* factor,
-                                 bool tiled, hipStream_t stream);
+hipError_t rmsnorm_quantize_hd32(const void* x, int dtype, const void* add, int add_dtype, void* xsum, const float* gain, float eps,
+                                 int64_t rows, int64_t cols, uint32_t sign_word, uint8_t* codes, uint8_t* scales, uint8_t* maskbits,
+                                 float* factor, bool tiled, hipStream_t stream);
 hipError_t swiglu_quantize_hd32(const void* h12, int dtype, int64_t rows, int64_t hidden, uint32_t sign_word,
                                 uint8_t* codes, uint8_t* scales, uint8_t* maskbits, bool tiled, hipStream_t stream);
 size_t rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols);
 hipError_t rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype, const float* gain,
                             const float* factor, int64_t rows, int64_t cols, const uint8_t* maskbits, uint32_t sign_word,
-                            int scale_dtype, const void* skip, void* dx, float* dgain, void* workspace, hipStream_t stream);
+                            int scale_dtype, const void* skip, void* dx, void* dx_bf16, float* dgain, void* workspace,
+                            hipStream_t stream);
 hipError_t swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
                            const uint8_t* maskbits, uint32_t sign_word, int scale_dtype, void* d_h12, hipStream_t stream);
 

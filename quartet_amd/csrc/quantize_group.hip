@@ -728,13 +728,19 @@ __device__ __forceinline__ void round_pair_to_bf16(float& a, float& b) {
     b = u2f(w & 0xffff0000u);
 }
 
-template <typename T>
+// TA = void: plain.  Otherwise the norm's input is x + add (the residual sum in front of the norm, src/models/llama.py:
+// 170-171), formed here in T's arithmetic and written to xsum, which the rest of the model continues with.
+template <typename T, typename TA = void>
 struct RmsNormProducer {
     static constexpr int kOutDtype = F32;  // bf16-or-fp32 normalised value times the fp32 gain is fp32
+    static constexpr bool kAdd = !std::is_void<TA>::value;
+    using TAdd = typename std::conditional<kAdd, TA, T>::type;
     const T* x;
     const float* gain;
     float* factor;  // [rows]: 1 / sqrt(mean(x^2) + eps), kept for the backward pass
     float eps;
+    const TAdd* add;
+    T* xsum;
 
     // The row's factor; `first` leaves with the raw elements of the lane's first group (if it has one).
     // Sum of squares in a fixed order: sixteen interleaved partial sums (partial j adds the sums of groups j, j+16,
@@ -748,6 +754,16 @@ struct RmsNormProducer {
             if (g < groups) {
                 float v[32];
                 load_group<T>(x + row * cols + g * 32, v);
+                if constexpr (kAdd) {
+                    static_assert(!kAdd || sizeof(T) == 4, "the residual sum is formed in fp32");
+                    float a[32];
+                    load_group<TAdd>(add + row * cols + g * 32, a);
+#pragma unroll
+                    for (int i = 0; i < 32; ++i) v[i] = v[i] + a[i];
+                    float4* dst = reinterpret_cast<float4*>(xsum + row * cols + g * 32);
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) dst[q] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+                }
                 if (base == 0) {
 #pragma unroll
                     for (int i = 0; i < 32; ++i) first[i] = v[i];
@@ -767,7 +783,8 @@ struct RmsNormProducer {
     }
     // v holds the group's raw elements on entry when have_raw
     __device__ __forceinline__ void load(int64_t row, int g, int64_t cols, float f, bool have_raw, float (&v)[32]) const {
-        if (!have_raw) load_group<T>(x + row * cols + g * 32, v);
+        // with a residual sum: the lane reads back what it stored in prepare()
+        if (!have_raw) load_group<T>((kAdd ? xsum : x) + row * cols + g * 32, v);
 #pragma unroll
         for (int i = 0; i < 32; ++i) v[i] = v[i] * f;
         if constexpr (sizeof(T) == 2) {  // .type_as(x)
@@ -860,17 +877,29 @@ void launch_produced(const P& prod, int64_t rows, int64_t cols, uint32_t sign_wo
 
 }  // namespace
 
-// Q(rmsnorm(x) * gain): Hadamard block 32, quest RTN, clip mask; factor [rows] receives 1 / sqrt(mean(x^2) + eps)
-hipError_t rmsnorm_quantize_hd32(const void* x, int dtype, const float* gain, float eps, int64_t rows, int64_t cols,
-                                 uint32_t sign_word, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, float* factor,
-                                 bool tiled, hipStream_t stream) {
+// Q(rmsnorm(x) * gain): Hadamard block 32, quest RTN, clip mask; factor [rows] receives 1 / sqrt(mean(x^2) + eps).
+// add != null (x fp32 only): the norm's input is x + add, also written to xsum [rows, cols] fp32.
+hipError_t rmsnorm_quantize_hd32(const void* x, int dtype, const void* add, int add_dtype, void* xsum, const float* gain, float eps,
+                                 int64_t rows, int64_t cols, uint32_t sign_word, uint8_t* codes, uint8_t* scales, uint8_t* maskbits,
+                                 float* factor, bool tiled, hipStream_t stream) {
     if (rows == 0) return hipSuccess;
-    if (dtype == BF16)
-        launch_produced(RmsNormProducer<uint16_t>{reinterpret_cast<const uint16_t*>(x), gain, factor, eps}, rows, cols,
+    if (add) {
+        if (dtype != F32) return hipErrorInvalidValue;
+        const float* xp = reinterpret_cast<const float*>(x);
+        float* sp = reinterpret_cast<float*>(xsum);
+        if (add_dtype == BF16)
+            launch_produced(RmsNormProducer<float, uint16_t>{xp, gain, factor, eps, reinterpret_cast<const uint16_t*>(add), sp}, rows,
+                            cols, sign_word, codes, scales, maskbits, tiled, stream);
+        else
+            launch_produced(RmsNormProducer<float, float>{xp, gain, factor, eps, reinterpret_cast<const float*>(add), sp}, rows, cols,
+                            sign_word, codes, scales, maskbits, tiled, stream);
+    } else if (dtype == BF16) {
+        launch_produced(RmsNormProducer<uint16_t>{reinterpret_cast<const uint16_t*>(x), gain, factor, eps, nullptr, nullptr}, rows,
+                        cols, sign_word, codes, scales, maskbits, tiled, stream);
+    } else {
+        launch_produced(RmsNormProducer<float>{reinterpret_cast<const float*>(x), gain, factor, eps, nullptr, nullptr}, rows, cols,
                         sign_word, codes, scales, maskbits, tiled, stream);
-    else
-        launch_produced(RmsNormProducer<float>{reinterpret_cast<const float*>(x), gain, factor, eps}, rows, cols, sign_word,
-                        codes, scales, maskbits, tiled, stream);
+    }
     return hipGetLastError();
 }
 

@@ -28,22 +28,29 @@ class RMSNormLinearFn(torch.autograd.Function):
 
     With `pass_input` the function also returns x itself: a block computes ``x + f(norm(x))``, and when the residual sum
     takes this second output instead of x, both gradients of x (through the norm and past it) arrive here together and
-    the RMSNorm backward kernel adds them, instead of autograd in a pass of its own."""
+    the RMSNorm backward kernel adds them, instead of autograd in a pass of its own.  With `add` (x fp32) the norm's
+    input is ``x + add``, formed inside the quantizer kernel; the sum is the second output."""
 
     @staticmethod
-    def forward(ctx, x, gain, weight, eps, a_q, w_q, g_q, weight_cache, pass_input=False):
+    def forward(ctx, x, add, gain, weight, eps, a_q, w_q, g_q, weight_cache, pass_input=False):
         I = weight.shape[1]
         x2 = x.reshape(-1, I).contiguous()
         T, O = x2.shape[0], weight.shape[0]
         tiled = _use_tiled_codes(T, I, O, a_q, w_q, g_q)
-        packed_x, factor = K.rmsnorm_quantize(x2, gain, eps, a_q.sign_bits, tiled)
+        if add is None:
+            packed_x, factor = K.rmsnorm_quantize(x2, gain, eps, a_q.sign_bits, tiled)
+        else:
+            packed_x, factor, x2 = K.rmsnorm_quantize(x2, gain, eps, a_q.sign_bits, tiled, add.reshape(-1, I).contiguous())
         # the normalised tensor times the fp32 gain is an fp32 tensor: that is the dtype the layer sees
         out_dtype = torch.bfloat16 if _autocast_bf16() else torch.float32
         y, packed_x, packed_w = _forward_packed(ctx, None, weight, a_q, w_q, g_q, weight_cache, tiled, out_dtype, torch.float32,
                                                 packed_x, T)
         ctx.save_for_backward(x2, gain, factor, packed_x, packed_w)
         ctx.x_shape = x.shape
+        ctx.add_dtype = None if add is None else add.dtype
         y = y.view(*x.shape[:-1], O)
+        if add is not None:
+            return y, x2.view(x.shape)
         return (y, x) if pass_input else y
 
     @staticmethod
@@ -53,8 +60,11 @@ class RMSNormLinearFn(torch.autograd.Function):
         gy, gw, (maskbits, signs, scale_dtype) = _backward_packed(ctx, e, packed_x, packed_w, gx_rotated=True)
         if skip is not None:
             skip = skip.reshape(x2.shape).to(x2.dtype).contiguous()
-        dx, dgain = K.rmsnorm_backward(gy, x2, gain, factor, maskbits, signs, scale_dtype, skip)
-        return dx.view(ctx.x_shape), dgain, gw.to(ctx.w_dtype), None, None, None, None, None, None
+        want_copy = ctx.add_dtype == torch.bfloat16
+        out = K.rmsnorm_backward(gy, x2, gain, factor, maskbits, signs, scale_dtype, skip, want_copy)
+        dx = out[0].view(ctx.x_shape)
+        d_add = None if ctx.add_dtype is None else (out[2].view(ctx.x_shape) if want_copy else dx)
+        return dx, d_add, out[1], gw.to(ctx.w_dtype), None, None, None, None, None, None
 
 
 class SwiGLULinearFn(torch.autograd.Function):
@@ -122,16 +132,23 @@ def rope_qkv(qkv, table, n_head):
     return q, k, v.view(B, T, n_head, hs)
 
 
-def rmsnorm_linear(norm, layer, x, pass_input=False):
+def rmsnorm_linear(norm, layer, x, pass_input=False, add=None):
     """layer(norm(x)) for an RMSNorm module `norm` (attributes ``weight`` and ``eps``) and a QuantizedLinear.  With
     `pass_input` returns (layer(norm(x)), x): use the second value for the residual sum around the norm, so that the sum
-    of x's two gradients happens inside the RMSNorm backward kernel."""
-    if (_layer_is_fusable(layer) and x.is_cuda and x.dtype in _KERNEL_DTYPES and norm.weight.dtype == torch.float32
-            and x.shape[-1] <= 8192):
-        return RMSNormLinearFn.apply(x, norm.weight, layer.weight, norm.eps, layer.activation_quantizer, layer.weight_quantizer,
+    of x's two gradients happens inside the RMSNorm backward kernel.  With `add` returns (layer(norm(x + add)), x + add):
+    the residual sum in front of the norm is formed inside the quantizer kernel."""
+    fusable = (_layer_is_fusable(layer) and x.is_cuda and x.dtype in _KERNEL_DTYPES and norm.weight.dtype == torch.float32
+               and x.shape[-1] <= 8192)
+    if fusable and add is not None and not (x.dtype == torch.float32 and add.dtype in _KERNEL_DTYPES and add.shape == x.shape):
+        x, add = x + add, None
+        pass_input = True
+    if fusable:
+        return RMSNormLinearFn.apply(x, add, norm.weight, layer.weight, norm.eps, layer.activation_quantizer, layer.weight_quantizer,
                                      layer.backward_scheme.g_quantizer, layer.packed_weight_cache, pass_input)
+    if add is not None:
+        x = x + add
     y = layer(norm(x))
-    return (y, x) if pass_input else y
+    return (y, x) if (pass_input or add is not None) else y
 
 
 def swiglu_linear(layer, h12):

@@ -182,17 +182,23 @@ def linear_forward(x2, w2, hd_x, signs_x, hd_w, signs_w, out_dtype, tiled, packe
     return y, packed_x, packed_w
 
 
-def rmsnorm_quantize(x2, gain, eps, signs, tiled):
-    """Q(rmsnorm(x2) * gain) without writing the normalised tensor: (packed operand buffer, per-row factor fp32)."""
-    _require_cuda(x2, gain)
+def rmsnorm_quantize(x2, gain, eps, signs, tiled, add=None):
+    """Q(rmsnorm(x2) * gain) without writing the normalised tensor: (packed operand buffer, per-row factor fp32).  With
+    `add` (x2 fp32, add like x2 in bf16 or fp32) the norm's input is x2 + add, returned as a third value."""
+    _require_cuda(x2, gain, add)
     assert x2.is_contiguous() and gain.is_contiguous() and gain.dtype == torch.float32 and gain.shape == (x2.shape[1],)
     rows, cols = x2.shape
     packed = packed_operand_buffer(rows, cols, x2.device)
     factor = torch.empty(rows, dtype=torch.float32, device=x2.device)
-    rc = _lib.lib().qm_rmsnorm_quantize_mxfp4(_ptr(x2), _dtype_code(x2.dtype), _ptr(gain), float(eps), rows, cols, sign_words(signs),
-                                              _ptr(packed), packed.numel(), _ptr(factor), _layout(tiled), _stream())
+    x_sum = None
+    if add is not None:
+        assert add.is_contiguous() and add.shape == x2.shape and x2.dtype == torch.float32
+        x_sum = torch.empty_like(x2)
+    rc = _lib.lib().qm_rmsnorm_quantize_mxfp4(_ptr(x2), _dtype_code(x2.dtype), _ptr(add), _dtype_code(add.dtype) if add is not None else 0,
+                                              _ptr(x_sum), _ptr(gain), float(eps), rows, cols, sign_words(signs), _ptr(packed),
+                                              packed.numel(), _ptr(factor), _layout(tiled), _stream())
     _lib.check(rc, "qm_rmsnorm_quantize_mxfp4")
-    return packed, factor
+    return (packed, factor) if add is None else (packed, factor, x_sum)
 
 
 def swiglu_quantize(h12, signs, tiled):
@@ -214,11 +220,11 @@ def packed_mask_bits(packed, rows, cols):
     return packed[off[2]: off[2] + rows * cols // 8].view(rows, cols // 8)
 
 
-def rmsnorm_backward(gy, x2, gain, factor, maskbits=None, signs=0, scale_dtype=torch.float32, skip=None):
+def rmsnorm_backward(gy, x2, gain, factor, maskbits=None, signs=0, scale_dtype=torch.float32, skip=None, want_bf16_copy=False):
     """gy [rows, cols] (gradient of the normalised, scaled tensor) -> (dx like x2, dgain fp32 [cols]).  With `maskbits`
     (and the rotation's `signs`, `scale_dtype`), gy is the gradient in the activation quantizer's rotated basis and its
     straight-through backward is applied first, inside the kernel.  `skip` (like x2) is added to dx: the gradient of a
-    residual connection around the norm."""
+    residual connection around the norm.  `want_bf16_copy`: returns dx rounded to bf16 as a third value."""
     _require_cuda(gy, x2, gain, factor, maskbits, skip)
     assert skip is None or (skip.is_contiguous() and skip.shape == x2.shape and skip.dtype == x2.dtype)
     assert gy.is_contiguous() and x2.is_contiguous() and gy.shape == x2.shape
@@ -228,11 +234,12 @@ def rmsnorm_backward(gy, x2, gain, factor, maskbits=None, signs=0, scale_dtype=t
     work = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=x2.device)
     dx = torch.empty_like(x2)
     dgain = torch.empty(cols, dtype=torch.float32, device=x2.device)
+    dx_bf16 = torch.empty(x2.shape, dtype=torch.bfloat16, device=x2.device) if want_bf16_copy else None
     rc = L.qm_rmsnorm_backward(_ptr(gy), _dtype_code(gy.dtype), _ptr(x2), _dtype_code(x2.dtype), _ptr(gain), _ptr(factor), rows, cols,
-                               _ptr(maskbits), sign_words(signs), _dtype_code(scale_dtype), _ptr(skip), _ptr(dx), _ptr(dgain),
-                               _ptr(work), nbytes, _stream())
+                               _ptr(maskbits), sign_words(signs), _dtype_code(scale_dtype), _ptr(skip), _ptr(dx), _ptr(dx_bf16),
+                               _ptr(dgain), _ptr(work), nbytes, _stream())
     _lib.check(rc, "qm_rmsnorm_backward")
-    return dx, dgain
+    return (dx, dgain, dx_bf16) if want_bf16_copy else (dx, dgain)
 
 
 def swiglu_backward(g, h12, maskbits=None, signs=0, scale_dtype=torch.float32):

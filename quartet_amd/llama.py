@@ -121,10 +121,11 @@ class LlamaMLP(nn.Module):
         self.w12 = _linear(config, config.n_embd, 2 * self.hidden_dim)
         self.c_proj = _linear(config, self.hidden_dim, config.n_embd)
 
-    def forward(self, x, norm=None):
-        """`norm`: the block's RMSNorm, applied to x here (fused into w12's quantizer) instead of by the caller."""
-        if norm is not None:   # returns (mlp output, x for the residual sum)
-            h12, x = rmsnorm_linear(norm, self.w12, x, pass_input=True)
+    def forward(self, x, norm=None, add=None):
+        """`norm`: the block's RMSNorm, applied to x (+ `add`, the attention branch's output) here, fused into w12's
+        quantizer, instead of by the caller."""
+        if norm is not None:   # returns (mlp output, x + add for the residual sum)
+            h12, x = rmsnorm_linear(norm, self.w12, x, pass_input=True, add=add)
             return swiglu_linear(self.c_proj, h12), x
         up, gate = self.w12(x).split(self.hidden_dim, dim=-1)
         return self.c_proj(F.silu(up) * gate)
@@ -139,13 +140,13 @@ class LlamaAttention(nn.Module):
         self.resid_dropout = nn.Dropout(config.dropout)
         self.n_head, self.n_embd, self.dropout = config.n_head, config.n_embd, config.dropout
 
-    def forward(self, x, table, norm=None):
+    def forward(self, x, table, norm=None, add=None):
         B, T, C = x.shape
         hs = C // self.n_head
         if norm is None:
             qkv = self.c_attn(x)
         else:
-            qkv, x = rmsnorm_linear(norm, self.c_attn, x, pass_input=True)
+            qkv, x = rmsnorm_linear(norm, self.c_attn, x, pass_input=True, add=add)
         if norm is not None:   # the fused path: split, rotate and convert in one kernel
             q, k, v = rope_qkv(qkv, table, self.n_head)
         else:
@@ -170,12 +171,12 @@ class LlamaBlock(nn.Module):
         self.mlp = LlamaMLP(config)
         self.fuse_producers = config.fuse_producers
 
-    def forward(self, x, table):
+    def forward(self, x, table, pending=None):
+        """Fused form: returns (x, m) with the block's output x + m left to whoever consumes it -- the next block's first
+        norm forms it inside its quantizer kernel (`pending`), as this block's second norm does with x + attention."""
         if self.fuse_producers:
-            a, x = self.attn(x, table, norm=self.ln_1)
-            x = x + a
-            m, x = self.mlp(x, norm=self.ln_2)
-            return x + m
+            a, x = self.attn(x, table, norm=self.ln_1, add=pending)
+            return self.mlp(x, norm=self.ln_2, add=a)[::-1]
         x = x + self.attn(self.ln_1(x), table)
         return x + self.mlp(self.ln_2(x))
 
@@ -221,8 +222,15 @@ class Llama(nn.Module):
         assert t <= self.config.sequence_length, f"sequence of length {t} exceeds block size {self.config.sequence_length}"
         x = self.transformer.drop(self.transformer.wte(idx))
         table = self.freqs_cis[:t]
+        pending = None   # a block's MLP output, not yet added to the residual stream (fused blocks only)
         for block in self.transformer.h:
-            x = block(x, table)
+            if block.fuse_producers:
+                x, pending = block(x, table, pending)
+            else:
+                x = block(x if pending is None else x + pending, table)
+                pending = None
+        if pending is not None:
+            x = x + pending
         x = self.transformer.ln_f(x)
         if targets is not None:
             logits = self.lm_head(x)

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_function():
 
 def test_host_only_entry_points():
     L = _lib.lib()
-    assert L.qm_version() == 7
+    assert L.qm_version() == 8
     T, I, O = 256, 128, 384
     off = (ctypes.c_size_t * 3)()
     for rows, cols in ((T, I), (O, I)):
@@ -63,14 +63,14 @@ def test_host_only_entry_points():
     (lambda L: L.qm_dequantize_mxfp4(None, None, 4, 40, 1.0, None, 0, None), b"C % 32"),
     (lambda L: L.qm_linear_forward(None, 0, None, 0, 64, 40, 64, 32, None, 32, None, None, 0, None, 0, 0, None, 0, 0, None), b"multiple of 32"),
     (lambda L: L.qm_linear_forward(None, 0, None, 0, 64, 64, 64, 32, None, 32, None, None, 0, None, 0, 0, None, 0, 0, None), b"packed operand buffers"),
-    (lambda L: L.qm_rmsnorm_quantize_mxfp4(None, 0, None, 1e-5, 16, 40, None, None, 0, None, 0, None), b"multiple of 32"),
-    (lambda L: L.qm_rmsnorm_quantize_mxfp4(None, 0, None, 1e-5, 20, 128, None, None, 0, None, 1, None), b"tiled codes"),
-    (lambda L: L.qm_rmsnorm_quantize_mxfp4(None, 0, None, 1e-5, 16, 128, None, None, 0, None, 0, None), b"non-null"),
+    (lambda L: L.qm_rmsnorm_quantize_mxfp4(None, 0, None, 0, None, None, 1e-5, 16, 40, None, None, 0, None, 0, None), b"multiple of 32"),
+    (lambda L: L.qm_rmsnorm_quantize_mxfp4(None, 0, None, 0, None, None, 1e-5, 20, 128, None, None, 0, None, 1, None), b"tiled codes"),
+    (lambda L: L.qm_rmsnorm_quantize_mxfp4(None, 0, None, 0, None, None, 1e-5, 16, 128, None, None, 0, None, 0, None), b"non-null"),
     (lambda L: L.qm_swiglu_quantize_mxfp4(None, 7, 16, 128, None, None, 0, 0, None), b"dtype"),
     (lambda L: L.qm_swiglu_quantize_mxfp4(None, 0, 16, 100, None, None, 0, 0, None), b"multiple of 32"),
     (lambda L: L.qm_swiglu_quantize_mxfp4(None, 0, 16, 128, None, None, 0, 0, None), b"non-null"),
-    (lambda L: L.qm_rmsnorm_backward(None, 0, None, 0, None, None, 16, 16384, None, None, 0, None, None, None, None, 0, None), b"[32, 8192]"),
-    (lambda L: L.qm_rmsnorm_backward(None, 0, None, 0, None, None, 16, 128, None, None, 0, None, None, None, None, 0, None), b"dgain"),
+    (lambda L: L.qm_rmsnorm_backward(None, 0, None, 0, None, None, 16, 16384, None, None, 0, None, None, None, None, None, 0, None), b"[32, 8192]"),
+    (lambda L: L.qm_rmsnorm_backward(None, 0, None, 0, None, None, 16, 128, None, None, 0, None, None, None, None, None, 0, None), b"dgain"),
     (lambda L: L.qm_swiglu_backward(None, 0, None, 0, 16, 30, None, None, 0, None, None), b"multiple of 4"),
     (lambda L: L.qm_swiglu_backward(None, 0, None, 0, 16, 32, None, None, 0, None, None), b"non-null"),
 ])
@@ -86,7 +86,7 @@ def test_empty_shapes_are_accepted_without_touching_pointers():
     assert L.qm_quantize_mxfp4(None, 0, 0, 64, 32, None, 0, 0, None, 0, None, None, None, None, 0, None) == 0
     assert L.qm_gemm_mxfp4_tn(None, None, None, None, 0, 64, 64, 1.0, None, 0, 0, 0, None, 0, None) == 0
     assert L.qm_linear_forward(None, 0, None, 0, 0, 64, 64, 32, None, 32, None, None, 0, None, 0, 0, None, 0, 0, None) == 0
-    assert L.qm_rmsnorm_quantize_mxfp4(None, 0, None, 1e-5, 0, 64, None, None, 0, None, 0, None) == 0
+    assert L.qm_rmsnorm_quantize_mxfp4(None, 0, None, 0, None, None, 1e-5, 0, 64, None, None, 0, None, 0, None) == 0
     assert L.qm_swiglu_quantize_mxfp4(None, 0, 0, 64, None, None, 0, 0, None) == 0
     assert L.qm_swiglu_backward(None, 0, None, 0, 0, 64, None, None, 0, None, None) == 0
 

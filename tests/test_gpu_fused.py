@@ -349,3 +349,63 @@ def test_residual_gradient_added_inside_the_norm_backward(q):
     dx0, dg0 = K.rmsnorm_backward(gy, x, gain, factor)
     dx1, dg1 = K.rmsnorm_backward(gy, x, gain, factor, skip=skip)
     assert torch.equal(dx1, dx0 + skip) and torch.equal(dg0, dg1)
+
+
+@pytest.mark.parametrize("add_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,cols,tiled", [(256, 640, True), (50, 96, False), (32, 4096, True)])
+def test_residual_sum_inside_the_norm_quantizer(q, rows, cols, tiled, add_dtype):
+    """x + add formed inside the fused kernel: the sum it writes and the packed operand are those of the plain kernel on
+    torch's x + add; the bf16 copy of the backward's dx is dx rounded."""
+    print(f"case fused residual sum rows={rows} cols={cols} tiled={tiled} add={add_dtype}", flush=True)
+    from quartet_amd import kernels as K
+    x = make_input(rows, cols, torch.float32, seed=rows, scale=2.0).to(DEV)
+    a = make_input(rows, cols, add_dtype, seed=rows + 1, scale=0.5).to(DEV)
+    gain = (1.0 + 0.2 * torch.randn(cols, generator=torch.Generator().manual_seed(2))).float().to(DEV)
+    want_sum = x + a
+    assert want_sum.dtype == torch.float32
+    p0, f0 = K.rmsnorm_quantize(want_sum, gain, 1e-5, 0x1234ABCD, tiled)
+    p1, f1, got_sum = K.rmsnorm_quantize(x, gain, 1e-5, 0x1234ABCD, tiled, add=a)
+    assert torch.equal(got_sum, want_sum) and torch.equal(f0, f1)
+    for u, v in zip(unpack(q, p0, rows, cols, tiled), unpack(q, p1, rows, cols, tiled)):   # (the buffers' padding is not set)
+        assert np.array_equal(u, v)
+    gy = make_input(rows, cols, torch.bfloat16, seed=9, scale=1e-2, outlier_frac=0).to(DEV)
+    dx, dg = K.rmsnorm_backward(gy, want_sum, gain, f0)
+    dx2, dg2, low = K.rmsnorm_backward(gy, want_sum, gain, f0, want_bf16_copy=True)
+    assert torch.equal(dx, dx2) and torch.equal(dg, dg2) and torch.equal(low, dx.to(torch.bfloat16))
+
+
+def test_block_with_deferred_residual_sums_matches_the_plain_block(q):
+    """Two fused blocks chained through `pending` against the same blocks with every residual sum done by torch."""
+    print("case fused blocks with pending sums", flush=True)
+    from quartet_amd import llama as L
+    from quartet_amd.fused import rmsnorm_linear
+    torch.manual_seed(0)
+    det = dict(g_quant_kwargs={"hadamard_dim": 32, "stochastic": False, "rerotate": None})
+    cfg = L.LlamaConfig(vocab_size=128, sequence_length=64, n_layer=2, n_head=2, n_embd=256, multiple_of=128, **det)
+    model = L.Llama(cfg).to(DEV)
+    idx = torch.randint(0, 128, (4, 64), device=DEV)
+    tgt = torch.randint(0, 128, (4, 64), device=DEV)
+
+    def run(plain_sums):
+        model.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            if not plain_sums:
+                loss = model(idx, targets=tgt)["loss"]
+            else:   # the fused kernels for norm, SwiGLU and rotary, but x + branch as separate torch adds
+                x = model.transformer.wte(idx)
+                table = model.freqs_cis[:64]
+                for blk in model.transformer.h:
+                    a, _ = blk.attn(x, table, norm=blk.ln_1)
+                    x = x + a
+                    m, _ = blk.mlp(x, norm=blk.ln_2)
+                    x = x + m
+                logits = model.lm_head(model.transformer.ln_f(x))
+                loss = F.cross_entropy(logits.view(-1, logits.size(-1)), tgt.view(-1), ignore_index=-1)
+            loss.backward()
+        return loss.detach().clone(), {n: p.grad.clone() for n, p in model.named_parameters()}
+
+    l0, g0 = run(False)
+    l1, g1 = run(True)
+    assert torch.equal(l0, l1)
+    for n in g0:
+        assert torch.equal(g0[n], g1[n]), n
