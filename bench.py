@@ -50,12 +50,30 @@ def build_layer(device):
     return layer
 
 
-def time_kernel(fn, reps=20, warmup=3):
-    """Average duration (ms) of one launch sequence `fn`, HIP events on the stream the kernels run on."""
+def time_kernel(fn, reps=20, warmup=3, graph=True):
+    """Average duration (ms) of one launch sequence `fn`, HIP events on the stream the kernels run on.
+
+    With `graph` the `reps` launches are recorded into one HIP graph and the replay is timed: the kernels then follow
+    each other as closely as the hardware dispatches them, so a 10-20 us kernel is not measured through the host's
+    launch rate (Python + allocator + ctypes cost about as much per call as such a kernel runs)."""
     for _ in range(warmup):
         fn()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
+    if graph:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(reps):
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        start.record()
+        g.replay()
+        stop.record()
+        stop.synchronize()
+        ms = start.elapsed_time(stop) / reps
+        del g
+        return ms
     start.record()
     for _ in range(reps):
         fn()
@@ -225,7 +243,7 @@ def library_gemm(device, reps=50):
         sa = torch.full((M, K // 32), 127, dtype=torch.uint8, device=device).view(torch.float8_e8m0fnu)
         sb = torch.full((N, K // 32), 127, dtype=torch.uint8, device=device).view(torch.float8_e8m0fnu)
         run = lambda: torch._scaled_mm(a, b.t(), sa, sb, out_dtype=torch.bfloat16)
-        ms = time_kernel(run, reps=reps, warmup=5)
+        ms = time_kernel(run, reps=reps, warmup=5, graph=False)
     except Exception as exc:  # the installed torch / hipBLASLt may not offer this product
         return {"error": f"{type(exc).__name__}: {str(exc)[:200]}"}
     return {"what": f"torch._scaled_mm float4_e2m1fn_x2 x float4_e2m1fn_x2, e8m0 scales per 32, {M}x{N}x{K}, bf16 out",
