@@ -250,6 +250,30 @@ def library_gemm(device, reps=50):
             "ms": round(ms, 4), "TFLOPs": round(2.0 * M * N * K / ms / 1e9, 1)}
 
 
+def gemm_operand_content(x, w, dy, rounds=3):
+    """The forward product's shape timed on operands of different content.  The kernel is power-limited: the clock the
+    chip holds, and with it the duration, follows how much the operand bits toggle, so constant operands show what the
+    kernel's structure alone costs."""
+    from quartet_amd import kernels as K
+    signs = 0x5A5AA5A5
+    xc, xs, _, _ = K.quantize_mxfp4(x, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=True)
+    wc, ws, _, _ = K.quantize_mxfp4(w, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=True)
+    ec, es, _, _ = K.quantize_mxfp4(dy, 32, signs, K.QM_ABSMAX_SR, seed=1, tiled=True)
+    wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=3, tiled_in=True,
+                                                tiled_out=True)
+    rand = lambda t: torch.randint(0, 256, t.shape, dtype=torch.uint8, device=t.device)
+    cases = [("quest_rtn_codes_of_gaussians", xc, xs, wc, ws), ("absmax_sr_codes_of_gaussians", ec, es, wtc, wts),
+             ("uniform_random_codes", rand(xc), xs, rand(wc), ws), ("all_zero_codes", torch.zeros_like(xc), xs, torch.zeros_like(wc), ws),
+             ("constant_codes_1.0", torch.full_like(xc, 0x22), xs, torch.full_like(wc, 0x22), ws)]
+    out = {}
+    for _ in range(rounds):  # interleaved rounds: the box's clock drifts over seconds
+        for name, a, sa, b, sb in cases:
+            ms = time_kernel(lambda: K.gemm_mxfp4_tn(a, sa, b, sb, 1.0, torch.bfloat16, a_tiled=True, b_tiled=True), reps=30)
+            out.setdefault(name, []).append(ms)
+    flops = 2.0 * T_TOKENS * IN_F * OUT_F
+    return {k: {"ms": round(sorted(v)[len(v) // 2], 4), "TFLOPs": round(flops / sorted(v)[len(v) // 2] / 1e9, 1)} for k, v in out.items()}
+
+
 def llama_step(args, device):
     """Whole-model step of a Llama configuration with every block linear on the Quartet path: bf16 autocast around
     forward and backward, cross-entropy on random ids, AdamW (fp32 state) for the ~800 M configuration."""
@@ -316,6 +340,8 @@ def main():
                     help="also run one plain 256 MiB device copy (a known-traffic kernel for scaling profiler byte counters)")
     ap.add_argument("--quantizer-sweep", action="store_true",
                     help="also time the quantizer alone on [rows x 4096] for rows 4096/16384/65536, three modes, hd 32/64/128")
+    ap.add_argument("--gemm-operand-content", action="store_true",
+                    help="also time the forward GEMM on operands of different content (real codes, random, constant): shows the power limit")
     ap.add_argument("--library-gemm", action="store_true",
                     help="also time the vendor library's MXFP4 product (torch._scaled_mm) on the forward GEMM's shape, for context")
     args = ap.parse_args()
@@ -388,6 +414,8 @@ def main():
         result["quantizer_sweep"] = quantizer_sweep(device)
     if args.library_gemm:
         result["library_gemm"] = library_gemm(device)
+    if args.gemm_operand_content:
+        result["gemm_operand_content"] = gemm_operand_content(x.detach(), w, dy)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
