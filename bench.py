@@ -280,6 +280,7 @@ def llama_step(args, device):
     from quartet_amd import llama as L
     torch.manual_seed(0)
     over = L.unquantized() if args.unquantized else {}
+    over["sdpa_backend"] = args.sdpa
     if args.workload == "llama30m":
         cfg, batch, seq, opt_step = L.llama_30m(**over), 64, 512, False
     else:
@@ -336,6 +337,8 @@ def main():
                          "over the block linears' flops")
     ap.add_argument("--unquantized", action="store_true",
                     help="with a llama workload: identity quantizers and the plain scheme (the bf16 model, for context)")
+    ap.add_argument("--sdpa", default="auto", choices=["auto", "default"],
+                    help="llama workloads: library attention kernels tried in the model's own order (auto) or the dispatcher's (default)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a known-traffic kernel for scaling profiler byte counters)")
     ap.add_argument("--quantizer-sweep", action="store_true",

@@ -10,12 +10,14 @@ linear is a ``QuantizedLinear`` built from registry names; init N(0, init_std) w
 (tiktoken) is not part of the numerics and is left out.
 
 Everything here except the block linears is stock PyTorch: this module is plumbing around the hot path."""
+import contextlib
 import math
 from dataclasses import dataclass, field
 
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
+from torch.nn.attention import SDPBackend, sdpa_kernel
 
 from .backward import BACKWARD_SCHEMES
 from .fused import rmsnorm_linear, rope_qkv, swiglu_linear
@@ -47,6 +49,11 @@ class LlamaConfig:
     # not in the reference: RMSNorm and the SwiGLU product are computed inside the activation quantizer of the linear
     # they feed (quartet_amd.fused) instead of being written out; False runs the reference's op-by-op composition
     fuse_producers: bool = True
+    # not in the reference (which leaves the choice to torch's dispatcher): which library kernel serves
+    # F.scaled_dot_product_attention.  "auto": on a GPU, the memory-efficient kernels first, then flash, then math --
+    # on MI355X with this PyTorch the memory-efficient pair runs a causal 16 x 12 x 2048 x 128 bf16 layer, forward and
+    # backward, in 2.1 ms against the 3.7 ms of the flash pair the dispatcher picks; "default": the dispatcher's order
+    sdpa_backend: str = "auto"
 
     @property
     def ffn_dim(self):
@@ -131,6 +138,15 @@ class LlamaMLP(nn.Module):
         return self.c_proj(F.silu(up) * gate)
 
 
+def _sdpa_choice(mode, q):
+    """Context manager that sets the order in which scaled_dot_product_attention tries its library kernels."""
+    if mode == "default" or not q.is_cuda:
+        return contextlib.nullcontext()
+    if mode != "auto":
+        raise ValueError(f"sdpa_backend must be 'auto' or 'default', got {mode!r}")
+    return sdpa_kernel([SDPBackend.EFFICIENT_ATTENTION, SDPBackend.FLASH_ATTENTION, SDPBackend.MATH], set_priority=True)
+
+
 class LlamaAttention(nn.Module):
     def __init__(self, config):
         super().__init__()
@@ -139,6 +155,7 @@ class LlamaAttention(nn.Module):
         self.c_proj = _linear(config, config.n_embd, config.n_embd)
         self.resid_dropout = nn.Dropout(config.dropout)
         self.n_head, self.n_embd, self.dropout = config.n_head, config.n_embd, config.dropout
+        self.sdpa_backend = config.sdpa_backend
 
     def forward(self, x, table, norm=None, add=None):
         B, T, C = x.shape
@@ -156,7 +173,8 @@ class LlamaAttention(nn.Module):
         q, k, v = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
         if not torch.is_autocast_enabled() and v.dtype != q.dtype:
             v = v.to(q.dtype)
-        y = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=self.dropout, is_causal=True)
+        with _sdpa_choice(self.sdpa_backend, q):
+            y = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=self.dropout, is_causal=True)
         y = y.transpose(1, 2).contiguous().view(B, T, C)
         out = self.resid_dropout(self.c_proj(y))
         return out if norm is None else (out, x)   # with the fused norm: also x for the residual sum
