@@ -562,6 +562,8 @@ struct Big4Plan {
     uint32_t lane_codes_a;  // this lane's byte offset inside a wave-load's source: row lane/4 + swizzled 16-byte column of a
     uint32_t lane_codes_b;  //   row-major panel, or the same pick inside the 1 KiB tile of a tiled one
     int kstep_a, kstep_b;   // bytes from one K step to the next: 64 row-major, 1024 tiled
+    uint32_t voff_a[4];     // lane_codes_a + i * (row16_bytes - 1024): wave-load i of a K step, issued with instruction
+    uint32_t voff_b[4];     //   offset i * 1024, which moves its LDS destination by as much (and the source back in place)
     uint32_t lane_scales;   // this lane's byte offset inside a panel's scales: row wave*64 + lane
     uint32_t lds_codes;     // wave-uniform LDS address of this wave's first A wave-load in stage 0
     uint32_t lds_scales;    // wave-uniform LDS address of this wave's A scale wave-load in buffer 0
@@ -579,6 +581,18 @@ __device__ __forceinline__ void big4_issue_scales(const Big4Plan& p, int qb, int
     const uint32_t base = p.lds_scales + buf * kScaleBufBytes;
     load_lds_b128_s(p.sa + qb * 16, p.lane_scales, base);
     load_lds_b128_s(p.sb + qb * 16, p.lane_scales, base + kBigM * 16);
+}
+
+// The LDS destination of a global->LDS load is M0 + the instruction's offset + lane * 16, and the same offset is added
+// to the source address: with the lane offsets of Big4Plan::voff_* one M0 value serves the four wave-loads of an
+// operand, and the loads themselves are single instructions between the MFMAs (every instruction a wave issues costs
+// it four to five cycles, and a K step has only 32 cycles per MFMA to hide them in).
+__device__ __forceinline__ void set_lds_dma_base(uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" ::"s"(lds_base));
+}
+template <int I>
+__device__ __forceinline__ void load_lds_b128_m0(const uint8_t* base, uint32_t lane_off) {
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(lane_off), "s"(base), "i"(I * 1024));
 }
 
 struct ScaleRegs {
@@ -628,6 +642,9 @@ __device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_by
     {
         const uint32_t base = plan.lds_codes + Q * kCodeStageBytes;
         if constexpr (Q == 3) __builtin_amdgcn_sched_barrier(0);
+        const uint8_t* src_a = plan.a + lks * plan.kstep_a;  // uniform: this wave's panel rows, K step lks
+        const uint8_t* src_b = plan.b + lks * plan.kstep_b;
+        set_lds_dma_base(base);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const v8i av = v8i{(int)st.f1.a[i].x, (int)st.f1.a[i].y, (int)st.f1.a[i].z, (int)st.f1.a[i].w, 0, 0, 0, 0};
@@ -641,10 +658,18 @@ __device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_by
                         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[i][j], 4, 4, 1, (int)sca[i], 1, (int)scb[j]);
                 }
             };
+            // per four MFMAs: two fragment reads of the next stage and two of the step's eight wave-loads (A's four,
+            // then B's four behind a second M0 value)
             st.f0.a[i] = *reinterpret_cast<const uint4*>(nxt + a_off0 + i * 32 * kRowBytes);
-            load_lds_b128_s(plan.a + i * plan.row16_bytes + lks * plan.kstep_a, plan.lane_codes_a, base + i * 1024);
+            if (i == 0) load_lds_b128_m0<0>(src_a, plan.voff_a[0]);
+            if (i == 1) load_lds_b128_m0<2>(src_a, plan.voff_a[2]);
+            if (i == 2) { set_lds_dma_base(base + kBOff); load_lds_b128_m0<0>(src_b, plan.voff_b[0]); }
+            if (i == 3) load_lds_b128_m0<2>(src_b, plan.voff_b[2]);
             st.f0.b[i] = *reinterpret_cast<const uint4*>(nxt + kBOff + b_off0 + i * 32 * kRowBytes);
-            load_lds_b128_s(plan.b + i * plan.row16_bytes + lks * plan.kstep_b, plan.lane_codes_b, base + kBOff + i * 1024);
+            if (i == 0) load_lds_b128_m0<1>(src_a, plan.voff_a[1]);
+            if (i == 1) load_lds_b128_m0<3>(src_a, plan.voff_a[3]);
+            if (i == 2) load_lds_b128_m0<1>(src_b, plan.voff_b[1]);
+            if (i == 3) load_lds_b128_m0<3>(src_b, plan.voff_b[3]);
             if constexpr (Q == 0) {
                 if (i == 3) big4_issue_scales(plan, lks >> 2, par ^ 1);
             }
@@ -747,6 +772,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         plan.kstep_a = a_tiled ? 1024 : kRowBytes;
         plan.kstep_b = b_tiled ? 1024 : kRowBytes;
         plan.lane_scales = (uint32_t)(lane * groups);
+        const uint32_t step16 = (uint32_t)plan.row16_bytes - 1024u;  // 16 rows are 8 K bytes in either layout, K >= 512
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            plan.voff_a[i] = plan.lane_codes_a + (uint32_t)i * step16;
+            plan.voff_b[i] = plan.lane_codes_b + (uint32_t)i * step16;
+        }
     }
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     int load_tm, load_tn, load_split;  // work item the load stream is in
