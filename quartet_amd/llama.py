@@ -140,10 +140,10 @@ class LlamaMLP(nn.Module):
 
 def _sdpa_choice(mode, q):
     """Context manager that sets the order in which scaled_dot_product_attention tries its library kernels."""
+    if mode not in ("auto", "default"):
+        raise ValueError(f"sdpa_backend must be 'auto' or 'default', got {mode!r}")
     if mode == "default" or not q.is_cuda:
         return contextlib.nullcontext()
-    if mode != "auto":
-        raise ValueError(f"sdpa_backend must be 'auto' or 'default', got {mode!r}")
     return sdpa_kernel([SDPBackend.EFFICIENT_ATTENTION, SDPBackend.FLASH_ATTENTION, SDPBackend.MATH], set_priority=True)
 
 

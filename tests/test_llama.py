@@ -139,3 +139,13 @@ def test_swiglu_split_order_is_up_then_gate():
     up, gate = x @ w[: cfg.ffn_dim].T, x @ w[cfg.ffn_dim:].T
     want = (torch.nn.functional.silu(up) * gate) @ mlp.c_proj.weight.T
     assert torch.allclose(mlp(x), want, atol=1e-6)
+
+
+def test_sdpa_backend_choice_is_validated_and_inert_on_cpu():
+    import contextlib
+    from quartet_amd.llama import _sdpa_choice
+    q = torch.zeros(1, 1, 4, 8)
+    assert isinstance(_sdpa_choice("auto", q), contextlib.nullcontext)      # CPU tensors: the dispatcher's own order
+    assert isinstance(_sdpa_choice("default", q), contextlib.nullcontext)
+    with pytest.raises(ValueError):
+        _sdpa_choice("flash", q)
