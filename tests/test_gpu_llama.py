@@ -149,3 +149,16 @@ def test_quartet_model_learns_with_the_training_loop():
     print(f"final losses {finals}", flush=True)
     assert finals["quartet"] < math.log(256) - 1.5
     assert finals["quartet"] < finals["bf16"] + 0.75
+
+
+def test_attention_kernel_choice_does_not_change_the_model(models):
+    """`sdpa_backend` only selects which library kernels serve scaled_dot_product_attention: the bf16-linear model must
+    give the same loss and the same gradients, to bf16 rounding, under the model's order and the dispatcher's."""
+    L, _, _, plain, idx, tgt = models
+    print("case llama30m sdpa auto vs default", flush=True)
+    other = L.Llama(L.llama_30m(**L.unquantized(sdpa_backend="default"))).to(idx.device)
+    other.load_state_dict(copy.deepcopy(plain.state_dict()))
+    la, lb = _step(plain, idx, tgt), _step(other, idx, tgt)
+    assert abs(la - lb) < 2e-3 * abs(la), (la, lb)
+    worst = min(_cosines(other, plain).values())
+    assert worst > 0.995, worst
