@@ -419,6 +419,7 @@ int qm_rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_dtype
     if (!dgain) return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: dgain must be non-null");
     if (rows > 0 && (!gy || !x || !gain || !factor || !dx || !workspace || workspace_bytes < qm::rmsnorm_backward_workspace_bytes(rows, cols)))
         return fail(QM_ERR_INVALID, "qm_rmsnorm_backward: null tensor, or workspace below %zu bytes", qm_rmsnorm_backward_workspace_bytes(rows, cols));
+    if (!aligned(maskbits, 4)) return fail(QM_ERR_UNALIGNED, "qm_rmsnorm_backward: maskbits needs 4-byte alignment");
     if (!aligned(skip, 16) || !aligned(dx_bf16, 8) || !aligned(gy, 8) || !aligned(x, 8) || !aligned(dx, 8) || !aligned(gain, 16) || !aligned(workspace, 16) ||
         (gy_dtype == QM_F32 && !aligned(gy, 16)) || (x_dtype == QM_F32 && (!aligned(x, 16) || !aligned(dx, 16))))
         return fail(QM_ERR_UNALIGNED, "qm_rmsnorm_backward: tensors need 16-byte alignment");
