@@ -191,7 +191,7 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
  * qm_swiglu_backward: autograd of silu(up) * gate: g [rows, hidden] -> d_h12 [rows, 2 hidden] of h12's dtype.
  *   Both backward kernels take the gradient either as it is (maskbits == NULL) or still in the rotated basis of the
  *   layer's activation quantizer (qm_linear_backward with gx_rotated): then maskbits [rows, cols/8] (the mask region of
- *   the layer's packed_x), sign_bits and scale_dtype describe that quantizer, and the masked inverse rotation of
+ *   the layer's packed_x; 4-byte aligned for qm_rmsnorm_backward), sign_bits and scale_dtype describe that quantizer, and the masked inverse rotation of
  *   qm_masked_hadamard_bwd (same operations, same bits, rounded to the gradient's dtype) is applied on the fly.
  * codes_layout QM_LAYOUT_TILED needs rows % 16 == 0 and cols (hidden) % 128 == 0; cols (hidden) % 32 == 0 always.
  */

@@ -71,6 +71,8 @@ def test_host_only_entry_points():
     (lambda L: L.qm_swiglu_quantize_mxfp4(None, 0, 16, 128, None, None, 0, 0, None), b"non-null"),
     (lambda L: L.qm_rmsnorm_backward(None, 0, None, 0, None, None, 16, 16384, None, None, 0, None, None, None, None, None, 0, None), b"[32, 8192]"),
     (lambda L: L.qm_rmsnorm_backward(None, 0, None, 0, None, None, 16, 128, None, None, 0, None, None, None, None, None, 0, None), b"dgain"),
+    # no rows: pointers are not dereferenced, the misaligned mask-bit pointer is still refused
+    (lambda L: L.qm_rmsnorm_backward(None, 0, None, 0, None, None, 0, 128, 0x1001, None, 0, None, None, None, 0x1000, None, 0, None), b"4-byte"),
     (lambda L: L.qm_swiglu_backward(None, 0, None, 0, 16, 30, None, None, 0, None, None), b"multiple of 4"),
     (lambda L: L.qm_swiglu_backward(None, 0, None, 0, 16, 32, None, None, 0, None, None), b"non-null"),
 ])
