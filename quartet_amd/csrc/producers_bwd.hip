@@ -363,6 +363,108 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const TG* __restrict__ 
     store4(d_h12 + row * 2 * hidden + hidden + col, make_float4(da[0], da[1], da[2], da[3]));
 }
 
+// Eight consecutive elements per lane: 16-byte accesses for bf16 tensors, and the clip mask of the lane's elements is
+// exactly one byte.  The four lanes that hold a group of 32 cooperate as in the stand-alone inverse rotation (three
+// butterfly strides inside the lane, two across lanes): the same operations on the same pairs, hence the same bits.
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float (&v)[8]) {
+    if constexpr (sizeof(T) == 2) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(p);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = u2f(w[i] << 16);
+            v[2 * i + 1] = u2f(w[i] & 0xffff0000u);
+        }
+    } else {
+        const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+}
+template <typename T>
+__device__ __forceinline__ void store8(T* p, const float (&v)[8]) {
+    if constexpr (sizeof(T) == 2) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2 * i], v[2 * i + 1]}, v2bf));
+        *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+}
+template <bool ROUND_BF16>
+__device__ __forceinline__ void inverse_rotate_oct(float (&v)[8], const InverseRotation& rot, int64_t elem) {
+    const int lic = (int)(elem >> 3) & 3;  // the lane's place in its group
+    const uint32_t keep = (uint32_t)rot.maskbits[elem >> 3];
+    const uint32_t sign = rot.sign_word >> (lic * 8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float x = v[i] * (((keep >> i) & 1u) ? 1.0f : 0.0f);
+        v[i] = u2f(f2u(x) ^ (((sign >> i) & 1u) << 31));
+    }
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (i & h) continue;
+            const float a = v[i], b = v[i + h];
+            v[i] = a + b;
+            v[i + h] = a - b;
+        }
+    }
+#pragma unroll
+    for (int m = 1; m < 4; m <<= 1) {  // lower lane of a butterfly: own + partner; upper lane: partner - own
+        const uint32_t flip = (lic & m) ? 0x80000000u : 0u;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float p = m == 1 ? quad_xor1(v[i]) : quad_xor2(v[i]);
+            v[i] = p + u2f(f2u(v[i]) ^ flip);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = v[i] * rot.c;
+    if constexpr (ROUND_BF16) {
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) {
+            const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[i], v[i + 1]}, v2bf));
+            v[i] = u2f(w << 16);
+            v[i + 1] = u2f(w & 0xffff0000u);
+        }
+    }
+}
+
+// hidden % 8 == 0: the same arithmetic per element as swiglu_bwd_kernel, half as many memory instructions per element
+// (used when the gradient arrives rotated: there the mask byte per quad of the other kernel is what it saves)
+template <typename TG, typename TH>
+__global__ __launch_bounds__(256) void swiglu_bwd_oct_kernel(const TG* __restrict__ g, const TH* __restrict__ h12,
+                                                             int64_t rows, int64_t hidden, InverseRotation rot,
+                                                             TH* __restrict__ d_h12) {
+    const int64_t octs_per_row = hidden / 8;
+    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (q >= rows * octs_per_row) return;
+    const int64_t row = q / octs_per_row, col = (q - row * octs_per_row) * 8;
+    float G[8], U[8], A[8], du[8], da[8];
+    load8(g + row * hidden + col, G);
+    load8(h12 + row * 2 * hidden + col, U);
+    load8(h12 + row * 2 * hidden + hidden + col, A);
+    if (rot.maskbits) inverse_rotate_oct<sizeof(TG) == 2>(G, rot, row * hidden + col);  // hidden % 32 == 0 then
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float s = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-U[i] * 1.44269504f));
+        float a = U[i] * s, t = G[i] * A[i];
+        if constexpr (sizeof(TH) == 2) {
+            a = bf16_to_f32(f32_to_bf16(a));
+            t = bf16_to_f32(f32_to_bf16(t));
+        }
+        da[i] = G[i] * a;
+        du[i] = t * s * (1.0f + U[i] * (1.0f - s));
+    }
+    store8(d_h12 + row * 2 * hidden + col, du);
+    store8(d_h12 + row * 2 * hidden + hidden + col, da);
+}
+
 // one wave per row for rows of at most 1536 columns (see rmsnorm_bwd_rows_kernel), the cooperative kernel above that
 inline bool rows_kernel_serves(int64_t cols) { return cols <= 1536; }
 int64_t rmsnorm_bwd_blocks(int64_t rows, int64_t cols) {
@@ -421,16 +523,23 @@ hipError_t rmsnorm_backward(const void* gy, int gy_dtype, const void* x, int x_d
 hipError_t swiglu_backward(const void* g, int g_dtype, const void* h12, int dtype, int64_t rows, int64_t hidden,
                            const uint8_t* maskbits, uint32_t sign_word, int scale_dtype, void* d_h12, hipStream_t stream) {
     if (rows == 0 || hidden == 0) return hipSuccess;
-    const dim3 grid((unsigned)((rows * (hidden / 4) + 255) / 256)), block(256);
     const InverseRotation rot{maskbits, sign_word, hadamard_scale(32, scale_dtype)};
-    if (g_dtype == BF16 && dtype == BF16)
-        swiglu_bwd_kernel<uint16_t, uint16_t><<<grid, block, 0, stream>>>(reinterpret_cast<const uint16_t*>(g), reinterpret_cast<const uint16_t*>(h12), rows, hidden, rot, reinterpret_cast<uint16_t*>(d_h12));
-    else if (g_dtype == BF16)
-        swiglu_bwd_kernel<uint16_t, float><<<grid, block, 0, stream>>>(reinterpret_cast<const uint16_t*>(g), reinterpret_cast<const float*>(h12), rows, hidden, rot, reinterpret_cast<float*>(d_h12));
-    else if (dtype == BF16)
-        swiglu_bwd_kernel<float, uint16_t><<<grid, block, 0, stream>>>(reinterpret_cast<const float*>(g), reinterpret_cast<const uint16_t*>(h12), rows, hidden, rot, reinterpret_cast<uint16_t*>(d_h12));
-    else
-        swiglu_bwd_kernel<float, float><<<grid, block, 0, stream>>>(reinterpret_cast<const float*>(g), reinterpret_cast<const float*>(h12), rows, hidden, rot, reinterpret_cast<float*>(d_h12));
+    // with the inverse rotation the octet kernel is 10 % faster (232 against 259 us at 32768 x 4096), without it 4 % slower
+    const bool oct = maskbits && hidden % 8 == 0;
+    const dim3 grid((unsigned)((rows * (hidden / (oct ? 8 : 4)) + 255) / 256)), block(256);
+    const auto go = [&](auto tg, auto th) {
+        using TG = decltype(tg);
+        using TH = decltype(th);
+        const TG* gp = reinterpret_cast<const TG*>(g);
+        const TH* hp = reinterpret_cast<const TH*>(h12);
+        TH* dp = reinterpret_cast<TH*>(d_h12);
+        if (oct) swiglu_bwd_oct_kernel<TG, TH><<<grid, block, 0, stream>>>(gp, hp, rows, hidden, rot, dp);
+        else swiglu_bwd_kernel<TG, TH><<<grid, block, 0, stream>>>(gp, hp, rows, hidden, rot, dp);
+    };
+    if (g_dtype == BF16 && dtype == BF16) go(uint16_t{}, uint16_t{});
+    else if (g_dtype == BF16) go(uint16_t{}, float{});
+    else if (dtype == BF16) go(float{}, uint16_t{});
+    else go(float{}, float{});
     return hipGetLastError();
 }
 
