@@ -746,7 +746,10 @@ struct RmsNormProducer {
     // Sum of squares in a fixed order: sixteen interleaved partial sums (partial j adds the sums of groups j, j+16,
     // j+32, ... in ascending order, each group summed by the pairwise tree), then the pairwise tree over the sixteen.
     // A lane without a group adds +0, which leaves a sum of squares unchanged.
-    __device__ __forceinline__ float prepare(int64_t row, int lane, int groups, int64_t cols, float (&first)[32]) const {
+    // W < 64: the wave holds 64 / W rows of at most W groups each, a row in the W lanes from `seg` on (`lane` counts
+    // from there); the partial sums then have W / 16 terms instead of four, the missing ones being the +0 of above.
+    template <int W = 64>
+    __device__ __forceinline__ float prepare(int64_t row, int lane, int groups, int64_t cols, float (&first)[32], int seg = 0) const {
         float acc = 0.0f;
         for (int base = 0; base < groups; base += 64) {
             const int g = base + lane;
@@ -773,7 +776,7 @@ struct RmsNormProducer {
                 s = tree_sum32(v);
             }
 #pragma unroll
-            for (int k = 0; k < 4; ++k) acc = acc + __shfl(s, (lane & 15) + 16 * k, 64);
+            for (int k = 0; k < W / 16; ++k) acc = acc + __shfl(s, seg + (lane & 15) + 16 * k, 64);
         }
 #pragma unroll
         for (int m = 1; m < 16; m <<= 1) acc = acc + __shfl_xor(acc, m, 64);
@@ -803,7 +806,8 @@ struct SwiGluProducer {
     static constexpr int kOutDtype = sizeof(T) == 2 ? BF16 : F32;
     const T* h12;  // [rows, 2 cols]: up, then gate
 
-    __device__ __forceinline__ float prepare(int64_t, int, int, int64_t, float (&)[32]) const { return 0.0f; }
+    template <int W = 64>
+    __device__ __forceinline__ float prepare(int64_t, int, int, int64_t, float (&)[32], int = 0) const { return 0.0f; }
     __device__ __forceinline__ void load(int64_t row, int g, int64_t cols, float, bool, float (&v)[32]) const {
         float gate[32];
         load_group<T>(h12 + row * 2 * cols + g * 32, v);
@@ -824,7 +828,8 @@ struct SwiGluProducer {
 };
 
 // quest RTN + clip mask (the forward quantizer) of rows that a producer computes
-template <typename P, bool TILED>
+// W: lanes per row (64, or 32 / 16 for rows of at most that many groups: two / four rows per wave)
+template <typename P, bool TILED, int W = 64>
 struct ProducedRowsJob {
     P prod;
     int64_t rows, cols;
@@ -835,17 +840,19 @@ struct ProducedRowsJob {
 
     ProducedRowsJob(const P& prod_, int64_t rows_, int64_t cols_, uint32_t sign_word_, const GroupOut& out_)
         : prod(prod_), rows(rows_), cols(cols_), c(hadamard_scale(32, P::kOutDtype)), sign_word(sign_word_), out(out_),
-          blocks((unsigned)((rows_ + 3) / 4)) {}
+          blocks((unsigned)((rows_ + 4 * (64 / W) - 1) / (4 * (64 / W)))) {}
 
     __device__ __forceinline__ void run(unsigned bid) const {
-        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-        const int64_t row = (int64_t)bid * 4 + wave;
-        if (row >= rows) return;  // a whole wave
+        const int wlane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const int lane = wlane & (W - 1), seg = wlane - lane;  // place in the row's segment of the wave
+        int64_t row = ((int64_t)bid * 4 + wave) * (64 / W) + seg / W;
+        if (row - seg / W >= rows) return;  // a whole wave
+        if (row >= rows) row = rows - 1;    // a segment past the end repeats the last row: same values to the same places
         const int groups = (int)(cols / 32);
         float v[32];
-        const float state = prod.prepare(row, lane, groups, cols, v);
+        const float state = prod.template prepare<W>(row, lane, groups, cols, v, seg);
         // TILED: cols % 128 == 0, so the four lanes of a quad run the same number of iterations
-        for (int g = lane; g < groups; g += 64) {
+        for (int g = lane; g < groups; g += W) {
             const int64_t gi = row * groups + g;
             const int64_t ci = TILED ? (row >> 4) * 16 * groups + ((g >> 2) * 64 + (int)(row & 15) * 4 + (g & 3)) : gi;
             prod.load(row, g, cols, state, g == lane, v);
@@ -867,12 +874,20 @@ struct ProducedRowsJob {
     }
 };
 
+template <typename P, int W>
+void launch_produced_w(const P& prod, int64_t rows, int64_t cols, uint32_t sign_word, const GroupOut& out, bool tiled,
+                       hipStream_t stream) {
+    if (tiled) launch_job(ProducedRowsJob<P, true, W>(prod, rows, cols, sign_word, out), stream);
+    else launch_job(ProducedRowsJob<P, false, W>(prod, rows, cols, sign_word, out), stream);
+}
+
 template <typename P>
 void launch_produced(const P& prod, int64_t rows, int64_t cols, uint32_t sign_word, uint8_t* codes, uint8_t* scales,
                      uint8_t* maskbits, bool tiled, hipStream_t stream) {
     const GroupOut out{reinterpret_cast<uint4*>(codes), scales, reinterpret_cast<uint32_t*>(maskbits), nullptr};
-    if (tiled) launch_job(ProducedRowsJob<P, true>(prod, rows, cols, sign_word, out), stream);
-    else launch_job(ProducedRowsJob<P, false>(prod, rows, cols, sign_word, out), stream);
+    if (cols <= 16 * 32) launch_produced_w<P, 16>(prod, rows, cols, sign_word, out, tiled, stream);
+    else if (cols <= 32 * 32) launch_produced_w<P, 32>(prod, rows, cols, sign_word, out, tiled, stream);
+    else launch_produced_w<P, 64>(prod, rows, cols, sign_word, out, tiled, stream);
 }
 
 }  // namespace
