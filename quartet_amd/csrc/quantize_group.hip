@@ -742,6 +742,12 @@ struct RmsNormProducer {
     const TAdd* add;
     T* xsum;
 
+    // 8 KiB of LDS per wave of the workgroup: staging of the residual sum on its way out
+    __device__ __forceinline__ static float4* xsum_area() {
+        __shared__ float4 xbuf[4][512];
+        return xbuf[threadIdx.x >> 6];
+    }
+
     // The row's factor; `first` leaves with the raw elements of the lane's first group (if it has one).
     // Sum of squares in a fixed order: sixteen interleaved partial sums (partial j adds the sums of groups j, j+16,
     // j+32, ... in ascending order, each group summed by the pairwise tree), then the pairwise tree over the sixteen.
@@ -763,9 +769,20 @@ struct RmsNormProducer {
                     load_group<TAdd>(add + row * cols + g * 32, a);
 #pragma unroll
                     for (int i = 0; i < 32; ++i) v[i] = v[i] + a[i];
-                    float4* dst = reinterpret_cast<float4*>(xsum + row * cols + g * 32);
+                    if constexpr (W == 64) {
+                        // the sum leaves through LDS so that an instruction stores whole 128-byte lines (a lane's own
+                        // 128 bytes would go out as eight 16-byte pieces of 64 different lines per instruction); slot
+                        // 8 l + (q ^ l % 8) of the wave's area holds piece q of lane l's group: writes and the
+                        // slot-ordered reads both spread over all banks
+                        float4* area = xsum_area();
 #pragma unroll
-                    for (int q = 0; q < 8; ++q) dst[q] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+                        for (int q = 0; q < 8; ++q)
+                            area[8 * lane + (q ^ (lane & 7))] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+                    } else {
+                        float4* dst = reinterpret_cast<float4*>(xsum + row * cols + g * 32);
+#pragma unroll
+                        for (int q = 0; q < 8; ++q) dst[q] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+                    }
                 }
                 if (base == 0) {
 #pragma unroll
@@ -774,6 +791,19 @@ struct RmsNormProducer {
 #pragma unroll
                 for (int i = 0; i < 32; ++i) v[i] = v[i] * v[i];
                 s = tree_sum32(v);
+            }
+            if constexpr (kAdd && W == 64) {
+                const float4* area = xsum_area();
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int slot = 64 * i + lane, gl = slot >> 3, piece = (slot & 7) ^ (gl & 7);
+                    if (base + gl < groups)
+                        reinterpret_cast<float4*>(xsum + row * cols + (int64_t)(base + gl) * 32)[piece] = area[slot];
+                }
+                __builtin_amdgcn_wave_barrier();  // the next pass over the row reuses the area
             }
 #pragma unroll
             for (int k = 0; k < W / 16; ++k) acc = acc + __shfl(s, seg + (lane & 15) + 16 * k, 64);
