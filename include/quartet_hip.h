@@ -107,6 +107,21 @@ int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint
                      void* stream);
 
 /*
+ * qm_gemm_mxfp4_tn for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses that forbid
+ * hipMalloc).  It has no counterpart in the reference.  Same arguments and the same results, bit for bit, as
+ * qm_gemm_mxfp4_tn offered qm_gemm_workspace_bytes(M, N, K) bytes of workspace; the split-K partial sums live in a
+ * device array built into the library (QM_GEMM_NOALLOC_SCRATCH_BYTES per GPU, held until the process ends) instead.
+ * A shape whose partial sums need more is rejected with QM_ERR_INVALID.  Nothing in the array has to start at zero
+ * (every partial sum that is read has been written by the same call), but every call on a GPU uses that GPU's one
+ * array: calls that overlap on one GPU (two streams, two threads) race.  Allocates nothing, frees nothing.
+ */
+#define QM_GEMM_NOALLOC_SCRATCH_BYTES ((size_t)64 << 20)
+size_t qm_gemm_noalloc_scratch_bytes(void);
+int qm_gemm_mxfp4_tn_noalloc(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                             const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c,
+                             int c_dtype, int a_layout, int b_layout, void* stream);
+
+/*
  * out = ((g * mask).view(-1, hd)) @ H^T: the straight-through backward of the forward quantizer,
  * QuestMXFP4QuantizerFn.backward (src/models/quantization/quantizers/mxfp4.py:143-146); with
  * maskbits == NULL it is AlbertTsengQuantizerFn.backward (mxfp4.py:31-34).

@@ -21,6 +21,8 @@ EXPORTS = (
     "qm_masked_hadamard_bwd",
     "qm_dequantize_mxfp4",
     "qm_gemm_workspace_bytes",
+    "qm_gemm_noalloc_scratch_bytes",
+    "qm_gemm_mxfp4_tn_noalloc",
     "qm_packed_operand_bytes",
     "qm_packed_operand_offsets",
     "qm_linear_backward_workspace_bytes",
@@ -64,6 +66,10 @@ def lib():
     L.qm_gemm_mxfp4_tn.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, i32, vp, ctypes.c_size_t, vp]
     L.qm_gemm_workspace_bytes.restype = ctypes.c_size_t
     L.qm_gemm_workspace_bytes.argtypes = [i64, i64, i64]
+    L.qm_gemm_noalloc_scratch_bytes.restype = ctypes.c_size_t
+    L.qm_gemm_noalloc_scratch_bytes.argtypes = []
+    L.qm_gemm_mxfp4_tn_noalloc.restype = i32
+    L.qm_gemm_mxfp4_tn_noalloc.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, i32, vp]
     L.qm_masked_hadamard_bwd.restype = i32
     L.qm_masked_hadamard_bwd.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp, i32, vp]
     L.qm_dequantize_mxfp4.restype = i32

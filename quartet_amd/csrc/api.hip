@@ -4,6 +4,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "../../include/quartet_hip.h"
 #include "qm_kernels.h"
 
@@ -42,7 +44,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 8; }
+int qm_version(void) { return 9; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -125,6 +127,60 @@ int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint
 size_t qm_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0 || K % 32) return 0;
     return qm::gemm_workspace_bytes(M, N, K);
+}
+
+}  // extern "C"
+
+// ---- the product without any allocation: split-K partial sums live in a file-scope device array ---------------
+namespace {
+constexpr size_t kNoAllocScratchBytes = QM_GEMM_NOALLOC_SCRATCH_BYTES;
+// One copy per GPU the library is loaded on, held until the process ends.  In host code this name is only a handle for
+// hipGetSymbolAddress: the device address of each GPU's copy is looked up once per device and used from then on.
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kNoAllocScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// device address of the current device's scratch array (nullptr + error code on failure)
+int scratch_of_current_device(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return from_hip(e, "qm_gemm_mxfp4_tn_noalloc: hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn_noalloc: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return from_hip(e == hipSuccess ? hipErrorInvalidSymbol : e, "qm_gemm_mxfp4_tn_noalloc: hipGetSymbolAddress");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+}  // namespace
+
+extern "C" {
+
+size_t qm_gemm_noalloc_scratch_bytes(void) { return kNoAllocScratchBytes; }
+
+int qm_gemm_mxfp4_tn_noalloc(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
+                             int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype, int a_layout, int b_layout,
+                             void* stream) {
+    if (M < 0 || N < 0 || K < 0 || K % 32)
+        return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn_noalloc: need K %% 32 == 0 (M=%lld N=%lld K=%lld)", (long long)M, (long long)N, (long long)K);
+    if (M == 0 || N == 0) return 0;
+    // the same cut into K ranges as qm_gemm_mxfp4_tn makes when it is offered qm_gemm_workspace_bytes() of scratch
+    const size_t need = qm::gemm_workspace_bytes(M, N, K);
+    if (need > kNoAllocScratchBytes)
+        return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn_noalloc: this shape's split-K partial sums need %zu bytes, the built-in scratch "
+                                    "holds %zu (M=%lld N=%lld K=%lld); use qm_gemm_mxfp4_tn with a caller-provided workspace",
+                    need, kNoAllocScratchBytes, (long long)M, (long long)N, (long long)K);
+    void* ws = nullptr;
+    if (need) {
+        if (int rc = scratch_of_current_device(&ws)) return rc;
+    }
+    return qm_gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, c_dtype, a_layout, b_layout, ws, need, stream);
 }
 
 int qm_masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t cols, int hadamard_dim, int scale_dtype,

@@ -119,6 +119,20 @@ def gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, alpha=1.0, out_dtype=tor
     return c
 
 
+def gemm_mxfp4_tn_noalloc(a_codes, a_scales, b_codes, b_scales, alpha, out):
+    """The same product through the library's allocation-free entry point: `out` [M,N] (bf16 or fp32) is written in
+    place and split-K partial sums go to the library's built-in device scratch.  Row-major code bytes."""
+    _require_cuda(a_codes, a_scales, b_codes, b_scales, out)
+    M, K = a_codes.shape[0], a_codes.shape[1] * 2
+    N = b_codes.shape[0]
+    assert out.shape == (M, N) and out.is_contiguous() and b_codes.shape[1] * 2 == K
+    rc = _lib.lib().qm_gemm_mxfp4_tn_noalloc(_ptr(a_codes), _ptr(a_scales), _ptr(b_codes), _ptr(b_scales), M, N, K, alpha,
+                                             _ptr(out), _dtype_code(out.dtype), QM_LAYOUT_ROWMAJOR, QM_LAYOUT_ROWMAJOR,
+                                             _stream())
+    _lib.check(rc, "qm_gemm_mxfp4_tn_noalloc")
+    return out
+
+
 def masked_hadamard_bwd(g, hadamard_dim=32, scale_dtype=torch.bfloat16, sign_bits=None, maskbits=None, out_dtype=None,
                         out=None):
     """g [R,C] -> ((g*mask).view(-1,hd) @ H^T) as [R,C] of out_dtype (default g.dtype); `out` may be pre-allocated."""
