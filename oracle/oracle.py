@@ -51,6 +51,7 @@ def lib():
         L.qo_philox_uniform16.restype = f32
         L.qo_philox_uniform16.argtypes = [u64, u64]
         L.qo_philox_uniform16_fill.argtypes = [u64, i64, vp]
+        L.qo_philox_uniform16_at.argtypes = [u64, i64, vp, vp]
         L.qo_quantize.restype = i32
         L.qo_quantize.argtypes = [vp, i32, i64, i64, i32, vp, i32, i32, vp, u64, vp, vp, vp, vp, vp]
         L.qo_dequantize.restype = i32
@@ -137,6 +138,14 @@ def philox4x32_10(ctr, key):
 def philox_uniform16(seed, n):
     u = np.empty(n, dtype=np.float32)
     lib().qo_philox_uniform16_fill(seed, n, _ptr(u))
+    return u
+
+
+def philox_uniform16_at(seed, offsets):
+    """The stream's uniforms at the given flat element offsets (any shape of int64), same shape back."""
+    off = np.ascontiguousarray(offsets, dtype=np.int64)
+    u = np.empty(off.shape, dtype=np.float32)
+    lib().qo_philox_uniform16_at(seed, off.size, _ptr(off), _ptr(u))
     return u
 
 

@@ -118,6 +118,11 @@ void qo_philox_uniform16_fill(uint64_t seed, int64_t n, float* u) {
     for (int64_t o = 0; o < n; ++o) u[o] = qo_philox_uniform16(seed, (uint64_t)o);
 }
 
+/* the uniforms of n arbitrary flat offsets (a sample of rows of a large tensor) */
+void qo_philox_uniform16_at(uint64_t seed, int64_t n, const int64_t* offsets, float* u) {
+    for (int64_t i = 0; i < n; ++i) u[i] = qo_philox_uniform16(seed, (uint64_t)offsets[i]);
+}
+
 /* ---- rotation --------------------------------------------------------------------- */
 /* v[0..hd) in place: Sylvester butterfly ascending strides, then * c, then column signs. */
 static void rotate_chunk(float* v, int hd, float c, const uint32_t* sign_bits) {

@@ -1,5 +1,6 @@
-"""Parity at the benchmark's full sizes (tokens 8192, features 4096; the quantizer also at 65536 x 4096), where the
-CPU oracle cannot process whole tensors in test time.  Each check is a size-independent property that reduces
+"""Parity at the benchmark's full sizes (tokens 8192, in 4096, out 4096 and 11008; the quantizer on [rows x 4096] for
+rows 4096, 16384 and 65536 with Hadamard blocks 32, 64 and 128), where the CPU oracle cannot process whole tensors in
+test time.  Each check is a size-independent property that reduces
 to an oracle comparison on a slice:
 
 * row-major quantization is row-local, so any subset of rows of the big result must equal the oracle's result on
@@ -19,6 +20,7 @@ from tests.util import to_oracle
 pytestmark = pytest.mark.gpu
 
 T, I, O = 8192, 4096, 4096
+OUTS = [4096, 11008]   # the two out-feature counts of the isolated-layer configuration
 
 
 @pytest.fixture(scope="module")
@@ -29,14 +31,18 @@ def K():
     return kernels
 
 
-@pytest.fixture(scope="module")
-def data():
+def _make_data(out_features):
     g = torch.Generator().manual_seed(123)
     x = torch.randn(T, I, generator=g)
     heavy = torch.rand(T, I, generator=g) < 0.01
     x = torch.where(heavy, 30.0 * torch.randn(T, I, generator=g), x).to(torch.bfloat16)
-    dy = (1e-3 * torch.randn(T, O, generator=g)).to(torch.bfloat16)
+    dy = (1e-3 * torch.randn(T, out_features, generator=g)).to(torch.bfloat16)
     return x, dy
+
+
+@pytest.fixture(scope="module")
+def data():
+    return _make_data(O)
 
 
 def _rows(t, idx):
@@ -71,6 +77,51 @@ def test_rowmajor_sampled_rows_match_oracle(oracle, K, rows, mode, want_mask):
     perm = torch.randperm(rows, generator=g)[:4096].to(dev)
     pc, ps, _, _ = K.quantize_mxfp4(xd[perm].contiguous(), 32, signs, mode)
     assert torch.equal(pc, codes[perm]) and torch.equal(ps, scales[perm])
+
+
+C4_ROWS = [4096, 16384, 65536]   # 16 Mi, 64 Mi and 256 Mi elements as [rows x 4096]
+
+
+@pytest.mark.parametrize("rows", C4_ROWS)
+@pytest.mark.parametrize("hd", [32, 64, 128])
+@pytest.mark.parametrize("mode", ["quest_rtn_mask", "absmax_rtn", "absmax_sr"])
+def test_quantizer_sweep_sampled_rows_match_oracle(oracle, K, rows, hd, mode):
+    """The quantizer-only configuration at its real sizes: Gaussian data with 0.1 % entries at +-1e3, three modes,
+    Hadamard blocks 32 / 64 / 128.  A Hadamard block never crosses a row, so sampled rows of the big result must equal
+    the oracle's result on those rows; with stochastic rounding the in-kernel stream is keyed by the flat element
+    offset, so the oracle is fed the stream's uniforms at the sampled rows' offsets."""
+    print(f"case quantizer sweep rows={rows} hd={hd} {mode}", flush=True)
+    dev = torch.device("cuda:0")
+    cols = 4096
+    seed = 1000 * hd + rows
+    gd = torch.Generator(device=dev).manual_seed(seed)
+    xd = torch.randn(rows, cols, generator=gd, device=dev)
+    spike = torch.rand(rows, cols, generator=gd, device=dev) < 1e-3
+    sgn = torch.where(torch.rand(rows, cols, generator=gd, device=dev) < 0.5, -1e3, 1e3)
+    xd = torch.where(spike, sgn, xd).to(torch.bfloat16)
+    signs = (0x9D2C5681 | (0x3A5F01C7 << 32) | (0xC0FFEE11 << 64) | (0x13579BDF << 96)) & ((1 << hd) - 1)
+    sv = np.array([-1 if (signs >> j) & 1 else 1 for j in range(hd)])
+    qmode = {"quest_rtn_mask": K.QM_QUEST_RTN, "absmax_rtn": K.QM_ABSMAX_RTN, "absmax_sr": K.QM_ABSMAX_SR}[mode]
+    omode = {"quest_rtn_mask": oracle.QUEST_RTN, "absmax_rtn": oracle.ABSMAX_RTN, "absmax_sr": oracle.ABSMAX_SR}[mode]
+    want_mask = mode == "quest_rtn_mask"
+    kseed = 0xC0DE_0000 + rows + hd
+    codes, scales, mask, _ = K.quantize_mxfp4(xd, hd, signs, qmode, want_mask=want_mask, seed=kseed)
+    torch.cuda.synchronize()
+    g = torch.Generator().manual_seed(seed)
+    idx = torch.cat([torch.arange(0, 8), torch.randint(0, rows, (80,), generator=g), torch.arange(rows - 8, rows)])
+    u = None
+    if mode == "absmax_sr":
+        offsets = idx.numpy().astype(np.int64)[:, None] * cols + np.arange(cols, dtype=np.int64)[None, :]
+        u = oracle.philox_uniform16_at(kseed, offsets)
+    ref = oracle.quantize(to_oracle(xd[idx.to(dev)]), hd, signs=sv, mode=omode, want_mask=want_mask, u=u)
+    assert np.array_equal(_rows(scales, idx.to(dev)), ref["scales"])
+    assert np.array_equal(_rows(codes, idx.to(dev)), ref["codes"])
+    if want_mask:
+        assert np.array_equal(_rows(mask, idx.to(dev)), ref["mask"])
+    if hd == 32:   # the tiled code layout (Hadamard block 32 only) holds the same bytes
+        tcodes, tscales, tmask, _ = K.quantize_mxfp4(xd, hd, signs, qmode, want_mask=want_mask, seed=kseed, tiled=True)
+        assert torch.equal(K.untile_codes(tcodes), codes) and torch.equal(tscales, scales)
+        assert not want_mask or torch.equal(tmask, mask)
 
 
 def test_stochastic_prefix_matches_oracle(oracle, K, data):
@@ -119,43 +170,67 @@ def test_transposed_and_requantize_column_slices(oracle, K, data):
         assert np.array_equal(to_oracle(xts[c0:c0 + 32]), ref["scales"]), c0
 
 
-def test_gemm_rows_and_sample(oracle, K, data):
-    print("case fullsize gemm 8192x4096x4096", flush=True)
+def _random_operand(K, rows, cols, seed, mode, dev):
+    """A packed [rows, cols] operand (tiled codes) quantized from seeded Gaussian data generated on the GPU."""
+    gd = torch.Generator(device=dev).manual_seed(seed)
+    t = torch.randn(rows, cols, generator=gd, device=dev).to(torch.bfloat16)
+    codes, scales, _, _ = K.quantize_mxfp4(t, 32, None, mode, tiled=True, seed=seed)
+    return codes, scales
+
+
+# the three products of the isolated layer at out = 4096 and out = 11008 (forward, grad-input, grad-weight: M x N x K)
+GEMM_SHAPES = [(T, 4096, I), (4096, I, T), (T, 11008, I), (T, I, 11008), (11008, I, T)]
+
+
+@pytest.mark.parametrize("M,N,Kdim", GEMM_SHAPES)
+def test_gemm_rows_and_sample(oracle, K, M, N, Kdim):
+    print(f"case fullsize gemm {M}x{N}x{Kdim}", flush=True)
+    from quartet_amd import _lib
     dev = torch.device("cuda:0")
-    x, _ = data
     g = torch.Generator().manual_seed(9)
-    w = (0.02 * torch.randn(O, I, generator=g)).to(torch.bfloat16)
-    xc, xs, _, _ = K.quantize_mxfp4(x.to(dev), 32, None, K.QM_QUEST_RTN, tiled=True)
-    wc, ws, _, _ = K.quantize_mxfp4(w.to(dev), 32, None, K.QM_QUEST_RTN, tiled=True)
-    y = K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.float32, a_tiled=True, b_tiled=True)
-    y16 = K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.bfloat16, a_tiled=True, b_tiled=True)
+    # forward-like operands for the token-major products, absmax-coded ones (whole E2M1 range, post-scale 4/3) for the
+    # weight-gradient shape
+    absmax = Kdim == T
+    mode = K.QM_ABSMAX_RTN if absmax else K.QM_QUEST_RTN
+    post = float(oracle.FOUR_THIRDS) if absmax else 1.0
+    ac, as_ = _random_operand(K, M, Kdim, 100 + M, mode, dev)
+    bc, bs = _random_operand(K, N, Kdim, 200 + N, mode, dev)
+    alpha = post * post
+    y = K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha, torch.float32, a_tiled=True, b_tiled=True)
+    y16 = K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha, torch.bfloat16, a_tiled=True, b_tiled=True)
     assert torch.equal(y16, y.to(torch.bfloat16))
-    # a 256-row panel alone (one tile row, same K order inside every tile): bitwise the same rows
-    xr = K.untile_codes(xc)
-    sub = K.gemm_mxfp4_tn(K.tile_codes(xr[4096:4352].contiguous()), xs[4096:4352].contiguous(), wc, ws, 1.0, torch.float32,
-                          a_tiled=True, b_tiled=True, split_k=False)
-    assert torch.equal(sub, y[4096:4352])
-    # sampled rows against the float64 product of the de-quantized operands
-    idx = torch.randint(0, T, (64,), generator=g)
-    A = oracle.dequantize(to_oracle(xr[idx.to(dev)]), to_oracle(xs[idx.to(dev)])).astype(np.float64)
-    B = oracle.dequantize(to_oracle(K.untile_codes(wc)), to_oracle(ws)).astype(np.float64)
+    ar = K.untile_codes(ac)
+    if _lib.lib().qm_gemm_workspace_bytes(M, N, Kdim) == 0:
+        # a 256-row panel alone (one tile row, same K order inside every tile): bitwise the same rows
+        r0 = (M // 2 // 256) * 256
+        sub = K.gemm_mxfp4_tn(K.tile_codes(ar[r0:r0 + 256].contiguous()), as_[r0:r0 + 256].contiguous(), bc, bs, alpha,
+                              torch.float32, a_tiled=True, b_tiled=True, split_k=False)
+        assert torch.equal(sub, y[r0:r0 + 256])
+    # sampled rows (first, last and random ones) against the float64 product of the de-quantized operands
+    idx = torch.cat([torch.tensor([0, M - 1]), torch.randint(0, M, (46,), generator=g)]).to(dev)
+    A = oracle.dequantize(to_oracle(ar[idx]), to_oracle(as_[idx]), post).astype(np.float64)
+    B = oracle.dequantize(to_oracle(K.untile_codes(bc)), to_oracle(bs), post).astype(np.float64)
     want = A @ B.T
-    got = y[idx.to(dev)].cpu().numpy().astype(np.float64)
+    got = y[idx].cpu().numpy().astype(np.float64)
     rel = np.linalg.norm(got - want) / np.linalg.norm(want)
     assert rel <= 1e-5, rel  # stated tolerance 1e-3
 
 
-def test_linear_step_rows_against_oracle_pipeline(oracle, K, data):
-    """Whole layer at full size: the first 64 token rows of y and of grad_x depend on those rows of x / dy and on W
-    only, so the oracle pipeline on (x[:64], W, dy[:64]) with the same seeds must reproduce them."""
-    print("case fullsize linear fwd+bwd", flush=True)
+@pytest.mark.parametrize("out_features", OUTS)
+def test_linear_step_rows_against_oracle_pipeline(oracle, K, out_features):
+    """Whole layer at full size.  The first 64 token rows of y and of grad_x depend on those rows of x / dy and on W
+    only, and the first 32 rows of grad_W on the first 32 columns of dy and on all of x: the oracle pipeline on those
+    slices with the same seeds must reproduce them (the random streams are keyed by flat offsets, which agree for a
+    prefix of rows)."""
+    print(f"case fullsize linear fwd+bwd out={out_features}", flush=True)
     import random
     import quartet_amd as q
     dev = torch.device("cuda:0")
-    x, dy = data
+    Of = out_features
+    x, dy = _make_data(Of)
     g = torch.Generator().manual_seed(11)
-    w = (0.02 * torch.randn(O, I, generator=g)).to(torch.bfloat16)
-    layer = q.QuantizedLinear(I, O, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(),
+    w = (0.02 * torch.randn(Of, I, generator=g)).to(torch.bfloat16)
+    layer = q.QuantizedLinear(I, Of, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(),
                               activation_quantizer=q.QuestMXFP4Quantizer(),
                               gradient_quantizer=q.AlbertTsengQuantizer(stochastic=True, rerotate=None),
                               backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]()).to(dev, torch.bfloat16)
@@ -170,19 +245,32 @@ def test_linear_step_rows_against_oracle_pipeline(oracle, K, data):
     seeds = [random.getrandbits(63) for _ in range(4)]
     d = float(oracle.FOUR_THIRDS)
     n = 64
-    qx = oracle.quantize(to_oracle(x[:n]), 32, mode=oracle.QUEST_RTN, want_mask=True)
-    qw = oracle.quantize(to_oracle(w), 32, mode=oracle.QUEST_RTN)
-    y_ref = oracle.gemm_tn(qx["codes"], qx["scales"], qw["codes"], qw["scales"])
+    qx = oracle.quantize(to_oracle(x), 32, mode=oracle.QUEST_RTN, want_mask=True)
+    qw = oracle.quantize(to_oracle(w), 32, mode=oracle.QUEST_RTN, want_mask=True)
+    y_ref = oracle.gemm_tn(qx["codes"][:n], qx["scales"][:n], qw["codes"], qw["scales"])
     got = y[:n].detach().float().cpu().numpy().astype(np.float64)
     assert np.linalg.norm(got - y_ref) / np.linalg.norm(y_ref) < 4e-3  # bf16 output rounding
+
+    def bf16_round(a):
+        return to_oracle(torch.from_numpy(a).to(torch.bfloat16))
+
+    def as_f64(bits):
+        return torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16).float().numpy().astype(np.float64)
+    # grad_x: B1, B2, B3, B7
     qe = oracle.quantize(to_oracle(dy[:n]), 32, mode=oracle.ABSMAX_SR, seed=seeds[0])
     qwt = oracle.requantize_transposed(qw["codes"], qw["scales"], val_dtype=oracle.BF16, hd=32, mode=oracle.ABSMAX_SR, seed=seeds[1])
     gxq = oracle.gemm_tn(qe["codes"], qe["scales"], qwt["codes"], qwt["scales"], a_post=d, b_post=d)
-    gxq16 = torch.from_numpy(gxq).to(torch.bfloat16)
-    gx_ref = oracle.masked_hadamard_bwd(to_oracle(gxq16), 32, oracle.BF16, None, qx["mask"])
-    gx_ref = torch.from_numpy(gx_ref.view(np.int16)).view(torch.bfloat16).float().numpy().astype(np.float64)
+    gx_ref = as_f64(oracle.masked_hadamard_bwd(bf16_round(gxq), 32, oracle.BF16, None, qx["mask"][:n]))
     gx = xd.grad[:n].float().cpu().numpy().astype(np.float64)
     assert np.linalg.norm(gx - gx_ref) / np.linalg.norm(gx_ref) < 1e-2  # two bf16 roundings on the way
+    # grad_W: B4, B5, B6, B8 (contraction over all 8192 tokens)
+    m = 32
+    qet = oracle.quantize(to_oracle(dy[:, :m].contiguous()), 32, mode=oracle.ABSMAX_SR, transposed_in=True, seed=seeds[2])
+    qxt = oracle.requantize_transposed(qx["codes"], qx["scales"], val_dtype=oracle.BF16, hd=32, mode=oracle.ABSMAX_SR, seed=seeds[3])
+    gwq = oracle.gemm_tn(qet["codes"], qet["scales"], qxt["codes"], qxt["scales"], a_post=d, b_post=d)
+    gw_ref = as_f64(oracle.masked_hadamard_bwd(bf16_round(gwq), 32, oracle.BF16, None, qw["mask"][:m]))
+    gw = layer.weight.grad[:m].float().cpu().numpy().astype(np.float64)
+    assert np.linalg.norm(gw - gw_ref) / np.linalg.norm(gw_ref) < 1e-2
 
 
 def _signs_from_word(word):

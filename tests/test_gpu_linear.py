@@ -321,3 +321,83 @@ def test_weight_gradient_widened_in_the_kernel(q, T, I, O):
     assert torch.equal(gw2, gw1)
     mask = K.packed_mask_bits(px, T, I)
     assert torch.equal(K.masked_hadamard_bwd(gx2, 32, torch.bfloat16, 0x5A5A5A5A, mask), gx0)
+
+
+@pytest.mark.parametrize("three_d", [False, True])
+@pytest.mark.parametrize("stochastic", [False, True])
+def test_error_only_scheme_against_oracle(oracle, q, three_d, stochastic):
+    """Scheme "Q(E)W_Q(Et)X" (src/models/quantization/backward.py:21-45 of the reference): only the error signal is
+    quantized; grad_x = Q(e) W and grad_W = Q(e^T) x with the saved operands as they are.  Checked against the oracle's
+    de-quantized Q(e), Q(e^T) (same seeds, same accumulated sign flips) multiplied in float64, for a 2-D and a 3-D
+    input."""
+    print(f"case scheme Q(E)W_Q(Et)X three_d={three_d} stochastic={stochastic}", flush=True)
+    dev = "cuda:0"
+    B, S, I, O = 4, 96, 256, 160
+    g_q = q.AlbertTsengQuantizer(stochastic=stochastic, rerotate="signs")
+    torch.manual_seed(5)
+    g_q.re_randomize()   # the scheme itself never re-randomises (the reference's does not either)
+    signs = np.array([-1 if (g_q.sign_bits >> j) & 1 else 1 for j in range(32)])
+    layer = q.QuantizedLinear(I, O, bias=False, gradient_quantizer=g_q,
+                              backward_scheme=q.BACKWARD_SCHEMES["Q(E)W_Q(Et)X"]()).to(dev)
+    assert type(layer.backward_scheme).__name__ == "QEW_QEtX_Scheme" and layer.backward_scheme.g_quantizer is g_q
+    x = make_input(B * S, I, torch.float32, 31, outlier_frac=0.0)
+    dy = make_input(B * S, O, torch.float32, 32, outlier_frac=0.0, scale=1e-3)
+    w = layer.weight.detach().cpu()
+    shape = (B, S) if three_d else (B * S,)
+    xd = x.view(*shape, I).to(dev).requires_grad_(True)
+    y = layer(xd)
+    assert y.shape == (*shape, O)
+    assert rel(y.detach().cpu().view(-1, O), x.double() @ w.double().T) < 1e-5   # identity quantizers in the forward pass
+    random.seed(77)
+    y.backward(dy.view(*shape, O).to(dev))
+    torch.cuda.synchronize()
+    random.seed(77)
+    seeds = [random.getrandbits(63) for _ in range(2)] if stochastic else [0, 0]
+    mode = oracle.ABSMAX_SR if stochastic else oracle.ABSMAX_RTN
+    qe = oracle.quantize(to_oracle(dy), 32, signs=signs, mode=mode, seed=seeds[0], want_dequant=True)
+    qet = oracle.quantize(to_oracle(dy), 32, signs=signs, mode=mode, transposed_in=True, seed=seeds[1], want_dequant=True)
+    gx_ref = qe["dequant"].astype(np.float64) @ w.double().numpy()
+    gw_ref = qet["dequant"].astype(np.float64) @ x.double().numpy()
+    assert xd.grad.shape == xd.shape and layer.weight.grad.shape == (O, I)
+    assert rel(xd.grad.cpu().view(-1, I), gx_ref) < 1e-5
+    assert rel(layer.weight.grad.cpu(), gw_ref) < 1e-5
+    # The MXFP4 quantizers return the tensor in the rotated basis (the reference's kernel never rotates back), so this
+    # scheme multiplies the rotated Q(e) with the unrotated W exactly as the reference does: the product is close to
+    # (e H) W, FP4 noise apart, not to e W.
+    rot = oracle.quantize(to_oracle(dy), 32, signs=signs, mode=oracle.ABSMAX_RTN, want_rotated=True)["rotated"]
+    assert 0.02 < rel(gx_ref, rot.astype(np.float64) @ w.double().numpy()) < 0.3
+
+
+def test_error_only_scheme_under_autocast(oracle, q):
+    """The same scheme the way the training loop runs it: bf16 autocast around forward and backward, so the products are
+    bf16 library GEMMs on the de-quantized bf16 Q(e)."""
+    print("case scheme Q(E)W_Q(Et)X under bf16 autocast", flush=True)
+    dev = "cuda:0"
+    T, I, O = 512, 384, 256
+    layer = q.QuantizedLinear(I, O, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(),
+                              activation_quantizer=q.QuestMXFP4Quantizer(),
+                              gradient_quantizer=q.AlbertTsengQuantizer(stochastic=False),
+                              backward_scheme=q.BACKWARD_SCHEMES["Q(E)W_Q(Et)X"]()).to(dev)
+    x = make_input(T, I, torch.bfloat16, 41, outlier_frac=0.0)
+    dy = make_input(T, O, torch.bfloat16, 42, outlier_frac=0.0, scale=1e-3)
+    xd = x.to(dev).requires_grad_(True)
+    with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+        y = layer(xd)
+        y.backward(dy.to(dev))
+    torch.cuda.synchronize()
+    qx = oracle.quantize(to_oracle(x), 32, mode=oracle.QUEST_RTN, want_mask=True, want_dequant=True)
+    qw = oracle.quantize(to_oracle(layer.weight.detach().cpu()), 32, mode=oracle.QUEST_RTN, want_mask=True, want_dequant=True)
+    qe = oracle.quantize(to_oracle(dy), 32, mode=oracle.ABSMAX_RTN, want_dequant=True)
+    qet = oracle.quantize(to_oracle(dy), 32, mode=oracle.ABSMAX_RTN, transposed_in=True, want_dequant=True)
+    from tests.util import from_oracle_bf16
+    # the scheme multiplies Q(e) with the saved pseudo-quantized operands (bf16 under autocast), then the forward
+    # quantizers' straight-through backward (clip mask + inverse rotation) maps the results to x and W
+    wq = qw["dequant"].astype(np.float64)
+    xq = from_oracle_bf16(qx["dequant"]).double().numpy()
+    eq, etq = from_oracle_bf16(qe["dequant"]).double().numpy(), from_oracle_bf16(qet["dequant"]).double().numpy()
+    gxq = torch.from_numpy(eq @ torch.from_numpy(wq).to(torch.bfloat16).double().numpy()).to(torch.bfloat16)
+    gwq = torch.from_numpy(etq @ xq).to(torch.bfloat16)
+    gx_ref = from_oracle_bf16(oracle.masked_hadamard_bwd(to_oracle(gxq), 32, oracle.BF16, None, qx["mask"])).double().numpy()
+    gw_ref = from_oracle_bf16(oracle.masked_hadamard_bwd(to_oracle(gwq), 32, oracle.BF16, None, qw["mask"])).double().numpy()
+    assert rel(xd.grad.float().cpu(), gx_ref) < 1e-2
+    assert rel(layer.weight.grad.float().cpu(), gw_ref) < 1e-2

@@ -75,6 +75,72 @@ def test_llama30m_quartet_step(models):
     assert min(full.values()) > 0.45 and sum(full.values()) / 24 > 0.55
 
 
+def _full_step(L, cfg, batch, seq, with_adamw):
+    """One whole step of a BASELINE configuration at its real batch: (model, loss, peak allocated GiB)."""
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    with torch.device(dev):   # parameters are drawn on the GPU: the 800 M model takes a while on the host
+        model = L.Llama(cfg)
+    opt = torch.optim.AdamW(model.parameters(), lr=1e-4, fused=True) if with_adamw else None
+    g = torch.Generator().manual_seed(1)
+    idx = torch.randint(0, cfg.vocab_size, (batch, seq), generator=g).to(dev)
+    tgt = torch.randint(0, cfg.vocab_size, (batch, seq), generator=g).to(dev)
+    before = model.transformer.h[0].attn.c_attn.weight.detach().clone()
+    torch.cuda.reset_peak_memory_stats()
+    with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+        loss = model(idx, targets=tgt)["loss"]
+        loss.backward()
+    torch.cuda.synchronize()
+    for name, p in model.named_parameters():
+        assert p.grad is not None and torch.isfinite(p.grad).all(), name
+    for name, m in model.block_linears():
+        assert float(m.weight.grad.float().norm()) > 0.0, name
+    if opt is not None:
+        opt.step()
+        torch.cuda.synchronize()
+        after = model.transformer.h[0].attn.c_attn.weight
+        assert torch.isfinite(after).all() and not torch.equal(after, before)
+        assert all(st["exp_avg"].dtype == torch.float32 for st in opt.state.values())
+    peak = torch.cuda.max_memory_allocated() / 2 ** 30
+    return model, float(loss.detach()), peak
+
+
+def test_llama30m_step_at_full_batch(models):
+    """The 30 M configuration at its real batch, 64 x 512 tokens: closed-form parameter count, loss at initialisation,
+    finite non-zero gradients in all 24 quantized linears."""
+    L = models[0]
+    print("case llama30m quartet fwd+bwd 64x512", flush=True)
+    cfg = L.llama_30m()
+    model, loss, peak = _full_step(L, cfg, 64, 512, with_adamw=False)
+    linears = 6 * (640 * 1920 + 640 * 640 + 640 * 3456 + 1728 * 640)
+    assert sum(m.weight.numel() for _, m in model.block_linears()) == linears == 29_736_960
+    assert model.get_num_params() == linears + 2 * 32000 * 640 + 13 * 640
+    assert len(model.block_linears()) == 24
+    assert abs(loss - (math.log(32000) + 640 * 0.02 ** 2 / 2)) < 0.1, loss
+    print(f"llama30m 64x512: loss {loss:.4f}, peak {peak:.2f} GiB", flush=True)
+
+
+def test_llama800m_step_with_adamw(models):
+    """The ~800 M configuration: 24 layers, d 1536, 12 heads, SwiGLU width 4096, 16 x 2048 tokens, AdamW with fp32
+    state.  Closed-form parameter count, loss at initialisation (ln V plus half the logit variance d * 0.02^2), finite
+    non-zero gradients in all 96 quantized linears, an optimizer step that moves the weights, peak memory."""
+    L = models[0]
+    print("case llama800m quartet fwd+bwd+AdamW 16x2048", flush=True)
+    cfg = L.llama_800m()
+    assert (cfg.n_layer, cfg.n_embd, cfg.n_head, cfg.ffn_dim, cfg.vocab_size) == (24, 1536, 12, 4096, 32000)
+    model, loss, peak = _full_step(L, cfg, 16, 2048, with_adamw=True)
+    linears = 24 * (1536 * 4608 + 1536 * 1536 + 1536 * 8192 + 4096 * 1536)
+    assert sum(m.weight.numel() for _, m in model.block_linears()) == linears == 679_477_248
+    assert model.get_num_params() == linears + 2 * 32000 * 1536 + 49 * 1536
+    assert len(model.block_linears()) == 96
+    assert abs(loss - (math.log(32000) + 1536 * 0.02 ** 2 / 2)) < 0.1, loss
+    # weights + gradients + two fp32 moments are 16 B per parameter = 11.6 GiB; packed activations keep the rest small
+    print(f"llama800m 16x2048: loss {loss:.4f}, peak {peak:.2f} GiB", flush=True)
+    assert peak < 80.0, peak
+    del model
+    torch.cuda.empty_cache()
+
+
 def test_llama_ragged_batch_shapes(models):
     # 4 x 40 tokens = 160 rows: a multiple of the Hadamard block but not of the 128-row tiles of the transposing kernels
     L, quartet, bwd_only, plain, idx, tgt = models
