@@ -16,16 +16,18 @@ import time
 
 import torch
 
-T_TOKENS, IN_F, OUT_F = 8192, 4096, 4096
+T_TOKENS, IN_F, OUT_F = 8192, 4096, 4096   # OUT_F: default of --out-features (the configuration's other value is 11008)
 PEAK_FP4_TFLOPS = 10100.0   # MI355X dense MXFP4 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
-# HBM bytes per launch from profiler byte counters (fetch + write), scaled by what the same counters read for a
-# plain 256 MiB device copy (fetch counter x 2.0 KiB, write counter x 1.0 KiB)
-GEMM_TRAFFIC_BYTES = 173.9e6      # mean of the three GEMMs: 108.7 MiB fetched (operand re-reads that miss L2) + 57.1 MiB written
-QUANTIZE_TRAFFIC_BYTES = 90.3e6   # two thirds (the X share) of the forward pair launch: 96.1 MiB fetched + 33.0 MiB written; algorithmic 89.1e6
+ROOT = os.path.dirname(os.path.abspath(__file__))
+# HBM bytes per launch come from profiler byte counters (two rocprofv3 --pmc runs of this script, FETCH_SIZE then
+# WRITE_SIZE, scaled by what the same counters read for a plain 256 MiB device copy).  `--counters-to-json` turns the
+# two runs' CSV files into this tracked file, which also records the commit and a hash of the kernel sources it was
+# taken at; the roofline entries quote it together with whether it still matches the sources of this build.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 
 
-def make_inputs(device, tokens=T_TOKENS, seed=0):
+def make_inputs(device, tokens=T_TOKENS, seed=0, out_f=OUT_F):
     """X ~ N(0,1) with 1% Student-t(3) entries, W ~ N(0, 0.02), dY ~ N(0, 1e-3); generated on the CPU
     with a seeded generator so the CPU baseline and the GPU see identical bits."""
     g = torch.Generator().manual_seed(seed)
@@ -33,15 +35,15 @@ def make_inputs(device, tokens=T_TOKENS, seed=0):
     heavy = torch.rand(tokens, IN_F, generator=g) < 0.01
     chi2 = (torch.randn(3, tokens, IN_F, generator=g) ** 2).sum(0)
     x = torch.where(heavy, torch.randn(tokens, IN_F, generator=g) / torch.sqrt(chi2 / 3.0), x)
-    w = 0.02 * torch.randn(OUT_F, IN_F, generator=g)
-    dy = 1e-3 * torch.randn(tokens, OUT_F, generator=g)
+    w = 0.02 * torch.randn(out_f, IN_F, generator=g)
+    dy = 1e-3 * torch.randn(tokens, out_f, generator=g)
     return x.to(torch.bfloat16).to(device), w.to(torch.bfloat16).to(device), dy.to(torch.bfloat16).to(device)
 
 
-def build_layer(device):
+def build_layer(device, out_f=OUT_F):
     import quartet_amd as q
     layer = q.QuantizedLinear(
-        IN_F, OUT_F, bias=False,
+        IN_F, out_f, bias=False,
         weight_quantizer=q.QUANTIZER_CLASSES["QuestMXFP4Quantizer"](hadamard_dim=32),
         activation_quantizer=q.QUANTIZER_CLASSES["QuestMXFP4Quantizer"](hadamard_dim=32),
         gradient_quantizer=q.QUANTIZER_CLASSES["AlbertTsengQuantizer"](hadamard_dim=32, stochastic=True, rerotate="signs"),
@@ -100,7 +102,7 @@ def time_kernel_cold(make_call, inputs, reps=24, warmup=2):
     return time_kernel(fn, reps=max(reps, n), warmup=warmup)
 
 
-def kernel_breakdown(x, w, dy):
+def kernel_breakdown(x, w, dy, only_gemms=False):
     """Per-kernel timings of the eleven launches of one step, with algorithmic bytes / flops.  HBM-bound kernels
     are timed HBM-cold (see time_kernel_cold) and, for reference, warm on one buffer."""
     from quartet_amd import kernels as K
@@ -127,6 +129,11 @@ def kernel_breakdown(x, w, dy):
         ms = time_kernel(fn)
         out[name] = {"ms": round(ms, 4), "TFLOPs": round(2.0 * m * n * k / ms / 1e9, 1), "shape": [m, n, k]}
 
+    if only_gemms:
+        mfma("gemm_fwd", T, O, I, lambda: K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
+        mfma("gemm_dgrad", T, I, O, lambda: K.gemm_mxfp4_tn(ec, es, wtc, wts, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
+        mfma("gemm_wgrad", O, I, T, lambda: K.gemm_mxfp4_tn(etc, ets, xtc, xts, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
+        return out
     hbm("quantize_x_quest_rtn_mask", T * I, 2.65625,
         lambda a: (lambda: K.quantize_mxfp4(a, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)), [x])
     hbm("quantize_w_quest_rtn_mask", O * I, 2.65625,
@@ -207,7 +214,7 @@ def _cpu_model():
     return "unknown"
 
 
-def cpu_baseline(sample_tokens=T_TOKENS):
+def cpu_baseline(sample_tokens=T_TOKENS, out_f=OUT_F):
     """The CPU restatement of the same pseudo-quantized linear (oracle quantizers + fp32 BLAS matmuls on
     de-quantized operands, i.e. the op sequence the reference runs) on a row sample of the workload."""
     import numpy as np
@@ -215,7 +222,7 @@ def cpu_baseline(sample_tokens=T_TOKENS):
     from tests.util import to_oracle
     threads = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(threads)
-    x, w, dy = make_inputs("cpu", tokens=sample_tokens)
+    x, w, dy = make_inputs("cpu", tokens=sample_tokens, out_f=out_f)
     xo, wo, eo = to_oracle(x), to_oracle(w), to_oracle(dy)
     o.lib()
     d = float(o.FOUR_THIRDS)
@@ -243,10 +250,10 @@ def cpu_baseline(sample_tokens=T_TOKENS):
         dt, y, gx, gw = one_pass()
         times.append(dt)
     dt = sorted(times)[1]
-    assert y.shape[0] == sample_tokens and gx.shape == (sample_tokens, IN_F) and gw.shape == (OUT_F, IN_F)
-    flops = 6.0 * sample_tokens * IN_F * OUT_F
+    assert y.shape[0] == sample_tokens and gx.shape == (sample_tokens, IN_F) and gw.shape == (out_f, IN_F)
+    flops = 6.0 * sample_tokens * IN_F * out_f
     return {"value": round(flops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"fwd+bwd on {sample_tokens} of {T_TOKENS} tokens (same I={IN_F}, O={OUT_F}), median of 3 passes; "
+            "sample": f"fwd+bwd on {sample_tokens} of {T_TOKENS} tokens (same I={IN_F}, O={out_f}), median of 3 passes; "
                       f"CPU oracle quantizers + fp32 BLAS matmuls on de-quantized operands, {dt:.2f} s per pass",
             "cpu_model": _cpu_model()}
 
@@ -342,13 +349,189 @@ def llama_step(args, device):
             "peak_allocated_GiB": round(peak_gib, 2)}
 
 
+def _csrc_sha16():
+    """Hash of the kernel sources this build was made from (the traffic profile records the same hash)."""
+    import hashlib
+    d = os.path.join(ROOT, "quartet_amd", "csrc")
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(d)):
+        if name.endswith((".hip", ".h")):
+            with open(os.path.join(d, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
+
+
+def traffic_profile():
+    """The tracked byte-counter profile, or None.  `current` says whether the kernel sources are still the ones it
+    was measured on."""
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            prof = json.load(f)
+    except (OSError, ValueError):
+        return None
+    prof["current"] = prof.get("csrc_sha16") == _csrc_sha16()
+    return prof
+
+
+def _traffic_entry(prof, key):
+    if prof is None or key not in prof.get("kernels", {}):
+        return None, {"file": None}
+    k = prof["kernels"][key]
+    return float(k["fetch_bytes"] + k["write_bytes"]), {"file": "profiles/hbm_traffic.json", "head": prof.get("head"),
+                                                         "matches_this_build": prof["current"],
+                                                         "fetch_bytes": k["fetch_bytes"], "write_bytes": k["write_bytes"]}
+
+
+def counters_to_json(fetch_dir, write_dir):
+    """Turn the CSV output of the two byte-counter runs
+
+        rocprofv3 --pmc FETCH_SIZE -d <fetch_dir> -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-extra --calibration-copy
+        rocprofv3 --pmc WRITE_SIZE -d <write_dir> -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-extra --calibration-copy
+
+    into profiles/hbm_traffic.json.  The calibration copy (the largest copyBuffer dispatch: 256 MiB read, 256 MiB
+    written) fixes how many bytes one counter unit stands for."""
+    import collections
+    import csv
+    import glob
+    import re
+    import subprocess
+
+    def read(d):
+        files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
+        if not files:
+            sys.exit(f"no *counter_collection.csv under {d}")
+        agg = collections.defaultdict(list)
+        for r in csv.DictReader(open(files[0])):
+            agg[re.sub(r"\(anonymous namespace\)::", "", r["Kernel_Name"])].append(float(r["Counter_Value"]))
+        return agg
+    fetch, write = read(fetch_dir), read(write_dir)
+    copy_bytes = 256 << 20
+
+    def unit(agg):
+        copies = [v for k, vs in agg.items() if "copyBuffer" in k for v in vs]
+        return copy_bytes / max(copies)
+    fu, wu = unit(fetch), unit(write)
+    groups = {"gemm_mxfp4_tn": lambda k: "gemm_mxfp4_tn" in k and "splitk" not in k,
+              "quantize_x_quest_rtn_mask_alone": lambda k: k.startswith("void qm::job_kernel<qm::RowmajorTiledJob") or k.startswith("qm::job_kernel<qm::RowmajorTiledJob"),
+              "forward_quantizer_pair": lambda k: "job_pair_kernel<qm::RowmajorTiledJob" in k,
+              "gradient_quantizer_pair": lambda k: "job_pair_kernel<qm::TransposedJob" in k,
+              "requantizer_pair": lambda k: "job_pair_kernel<qm::RequantJob" in k,
+              "inverse_rotation_pair": lambda k: "job_pair_kernel<qm::HadamardBwdJob" in k}
+    out = {}
+    for name, match in groups.items():
+        f = [v for k, vs in fetch.items() if match(k) for v in vs]
+        w = [v for k, vs in write.items() if match(k) for v in vs]
+        if f and w:
+            out[name] = {"fetch_bytes": round(sum(f) / len(f) * fu), "write_bytes": round(sum(w) / len(w) * wu), "dispatches": len(f)}
+    head = subprocess.run(["git", "-C", ROOT, "rev-parse", "HEAD"], capture_output=True, text=True).stdout.strip()
+    dirty = subprocess.run(["git", "-C", ROOT, "status", "--porcelain", "--", "quartet_amd/csrc"], capture_output=True, text=True).stdout.strip()
+    prof = {"what": "HBM-side bytes per launch (mean over the dispatches of a 2-step run) of the isolated linear, tokens 8192 x in 4096 x out 4096",
+            "head": head + (" + uncommitted kernel changes" if dirty else ""), "csrc_sha16": _csrc_sha16(),
+            "calibration": {"copy_bytes": copy_bytes, "bytes_per_fetch_unit": round(fu, 2), "bytes_per_write_unit": round(wu, 2)},
+            "commands": ["rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof_fetch -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-extra --calibration-copy",
+                         "rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof_write -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-extra --calibration-copy",
+                         "python3 bench.py --counters-to-json gpurun_out/prof_fetch gpurun_out/prof_write"],
+            "kernels": out}
+    with open(TRAFFIC_PROFILE, "w") as f:
+        json.dump(prof, f, indent=1)
+        f.write("\n")
+    print(json.dumps(prof, indent=1))
+
+
+def time_layer_steps(step, steps, warmup, sustain_s=1.0):
+    """(ms per step over exactly `steps` steps, sustained statistics).  The first figure is the contract's: warm-up, then
+    `steps` steps between two synchronisations.  The block is then repeated until `sustain_s` seconds have been spent
+    inside timed blocks: the GEMMs run against the chip's power limit, and a window of a few milliseconds after an idle
+    period says little about the clock it holds over seconds."""
+    for _ in range(warmup):
+        step()
+    blocks = []
+    total = 0.0
+    while not blocks or total < sustain_s:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        blocks.append(dt / steps * 1e3)
+        total += dt
+    srt = sorted(blocks)
+    return blocks[0], {"blocks": len(blocks), "steps_per_block": steps, "seconds": round(total, 3),
+                       "ms_per_step_median": round(srt[len(srt) // 2], 4), "ms_per_step_min": round(srt[0], 4),
+                       "ms_per_step_max": round(srt[-1], 4)}
+
+
+def make_step(layer, x, dy):
+    def step():
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            y = layer(x)
+        y.backward(dy)
+        x.grad = None
+        layer.weight.grad = None
+    return step
+
+
+def gemm_summary(kb, tokens, out_f):
+    gemms = [kb[k] for k in ("gemm_fwd", "gemm_dgrad", "gemm_wgrad")]
+    ms = sum(g["ms"] for g in gemms) / 3.0
+    return ms, 2.0 * tokens * IN_F * out_f / ms / 1e9
+
+
+def out11008_block(device, args):
+    """The configuration's second out-feature count: layer step and the three products (8192x11008x4096,
+    8192x4096x11008, 11008x4096x8192), same method as the main figures."""
+    out_f = 11008
+    x, w, dy = make_inputs(device, out_f=out_f)
+    layer = build_layer(device, out_f)
+    with torch.no_grad():
+        layer.weight.copy_(w)
+    x.requires_grad_(True)
+    ms, sustained = time_layer_steps(make_step(layer, x, dy), args.steps, args.warmup, sustain_s=0.5)
+    flops = 6.0 * T_TOKENS * IN_F * out_f
+    x.requires_grad_(False)
+    kb = kernel_breakdown(x.detach(), w, dy, only_gemms=True)
+    gemm_ms, gemm_tf = gemm_summary(kb, T_TOKENS, out_f)
+    return {"workload": f"isolated Quartet linear, tokens {T_TOKENS} x in {IN_F} x out {out_f}", "ms_per_step": round(ms, 4),
+            "TFLOPs": round(flops / ms / 1e9, 1), "sustained": sustained, "gemms": kb,
+            "gemm_mean": {"ms": round(gemm_ms, 4), "TFLOPs": round(gemm_tf, 1), "frac_of_peak": round(gemm_tf / PEAK_FP4_TFLOPS, 4)}}
+
+
+def quantizer_sizes_block(device):
+    """Quantizer-only configuration in brief: for each tensor size, the slowest and fastest of the nine (mode x Hadamard
+    block) cells, HBM-cold."""
+    from quartet_amd import kernels as K
+    out = {}
+    for rows in (4096, 16384, 65536):
+        gd = torch.Generator(device=device).manual_seed(rows)
+        x = torch.randn(rows, 4096, generator=gd, device=device)
+        spike = torch.rand(rows, 4096, generator=gd, device=device) < 1e-3
+        x = torch.where(spike, torch.where(torch.rand(rows, 4096, generator=gd, device=device) < 0.5, -1e3, 1e3), x).to(torch.bfloat16)
+        cells = []
+        for hd in (32, 64, 128):
+            for name, mode, mask, bpe in (("quest_rtn_mask", K.QM_QUEST_RTN, True, 2.65625), ("absmax_rtn", K.QM_ABSMAX_RTN, False, 2.53125),
+                                          ("absmax_sr", K.QM_ABSMAX_SR, False, 2.53125)):
+                ms = time_kernel_cold(lambda a: (lambda: K.quantize_mxfp4(a, hd, None, mode, want_mask=mask, seed=7)), [x], reps=8, warmup=1)
+                cells.append((rows * 4096 * bpe / ms / 1e6, f"hd{hd}_{name}"))
+        cells.sort()
+        out[f"{rows}x4096"] = {"worst": {"cell": cells[0][1], "GBps": round(cells[0][0], 1)},
+                               "best": {"cell": cells[-1][1], "GBps": round(cells[-1][0], 1)},
+                               "median_GBps": round(cells[len(cells) // 2][0], 1)}
+        del x
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--out-features", type=int, default=OUT_F,
+                    help="out features of the isolated layer: 4096 (default, the shape the metric is quoted on) or 11008")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the brief out=11008 and quantizer-size blocks the default run appends")
     ap.add_argument("--workload", default="linear", choices=["linear", "llama30m", "llama800m"],
                     help="linear (default): the isolated 8192x4096x4096 layer the metric is quoted on; llama30m / llama800m: "
                          "whole-model fwd+bwd(+AdamW) step of the 30 M / ~800 M Llama configurations, reported in the same unit "
@@ -358,7 +541,10 @@ def main():
     ap.add_argument("--sdpa", default="auto", choices=["auto", "default"],
                     help="llama workloads: library attention kernels tried in the model's own order (auto) or the dispatcher's (default)")
     ap.add_argument("--calibration-copy", action="store_true",
-                    help="also run one plain 256 MiB device copy (a known-traffic kernel for scaling profiler byte counters)")
+                    help="also run one plain 256 MiB device copy (a known-traffic kernel for scaling profiler byte counters) and one "
+                         "forward quantizer launch on its own")
+    ap.add_argument("--counters-to-json", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="no GPU work: summarise the CSV output of the two byte-counter runs into profiles/hbm_traffic.json")
     ap.add_argument("--quantizer-sweep", action="store_true",
                     help="also time the quantizer alone on [rows x 4096] for rows 4096/16384/65536, three modes, hd 32/64/128")
     ap.add_argument("--gemm-operand-content", action="store_true",
@@ -366,71 +552,68 @@ def main():
     ap.add_argument("--library-gemm", action="store_true",
                     help="also time the vendor library's MXFP4 product (torch._scaled_mm) on the forward GEMM's shape, for context")
     args = ap.parse_args()
+    if args.counters_to_json:
+        counters_to_json(*args.counters_to_json)
+        return
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)")
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU: the quantized-linear path has no CPU fallback")
-    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    sys.path.insert(0, ROOT)
     device = torch.device("cuda:0")
     if args.workload != "linear":
         print(json.dumps(llama_step(args, device)))
         return
-    x, w, dy = make_inputs(device)
-    layer = build_layer(device)
+    out_f = args.out_features
+    x, w, dy = make_inputs(device, out_f=out_f)
+    layer = build_layer(device, out_f)
     with torch.no_grad():
         layer.weight.copy_(w)
     x.requires_grad_(True)
-
-    def step():
-        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
-            y = layer(x)
-        y.backward(dy)
-        x.grad = None
-        layer.weight.grad = None
-
     if args.calibration_copy:
+        from quartet_amd import kernels as K
         src = torch.empty(256 << 20, dtype=torch.uint8, device=device).fill_(1)
         dst = torch.empty_like(src)
         dst.copy_(src)
+        K.quantize_mxfp4(x.detach(), 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=True)
         torch.cuda.synchronize()
         del src, dst
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
-    flops = 6.0 * T_TOKENS * IN_F * OUT_F
+    ms_per_step, sustained = time_layer_steps(make_step(layer, x, dy), args.steps, args.warmup,
+                                              sustain_s=0.0 if args.calibration_copy else 1.0)
+    flops = 6.0 * T_TOKENS * IN_F * out_f
     result = {
         "metric": "Quartet linear fwd+bwd TFLOPS (MXFP4 MFMA) + Hadamard/quantize HBM GB/s",
         "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "mxfp4", "data": "synthetic",
-        "config": {"workload": "isolated Quartet linear fwd+dgrad+wgrad, tokens 8192 x in 4096 x out 4096, "
+        "config": {"workload": f"isolated Quartet linear fwd+dgrad+wgrad, tokens {T_TOKENS} x in {IN_F} x out {out_f}, "
                                "bf16 X/W/dY, quest-RTN forward, absmax-SR backward, Hadamard 32"},
+        "sustained": {**sustained, "TFLOPs_median": round(flops / sustained["ms_per_step_median"] / 1e9, 1)},
     }
+    prof = traffic_profile() if out_f == OUT_F else None
     if not args.no_breakdown:
         x.requires_grad_(False)
         kb = kernel_breakdown(x.detach(), w, dy)
         result["kernels"] = kb
         # the three GEMMs of a step (fwd, dgrad, wgrad) run the same kernel on the same flop count: the roofline
         # entry is their mean, which is what a profiler's per-kernel average over the run reports
-        gemms = [kb[k] for k in ("gemm_fwd", "gemm_dgrad", "gemm_wgrad")]
-        gemm_ms = sum(g["ms"] for g in gemms) / 3.0
-        gemm_tf = 2.0 * T_TOKENS * IN_F * OUT_F / gemm_ms / 1e9
-        result["roofline"] = {"bound": "mfma", "kernel": "gemm_mxfp4_tn_big4_kernel (8192x4096x4096, 8192x4096x4096, 4096x4096x8192)",
+        gemm_ms, gemm_tf = gemm_summary(kb, T_TOKENS, out_f)
+        traffic, source = _traffic_entry(prof, "gemm_mxfp4_tn")
+        result["roofline"] = {"bound": "mfma", "kernel": f"gemm_mxfp4_tn ({T_TOKENS}x{out_f}x{IN_F}, {T_TOKENS}x{IN_F}x{out_f}, {out_f}x{IN_F}x{T_TOKENS})",
                               "achieved": round(gemm_tf, 1), "peak": PEAK_FP4_TFLOPS, "unit": "TFLOP/s",
-                              "frac": round(gemm_tf / PEAK_FP4_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
+                              "frac": round(gemm_tf / PEAK_FP4_TFLOPS, 4), "traffic": traffic, "traffic_source": source,
                               "avg_launch_ms": round(gemm_ms, 4)}
         qk = kb["quantize_x_quest_rtn_mask"]
-        result["roofline_quantize"] = {"bound": "hbm", "kernel": "quantize_rowmajor (quest RTN + mask, 8192x4096 bf16)",
+        traffic, source = _traffic_entry(prof, "quantize_x_quest_rtn_mask_alone")
+        result["roofline_quantize"] = {"bound": "hbm", "kernel": f"quantize_rowmajor (quest RTN + mask, {T_TOKENS}x{IN_F} bf16)",
                                        "achieved": qk["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                       "frac": round(qk["GBps"] / PEAK_HBM_GBS, 4), "traffic": QUANTIZE_TRAFFIC_BYTES,
+                                       "frac": round(qk["GBps"] / PEAK_HBM_GBS, 4), "traffic": traffic, "traffic_source": source,
                                        "avg_launch_ms": qk["ms"]}
+    if not args.no_extra and not args.no_breakdown and out_f == OUT_F:
+        del layer
+        result["out11008"] = out11008_block(device, args)
+        result["quantizer_sizes"] = quantizer_sizes_block(device)
     if args.quantizer_sweep:
         result["quantizer_sweep"] = quantizer_sweep(device)
     if args.library_gemm:
@@ -438,7 +621,7 @@ def main():
     if args.gemm_operand_content:
         result["gemm_operand_content"] = gemm_operand_content(x.detach(), w, dy)
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline()
+        result["cpu_baseline"] = cpu_baseline(out_f=out_f)
     print(json.dumps(result))
 
 
