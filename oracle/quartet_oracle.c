@@ -98,19 +98,23 @@ void qo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out
  * Uniform for the element at flat offset o of the tensor being quantized (the role of
  * tl.rand(seed, offsets), mxfp4_triton.py:124).  One Philox4x32-10 call serves sixteen
  * consecutive elements: counter = (o/16 low, o/16 high, 0, 0), key = (seed low, seed high);
- * element o takes the 8 bits r8 = byte (o%4) of word (o%16)/4 -- 8 random bits per element,
- * as hardware FP4 stochastic-rounding converts consume.  The uniform is the largest float
- * below (r8 + 1/2) / 256 + 2^-22, so that "u < p" holds exactly when
- * floor(p * 2^22) > r8 * 2^14 + 2^13: a comparison at 22 fractional bits, which is what
- * gfx950's stochastic-rounding convert evaluates, centred in the r8-th of 256 equal bins.
+ * element o takes 16 random bits r16: byte (o%4) of word (o%16)/4 as the high half and the next byte
+ * of the same word (byte (o+1)%4) as the low half.  Every element's r16 is uniform over 65536
+ * values; neighbours inside a word share one byte, which correlates their rounding decisions by
+ * less than 2^-8.  The uniform is the largest float below (r16 + 1/2) / 65536 + 2^-22, so that
+ * "u < p" holds exactly when floor(p * 2^22) > r16 * 2^6 + 2^5: a comparison at 22 fractional
+ * bits, which is what gfx950's stochastic-rounding convert evaluates, centred in the r16-th of
+ * 65536 equal bins.  E[round up] differs from p by at most 2^-17 (mxfp4_triton.py:124 draws a
+ * 24-bit uniform).
  */
 float qo_philox_uniform16(uint64_t seed, uint64_t o) {
     uint32_t ctr[4] = {(uint32_t)(o >> 4), (uint32_t)((o >> 4) >> 32), 0u, 0u};
     uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
     uint32_t w[4];
     qo_philox4x32_10(ctr, key, w);
-    uint32_t r8 = (w[(o & 15) >> 2] >> (8 * (o & 3))) & 0xffu;
-    float bound = (float)(16384u * r8 + 8193u) * (1.0f / 4194304.0f); /* exact: 22 significant bits */
+    uint32_t word = w[(o & 15) >> 2];
+    uint32_t r16 = (((word >> (8 * (o & 3))) & 0xffu) << 8) | ((word >> (8 * ((o + 1) & 3))) & 0xffu);
+    float bound = (float)(64u * r16 + 33u) * (1.0f / 4194304.0f); /* exact: 22 significant bits */
     return bits_to_f32(f32_to_bits(bound) - 1u);
 }
 

@@ -150,13 +150,17 @@ QM_HD Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, 
     return o;
 }
 // Random bits of element `o` (flat offset in the tensor being quantized): one Philox call per sixteen
-// consecutive elements, counter = o/16; element j of the sixteen takes byte j%4 of word j/4 (8 random bits
-// per element, as hardware FP4 stochastic-rounding converts consume).  Its uniform is the largest float
-// below (r8 * 2^14 + 2^13 + 1) * 2^-22: "u < p" is then exactly the 22-bit comparison
-// floor(p * 2^22) > r8 * 2^14 + 2^13 that the hardware convert performs, centred in the r8-th of 256 bins.
-QM_HD uint32_t philox_r8(const Philox4& p, int j) { return (p.w[j >> 2] >> (8 * (j & 3))) & 0xffu; }
-QM_HD float uniform_from_r8(uint32_t r8) {
-    return u2f(f2u((float)(16384u * r8 + 8193u) * (1.0f / 4194304.0f)) - 1u);
+// consecutive elements, counter = o/16; element j of the sixteen takes byte j%4 of word j/4 as the high half
+// and byte (j+1)%4 of the same word as the low half of its 16 random bits (uniform over 65536 values per
+// element; neighbours inside a word share one byte).  Its uniform is the largest float below
+// (r16 * 2^6 + 2^5 + 1) * 2^-22: "u < p" is then exactly the 22-bit comparison
+// floor(p * 2^22) > r16 * 2^6 + 2^5 that the hardware convert performs, centred in the r16-th of 65536 bins.
+QM_HD uint32_t philox_r16(const Philox4& p, int j) {
+    const uint32_t w = p.w[j >> 2];
+    return (((w >> (8 * (j & 3))) & 0xffu) << 8) | ((w >> (8 * ((j + 1) & 3))) & 0xffu);
+}
+QM_HD float uniform_from_r16(uint32_t r16) {
+    return u2f(f2u((float)(64u * r16 + 33u) * (1.0f / 4194304.0f)) - 1u);
 }
 QM_HD Philox4 philox_for_hexadecad(uint64_t seed, uint64_t block16) {
     return philox4x32_10((uint32_t)block16, (uint32_t)(block16 >> 32), 0u, 0u, (uint32_t)seed, (uint32_t)(seed >> 32));

@@ -77,16 +77,25 @@ int main() {
     }
     if (rtn_code(1e9f) != 7 || sr_code(7.5f, 0.f) != 7) fail("saturation", 0);
 
-    // the uniform of a random byte turns "u < p" into the integer comparison floor(p 2^22) > r8 2^14 + 2^13
-    for (uint32_t r8 = 0; r8 < 256; ++r8) {
-        const float u = uniform_from_r8(r8);
-        const uint32_t R = r8 * 16384u + 8192u;
+    // the uniform of 16 random bits turns "u < p" into the integer comparison floor(p 2^22) > r16 2^6 + 2^5
+    for (uint32_t r16 = 0; r16 < 65536; ++r16) {
+        const float u = uniform_from_r16(r16);
+        const uint32_t R = r16 * 64u + 32u;
         for (int d = -2; d <= 2; ++d) {
             const uint32_t k = R + (uint32_t)d;  // p = k 2^-22, exact in fp32
             const float p = (float)k * (1.0f / 4194304.0f);
-            if ((u < p) != (k > R)) fail("uniform_from_r8", r8);
+            if ((u < p) != (k > R)) fail("uniform_from_r16", r16);
             const float p_half = ((float)k + 0.5f) * (1.0f / 4194304.0f);  // p with bits below 2^-22
-            if ((u < p_half) != (k > R)) fail("uniform_from_r8 (sub-grid p)", r8);
+            if ((u < p_half) != (k > R)) fail("uniform_from_r16 (sub-grid p)", r16);
+        }
+    }
+    // an element's 16 bits: its own byte of the word above the next byte of the same word
+    {
+        Philox4 ph;
+        ph.w[0] = 0x04030201u; ph.w[1] = 0x08070605u; ph.w[2] = 0x0c0b0a09u; ph.w[3] = 0x100f0e0du;
+        for (int j = 0; j < 16; ++j) {
+            const uint32_t own = (uint32_t)j + 1u, next = (uint32_t)((j & ~3) + ((j + 1) & 3)) + 1u;
+            if (philox_r16(ph, j) != ((own << 8) | next)) fail("philox_r16", (uint32_t)j);
         }
     }
 

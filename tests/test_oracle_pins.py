@@ -147,7 +147,8 @@ def test_philox_known_answer_vectors(oracle):
 
 
 def test_philox_uniform16_mapping(oracle):
-    # u(r8) = largest float below (r8 * 2^14 + 2^13 + 1) / 2^22, r8 = bytes of Philox words, 16 elements per call
+    # u(r16) = largest float below (r16 * 2^6 + 2^5 + 1) / 2^22; r16 = a byte of a Philox word above the next byte of
+    # the same word; 16 elements per call
     seed = 0x1234_5678_9ABC
     u = oracle.philox_uniform16(seed, 64)
     for blk in range(4):
@@ -155,24 +156,64 @@ def test_philox_uniform16_mapping(oracle):
         want = []
         for word in w.tolist():
             for b in range(4):
-                r8 = (word >> (8 * b)) & 0xFF
-                bound = np.float32((16384 * r8 + 8193) / 4194304.0)
-                assert float(bound) == (16384 * r8 + 8193) / 4194304.0  # exactly representable
+                r16 = (((word >> (8 * b)) & 0xFF) << 8) | ((word >> (8 * ((b + 1) % 4))) & 0xFF)
+                bound = np.float32((64 * r16 + 33) / 4194304.0)
+                assert float(bound) == (64 * r16 + 33) / 4194304.0  # exactly representable
                 want.append(float(np.nextafter(bound, np.float32(0))))
         assert u[16 * blk:16 * blk + 16].tolist() == want
+    off = np.array([[5, 1 << 20], [(1 << 33) + 7, 63]], dtype=np.int64)
+    at = oracle.philox_uniform16_at(seed, off)
+    assert at.shape == off.shape and at[0, 0] == u[5] and at[1, 1] == u[63]
+    w = oracle.philox4x32_10([((1 << 33) + 7) >> 4 & 0xFFFFFFFF, ((1 << 33) + 7) >> 36, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
+    word = int(w[1])   # element 7 of its call: word 1, byte 3 above byte 0
+    r16 = ((word >> 24) << 8) | (word & 0xFF)
+    assert at[1, 0] == np.nextafter(np.float32((64 * r16 + 33) / 4194304.0), np.float32(0))
     big = oracle.philox_uniform16(7, 1 << 16)
     assert 0 <= big.min() and big.max() < 1 and abs(big.mean() - 0.5) < 5e-3
-    # "u < p" is the 22-bit comparison "floor(p * 2^22) > r8 * 2^14 + 2^13" for every float p in [0, 1]
+    # "u < p" is the 22-bit comparison "floor(p * 2^22) > r16 * 2^6 + 2^5" for every float p in [0, 1]
     rng = np.random.default_rng(0)
-    r8 = rng.integers(0, 256, 20000)
-    bound = ((16384 * r8 + 8193) / 4194304.0).astype(np.float32)
+    r16 = rng.integers(0, 65536, 20000)
+    bound = ((64 * r16 + 33) / 4194304.0).astype(np.float32)
     uu = np.nextafter(bound, np.float32(0))
     p = np.concatenate([rng.random(10000, dtype=np.float32), bound[:5000], uu[:2500], np.nextafter(bound[:2500], np.float32(2))])
-    assert np.array_equal(uu < p, np.floor(p.astype(np.float64) * 4194304.0) > 16384 * r8 + 8192)
-    # centred bins: averaged over r8 the round-up probability of p is p to within 2^-9
-    for pv in (0.1, 0.37, 0.5, 0.93):
-        allu = np.nextafter(((16384 * np.arange(256) + 8193) / 4194304.0).astype(np.float32), np.float32(0))
-        assert abs(np.mean(allu < np.float32(pv)) - pv) <= 1 / 512 + 1e-9
+    assert np.array_equal(uu < p, np.floor(p.astype(np.float64) * 4194304.0) > 64 * r16 + 32)
+    # centred bins: averaged over r16 the round-up probability of p is p to within 2^-17, also for p below 1/512
+    allu = np.nextafter(((64 * np.arange(65536) + 33) / 4194304.0).astype(np.float32), np.float32(0))
+    for pv in (1e-4, 1 / 700, 0.1, 0.37, 0.5, 0.93, 1 - 1e-4):
+        assert abs(np.mean(allu < np.float32(pv)) - float(np.float32(pv))) <= 2.0 ** -17 + 1e-12
+
+
+def test_stochastic_rounding_is_unbiased_over_seeds(oracle):
+    """E[Q(x)] = x: the de-quantized result of absmax stochastic rounding, averaged over many seeds of the in-kernel
+    stream, approaches the rotated input element by element -- including elements whose round-up probability is far
+    below 1/256 (which a stream with 8 random bits per element would always round down)."""
+    rng = np.random.default_rng(5)
+    hd, rows = 32, 4
+    g = rng.standard_normal((rows, hd)).astype(np.float32)
+    g[:, 0] = 5.5                      # fixes the scale: 2^k = 1, values are t * 4/3
+    four_thirds = np.float32(1.0 / 0.75)
+    tiny = np.float32(0.5 * 1e-3) * four_thirds      # t = 0.0005: rounds up to 0.5 with probability 1e-3
+    g[0, 1:9] = tiny
+    g[1, 1:9] = np.float32(1.0 + 0.5 * 2e-3) * four_thirds   # just above a grid point
+    S = oracle.sylvester(hd).astype(np.float64)
+    c = float(oracle.hadamard_scale(hd, oracle.F32))
+    x = ((g.astype(np.float64) @ S.T) / (hd * c)).astype(np.float32)   # x @ H = g up to rounding
+    n_seeds = 6000
+    acc = np.zeros((rows, hd))
+    rot = None
+    for seed in range(n_seeds):
+        r = oracle.quantize(x, hd, mode=oracle.ABSMAX_SR, seed=1000 + seed, want_dequant=True, want_rotated=(seed == 0))
+        if seed == 0:
+            rot = r["rotated"].astype(np.float64)
+        acc += r["dequant"].astype(np.float64)
+    mean = acc / n_seeds
+    step = 0.5 * float(four_thirds)     # finest grid spacing at this scale
+    # per element: |bias| below 4 standard errors of the mean of a two-point variable (at most step/2 / sqrt(n)) + 2^-17 step
+    assert np.all(np.abs(mean - rot) <= 4 * (2 * step) / (2 * np.sqrt(n_seeds)) + step * 2.0 ** -17 + 1e-6)
+    # the tiny elements are not rounded away: their mean over seeds and over the eight copies is the value itself
+    got = mean[0, 1:9].mean()
+    want = rot[0, 1:9].mean()
+    assert got > 0 and abs(got - want) < 0.35 * want, (got, want)
 
 
 # ---- scales, codes, mask, packing ---------------------------------------------------------------
