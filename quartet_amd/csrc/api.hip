@@ -114,8 +114,8 @@ int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint
     if (M < 0 || N < 0 || K < 0 || K % 32) return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn: need K %% 32 == 0 (M=%lld N=%lld K=%lld)", (long long)M, (long long)N, (long long)K);
     if (M == 0 || N == 0) return 0;
     if (!c || (K > 0 && (!a_codes || !a_scales || !b_codes || !b_scales))) return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn: null tensor");
-    if (!aligned(a_codes, 16) || !aligned(b_codes, 16) || !aligned(a_scales, 4) || !aligned(b_scales, 4) || !aligned(c, 4))
-        return fail(QM_ERR_UNALIGNED, "qm_gemm_mxfp4_tn: codes need 16-byte, scales and c 4-byte alignment");
+    if (!aligned(a_codes, 16) || !aligned(b_codes, 16) || !aligned(a_scales, 4) || !aligned(b_scales, 4) || !aligned(c, 16))
+        return fail(QM_ERR_UNALIGNED, "qm_gemm_mxfp4_tn: codes and c need 16-byte, scales 4-byte alignment");
     if ((a_layout == QM_LAYOUT_TILED || b_layout == QM_LAYOUT_TILED) && !qm::gemm_supports_tiled(M, N, K))
         return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn: tiled operands need M, N multiples of 64 and >= 256, K %% 128 == 0 (M=%lld N=%lld K=%lld)",
                     (long long)M, (long long)N, (long long)K);

@@ -59,6 +59,8 @@ def test_host_only_entry_points():
     (lambda L: L.qm_quantize_mxfp4(None, 0, 4, 32, 32, None, 0, 0, None, 0, None, None, None, None, 0, None), b"non-null"),
     (lambda L: L.qm_requantize_transposed_mxfp4(None, None, 30, 64, 1.0, 0, 32, None, 2, None, 0, None, None, None, 0, 0, None), b"hadamard_dim"),
     (lambda L: L.qm_gemm_mxfp4_tn(None, None, None, None, 64, 64, 48, 1.0, None, 0, 0, 0, None, 0, None), b"qm_gemm_mxfp4_tn"),
+    # an output offset by 4 bytes: the tile kernels store 16-byte pieces, so the call is refused before any launch
+    (lambda L: L.qm_gemm_mxfp4_tn(0x1000, 0x2000, 0x3000, 0x4000, 256, 256, 128, 1.0, 0x5004, 0, 0, 0, None, 0, None), b"c need 16-byte"),
     (lambda L: L.qm_masked_hadamard_bwd(None, 0, 4, 40, 32, 0, None, None, None, 0, None), b"multiple of hadamard_dim"),
     (lambda L: L.qm_dequantize_mxfp4(None, None, 4, 40, 1.0, None, 0, None), b"C % 32"),
     (lambda L: L.qm_linear_forward(None, 0, None, 0, 64, 40, 64, 32, None, 32, None, None, 0, None, 0, 0, None, 0, 0, None), b"multiple of 32"),
