@@ -90,6 +90,27 @@ int qm_requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scale
                                    void* dequant, int in_layout, int out_layout, void* stream);
 
 /*
+ * The two quantizers with a dense 32 x 32 rotation in place of the Hadamard block: the matrix a quantizer holds after
+ * re_randomize with rerotate="O32" (U V^T of a Gaussian matrix's SVD, quantizers/mxfp4.py:61-64), which the reference
+ * applies with tl.dot inside its kernel (mxfp4_triton.py:44-45).  Each group of 32 consecutive elements g becomes
+ * g . matrix, evaluated on the matrix pipe as out[j] = fma(g[31], H[31][j], ... fma(g[0], H[0][j], 0)), then quantized
+ * as by qm_quantize_mxfp4 / qm_requantize_transposed_mxfp4.
+ *   matrix  DEVICE pointer to [32][32] fp32, row-major (H[k][j]); entries are rounded to x_dtype / val_dtype first,
+ *           as the reference casts its matrix to the tensor's dtype (mxfp4.py:49)
+ *   SR modes draw from the in-kernel Philox stream of `seed`.
+ * qm_quantize_mxfp4_dense: cols % 32 == 0; transposed_in needs cols % 128 == 0, rows % 8 == 0 and maskbits == NULL;
+ *   QM_LAYOUT_TILED needs rows % 16 == 0 and cols % 128 == 0.
+ * qm_requantize_transposed_mxfp4_dense: R % 128 == 0, C % 32 == 0; QM_LAYOUT_TILED on either side needs C % 128 == 0.
+ */
+int qm_quantize_mxfp4_dense(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* matrix, int mode,
+                            int transposed_in, uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits,
+                            void* dequant, int codes_layout, void* stream);
+int qm_requantize_transposed_mxfp4_dense(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C,
+                                         float post, int val_dtype, const float* matrix, int mode, uint64_t seed,
+                                         uint8_t* codes_out, uint8_t* scales_out, void* dequant, int in_layout,
+                                         int out_layout, void* stream);
+
+/*
  * C[M, N] = alpha * A[M, K] . B[N, K]^T on packed MXFP4 operands, fp32 accumulation.
  * Replaces F.linear / einsum on de-quantized operands (src/models/quantization/backward.py:62,
  * 71-75, 79-83) and matmul_mxf4_bf16_tn of notebooks/benchmark_mxfp4.ipynb.  K % 32 == 0.
@@ -163,6 +184,9 @@ int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, 
  *   workspace         qm_linear_backward_workspace_bytes(T, I, O, mid_dtype) bytes of scratch, 256-byte aligned
  *   gw_dtype          dtype of gw: mid_dtype, or QM_F32 with a bf16 mid_dtype -- then gw holds the bf16-rounded values
  *                     widened to fp32, i.e. what autograd's cast of a bf16 gradient to an fp32 weight's dtype produces
+ *   g_matrix          NULL, or a DEVICE pointer to the gradient quantizer's dense rotation ([32][32] fp32, as for
+ *                     qm_quantize_mxfp4_dense; AlbertTsengQuantizer with rerotate="O32"): replaces hd_g / signs_g in the
+ *                     four gradient quantizations; needs hd_g == 32 and T, I, O multiples of 128
  *   gx_rotated        != 0: gx receives the gradient w.r.t. the activation quantizer's rotated output (the first
  *                     product, B3) and its straight-through backward is left to the caller, who folds it into the
  *                     next kernel (maskbits argument of qm_rmsnorm_backward / qm_swiglu_backward); needs hd_x == 32
@@ -182,7 +206,7 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                        int hd_g, const uint32_t* signs_g, int g_mode, const uint64_t* seeds, int x_val_dtype,
                        int w_val_dtype, int mid_dtype, int x_scale_dtype, int w_scale_dtype, void* workspace,
                        size_t workspace_bytes, void* gx, void* gw, int gw_dtype, int codes_layout, int gx_rotated,
-                       void* stream);
+                       const float* g_matrix, void* stream);
 
 /*
  * Producers fused into the activation quantizer.  The tensor the model would hand to a quantized linear is computed

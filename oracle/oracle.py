@@ -54,6 +54,10 @@ def lib():
         L.qo_philox_uniform16_at.argtypes = [u64, i64, vp, vp]
         L.qo_quantize.restype = i32
         L.qo_quantize.argtypes = [vp, i32, i64, i64, i32, vp, i32, i32, vp, u64, vp, vp, vp, vp, vp]
+        L.qo_quantize_dense.restype = i32
+        L.qo_quantize_dense.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, u64, vp, vp, vp, vp, vp]
+        L.qo_requantize_transposed_dense.restype = i32
+        L.qo_requantize_transposed_dense.argtypes = [vp, vp, i64, i64, f32, i32, vp, i32, vp, u64, vp, vp, vp, vp]
         L.qo_dequantize.restype = i32
         L.qo_dequantize.argtypes = [vp, vp, i64, i64, f32, vp, i32]
         L.qo_requantize_transposed.restype = i32
@@ -150,10 +154,11 @@ def philox_uniform16_at(seed, offsets):
 
 
 def quantize(x, hd=32, signs=None, mode=QUEST_RTN, transposed_in=False, u=None, seed=0,
-             want_mask=False, want_dequant=False, want_rotated=False):
+             want_mask=False, want_dequant=False, want_rotated=False, matrix=None):
     """Returns dict(codes [R,C/2] u8, scales [R,C/32] u8, mask [R,C/8] u8|None,
     dequant like logical x|None, rotated f32|None).  Logical shape is x.shape, or its transpose
-    when transposed_in."""
+    when transposed_in.  `matrix` (float32 [32, 32]): a dense rotation replaces the Hadamard block
+    (hd and signs are then unused); it is rounded to x's dtype first."""
     x = np.ascontiguousarray(x)
     dt = _dtype_of(x)
     rows, cols = (x.shape[1], x.shape[0]) if transposed_in else x.shape
@@ -166,9 +171,15 @@ def quantize(x, hd=32, signs=None, mode=QUEST_RTN, transposed_in=False, u=None, 
     if u is not None:
         u = np.ascontiguousarray(u, dtype=np.float32)
         assert u.size == rows * cols
-    rc = lib().qo_quantize(_ptr(x), dt, rows, cols, hd, _ptr(sb), mode, int(transposed_in),
-                           _ptr(u), seed, _ptr(codes), _ptr(scales), _ptr(mask), _ptr(deq),
-                           _ptr(rot))
+    if matrix is not None:
+        m = np.ascontiguousarray(matrix, dtype=np.float32)
+        assert m.shape == (32, 32)
+        rc = lib().qo_quantize_dense(_ptr(x), dt, rows, cols, _ptr(m), mode, int(transposed_in), _ptr(u), seed,
+                                     _ptr(codes), _ptr(scales), _ptr(mask), _ptr(deq), _ptr(rot))
+    else:
+        rc = lib().qo_quantize(_ptr(x), dt, rows, cols, hd, _ptr(sb), mode, int(transposed_in),
+                               _ptr(u), seed, _ptr(codes), _ptr(scales), _ptr(mask), _ptr(deq),
+                               _ptr(rot))
     if rc != 0:
         raise ValueError(f"qo_quantize rejected its arguments (rc={rc})")
     return dict(codes=codes, scales=scales, mask=mask, dequant=deq, rotated=rot)
@@ -185,7 +196,7 @@ def dequantize(codes, scales, post=1.0, out_dtype=F32):
 
 
 def requantize_transposed(codes, scales, post=1.0, val_dtype=BF16, hd=32, signs=None,
-                          mode=ABSMAX_SR, u=None, seed=0, want_dequant=False, want_rotated=False):
+                          mode=ABSMAX_SR, u=None, seed=0, want_dequant=False, want_rotated=False, matrix=None):
     R, C = codes.shape[0], codes.shape[1] * 2
     sb = sign_bits_from_signs(signs)
     codes_out = np.empty((C, R // 2), dtype=np.uint8)
@@ -195,10 +206,17 @@ def requantize_transposed(codes, scales, post=1.0, val_dtype=BF16, hd=32, signs=
     if u is not None:
         u = np.ascontiguousarray(u, dtype=np.float32)
         assert u.size == R * C
-    rc = lib().qo_requantize_transposed(_ptr(np.ascontiguousarray(codes)),
-                                        _ptr(np.ascontiguousarray(scales)), R, C, post, val_dtype,
-                                        hd, _ptr(sb), mode, _ptr(u), seed, _ptr(codes_out),
-                                        _ptr(scales_out), _ptr(deq), _ptr(rot))
+    if matrix is not None:
+        m = np.ascontiguousarray(matrix, dtype=np.float32)
+        assert m.shape == (32, 32)
+        rc = lib().qo_requantize_transposed_dense(_ptr(np.ascontiguousarray(codes)), _ptr(np.ascontiguousarray(scales)),
+                                                  R, C, post, val_dtype, _ptr(m), mode, _ptr(u), seed, _ptr(codes_out),
+                                                  _ptr(scales_out), _ptr(deq), _ptr(rot))
+    else:
+        rc = lib().qo_requantize_transposed(_ptr(np.ascontiguousarray(codes)),
+                                            _ptr(np.ascontiguousarray(scales)), R, C, post, val_dtype,
+                                            hd, _ptr(sb), mode, _ptr(u), seed, _ptr(codes_out),
+                                            _ptr(scales_out), _ptr(deq), _ptr(rot))
     if rc != 0:
         raise ValueError(f"qo_requantize_transposed rc={rc}")
     return dict(codes=codes_out, scales=scales_out, dequant=deq, rotated=rot)

@@ -17,6 +17,8 @@ EXPORTS = (
     "qm_last_error",
     "qm_quantize_mxfp4",
     "qm_requantize_transposed_mxfp4",
+    "qm_quantize_mxfp4_dense",
+    "qm_requantize_transposed_mxfp4_dense",
     "qm_gemm_mxfp4_tn",
     "qm_masked_hadamard_bwd",
     "qm_dequantize_mxfp4",
@@ -62,6 +64,10 @@ def lib():
     L.qm_quantize_mxfp4.argtypes = [vp, i32, i64, i64, i32, vp, i32, i32, vp, u64, vp, vp, vp, vp, i32, vp]
     L.qm_requantize_transposed_mxfp4.restype = i32
     L.qm_requantize_transposed_mxfp4.argtypes = [vp, vp, i64, i64, f32, i32, i32, vp, i32, vp, u64, vp, vp, vp, i32, i32, vp]
+    L.qm_quantize_mxfp4_dense.restype = i32
+    L.qm_quantize_mxfp4_dense.argtypes = [vp, i32, i64, i64, vp, i32, i32, u64, vp, vp, vp, vp, i32, vp]
+    L.qm_requantize_transposed_mxfp4_dense.restype = i32
+    L.qm_requantize_transposed_mxfp4_dense.argtypes = [vp, vp, i64, i64, f32, i32, vp, i32, u64, vp, vp, vp, i32, i32, vp]
     L.qm_gemm_mxfp4_tn.restype = i32
     L.qm_gemm_mxfp4_tn.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, i32, vp, ctypes.c_size_t, vp]
     L.qm_gemm_workspace_bytes.restype = ctypes.c_size_t
@@ -99,7 +105,7 @@ def lib():
     L.qm_rope_merge_qkv_grad.argtypes = [vp, vp, vp, i32, i64, i64, i64, i32, vp, vp, i32, vp]
     L.qm_linear_backward.restype = i32
     L.qm_linear_backward.argtypes = [vp, i32, i64, i64, i64, vp, vp, i32, vp, i32, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32,
-                                     vp, sz, vp, vp, i32, i32, i32, vp]
+                                     vp, sz, vp, vp, i32, i32, i32, vp, vp]
     _lib = L
     return L
 

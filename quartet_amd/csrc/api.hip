@@ -44,7 +44,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 9; }
+int qm_version(void) { return 10; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -103,6 +103,50 @@ int qm_requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scale
                                                     scales_out, dequant, in_layout, out_layout,
                                                     reinterpret_cast<hipStream_t>(stream)),
                     "qm_requantize_transposed_mxfp4");
+}
+
+int qm_quantize_mxfp4_dense(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* matrix, int mode,
+                            int transposed_in, uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
+                            int codes_layout, void* stream) {
+    if (!valid_layout(codes_layout)) return fail(QM_ERR_INVALID, "qm_quantize_mxfp4_dense: unknown codes_layout %d", codes_layout);
+    if (!valid_dtype(x_dtype)) return fail(QM_ERR_INVALID, "qm_quantize_mxfp4_dense: x_dtype %d is not QM_BF16/QM_F32", x_dtype);
+    if (!valid_mode(mode)) return fail(QM_ERR_INVALID, "qm_quantize_mxfp4_dense: unknown mode %d", mode);
+    if (rows < 0 || cols < 0 || cols % 32)
+        return fail(QM_ERR_INVALID, "qm_quantize_mxfp4_dense: cols %lld not a multiple of 32", (long long)cols);
+    if (rows == 0 || cols == 0) return 0;
+    if (!x || !codes || !scales || !matrix) return fail(QM_ERR_INVALID, "qm_quantize_mxfp4_dense: x, matrix, codes and scales must be non-null");
+    if (!aligned(x, 16) || !aligned(codes, 16) || !aligned(matrix, 4) || !aligned(maskbits, 4) || (dequant && !aligned(dequant, 16)))
+        return fail(QM_ERR_UNALIGNED, "qm_quantize_mxfp4_dense: x/codes/dequant need 16-byte, matrix and maskbits 4-byte alignment");
+    if (transposed_in && (maskbits || cols % 128 || rows % 8 || !aligned(scales, 4)))
+        return fail(QM_ERR_INVALID, "qm_quantize_mxfp4_dense: transposed input needs cols %% 128 == 0, rows %% 8 == 0, no clip mask, "
+                                    "4-byte aligned scales (rows=%lld cols=%lld)", (long long)rows, (long long)cols);
+    if (codes_layout == QM_LAYOUT_TILED && (rows % 16 || cols % 128))
+        return fail(QM_ERR_INVALID, "qm_quantize_mxfp4_dense: tiled codes need rows %% 16 == 0 and cols %% 128 == 0 (rows=%lld cols=%lld)",
+                    (long long)rows, (long long)cols);
+    return from_hip(qm::quantize_mxfp4_dense(x, x_dtype, rows, cols, matrix, mode, transposed_in != 0, seed, codes, scales, maskbits,
+                                             dequant, codes_layout, reinterpret_cast<hipStream_t>(stream)),
+                    "qm_quantize_mxfp4_dense");
+}
+
+int qm_requantize_transposed_mxfp4_dense(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C, float post,
+                                         int val_dtype, const float* matrix, int mode, uint64_t seed, uint8_t* codes_out,
+                                         uint8_t* scales_out, void* dequant, int in_layout, int out_layout, void* stream) {
+    if (!valid_layout(in_layout) || !valid_layout(out_layout))
+        return fail(QM_ERR_INVALID, "qm_requantize_transposed_mxfp4_dense: unknown layout %d / %d", in_layout, out_layout);
+    if (!valid_dtype(val_dtype)) return fail(QM_ERR_INVALID, "qm_requantize_transposed_mxfp4_dense: val_dtype %d", val_dtype);
+    if (!valid_mode(mode)) return fail(QM_ERR_INVALID, "qm_requantize_transposed_mxfp4_dense: unknown mode %d", mode);
+    if (R < 0 || C < 0 || C % 32 || R % 128)
+        return fail(QM_ERR_INVALID, "qm_requantize_transposed_mxfp4_dense: need C %% 32 == 0 and R %% 128 == 0 (R=%lld C=%lld)", (long long)R, (long long)C);
+    if (R == 0 || C == 0) return 0;
+    if (!codes_in || !scales_in || !codes_out || !scales_out || !matrix) return fail(QM_ERR_INVALID, "qm_requantize_transposed_mxfp4_dense: null tensor");
+    if (!aligned(codes_in, 16) || !aligned(codes_out, 16) || !aligned(scales_out, 4) || !aligned(matrix, 4) || (dequant && !aligned(dequant, 16)))
+        return fail(QM_ERR_UNALIGNED, "qm_requantize_transposed_mxfp4_dense: codes and dequant need 16-byte, scales_out and matrix 4-byte alignment");
+    if ((in_layout == QM_LAYOUT_TILED || out_layout == QM_LAYOUT_TILED) && C % 128)
+        return fail(QM_ERR_INVALID, "qm_requantize_transposed_mxfp4_dense: tiled codes need C %% 128 == 0 (C=%lld)", (long long)C);
+    return from_hip(qm::requantize_transposed_mxfp4_dense(codes_in, scales_in, R, C, post, val_dtype, matrix, mode, seed, codes_out,
+                                                          scales_out, dequant, in_layout, out_layout,
+                                                          reinterpret_cast<hipStream_t>(stream)),
+                    "qm_requantize_transposed_mxfp4_dense");
 }
 
 int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
@@ -322,7 +366,7 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                        int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, int hd_g, const uint32_t* signs_g,
                        int g_mode, const uint64_t* seeds, int x_val_dtype, int w_val_dtype, int mid_dtype, int x_scale_dtype,
                        int w_scale_dtype, void* workspace, size_t workspace_bytes, void* gx, void* gw, int gw_dtype,
-                       int codes_layout, int gx_rotated, void* stream) {
+                       int codes_layout, int gx_rotated, const float* g_matrix, void* stream) {
     if (T < 0 || I < 0 || O < 0) return fail(QM_ERR_INVALID, "qm_linear_backward: negative extent");
     if (T == 0 || O == 0 || I == 0) return 0;
     if (g_mode != QM_ABSMAX_RTN && g_mode != QM_ABSMAX_SR)
@@ -362,6 +406,33 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                                                 gw_dtype, true, hs), "qm_linear_backward");
     };
     if (gx_rotated && hd_x != 32) return fail(QM_ERR_INVALID, "qm_linear_backward: gx_rotated needs hd_x == 32");
+    if (g_matrix) {
+        // a dense rotation in the gradient quantizer (rerotate="O32"): the same eight steps on the dense-rotation kernels
+        if (hd_g != 32 || T % 128 || I % 128 || O % 128)
+            return fail(QM_ERR_INVALID, "qm_linear_backward: a dense gradient rotation needs hd_g == 32 and T, I, O multiples of 128 "
+                                        "(T=%lld I=%lld O=%lld)", (long long)T, (long long)I, (long long)O);
+        rc = qm_quantize_mxfp4_dense(e, e_dtype, T, O, g_matrix, g_mode, 0, seeds[0], k + wl.ec, k + wl.es, nullptr, nullptr, codes_layout, stream);
+        if (rc) return rc;
+        rc = qm_requantize_transposed_mxfp4_dense(pw + lw.c, pw + lw.s, O, I, 1.0f, w_val_dtype, g_matrix, g_mode, seeds[1], k + wl.wtc,
+                                                  k + wl.wts, nullptr, codes_layout, codes_layout, stream);
+        if (rc) return rc;
+        rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, gx_product, mid_dtype, codes_layout,
+                              codes_layout, gws, wl.gemm_ws_bytes, stream);
+        if (rc) return rc;
+        rc = qm_quantize_mxfp4_dense(e, e_dtype, O, T, g_matrix, g_mode, 1, seeds[2], k + wl.etc, k + wl.ets, nullptr, nullptr, codes_layout, stream);
+        if (rc) return rc;
+        rc = qm_requantize_transposed_mxfp4_dense(px + lx.c, px + lx.s, T, I, 1.0f, x_val_dtype, g_matrix, g_mode, seeds[3], k + wl.xtc,
+                                                  k + wl.xts, nullptr, codes_layout, codes_layout, stream);
+        if (rc) return rc;
+        rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, k + wl.gwq, mid_dtype, codes_layout,
+                              codes_layout, gws, wl.gemm_ws_bytes, stream);
+        if (rc) return rc;
+        if (!gx_rotated) {
+            rc = qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, px + lx.m, gx, mid_dtype, stream);
+            if (rc) return rc;
+        }
+        return rotate_gw();
+    }
     if (pair_launches(codes_layout, T, I, O, hd_x, hd_w, hd_g) && e && gx && gw && valid_dtype(e_dtype) && aligned(e, 16) &&
         aligned(gx, 16) && aligned(gw, 16) && valid_dtype(x_val_dtype) && valid_dtype(w_val_dtype) &&
         valid_dtype(x_scale_dtype) && valid_dtype(w_scale_dtype)) {

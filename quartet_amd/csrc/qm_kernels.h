@@ -44,6 +44,25 @@ hipError_t requantize_transposed_hd32(const uint8_t* codes_in, const uint8_t* sc
                                       int val_dtype, uint32_t sign_word, int mode, uint64_t seed, uint8_t* codes,
                                       uint8_t* scales, void* dequant, bool tiled_in, bool tiled_out, hipStream_t stream);
 
+// The same with a dense 32x32 rotation instead of the Hadamard block (matrix: device pointer, [32][32] fp32, H[k][j])
+hipError_t quantize_rowmajor_dense(const void* x, int dtype, int64_t rows, int64_t cols, const float* matrix, int mode,
+                                   uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
+                                   bool tiled, hipStream_t stream);
+hipError_t quantize_transposed_dense(const void* x, int dtype, int64_t P, int64_t Q, const float* matrix, int mode,
+                                     uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant, bool tiled,
+                                     hipStream_t stream);
+hipError_t requantize_transposed_dense(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C, float post,
+                                       int val_dtype, const float* matrix, int mode, uint64_t seed, uint8_t* codes,
+                                       uint8_t* scales, void* dequant, bool tiled_in, bool tiled_out, hipStream_t stream);
+// shape-checked front ends of the three (what the C ABI calls); hipErrorInvalidValue for shapes they do not serve
+hipError_t quantize_mxfp4_dense(const void* x, int dtype, int64_t rows, int64_t cols, const float* matrix, int mode,
+                                bool transposed_in, uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits,
+                                void* dequant, int codes_layout, hipStream_t stream);
+hipError_t requantize_transposed_mxfp4_dense(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C,
+                                             float post, int val_dtype, const float* matrix, int mode, uint64_t seed,
+                                             uint8_t* codes_out, uint8_t* scales_out, void* dequant, int in_layout,
+                                             int out_layout, hipStream_t stream);
+
 // Pairs of independent quantizer launches issued as one grid (Hadamard block 32, tiled codes in and out).
 struct RowmajorArgs {
     const void* x;

@@ -445,6 +445,36 @@ hipError_t quantize_mxfp4(const void* x, int dtype, int64_t rows, int64_t cols, 
     return hipGetLastError();
 }
 
+// Dense 32x32 rotation: served by the group-layout kernels only.  Row-major input: any rows, cols % 32 == 0.
+// Transposed input (logical [rows, cols] = physical [cols, rows]): cols % 128 == 0, rows % 8 == 0, no clip mask.
+hipError_t quantize_mxfp4_dense(const void* x, int dtype, int64_t rows, int64_t cols, const float* matrix, int mode,
+                                bool transposed_in, uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits,
+                                void* dequant, int codes_layout, hipStream_t stream) {
+    if (rows == 0 || cols == 0) return hipSuccess;
+    const bool tiled = codes_layout == LAYOUT_TILED;
+    const auto al = [](const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
+    if (!matrix || cols % 32 || !al(codes, 16) || !al(maskbits, 4) || !al(matrix, 4)) return hipErrorInvalidValue;
+    if (tiled && (rows % 16 || cols % 128)) return hipErrorInvalidValue;
+    if (!transposed_in)
+        return quantize_rowmajor_dense(x, dtype, rows, cols, matrix, mode, seed, codes, scales, maskbits, dequant, tiled, stream);
+    if (maskbits || cols % 128 || rows % 8 || !al(scales, 4)) return hipErrorInvalidValue;
+    return quantize_transposed_dense(x, dtype, cols, rows, matrix, mode, seed, codes, scales, dequant, tiled, stream);
+}
+
+// R % 128 == 0, C % 32 == 0; tiled code bytes on either side need C % 128 == 0 as well
+hipError_t requantize_transposed_mxfp4_dense(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C,
+                                             float post, int val_dtype, const float* matrix, int mode, uint64_t seed,
+                                             uint8_t* codes_out, uint8_t* scales_out, void* dequant, int in_layout,
+                                             int out_layout, hipStream_t stream) {
+    if (R == 0 || C == 0) return hipSuccess;
+    const bool tiled_in = in_layout == LAYOUT_TILED, tiled_out = out_layout == LAYOUT_TILED;
+    const auto al = [](const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
+    if (!matrix || R % 128 || C % 32 || !al(codes_out, 16) || !al(scales_out, 4) || !al(codes_in, 16)) return hipErrorInvalidValue;
+    if ((tiled_in || tiled_out) && C % 128) return hipErrorInvalidValue;
+    return requantize_transposed_dense(codes_in, scales_in, R, C, post, val_dtype, matrix, mode, seed, codes_out, scales_out,
+                                       dequant, tiled_in, tiled_out, stream);
+}
+
 hipError_t requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C,
                                        float post, int val_dtype, int hd, const SignBits& sb, int mode, const float* u,
                                        uint64_t seed, uint8_t* codes_out, uint8_t* scales_out, void* dequant,

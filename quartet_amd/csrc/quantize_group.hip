@@ -274,6 +274,47 @@ __device__ __forceinline__ void rotate_group(float (&v)[32], float c, uint32_t s
     }
 }
 
+// ---- dense 32x32 rotation (rerotate="O32", quantizers/mxfp4.py:61-64 of the reference) on the matrix pipe ----------
+// The reference applies the matrix with tl.dot inside its kernel (mxfp4_triton.py:44-45).  Here each lane owns one
+// group of 32 values; v_mfma_f32_32x32x2_f32 computes D[j][n] += H[k][j] x[n][k] for 32 groups n at a time, and sixteen
+// chained instructions walk k = 0..31.  The instruction evaluates acc = fma(a, b, acc) per term in ascending k
+// (measured against every candidate order on random fp32 data: no mismatch), which is the order the test oracle states.
+// Lanes 0..31 hold groups "lo", lanes 32..63 groups "hi": v_permlane32_swap deals a lane's pair (k, k+1) out as the two
+// k rows the instruction wants from the two half-waves, and collects the results (a lane gets the 16 rotated values of
+// its group that the other half-wave computed).  Every lane of the wave must be active.
+typedef float v16f __attribute__((ext_vector_type(16)));
+struct DenseFrag {
+    float a[16];  // H[2t + lane/32][lane%32], t = 0..15, rounded to the tensor's dtype
+};
+__device__ __forceinline__ void load_dense_frag(const float* __restrict__ matrix, int dtype, DenseFrag& f) {
+    const int lane = threadIdx.x & 63, j = lane & 31, half = lane >> 5;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+        float h = matrix[(2 * t + half) * 32 + j];
+        if (dtype == BF16) h = bf16_to_f32(f32_to_bf16(h));
+        f.a[t] = h;
+    }
+}
+__device__ __forceinline__ void dense_rotate(float (&v)[32], const DenseFrag& f) {
+    v16f lo, hi;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) lo[e] = hi[e] = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+        // after the swap: first = (k = 2t of groups lo | k = 2t+1 of groups lo), second = the same of groups hi
+        const auto r = __builtin_amdgcn_permlane32_swap(f2u(v[2 * t]), f2u(v[2 * t + 1]), false, false);
+        lo = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[t], u2f(r[0]), lo, 0, 0, 0);
+        hi = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[t], u2f(r[1]), hi, 0, 0, 0);
+    }
+    // accumulator element e of a lane is output row j = 8 (e / 4) + 4 (lane / 32) + e % 4 of group lane % 32
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const auto r = __builtin_amdgcn_permlane32_swap(f2u(lo[e]), f2u(hi[e]), false, false);
+        v[8 * (e / 4) + (e % 4)] = u2f(r[0]);
+        v[8 * (e / 4) + 4 + (e % 4)] = u2f(r[1]);
+    }
+}
+
 // rotate (hd = 32) + quantize the group in v; gi is its logical (row-major) group index, which also keys the
 // random stream; ci is the index of its 16 code bytes in the code buffer (= gi for row-major codes)
 template <typename T, int MODE, bool WANT_MASK>
@@ -297,6 +338,53 @@ __global__ __launch_bounds__(256) void quantize_rowmajor_g32_kernel(const T* __r
     float v[32];
     load_group<T>(x + gi * 32, v);
     finish_group<T, MODE, WANT_MASK>(v, gi, gi, c, sign_word, seed, out, rotate != 0);
+}
+
+// Row-major input with a dense rotation: one group per lane, flat over the tensor; row-major or tiled code bytes.
+template <typename T, int MODE, bool WANT_MASK>
+__global__ __launch_bounds__(256) void quantize_rowmajor_dense_kernel(const T* __restrict__ x, int64_t n_groups, int groups_per_row,
+                                                                      const float* __restrict__ matrix, uint64_t seed,
+                                                                      GroupOut out, int tiled) {
+    const int64_t gi = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const bool valid = gi < n_groups;
+    DenseFrag frag;
+    load_dense_frag(matrix, sizeof(T) == 2 ? BF16 : F32, frag);
+    float v[32];
+    if (valid) {
+        load_group<T>(x + gi * 32, v);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 32; ++i) v[i] = 0.0f;
+    }
+    dense_rotate(v, frag);  // the whole wave, also past the end of the tensor
+    if (!valid) return;
+    GroupCodes o;
+    quantize_group_regs<MODE, WANT_MASK>(v, seed, gi, o);
+    int64_t ci = gi;
+    if (tiled) {
+        const int64_t row = gi / groups_per_row;
+        const int g = (int)(gi - row * groups_per_row);
+        ci = (row >> 4) * 16 * groups_per_row + ((g >> 2) * 64 + (int)(row & 15) * 4 + (g & 3));
+    }
+    out.codes[ci] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
+    out.scales[gi] = (uint8_t)o.scale_byte;
+    if constexpr (WANT_MASK) out.maskbits[gi] = o.keep;
+    if (out.dequant) store_dequant<T>(reinterpret_cast<T*>(out.dequant) + gi * 32, o);
+}
+
+template <typename T, bool WANT_MASK>
+void launch_rowmajor_dense(int mode, const void* x, int64_t rows, int64_t cols, const float* matrix, uint64_t seed,
+                           const GroupOut& out, bool tiled, hipStream_t stream) {
+    const T* xp = reinterpret_cast<const T*>(x);
+    const int64_t n_groups = rows * cols / 32;
+    const int gpr = (int)(cols / 32);
+    dim3 grid((unsigned)((n_groups + 255) / 256)), block(256);
+    switch (mode) {
+        case QUEST_RTN: quantize_rowmajor_dense_kernel<T, QUEST_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, gpr, matrix, seed, out, (int)tiled); break;
+        case ABSMAX_RTN: quantize_rowmajor_dense_kernel<T, ABSMAX_RTN, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, gpr, matrix, seed, out, (int)tiled); break;
+        case ABSMAX_SR: quantize_rowmajor_dense_kernel<T, ABSMAX_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, gpr, matrix, seed, out, (int)tiled); break;
+        default: quantize_rowmajor_dense_kernel<T, QUEST_SR, WANT_MASK><<<grid, block, 0, stream>>>(xp, n_groups, gpr, matrix, seed, out, (int)tiled); break;
+    }
 }
 
 // Tiled code layout ([rows/16][cols/128][16 rows][64 bytes]).  Workgroup b owns block b / chunks of 16 rows and run
@@ -440,7 +528,7 @@ struct TrTile {
 };
 constexpr int kTrP = 128;
 
-template <typename T, int MODE>
+template <typename T, int MODE, bool DENSE = false>
 struct TransposedJob {
     const T* x;
     int64_t P, Q;
@@ -451,12 +539,13 @@ struct TransposedJob {
     uint8_t* scales;
     void* dequant;
     bool tiled_out;
+    const float* matrix;  // DENSE: the rotation, [32][32] fp32 (c and sign_word are then unused)
     unsigned grid_p, blocks;
 
     TransposedJob(const void* x_, int64_t P_, int64_t Q_, float c_, uint32_t sign_word_, uint64_t seed_, uint8_t* codes_,
-                  uint8_t* scales_, void* dequant_, bool tiled_out_)
+                  uint8_t* scales_, void* dequant_, bool tiled_out_, const float* matrix_ = nullptr)
         : x(reinterpret_cast<const T*>(x_)), P(P_), Q(Q_), c(c_), sign_word(sign_word_), seed(seed_), codes(codes_),
-          scales(scales_), dequant(dequant_), tiled_out(tiled_out_), grid_p((unsigned)((P_ + kTrP - 1) / kTrP)),
+          scales(scales_), dequant(dequant_), tiled_out(tiled_out_), matrix(matrix_), grid_p((unsigned)((P_ + kTrP - 1) / kTrP)),
           blocks((unsigned)(((P_ + kTrP - 1) / kTrP) * ((Q_ + TrTile<T>::kQ - 1) / TrTile<T>::kQ))) {}
 
     __device__ __forceinline__ void run(unsigned bid) const {
@@ -471,8 +560,8 @@ struct TransposedJob {
         const int64_t pbase = p0 + wave * 32;       // this wave's group along p
         const int64_t qa = q0 + lane * GPL;         // this lane's first column
         const bool active = pbase < P && qa < Q;    // P % 32 == 0 and Q % 8 == 0: all of a lane's groups or none
+        float v[GPL][32];
         if (active) {
-            float v[GPL][32];
             // uniform row pointers (scalar unit) + the lane's 32-bit dword offset: no per-lane 64-bit address math
             const uint32_t* row = reinterpret_cast<const uint32_t*>(x + pbase * Q + q0);
             const int64_t row_dw = Q * (int64_t)sizeof(T) / 4;
@@ -486,11 +575,24 @@ struct TransposedJob {
                     v[0][i] = u2f(w);
                 }
             }
+        } else if constexpr (DENSE) {
+#pragma unroll
+            for (int gq = 0; gq < GPL; ++gq)
+#pragma unroll
+                for (int i = 0; i < 32; ++i) v[gq][i] = 0.0f;
+        }
+        if constexpr (DENSE) {  // the matrix instruction needs the whole wave, lanes outside the tensor included
+            DenseFrag frag;
+            load_dense_frag(matrix, sizeof(T) == 2 ? BF16 : F32, frag);
+#pragma unroll
+            for (int gq = 0; gq < GPL; ++gq) dense_rotate(v[gq], frag);
+        }
+        if (active) {
 #pragma unroll
             for (int gq = 0; gq < GPL; ++gq) {
                 const int64_t gi = (qa + gq) * (P / 32) + pbase / 32;
                 GroupCodes res;
-                rotate_group(v[gq], c, sign_word);
+                if constexpr (!DENSE) rotate_group(v[gq], c, sign_word);
                 quantize_group_regs<MODE, false>(v[gq], seed, gi, res);
                 if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res);
                 ocodes[(lane * GPL + gq) * 4 + wave] = make_uint4(res.w[0], res.w[1], res.w[2], res.w[3]);
@@ -522,14 +624,16 @@ struct TransposedJob {
 };
 
 // ---- packed MXFP4 in, transposed + rotated + re-quantized out --------------------------------------------
-// in: codes [R, C/2], scales [R, C/32]; out: the [C, R] tensor quantized along R.  A workgroup owns 128
-// columns (64 code bytes per row) by 128 rows; wave w owns r-group w; a lane handles one byte column = two
-// adjacent c, 32 rows deep, read straight from global memory (one contiguous 64-byte row segment per wave
-// load, plus the row's E8M0 byte of the lane's column group).  The hardware FP4 de-quantizing convert turns
-// each byte into two floats.  Outputs leave through LDS as in the transposed quantizer.
-constexpr int kRqR = 128, kRqC = 128;
+// in: codes [R, C/2], scales [R, C/32]; out: the [C, R] tensor quantized along R.  A wave owns 128 rows by 128
+// columns: lane l reads, for the 32 rows of row group l / 16, the four code bytes (eight columns c) at byte column
+// 4 (l % 16) straight from global memory as dwords -- a wave load is four contiguous 64-byte row segments -- plus the
+// rows' E8M0 byte of its column group.  It then handles its eight columns two at a time: the hardware FP4
+// de-quantizing convert turns byte p of each dword into two floats, which gives two groups of 32 along r in registers.
+// A workgroup stacks its four waves along r (512 rows), so that a column's scale bytes leave as one 16-byte piece;
+// codes leave through LDS as whole 64-byte row pieces (tiled output: eight contiguous 1 KiB tiles per wave).
+constexpr int kRqR = 512, kRqC = 128;
 
-template <int VAL_DTYPE, int MODE>
+template <int VAL_DTYPE, int MODE, bool DENSE = false>
 struct RequantJob {
     const uint8_t* codes_in;
     const uint8_t* scales_in;
@@ -541,113 +645,149 @@ struct RequantJob {
     uint8_t* scales;
     void* dequant;
     bool tiled_in, tiled_out;
+    const float* matrix;  // DENSE: the rotation, [32][32] fp32 (c and sign_word are then unused)
     unsigned grid_r, blocks;
 
     RequantJob(const uint8_t* codes_in_, const uint8_t* scales_in_, int64_t R_, int64_t C_, float post_, float c_,
                uint32_t sign_word_, uint64_t seed_, uint8_t* codes_, uint8_t* scales_, void* dequant_, bool tiled_in_,
-               bool tiled_out_)
+               bool tiled_out_, const float* matrix_ = nullptr)
         : codes_in(codes_in_), scales_in(scales_in_), R(R_), C(C_), post(post_), c(c_), sign_word(sign_word_), seed(seed_),
-          codes(codes_), scales(scales_), dequant(dequant_), tiled_in(tiled_in_), tiled_out(tiled_out_),
+          codes(codes_), scales(scales_), dequant(dequant_), tiled_in(tiled_in_), tiled_out(tiled_out_), matrix(matrix_),
           grid_r((unsigned)((R_ + kRqR - 1) / kRqR)),
           blocks((unsigned)(((R_ + kRqR - 1) / kRqR) * ((C_ + kRqC - 1) / kRqC))) {}
 
-    __device__ __forceinline__ void run(unsigned bid) const {
+    // columns 2 P and 2 P + 1 of the lane's eight: de-quantize byte P of the 32 row dwords, rotate, quantize, stage
+    template <int P>
+    __device__ __forceinline__ void column_pair(const uint32_t (&cw)[32], const float (&sc)[32], const DenseFrag& frag, bool active,
+                                                int64_t ca, int64_t rbase, int co, int rg, int wave, uint4* ocodes,
+                                                uint8_t* oscales) const {
         using T = typename std::conditional<VAL_DTYPE == BF16, uint16_t, float>::type;
-        __shared__ uint4 ocodes[kRqC * 4];
-        __shared__ uint32_t oscales[kRqC];
+        float v[2][32];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const v2f pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(cw[i], sc[i], P);
+            float a = pr.x, b = pr.y;
+            if (post != 1.0f) {  // absmax-coded input: value = code * 2^k * post, held in val_dtype
+                a *= post;
+                b *= post;
+                if constexpr (VAL_DTYPE == BF16) {
+                    a = bf16_to_f32(f32_to_bf16(a));
+                    b = bf16_to_f32(f32_to_bf16(b));
+                }
+            }
+            v[0][i] = a;
+            v[1][i] = b;
+        }
+        if constexpr (DENSE) {  // the matrix instruction needs the whole wave, lanes outside the tensor included
+            dense_rotate(v[0], frag);
+            dense_rotate(v[1], frag);
+        }
+        if (!active) return;
+#pragma unroll
+        for (int gq = 0; gq < 2; ++gq) {
+            const int64_t gi = (ca + 2 * P + gq) * (R / 32) + rbase / 32;
+            GroupCodes res;
+            if constexpr (!DENSE) rotate_group(v[gq], c, sign_word);
+            quantize_group_regs<MODE, false>(v[gq], seed, gi, res);
+            if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res);
+            const int cl = 8 * co + 2 * P + gq;
+            ocodes[cl * 4 + rg] = make_uint4(res.w[0], res.w[1], res.w[2], res.w[3]);
+            oscales[cl * 16 + wave * 4 + rg] = (uint8_t)res.scale_byte;
+        }
+    }
+
+    __device__ __forceinline__ void run(unsigned bid) const {
+        __shared__ uint4 ocodes_all[4][kRqC * 4];  // per wave: [c][4 row groups x 16 B]
+        __shared__ uint4 oscales_all[kRqC];        // [c][16 scale bytes: wave-major, then row group]
         const int tid = threadIdx.x, lane = tid & 63;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // tells the compiler it is wave-uniform
         const unsigned bc = bid / grid_r;
         const int64_t r0 = (int64_t)(bid - bc * grid_r) * kRqR, c0 = (int64_t)bc * kRqC;
         const int64_t in_code_pitch = C / 2, in_scale_pitch = C / 32;
-        const int64_t rbase = r0 + wave * 32;
-        const int64_t ca = c0 + 2 * lane;            // this lane's column pair
-        const bool active = rbase < R && ca < C;     // C % 32 == 0: both columns of the pair or none
+        const int64_t rw = r0 + wave * 128;          // this wave's first row
+        const int rg = lane >> 4, co = lane & 15;    // row group within the wave, column octet
+        const int64_t rbase = rw + 32 * rg;
+        const int64_t ca = c0 + 8 * co;              // this lane's first column
+        const bool active = rbase < R && ca < C;     // R % 32 == 0 and C % 32 == 0: all of a lane's groups or none
+        uint32_t cw[32];
+        float sc[32];
         if (active) {
-            float v[2][32];
             // Uniform row pointers (scalar unit) + the lane's 32-bit byte offset: no per-lane 64-bit address math.
-            // Tiled input: the lane's byte column sits at offset `lane` of the 64-byte rows of column block c0/128.
-            const uint8_t* cu = tiled_in ? codes_in + tiled_code_offset(rbase, c0 / 128, C / 128)
-                                         : codes_in + rbase * in_code_pitch + c0 / 2;
-            const int64_t row_step = tiled_in ? 64 : in_code_pitch;                            // next row of a 16-row block
-            const int64_t block_step = tiled_in ? (C / 128) * 1024 - 16 * 64 : 0;              // extra hop into the next block
-            const uint8_t* su = scales_in + rbase * in_scale_pitch + c0 / 32;
-            const uint32_t sl = (uint32_t)lane >> 4;  // which of the workgroup's four column groups the lane is in
-            uint32_t byte[32], sbyte[32];
+            // Tiled input: rows are 64 bytes apart inside a 16-row block, blocks (C / 128) KiB apart.
+            const int64_t blk = (C / 128) * 1024;
+            const uint8_t* cu = tiled_in ? codes_in + tiled_code_offset(rw, c0 / 128, C / 128) : codes_in + rw * in_code_pitch + c0 / 2;
+            const uint32_t lane_off = (uint32_t)((tiled_in ? 2 * rg * blk : 32 * rg * in_code_pitch) + 4 * co);
+            const int64_t row_step = tiled_in ? 64 : in_code_pitch;                 // next row of a 16-row block
+            const int64_t block_step = tiled_in ? blk - 16 * 64 : 0;                // extra hop into the next block
+            const uint8_t* su = scales_in + rw * in_scale_pitch + c0 / 32;
+            const uint32_t slane_off = (uint32_t)(32 * rg * in_scale_pitch + (co >> 2));
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
-                byte[i] = (cu + i * row_step + (i >> 4) * block_step)[(uint32_t)lane];
-                sbyte[i] = (su + i * in_scale_pitch)[sl];
+                cw[i] = *reinterpret_cast<const uint32_t*>(cu + i * row_step + (i >> 4) * block_step + lane_off);
+                sc[i] = u2f((uint32_t)(su + i * in_scale_pitch)[slane_off] << 23);
             }
+        } else {
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
-                const v2f pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(byte[i], u2f(sbyte[i] << 23), 0);
-                float a = pr.x, b = pr.y;
-                if (post != 1.0f) {  // absmax-coded input: value = code * 2^k * post, held in val_dtype
-                    a *= post;
-                    b *= post;
-                    if constexpr (VAL_DTYPE == BF16) {
-                        a = bf16_to_f32(f32_to_bf16(a));
-                        b = bf16_to_f32(f32_to_bf16(b));
-                    }
-                }
-                v[0][i] = a;
-                v[1][i] = b;
-            }
-#pragma unroll
-            for (int gq = 0; gq < 2; ++gq) {
-                const int64_t gi = (ca + gq) * (R / 32) + rbase / 32;
-                GroupCodes res;
-                rotate_group(v[gq], c, sign_word);
-                quantize_group_regs<MODE, false>(v[gq], seed, gi, res);
-                if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res);
-                ocodes[(lane * 2 + gq) * 4 + wave] = make_uint4(res.w[0], res.w[1], res.w[2], res.w[3]);
-                reinterpret_cast<uint8_t*>(oscales)[(lane * 2 + gq) * 4 + wave] = (uint8_t)res.scale_byte;
+                cw[i] = 0u;
+                sc[i] = 1.0f;
             }
         }
+        DenseFrag frag;
+        if constexpr (DENSE) load_dense_frag(matrix, VAL_DTYPE, frag);
+        uint4* ocodes = ocodes_all[wave];
+        uint8_t* oscales = reinterpret_cast<uint8_t*>(oscales_all);
+        column_pair<0>(cw, sc, frag, active, ca, rbase, co, rg, wave, ocodes, oscales);
+        column_pair<1>(cw, sc, frag, active, ca, rbase, co, rg, wave, ocodes, oscales);
+        column_pair<2>(cw, sc, frag, active, ca, rbase, co, rg, wave, ocodes, oscales);
+        column_pair<3>(cw, sc, frag, active, ca, rbase, co, rg, wave, ocodes, oscales);
         __syncthreads();
         const int64_t code_pitch = R / 2, scale_pitch = R / 32;
-        for (int idx = tid; idx < kRqC * 4; idx += 256) {
-            const int cl = idx >> 2, part = idx & 3;
-            if (c0 + cl < C && r0 + part * 32 < R) {
-                const int64_t off = tiled_out ? tiled_code_offset(c0 + cl, r0 / 128, R / 128) + part * 16
-                                              : (c0 + cl) * code_pitch + r0 / 2 + part * 16;
+        // codes: each wave writes its own 128 x 64-byte tile
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int idx = it * 64 + lane, cl = idx >> 2, part = idx & 3;
+            if (c0 + cl < C && rw + part * 32 < R) {
+                const int64_t off = tiled_out ? tiled_code_offset(c0 + cl, rw / 128, R / 128) + part * 16
+                                              : (c0 + cl) * code_pitch + rw / 2 + part * 16;
                 *reinterpret_cast<uint4*>(codes + off) = ocodes[idx];
             }
         }
+        // scales: one column's 16 bytes (the workgroup's 512 rows) per thread
         if (tid < kRqC && c0 + tid < C) {
-            const uint32_t sw = oscales[tid];
+            const uint4 sw = oscales_all[tid];
             uint8_t* dst = scales + (c0 + tid) * scale_pitch + r0 / 32;
-            if (r0 + kRqR <= R) {
-                *reinterpret_cast<uint32_t*>(dst) = sw;
+            if (r0 + kRqR <= R && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+                *reinterpret_cast<uint4*>(dst) = sw;
             } else {
-                for (int b = 0; b < 4; ++b)
-                    if (r0 + b * 32 < R) dst[b] = (uint8_t)(sw >> (8 * b));
+                const uint32_t w4[4] = {sw.x, sw.y, sw.z, sw.w};
+                for (int b = 0; b < 16; ++b)
+                    if (r0 + b * 32 < R) dst[b] = (uint8_t)(w4[b >> 2] >> (8 * (b & 3)));
             }
         }
     }
 };
 
-template <typename T>
+template <typename T, bool DENSE>
 void launch_transposed_g32(int mode, const void* x, int64_t P, int64_t Q, float c, uint32_t sign_word, uint64_t seed,
-                           uint8_t* codes, uint8_t* scales, void* dequant, bool tiled, hipStream_t stream) {
+                           uint8_t* codes, uint8_t* scales, void* dequant, bool tiled, const float* matrix, hipStream_t stream) {
     switch (mode) {
-        case QUEST_RTN: launch_job(TransposedJob<T, QUEST_RTN>(x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled), stream); break;
-        case ABSMAX_RTN: launch_job(TransposedJob<T, ABSMAX_RTN>(x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled), stream); break;
-        case ABSMAX_SR: launch_job(TransposedJob<T, ABSMAX_SR>(x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled), stream); break;
-        default: launch_job(TransposedJob<T, QUEST_SR>(x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled), stream); break;
+        case QUEST_RTN: launch_job(TransposedJob<T, QUEST_RTN, DENSE>(x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled, matrix), stream); break;
+        case ABSMAX_RTN: launch_job(TransposedJob<T, ABSMAX_RTN, DENSE>(x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled, matrix), stream); break;
+        case ABSMAX_SR: launch_job(TransposedJob<T, ABSMAX_SR, DENSE>(x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled, matrix), stream); break;
+        default: launch_job(TransposedJob<T, QUEST_SR, DENSE>(x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled, matrix), stream); break;
     }
 }
 
-template <int VAL_DTYPE>
+template <int VAL_DTYPE, bool DENSE>
 void launch_requant_g32(int mode, const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C, float post,
                         float c, uint32_t sign_word, uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant,
-                        bool tiled_in, bool tiled_out, hipStream_t stream) {
+                        bool tiled_in, bool tiled_out, const float* matrix, hipStream_t stream) {
     switch (mode) {
-        case QUEST_RTN: launch_job(RequantJob<VAL_DTYPE, QUEST_RTN>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out), stream); break;
-        case ABSMAX_RTN: launch_job(RequantJob<VAL_DTYPE, ABSMAX_RTN>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out), stream); break;
-        case ABSMAX_SR: launch_job(RequantJob<VAL_DTYPE, ABSMAX_SR>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out), stream); break;
-        default: launch_job(RequantJob<VAL_DTYPE, QUEST_SR>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out), stream); break;
+        case QUEST_RTN: launch_job(RequantJob<VAL_DTYPE, QUEST_RTN, DENSE>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out, matrix), stream); break;
+        case ABSMAX_RTN: launch_job(RequantJob<VAL_DTYPE, ABSMAX_RTN, DENSE>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out, matrix), stream); break;
+        case ABSMAX_SR: launch_job(RequantJob<VAL_DTYPE, ABSMAX_SR, DENSE>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out, matrix), stream); break;
+        default: launch_job(RequantJob<VAL_DTYPE, QUEST_SR, DENSE>(codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out, matrix), stream); break;
     }
 }
 
@@ -699,8 +839,8 @@ hipError_t quantize_transposed_hd32(const void* x, int dtype, int64_t P, int64_t
                                     uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant, bool tiled,
                                     hipStream_t stream) {
     const float c = hadamard_scale(32, dtype);
-    if (dtype == BF16) launch_transposed_g32<uint16_t>(mode, x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled, stream);
-    else launch_transposed_g32<float>(mode, x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled, stream);
+    if (dtype == BF16) launch_transposed_g32<uint16_t, false>(mode, x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled, nullptr, stream);
+    else launch_transposed_g32<float, false>(mode, x, P, Q, c, sign_word, seed, codes, scales, dequant, tiled, nullptr, stream);
     return hipGetLastError();
 }
 
@@ -708,8 +848,40 @@ hipError_t requantize_transposed_hd32(const uint8_t* codes_in, const uint8_t* sc
                                       int val_dtype, uint32_t sign_word, int mode, uint64_t seed, uint8_t* codes,
                                       uint8_t* scales, void* dequant, bool tiled_in, bool tiled_out, hipStream_t stream) {
     const float c = hadamard_scale(32, val_dtype);
-    if (val_dtype == BF16) launch_requant_g32<BF16>(mode, codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out, stream);
-    else launch_requant_g32<F32>(mode, codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out, stream);
+    if (val_dtype == BF16) launch_requant_g32<BF16, false>(mode, codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out, nullptr, stream);
+    else launch_requant_g32<F32, false>(mode, codes_in, scales_in, R, C, post, c, sign_word, seed, codes, scales, dequant, tiled_in, tiled_out, nullptr, stream);
+    return hipGetLastError();
+}
+
+// ---- the same three with a dense 32x32 rotation (matrix: device pointer to [32][32] fp32, H[k][j]; its entries are
+// rounded to the tensor's dtype as the reference casts its matrix, quantizers/mxfp4.py:49) ---------------------------
+hipError_t quantize_rowmajor_dense(const void* x, int dtype, int64_t rows, int64_t cols, const float* matrix, int mode,
+                                   uint64_t seed, uint8_t* codes, uint8_t* scales, uint8_t* maskbits, void* dequant,
+                                   bool tiled, hipStream_t stream) {
+    GroupOut out{reinterpret_cast<uint4*>(codes), scales, reinterpret_cast<uint32_t*>(maskbits), dequant};
+    if (maskbits) {
+        if (dtype == BF16) launch_rowmajor_dense<uint16_t, true>(mode, x, rows, cols, matrix, seed, out, tiled, stream);
+        else launch_rowmajor_dense<float, true>(mode, x, rows, cols, matrix, seed, out, tiled, stream);
+    } else {
+        if (dtype == BF16) launch_rowmajor_dense<uint16_t, false>(mode, x, rows, cols, matrix, seed, out, tiled, stream);
+        else launch_rowmajor_dense<float, false>(mode, x, rows, cols, matrix, seed, out, tiled, stream);
+    }
+    return hipGetLastError();
+}
+
+hipError_t quantize_transposed_dense(const void* x, int dtype, int64_t P, int64_t Q, const float* matrix, int mode,
+                                     uint64_t seed, uint8_t* codes, uint8_t* scales, void* dequant, bool tiled,
+                                     hipStream_t stream) {
+    if (dtype == BF16) launch_transposed_g32<uint16_t, true>(mode, x, P, Q, 1.0f, 0u, seed, codes, scales, dequant, tiled, matrix, stream);
+    else launch_transposed_g32<float, true>(mode, x, P, Q, 1.0f, 0u, seed, codes, scales, dequant, tiled, matrix, stream);
+    return hipGetLastError();
+}
+
+hipError_t requantize_transposed_dense(const uint8_t* codes_in, const uint8_t* scales_in, int64_t R, int64_t C, float post,
+                                       int val_dtype, const float* matrix, int mode, uint64_t seed, uint8_t* codes,
+                                       uint8_t* scales, void* dequant, bool tiled_in, bool tiled_out, hipStream_t stream) {
+    if (val_dtype == BF16) launch_requant_g32<BF16, true>(mode, codes_in, scales_in, R, C, post, 1.0f, 0u, seed, codes, scales, dequant, tiled_in, tiled_out, matrix, stream);
+    else launch_requant_g32<F32, true>(mode, codes_in, scales_in, R, C, post, 1.0f, 0u, seed, codes, scales, dequant, tiled_in, tiled_out, matrix, stream);
     return hipGetLastError();
 }
 

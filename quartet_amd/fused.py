@@ -18,8 +18,8 @@ from .quantizers.mxfp4 import _autocast_bf16
 _KERNEL_DTYPES = (torch.float32, torch.bfloat16)
 
 
-def _layer_is_fusable(layer):
-    return (isinstance(layer, QuantizedLinear) and layer._is_production_config() and layer.weight.is_cuda
+def _layer_is_fusable(layer, x):
+    return (isinstance(layer, QuantizedLinear) and layer._is_production_config(x.numel() // max(x.shape[-1], 1)) and layer.weight.is_cuda
             and layer.activation_quantizer.hadamard_dim == 32 and layer.weight.dtype in _KERNEL_DTYPES)
 
 
@@ -137,7 +137,7 @@ def rmsnorm_linear(norm, layer, x, pass_input=False, add=None):
     `pass_input` returns (layer(norm(x)), x): use the second value for the residual sum around the norm, so that the sum
     of x's two gradients happens inside the RMSNorm backward kernel.  With `add` returns (layer(norm(x + add)), x + add):
     the residual sum in front of the norm is formed inside the quantizer kernel."""
-    fusable = (_layer_is_fusable(layer) and x.is_cuda and x.dtype in _KERNEL_DTYPES and norm.weight.dtype == torch.float32
+    fusable = (_layer_is_fusable(layer, x) and x.is_cuda and x.dtype in _KERNEL_DTYPES and norm.weight.dtype == torch.float32
                and x.shape[-1] <= 8192)
     if fusable and add is not None and not (x.dtype == torch.float32 and add.dtype in _KERNEL_DTYPES and add.shape == x.shape):
         x, add = x + add, None
@@ -153,7 +153,7 @@ def rmsnorm_linear(norm, layer, x, pass_input=False, add=None):
 
 def swiglu_linear(layer, h12):
     """layer(silu(up) * gate) with (up, gate) the two halves of h12's last dimension."""
-    if _layer_is_fusable(layer) and h12.is_cuda and h12.dtype in _KERNEL_DTYPES:
+    if _layer_is_fusable(layer, h12) and h12.is_cuda and h12.dtype in _KERNEL_DTYPES:
         return SwiGLULinearFn.apply(h12, layer.weight, layer.activation_quantizer, layer.weight_quantizer,
                                     layer.backward_scheme.g_quantizer, layer.packed_weight_cache)
     up, gate = h12.split(h12.shape[-1] // 2, dim=-1)

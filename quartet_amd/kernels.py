@@ -82,6 +82,51 @@ def quantize_mxfp4(x, hadamard_dim=32, sign_bits=None, mode=QM_QUEST_RTN, transp
     return codes, scales, mask, deq
 
 
+def _matrix_arg(matrix, device):
+    """A dense rotation as the kernels read it: contiguous fp32 [32, 32] on the tensors' device."""
+    m = matrix.detach().to(device=device, dtype=torch.float32).contiguous()
+    if tuple(m.shape) != (32, 32):
+        raise _lib.QuartetHipError(f"a dense rotation must be 32 x 32, got {tuple(m.shape)}")
+    return m
+
+
+def quantize_mxfp4_dense(x, matrix, mode=QM_ABSMAX_RTN, transposed_in=False, seed=0, want_mask=False, want_dequant=False,
+                         tiled=False):
+    """quantize_mxfp4 with a dense 32 x 32 rotation (`matrix`, H[k][j]) applied to every group of 32 in place of the
+    Hadamard block.  Same return value."""
+    _require_cuda(x)
+    assert x.dim() == 2 and x.is_contiguous()
+    rows, cols = (x.shape[1], x.shape[0]) if transposed_in else x.shape
+    dev = x.device
+    m = _matrix_arg(matrix, dev)
+    codes = torch.empty((rows, cols // 2), dtype=torch.uint8, device=dev)
+    scales = torch.empty((rows, cols // 32), dtype=torch.uint8, device=dev)
+    mask = torch.empty((rows, cols // 8), dtype=torch.uint8, device=dev) if want_mask else None
+    deq = torch.empty((rows, cols), dtype=x.dtype, device=dev) if want_dequant else None
+    rc = _lib.lib().qm_quantize_mxfp4_dense(_ptr(x), _dtype_code(x.dtype), rows, cols, _ptr(m), mode, int(transposed_in), seed,
+                                            _ptr(codes), _ptr(scales), _ptr(mask), _ptr(deq), _layout(tiled), _stream())
+    _lib.check(rc, "qm_quantize_mxfp4_dense")
+    return codes, scales, mask, deq
+
+
+def requantize_transposed_mxfp4_dense(codes, scales, matrix, post=1.0, val_dtype=torch.bfloat16, mode=QM_ABSMAX_SR, seed=0,
+                                      want_dequant=False, tiled_in=False, tiled_out=False):
+    """requantize_transposed_mxfp4 with a dense 32 x 32 rotation.  Same return value."""
+    _require_cuda(codes, scales)
+    assert codes.is_contiguous() and scales.is_contiguous()
+    R, C = codes.shape[0], codes.shape[1] * 2
+    dev = codes.device
+    m = _matrix_arg(matrix, dev)
+    codes_out = torch.empty((C, R // 2), dtype=torch.uint8, device=dev)
+    scales_out = torch.empty((C, R // 32), dtype=torch.uint8, device=dev)
+    deq = torch.empty((C, R), dtype=val_dtype, device=dev) if want_dequant else None
+    rc = _lib.lib().qm_requantize_transposed_mxfp4_dense(_ptr(codes), _ptr(scales), R, C, post, _dtype_code(val_dtype), _ptr(m), mode,
+                                                         seed, _ptr(codes_out), _ptr(scales_out), _ptr(deq), _layout(tiled_in),
+                                                         _layout(tiled_out), _stream())
+    _lib.check(rc, "qm_requantize_transposed_mxfp4_dense")
+    return codes_out, scales_out, deq
+
+
 def requantize_transposed_mxfp4(codes, scales, post=1.0, val_dtype=torch.bfloat16, hadamard_dim=32, sign_bits=None,
                                 mode=QM_ABSMAX_SR, u=None, seed=0, want_dequant=False, tiled_in=False, tiled_out=False):
     """codes [R,C/2], scales [R,C/32] -> (codes [C,R/2], scales [C,R/32], dequant [C,R] | None)."""
@@ -294,7 +339,7 @@ def rope_merge_qkv_grad(dq, dk, dv, table, n_embd, head_dim, seq_len, out_dtype)
 
 
 def linear_backward(e2, packed_x, packed_w, T, I, O, hd_x, signs_x, hd_w, signs_w, hd_g, signs_g, mode, seeds, x_val_dtype,
-                    w_val_dtype, mid_dtype, x_scale_dtype, w_scale_dtype, tiled, gx_rotated=False, gw_dtype=None):
+                    w_val_dtype, mid_dtype, x_scale_dtype, w_scale_dtype, tiled, gx_rotated=False, gw_dtype=None, g_matrix=None):
     """Whole backward pass in one foreign call: e [T,O] -> (gx [T,I], gw [O,I]) of mid_dtype.  With `gx_rotated`, gx is
     still in the rotated basis of the activation quantizer: its masked inverse rotation is left to the kernel that
     consumes gx (rmsnorm_backward / swiglu_backward with `maskbits`).  `gw_dtype` = float32 with a bf16 mid_dtype returns
@@ -312,6 +357,6 @@ def linear_backward(e2, packed_x, packed_w, T, I, O, hd_x, signs_x, hd_w, signs_
                               hd_w, sign_words(signs_w), hd_g, sign_words(signs_g), mode, (ctypes.c_uint64 * 4)(*seeds),
                               _dtype_code(x_val_dtype), _dtype_code(w_val_dtype), mid, _dtype_code(x_scale_dtype),
                               _dtype_code(w_scale_dtype), _ptr(work), nbytes, _ptr(gx), _ptr(gw), _dtype_code(gw_dtype), _layout(tiled),
-                              int(gx_rotated), _stream())
+                              int(gx_rotated), _ptr(g_matrix), _stream())
     _lib.check(rc, "qm_linear_backward")
     return gx, gw

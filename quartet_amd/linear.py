@@ -51,6 +51,8 @@ def _backward_packed(ctx, e, packed_x, packed_w, gx_rotated=False):
     T, I, O = ctx.dims
     g_q.re_randomize()
     hd, signs = g_q.hadamard_dim, g_q.sign_bits
+    # rerotate="O32": the four gradient quantizations rotate by the dense matrix drawn just now, on the matrix pipe
+    g_matrix = g_q.dense_matrix(e.device) if g_q.is_dense else None
     mode = K.QM_ABSMAX_SR if g_q.stochastic else K.QM_ABSMAX_RTN
     # one host-side draw per stochastic quantization, in the order e, W^T, e^T, x^T
     seeds = [_fresh_seed() if g_q.stochastic else 0 for _ in range(4)]
@@ -61,7 +63,7 @@ def _backward_packed(ctx, e, packed_x, packed_w, gx_rotated=False):
     sd_w = torch.bfloat16 if low else ctx.w_dtype
     gx, gw = K.linear_backward(e2, packed_x, packed_w, T, I, O, a_hd, a_signs, w_hd, w_signs, hd, signs, mode, seeds, ctx.x_dtype,
                                ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled, gx_rotated,
-                               ctx.w_dtype if ctx.w_dtype in (torch.float32, torch.bfloat16) else None)
+                               ctx.w_dtype if ctx.w_dtype in (torch.float32, torch.bfloat16) else None, g_matrix)
     if gx_rotated:
         return gx, gw, (K.packed_mask_bits(packed_x, T, I), a_signs, sd_x)
     return gx, gw
@@ -154,11 +156,15 @@ class QuantizedLinear(nn.Linear):
         self.use_packed_path = True
         self.packed_weight_cache = None  # see enable_packed_weight_cache
 
-    def _is_production_config(self):
+    def _is_production_config(self, tokens):
         g_q = self.backward_scheme.g_quantizer
-        # a dense rotation (rerotate="O32") anywhere, now or after the next re_randomize, needs the generic path
+        # a dense rotation (rerotate="O32") in a forward quantizer, now or after the next re_randomize, needs the generic
+        # path; in the gradient quantizer the packed path serves it when every extent is a multiple of 128 and the
+        # Hadamard block it replaces is 32
         dense = any(getattr(q_, "is_dense", False) or getattr(q_, "rerotate", None) == "O32"
-                    for q_ in (self.activation_quantizer, self.weight_quantizer, g_q))
+                    for q_ in (self.activation_quantizer, self.weight_quantizer))
+        if getattr(g_q, "is_dense", False) or getattr(g_q, "rerotate", None) == "O32":
+            dense = dense or g_q.hadamard_dim != 32 or any(d % 128 for d in (tokens, self.in_features, self.out_features))
         return (self.use_packed_path and not dense
                 and type(self.activation_quantizer) is QuestMXFP4Quantizer
                 and type(self.weight_quantizer) is QuestMXFP4Quantizer
@@ -166,7 +172,7 @@ class QuantizedLinear(nn.Linear):
                 and type(self.backward_scheme) is QEQWtt_QEtQXtt_Scheme)
 
     def forward(self, x):
-        if self._is_production_config():
+        if self._is_production_config(x.numel() // max(x.shape[-1], 1)):
             return QuartetLinearFn.apply(x, self.weight, self.activation_quantizer, self.weight_quantizer,
                                          self.backward_scheme.g_quantizer, self.packed_weight_cache)
         xq = self.activation_quantizer(x)

@@ -5,10 +5,9 @@ Differences in representation, not in results:
   * the rotation H = hd^-1/2 * Sylvester * diag(signs) is kept as a sign bit mask; the dense
     ``hadamard_matrix`` attribute is materialised on demand (same values the reference holds);
   * the clip mask saved for backward is bit-packed (1 bit per element);
-  * ``rerotate="O32"`` replaces H by a dense random orthogonal matrix (mxfp4.py:61-64).  The butterfly kernels cannot
-    apply it, so the rotation runs as a library matrix product (fp32 accumulation over the tensor's dtype, which is
-    what the reference's in-kernel ``tl.dot`` does) and the kernel quantizes the rotated groups as they are; a layer
-    whose quantizers hold a dense rotation takes the generic (pseudo-quantized) path.
+  * ``rerotate="O32"`` replaces H by a dense random orthogonal matrix (mxfp4.py:61-64).  The kernels apply it on the
+    matrix pipe (fp32 multiply-adds over the matrix rounded to the tensor's dtype, the role of the reference's
+    in-kernel ``tl.dot``); a layer whose *gradient* quantizer holds a dense rotation stays on the packed FP4 path.
 """
 import random
 import weakref
@@ -95,7 +94,10 @@ def mxfp4_forward_kernel_wrapper(x, hadamard_matrix, return_clip_mask=False, gau
         (K.QM_ABSMAX_SR if stochastic_round else K.QM_ABSMAX_RTN)
     seed = _fresh_seed() if stochastic_round else 0
     sign_bits = sylvester_sign_bits(hadamard_matrix)
-    if sign_bits is None:
+    if sign_bits is None and hd == 32:
+        _, _, mask, deq = K.quantize_mxfp4_dense(_as_2d(x, 32), hadamard_matrix, mode, seed=seed, want_mask=return_clip_mask,
+                                                 want_dequant=True)
+    elif sign_bits is None:   # a dense matrix of another size: library product, then the kernel quantizes the groups as they are
         _, _, mask, deq = K.quantize_mxfp4(_rotate_dense(x, hadamard_matrix), 1, None, mode, seed=seed,
                                            want_mask=return_clip_mask, want_dequant=True)
         deq = deq.to(x.dtype)
@@ -117,6 +119,7 @@ class _HadamardQuantizer(BaseQuantizer):
         self.rerotate = rerotate
         self.sign_bits = 0  # bit j set = column j of H negated
         self._dense = None  # fp32 [hd, hd] orthogonal matrix once re_randomize("O32") has replaced H
+        self._dense_dev = None  # its copy on the device of the tensors being quantized
         self._matrix_dtype = torch.float32
         self._matrix_device = torch.device("cpu")
 
@@ -133,6 +136,15 @@ class _HadamardQuantizer(BaseQuantizer):
         h = sylvester_matrix(hd) * torch.tensor(hd ** -0.5, dtype=torch.float32) * signs[None, :]
         return h.to(self._matrix_device).to(self._matrix_dtype)
 
+    def dense_matrix(self, device):
+        """The dense rotation as the kernels read it (fp32 [32, 32] on `device`), or None while H is a signed Hadamard
+        matrix.  Kept on the device until the next re_randomize replaces it."""
+        if self._dense is None:
+            return None
+        if self._dense_dev is None or self._dense_dev.device != torch.device(device):
+            self._dense_dev = self._dense.to(device=device, dtype=torch.float32).contiguous()
+        return self._dense_dev
+
     def _note_input(self, x):
         # the reference re-casts its matrix to the input's device and dtype on every call (mxfp4.py:49,160)
         self._matrix_dtype, self._matrix_device = x.dtype, x.device
@@ -148,6 +160,7 @@ class _HadamardQuantizer(BaseQuantizer):
             # H <- U V^T of the SVD of a Gaussian matrix (mxfp4.py:61-64): Haar-distributed up to signs
             u, _, vh = torch.linalg.svd(torch.randn(self.hadamard_dim, self.hadamard_dim))
             self._dense = (u @ vh).contiguous()
+            self._dense_dev = None
             self.sign_bits = 0
         elif self.rerotate is None:
             pass
@@ -168,15 +181,14 @@ def _unpack_mask(maskbits, shape):
 
 
 class DenseRotationQuantizerFn(torch.autograd.Function):
-    """Either quantizer with a dense rotation: rotate by a matrix product, quantize the rotated groups of 32 as they
-    are (kernel block size 1), straight-through backward ``(g * mask) @ matrix^T`` (mxfp4.py:30-34,143-146)."""
+    """Either quantizer with a dense 32 x 32 rotation: the kernel rotates every group of 32 on the matrix pipe and
+    quantizes it; straight-through backward ``(g * mask) @ matrix^T`` (mxfp4.py:30-34,143-146)."""
 
     @staticmethod
     def forward(ctx, x, matrix, mode, want_mask, post_scale):
-        xr = _rotate_dense(x, matrix)
         stochastic = mode in (K.QM_ABSMAX_SR, K.QM_QUEST_SR)
-        _, _, maskbits, deq = K.quantize_mxfp4(xr, 1, None, mode, seed=_fresh_seed() if stochastic else 0,
-                                               want_mask=want_mask, want_dequant=True)
+        _, _, maskbits, deq = K.quantize_mxfp4_dense(_as_2d(x, 32), matrix, mode, seed=_fresh_seed() if stochastic else 0,
+                                                     want_mask=want_mask, want_dequant=True)
         if post_scale != 1.0:
             deq *= post_scale
         ctx.save_for_backward(matrix, maskbits) if want_mask else ctx.save_for_backward(matrix)

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_function():
 
 def test_host_only_entry_points():
     L = _lib.lib()
-    assert L.qm_version() == 9
+    assert L.qm_version() == 10
     T, I, O = 256, 128, 384
     off = (ctypes.c_size_t * 3)()
     for rows, cols in ((T, I), (O, I)):
@@ -61,6 +61,11 @@ def test_host_only_entry_points():
     (lambda L: L.qm_gemm_mxfp4_tn(None, None, None, None, 64, 64, 48, 1.0, None, 0, 0, 0, None, 0, None), b"qm_gemm_mxfp4_tn"),
     # an output offset by 4 bytes: the tile kernels store 16-byte pieces, so the call is refused before any launch
     (lambda L: L.qm_gemm_mxfp4_tn(0x1000, 0x2000, 0x3000, 0x4000, 256, 256, 128, 1.0, 0x5004, 0, 0, 0, None, 0, None), b"c need 16-byte"),
+    (lambda L: L.qm_quantize_mxfp4_dense(None, 0, 4, 40, None, 1, 0, 0, None, None, None, None, 0, None), b"multiple of 32"),
+    (lambda L: L.qm_quantize_mxfp4_dense(None, 0, 4, 64, None, 1, 0, 0, None, None, None, None, 0, None), b"non-null"),
+    (lambda L: L.qm_quantize_mxfp4_dense(0x1000, 0, 64, 64, 0x2000, 1, 1, 0, 0x3000, 0x4000, None, None, 0, None), b"transposed input needs"),
+    (lambda L: L.qm_requantize_transposed_mxfp4_dense(None, None, 64, 64, 1.0, 0, None, 2, 0, None, None, None, 0, 0, None), b"R % 128"),
+    (lambda L: L.qm_requantize_transposed_mxfp4_dense(None, None, 128, 64, 1.0, 0, None, 2, 0, None, None, None, 0, 0, None), b"null tensor"),
     (lambda L: L.qm_masked_hadamard_bwd(None, 0, 4, 40, 32, 0, None, None, None, 0, None), b"multiple of hadamard_dim"),
     (lambda L: L.qm_dequantize_mxfp4(None, None, 4, 40, 1.0, None, 0, None), b"C % 32"),
     (lambda L: L.qm_linear_forward(None, 0, None, 0, 64, 40, 64, 32, None, 32, None, None, 0, None, 0, 0, None, 0, 0, None), b"multiple of 32"),

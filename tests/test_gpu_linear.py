@@ -184,9 +184,9 @@ def test_notebook_error_bands_on_gpu(q):
                                                      ("AlbertTsengQuantizer", "ABSMAX_SR", 1.0),
                                                      ("AlignedAlbertTsengQuantizer", "ABSMAX_RTN", 1.009276)])
 def test_dense_rotation_quantizers_against_oracle(oracle, q, cls_name, mode_name, post):
-    """rerotate="O32": the module rotates by a matrix product and the kernel quantizes the rotated groups; on the
-    same rotated tensor the oracle must give the same pseudo-quantized values, and the backward pass is the
-    (masked) product with the transposed matrix."""
+    """rerotate="O32": the kernel rotates every group of 32 by the module's dense matrix and quantizes it; the oracle
+    with the same matrix must give the same pseudo-quantized values bit for bit, and the backward pass is the (masked)
+    product with the transposed matrix."""
     print(f"case dense rotation {cls_name}", flush=True)
     import random
     dev = "cuda:0"
@@ -198,14 +198,15 @@ def test_dense_rotation_quantizers_against_oracle(oracle, q, cls_name, mode_name
     y = quant(x)
     R = quant.hadamard_matrix
     assert R.dtype == torch.bfloat16 and R.device.type == "cuda"
-    xr = (x.detach().reshape(-1, 32).float() @ R.float()).view(48, 256)
     random.seed(4)
     seed = random.getrandbits(63) if "SR" in mode_name else 0
-    want = oracle.quantize(xr.cpu().numpy(), 1, mode=getattr(oracle, mode_name), seed=seed, want_mask=True, want_dequant=True)
-    ref = torch.from_numpy(want["dequant"])
+    want = oracle.quantize(to_oracle(x.detach()), mode=getattr(oracle, mode_name), seed=seed, want_mask=True, want_dequant=True,
+                           matrix=quant._dense.numpy())
+    from tests.util import from_oracle_bf16
+    ref = from_oracle_bf16(want["dequant"])
     if post != 1.0:
-        ref = ref * post
-    assert torch.equal(y.detach().cpu(), ref.to(torch.bfloat16))
+        ref = ref * post   # the module scales the kernel's bf16 result in place
+    assert torch.equal(y.detach().cpu(), ref)
     g = make_input(48, 256, torch.bfloat16, seed=13).to(dev)
     y.backward(g)
     gm = g.float()
@@ -216,30 +217,54 @@ def test_dense_rotation_quantizers_against_oracle(oracle, q, cls_name, mode_name
     assert float((x.grad.float() - gref).norm() / gref.norm()) < 1e-2   # the module's product runs in bf16
 
 
-def test_layer_with_dense_gradient_rotation(q):
-    """The production configuration with rerotate="O32" on the gradient quantizer (generic path): gradients stay as
-    close to the unquantized ones as with sign flips."""
+def test_layer_with_dense_gradient_rotation(oracle, q):
+    """The production configuration with rerotate="O32" on the gradient quantizer stays on the packed FP4 path (the
+    four gradient quantizations rotate by the dense matrix on the matrix pipe): the step must equal the oracle pipeline
+    with the same matrix and seeds, and gradients stay as close to the unquantized ones as with sign flips."""
     print("case layer with O32 gradient rotation", flush=True)
+    T, I, O = 256, 512, 128
     g = torch.Generator().manual_seed(0)
-    x = torch.randn(256, 512, generator=g).to(torch.bfloat16).to("cuda:0")
-    w = torch.randn(128, 512, generator=g).to(torch.bfloat16).to("cuda:0")
-    dy = torch.randn(256, 128, generator=g).to(torch.bfloat16).to("cuda:0")
+    x = torch.randn(T, I, generator=g).to(torch.bfloat16)
+    w = torch.randn(O, I, generator=g).to(torch.bfloat16)
+    dy = torch.randn(T, O, generator=g).to(torch.bfloat16)
     wref = w.clone().float().requires_grad_(True)
     xref = x.clone().float().requires_grad_(True)
     torch.nn.functional.linear(xref, wref).backward(dy.float())
-    err = lambda a, b: float(((a.detach().float() - b.detach().float()) ** 2).sum() / (b.detach().float() ** 2).sum())
+    err = lambda a, b: float(((a.detach().float().cpu() - b.detach().float()) ** 2).sum() / (b.detach().float() ** 2).sum())
     errs = {}
     for rr in ("signs", "O32"):
         torch.manual_seed(1)
-        layer = production_layer(q, 512, 128, True, rr, torch.bfloat16)
+        random.seed(9)
+        layer = production_layer(q, I, O, True, rr, torch.bfloat16)
+        assert layer._is_production_config(T)
         with torch.no_grad():
             layer.weight.copy_(w)
-        xin = x.clone().requires_grad_(True)
+        xin = x.clone().to("cuda:0").requires_grad_(True)
         with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
             y = layer(xin)
-        y.backward(dy)
-        assert layer.backward_scheme.g_quantizer.is_dense == (rr == "O32")
+        y.backward(dy.to("cuda:0"))
+        g_q = layer.backward_scheme.g_quantizer
+        assert g_q.is_dense == (rr == "O32")
         errs[rr] = (err(xin.grad, xref.grad), err(layer.weight.grad, wref.grad))
+        if rr == "O32":
+            # the oracle pipeline with the matrix the layer drew and the seeds it used
+            random.seed(9)
+            seeds = [random.getrandbits(63) for _ in range(4)]
+            H = g_q._dense.numpy()
+            d = float(oracle.FOUR_THIRDS)
+            qx = oracle.quantize(to_oracle(x), 32, mode=oracle.QUEST_RTN, want_mask=True)
+            qw = oracle.quantize(to_oracle(w), 32, mode=oracle.QUEST_RTN, want_mask=True)
+            qe = oracle.quantize(to_oracle(dy), mode=oracle.ABSMAX_SR, seed=seeds[0], matrix=H)
+            qwt = oracle.requantize_transposed(qw["codes"], qw["scales"], val_dtype=oracle.BF16, mode=oracle.ABSMAX_SR, seed=seeds[1], matrix=H)
+            gxq = oracle.gemm_tn(qe["codes"], qe["scales"], qwt["codes"], qwt["scales"], a_post=d, b_post=d)
+            qet = oracle.quantize(to_oracle(dy), mode=oracle.ABSMAX_SR, transposed_in=True, seed=seeds[2], matrix=H)
+            qxt = oracle.requantize_transposed(qx["codes"], qx["scales"], val_dtype=oracle.BF16, mode=oracle.ABSMAX_SR, seed=seeds[3], matrix=H)
+            gwq = oracle.gemm_tn(qet["codes"], qet["scales"], qxt["codes"], qxt["scales"], a_post=d, b_post=d)
+            from tests.util import from_oracle_bf16
+            gx_ref = from_oracle_bf16(oracle.masked_hadamard_bwd(to_oracle(torch.from_numpy(gxq).to(torch.bfloat16)), 32, oracle.BF16, None, qx["mask"]))
+            gw_ref = from_oracle_bf16(oracle.masked_hadamard_bwd(to_oracle(torch.from_numpy(gwq).to(torch.bfloat16)), 32, oracle.BF16, None, qw["mask"]))
+            assert rel(xin.grad.float().cpu(), gx_ref.float()) < 1e-2
+            assert rel(layer.weight.grad.float().cpu(), gw_ref.float()) < 1e-2
     print(f"relative squared gradient errors {errs}", flush=True)
     for k in (0, 1):
         assert 0.03 < errs["O32"][k] < 0.3 and abs(errs["O32"][k] - errs["signs"][k]) < 0.5 * errs["signs"][k]

@@ -338,3 +338,76 @@ def test_empty_and_rejected_inputs(K):
         K.quantize_mxfp4(torch.zeros(4, 64, dtype=torch.bfloat16, device=dev), hadamard_dim=16)
     with pytest.raises(QuartetHipError):
         K.quantize_mxfp4(torch.zeros(4, 64, dtype=torch.bfloat16))  # CPU tensor: no fallback
+
+
+def _orthogonal(seed):
+    """A dense 32 x 32 rotation as re_randomize("O32") draws it: U V^T of a Gaussian matrix's SVD."""
+    g = torch.Generator().manual_seed(seed)
+    u, _, vh = torch.linalg.svd(torch.randn(32, 32, generator=g))
+    return (u @ vh).contiguous()
+
+
+def _same_bits(got, want, tag):
+    for name in ("scales", "codes", "mask", "dequant"):
+        if want.get(name) is None or got.get(name) is None:
+            continue
+        g, w = to_oracle(got[name]), want[name]
+        if g.dtype == np.float32:
+            g, w = g.view(np.uint32), w.view(np.uint32)
+        bad = int((g != w).sum())
+        assert bad == 0, f"{tag}: {name} differs in {bad} of {w.size} entries"
+
+
+@pytest.mark.parametrize("mode", ["quest_rtn", "absmax_rtn", "absmax_sr"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_dense_rotation_kernels_bit_exact(oracle, K, mode, dtype):
+    """rerotate="O32": every group of 32 is multiplied by a dense 32 x 32 matrix on the matrix pipe (one fused
+    multiply-add per term, ascending k) and quantized.  Codes, scales, mask bits and de-quantized values must equal
+    the oracle's bit for bit: row-major input (ragged and tiled shapes), transposed input, and the transposing
+    re-quantizer of a packed tensor, with the in-kernel random stream for stochastic rounding."""
+    print(f"case dense rotation mode={mode} dtype={dtype}", flush=True)
+    dev = torch.device("cuda:0")
+    H = _orthogonal(17)
+    m = MODES[mode]
+    want_mask = mode == "quest_rtn"
+    seed = 0xABCD_1234_5678 if "sr" in mode else 0
+    odt = oracle.BF16 if dtype == torch.bfloat16 else oracle.F32
+    for rows, cols, tiled in ((100, 96, False), (272, 640, False), (128, 256, True)):
+        x = make_input(rows, cols, dtype, seed=rows + cols, zero_rows=1)
+        codes, scales, mask, deq = K.quantize_mxfp4_dense(x.to(dev), H.to(dev), m, seed=seed, want_mask=want_mask, want_dequant=True,
+                                                          tiled=tiled)
+        ref = oracle.quantize(to_oracle(x), mode=m, seed=seed, want_mask=want_mask, want_dequant=True, matrix=H.numpy())
+        _same_bits(dict(scales=scales, codes=K.untile_codes(codes) if tiled else codes, mask=mask, dequant=deq), ref,
+                   f"dense rowmajor {rows}x{cols} tiled={tiled}")
+    if mode != "quest_rtn":   # the transposing kernels serve the gradient quantizer: no clip mask
+        for p, q_, tiled in ((256, 72, False), (128, 200, False), (256, 80, True)):
+            x = make_input(p, q_, dtype, seed=p + q_)   # physical [P, Q]; logical [Q, P]
+            codes, scales, _, deq = K.quantize_mxfp4_dense(x.to(dev), H.to(dev), m, transposed_in=True, seed=seed, want_dequant=True,
+                                                           tiled=tiled)
+            ref = oracle.quantize(to_oracle(x), mode=m, seed=seed, transposed_in=True, want_dequant=True, matrix=H.numpy())
+            _same_bits(dict(scales=scales, codes=K.untile_codes(codes) if tiled else codes, dequant=deq), ref,
+                       f"dense transposed {p}x{q_} tiled={tiled}")
+        for R, C, tiled in ((256, 96, False), (640, 160, False), (512, 256, True), (1152, 128, True)):
+            src = make_input(R, C, torch.bfloat16, seed=R + C)
+            qc = oracle.quantize(to_oracle(src), 32, mode=oracle.QUEST_RTN)
+            cin = torch.from_numpy(qc["codes"]).to(dev)
+            sin = torch.from_numpy(qc["scales"]).to(dev)
+            codes, scales, deq = K.requantize_transposed_mxfp4_dense(K.tile_codes(cin) if tiled else cin, sin, H.to(dev), 1.0, dtype, m,
+                                                                     seed=seed, want_dequant=True, tiled_in=tiled, tiled_out=tiled)
+            ref = oracle.requantize_transposed(qc["codes"], qc["scales"], 1.0, odt, mode=m, seed=seed, want_dequant=True,
+                                               matrix=H.numpy())
+            _same_bits(dict(scales=scales, codes=K.untile_codes(codes) if tiled else codes, dequant=deq), ref,
+                       f"dense requantize {R}x{C} tiled={tiled}")
+
+
+def test_dense_rotation_with_the_hadamard_matrix_is_close_to_the_butterfly(oracle, K):
+    """The Hadamard matrix handed over as a dense matrix: same scales, and codes that differ only where the two
+    summation orders round a rotated value differently."""
+    dev = torch.device("cuda:0")
+    x = make_input(256, 512, torch.bfloat16, seed=5)
+    c = float(oracle.hadamard_scale(32, oracle.BF16))
+    Hd = torch.from_numpy(oracle.sylvester(32).astype(np.float32) * np.float32(c))
+    a = K.quantize_mxfp4(x.to(dev), 32, None, K.QM_QUEST_RTN, want_mask=True)
+    b = K.quantize_mxfp4_dense(x.to(dev), Hd.to(dev), K.QM_QUEST_RTN, want_mask=True)
+    assert torch.equal(a[1], b[1])
+    assert float((a[0] != b[0]).float().mean()) < 0.01

@@ -57,13 +57,84 @@ def test_classifier_tells_signed_sylvester_from_everything_else():
     assert sylvester_sign_bits(torch.linalg.qr(torch.randn(32, 32))[0]) is None
 
 
-def test_layer_with_a_dense_rotation_takes_the_generic_path():
-    make = lambda rr: q.QuantizedLinear(64, 64, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(),
-                                        activation_quantizer=q.QuestMXFP4Quantizer(),
-                                        gradient_quantizer=q.AlbertTsengQuantizer(stochastic=True, rerotate=rr),
-                                        backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]())
-    assert make("signs")._is_production_config()
-    assert not make("O32")._is_production_config()
+def test_which_layers_with_a_dense_rotation_stay_on_the_packed_path():
+    """A dense rotation in the gradient quantizer is served by the packed FP4 path when every extent is a multiple of
+    128; in a forward quantizer, or at other shapes, the layer takes the generic path."""
+    def make(rr, fwd_rr=None, features=256):
+        return q.QuantizedLinear(features, features, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(rerotate=fwd_rr),
+                                 activation_quantizer=q.QuestMXFP4Quantizer(),
+                                 gradient_quantizer=q.AlbertTsengQuantizer(stochastic=True, rerotate=rr),
+                                 backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]())
+    assert make("signs")._is_production_config(256) and make("signs", features=64)._is_production_config(32)
+    assert make("O32")._is_production_config(256)
+    assert not make("O32")._is_production_config(160)          # tokens not a multiple of 128
+    assert not make("O32", features=64)._is_production_config(256)
+    assert not make("signs", fwd_rr="O32")._is_production_config(256)
+    dense64 = make("O32")
+    dense64.backward_scheme.g_quantizer.hadamard_dim = 64
+    assert not dense64._is_production_config(256)
+
+
+def test_oracle_dense_rotation_is_the_fma_chain_and_reduces_to_known_cases(oracle):
+    """The dense rotation's canonical order: out[j] = fma(g[31], H[31][j], ... fma(g[0], H[0][j], 0)).  Pinned by a
+    float64 evaluation (every fused step rounds once: emulated exactly with Python fractions on a small case), by the
+    identity matrix (pass-through mode), by a permutation matrix, and by the Hadamard matrix itself (same rotated
+    values as the butterfly to rounding)."""
+    from fractions import Fraction
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((2, 32)).astype(np.float32)
+    H = np.linalg.qr(rng.standard_normal((32, 32)))[0].astype(np.float32)
+    got = oracle.quantize(x, mode=oracle.ABSMAX_RTN, want_rotated=True, matrix=H)["rotated"]
+
+    def fl32(fr):   # round a Fraction to the nearest float32 (ties to even), via exact integer arithmetic
+        if fr == 0:
+            return np.float32(0.0)
+        sign = -1 if fr < 0 else 1
+        fr = abs(fr)
+        e = 0
+        while fr >= 2:
+            fr /= 2
+            e += 1
+        while fr < 1:
+            fr *= 2
+            e -= 1
+        scaled = fr * (1 << 23)
+        n = scaled.numerator // scaled.denominator
+        rem = scaled - n
+        if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and n % 2 == 1):
+            n += 1
+        return np.float32(sign * float(Fraction(n, 1 << 23) * Fraction(2) ** e))
+    for r in range(2):
+        for j in (0, 7, 31):
+            acc = Fraction(0)
+            for k in range(32):
+                acc = Fraction(float(fl32(Fraction(float(x[r, k])) * Fraction(float(H[k, j])) + acc)))
+            assert np.float32(float(acc)) == got[r, j], (r, j)
+    # identity = pass-through, permutation = reordering, both exact
+    same = oracle.quantize(x, mode=oracle.ABSMAX_RTN, want_rotated=True, matrix=np.eye(32, dtype=np.float32))
+    assert np.array_equal(same["rotated"], x)
+    perm = rng.permutation(32)
+    P = np.zeros((32, 32), dtype=np.float32)
+    P[perm, np.arange(32)] = 1.0
+    assert np.array_equal(oracle.quantize(x, mode=oracle.ABSMAX_RTN, want_rotated=True, matrix=P)["rotated"], x[:, perm])
+    # the Hadamard matrix as a dense matrix: the butterfly's values up to summation order
+    xb = make_input(8, 128, torch.bfloat16, seed=2)
+    c = float(oracle.hadamard_scale(32, oracle.BF16))
+    Hd = oracle.sylvester(32).astype(np.float32) * np.float32(c)
+    a = oracle.quantize(to_oracle(xb), 32, mode=oracle.QUEST_RTN, want_rotated=True, want_mask=True)
+    b = oracle.quantize(to_oracle(xb), mode=oracle.QUEST_RTN, want_rotated=True, want_mask=True, matrix=Hd)
+    assert np.abs(a["rotated"] - b["rotated"]).max() <= 1e-6 * np.abs(a["rotated"]).max()
+    assert (a["codes"] != b["codes"]).mean() < 0.01 and np.array_equal(a["scales"], b["scales"])
+    # the matrix is rounded to the tensor's dtype first (the reference casts it, mxfp4.py:49)
+    Hb = torch.from_numpy(H).to(torch.bfloat16).float().numpy()
+    r1 = oracle.quantize(to_oracle(xb), mode=oracle.ABSMAX_RTN, want_rotated=True, matrix=H)
+    r2 = oracle.quantize(to_oracle(xb), mode=oracle.ABSMAX_RTN, want_rotated=True, matrix=Hb)
+    assert np.array_equal(r1["rotated"], r2["rotated"]) and np.array_equal(r1["codes"], r2["codes"])
+    # the transposing re-quantizer rotates the same way: against quantizing the de-quantized, transposed tensor
+    qx = oracle.quantize(to_oracle(make_input(128, 64, torch.bfloat16, seed=4)), 32, mode=oracle.QUEST_RTN, want_dequant=True)
+    rq = oracle.requantize_transposed(qx["codes"], qx["scales"], val_dtype=oracle.BF16, mode=oracle.ABSMAX_RTN, matrix=H)
+    direct = oracle.quantize(np.ascontiguousarray(qx["dequant"].T), mode=oracle.ABSMAX_RTN, matrix=H)
+    assert np.array_equal(rq["codes"], direct["codes"]) and np.array_equal(rq["scales"], direct["scales"])
 
 
 @pytest.mark.parametrize("mode", ["QUEST_RTN", "ABSMAX_RTN", "ABSMAX_SR"])
