@@ -15,10 +15,12 @@
 // instruction needs.
 //
 // Three kernels, picked by shape in gemm_mxfp4_tn() at the end of the file:
-//   gemm_mxfp4_tn_big4_kernel  M, N multiples of 64 and >= 256, K % 512 == 0.  Persistent, 256x256 macro tile,
-//                              4 waves x 128x128, operands global -> LDS directly into a 4-stage ring, scales in
-//                              blocks of four K steps, row-major or tiled code bytes, optional split-K.
-//   gemm_mxfp4_tn_big_kernel   same tile for other K % 128 == 0: one workgroup per tile, scales per K step.
+//   gemm_mxfp4_tn_big4_kernel  M, N multiples of 64 and >= 256, K % 512 == 0, or another multiple of 128 that pads to
+//                              whole blocks of four K steps with at most an eighth more work.  Persistent, 256x256
+//                              macro tile, 4 waves x 128x128, operands global -> LDS directly into a 4-stage ring,
+//                              scales in blocks of four K steps, row-major or tiled code bytes, optional split-K.
+//   gemm_mxfp4_tn_big_kernel   same tile for the remaining K % 128 == 0 (short K): one workgroup per tile, scales per
+//                              K step.
 //   gemm_mxfp4_tn_kernel       any M, N and K % 32 == 0: 128x128 macro tile, 4 waves x 64x64, operands staged
 //                              global -> registers -> LDS (rows padded from 64 to 80 bytes so the 16-byte fragment
 //                              reads of 16 consecutive rows hit 64 distinct banks), double buffered.
@@ -541,7 +543,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                        (int)(N - n0) - wn * 128);
 }
 
-// ---- variant for K % 512 == 0: scales travel in blocks of four K steps -----------------------------
+// ---- persistent variant: scales travel in blocks of four K steps ------------------------------------
 // Fetching one scale dword per row per K step costs as many L2 requests as the codes themselves (each
 // row's 4 bytes sit in a different cache line).  Here a wave-load brings 16 bytes per row = the scales of
 // four K steps, into a small double-buffered LDS area behind the four code stages; a lane reads the
@@ -577,10 +579,11 @@ __device__ __forceinline__ void big4_issue_codes(const Big4Plan& p, int stage, i
         load_lds_b128_s(p.b + j * p.row16_bytes + ks * p.kstep_b, p.lane_codes_b, base + kBOff + j * 1024);
     }
 }
-__device__ __forceinline__ void big4_issue_scales(const Big4Plan& p, int qb, int buf) {
+// soff: byte offset, within a row's scales, of the 16 bytes (four K steps) to request
+__device__ __forceinline__ void big4_issue_scales(const Big4Plan& p, int soff, int buf) {
     const uint32_t base = p.lds_scales + buf * kScaleBufBytes;
-    load_lds_b128_s(p.sa + qb * 16, p.lane_scales, base);
-    load_lds_b128_s(p.sb + qb * 16, p.lane_scales, base + kBigM * 16);
+    load_lds_b128_s(p.sa + soff, p.lane_scales, base);
+    load_lds_b128_s(p.sb + soff, p.lane_scales, base + kBigM * 16);
 }
 
 // The LDS destination of a global->LDS load is M0 + the instruction's offset + lane * 16, and the same offset is added
@@ -619,15 +622,19 @@ struct Big4State {
 
 // One K step of the flat (tile, K step) stream; the step's index in its tile is congruent to Q mod 4, so
 // the ring stage it consumes is Q.  `lks` is the K step (of the tile `plan` points at) whose codes it
-// requests into the stage it has just freed; `par` selects the scale buffer the current block lives in.
+// requests into the stage it has just freed, `soff` (Q = 0 only) the byte offset of the scale block it requests;
+// `sw` = 16, or 0 for a step whose scale bytes are to read as zero (2^-127: its products vanish); `par` selects the
+// scale buffer the current block lives in.
 template <int Q, bool SWAP, bool FIRST = false>
-__device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_bytes, int lks, int par, int a_off0,
+__device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_bytes, int lks, int soff, int sw, int par, int a_off0,
                                           int a_off1, int b_off0, int b_off1, int a_sc_off, int b_sc_off, int sh,
                                           Big4State& st, v16f (&acc)[4][4]) {
     const uint8_t* cur = smem_bytes + Q * kCodeStageBytes;
     const uint8_t* nxt = smem_bytes + ((Q + 1) & 3) * kCodeStageBytes;
-    const uint32_t sca[4] = {pick<Q>(st.sr.a[0]) >> sh, pick<Q>(st.sr.a[1]) >> sh, pick<Q>(st.sr.a[2]) >> sh, pick<Q>(st.sr.a[3]) >> sh};
-    const uint32_t scb[4] = {pick<Q>(st.sr.b[0]) >> sh, pick<Q>(st.sr.b[1]) >> sh, pick<Q>(st.sr.b[2]) >> sh, pick<Q>(st.sr.b[3]) >> sh};
+    // the lane half's two scale bytes of this step: bits [sh, sh + 16) of the row's dword; sw = 0 mutes the step
+    const auto two = [&](const uint4& v) { return __builtin_amdgcn_ubfe(pick<Q>(v), (uint32_t)sh, (uint32_t)sw); };
+    const uint32_t sca[4] = {two(st.sr.a[0]), two(st.sr.a[1]), two(st.sr.a[2]), two(st.sr.a[3])};
+    const uint32_t scb[4] = {two(st.sr.b[0]), two(st.sr.b[1]), two(st.sr.b[2]), two(st.sr.b[3])};
     big_read_sub(cur, a_off1, b_off1, st.f1);
     big_mfma_sub<0, SWAP, FIRST>(st.f0, sca, scb, acc);
     QM_SCHED_PAIR(0x100, 8)
@@ -671,7 +678,7 @@ __device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_by
             if (i == 2) load_lds_b128_m0<1>(src_b, plan.voff_b[1]);
             if (i == 3) load_lds_b128_m0<3>(src_b, plan.voff_b[3]);
             if constexpr (Q == 0) {
-                if (i == 3) big4_issue_scales(plan, lks >> 2, par ^ 1);
+                if (i == 3) big4_issue_scales(plan, soff, par ^ 1);
             }
             products(0, 4);
             __builtin_amdgcn_sched_barrier(0);
@@ -746,7 +753,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int code_pitch = K / 2, groups = K / 32;
     // Split K: a work item is (tile, K range); with splits > 1 (fp32 instantiation only) item (t, s) covers K steps
     // [s * nk, (s + 1) * nk) and stores its partial sums, unscaled, into slab s of c = [splits][M][N].
-    const int nk = K / kBK / splits;  // K steps per work item, a multiple of 4
+    // K steps per work item.  The pipeline walks blocks of four steps.  When K is not a multiple of 512 (one work item
+    // then) the last block covers the row's final four steps, and those of them that the block before has already
+    // added are muted: their scale bytes read as zero (2^-127 each), so every product is below the smallest fp32
+    // denormal and adds an exact zero.  No request leaves the operand's rows.
+    const int nk_real = K / kBK / splits;
+    const int nk = (nk_real + 3) & ~3;
+    const int muted = nk - nk_real;  // steps of the last block that repeat the block before (0: K steps in whole blocks)
     const int total_items = total * splits;
     const int stride = (int)gridDim.x;
 
@@ -790,7 +803,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         int64_t m0 = (int64_t)load_tm * kBigM + wave_u * 64, n0 = (int64_t)load_tn * kBigN + wave_u * 64;
         m0 = m0 < M ? m0 : (int64_t)M - 64;
         n0 = n0 < N ? n0 : (int64_t)N - 64;
-        const int64_t k0 = (int64_t)load_split * nk;  // first K step of the item
+        const int64_t k0 = (int64_t)load_split * nk_real;  // first K step of the item
         plan.a = a_codes + m0 * code_pitch + k0 * plan.kstep_a;
         plan.b = b_codes + n0 * code_pitch + k0 * plan.kstep_b;
         plan.sa = a_scales + m0 * groups + k0 * 4;
@@ -798,7 +811,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     };
 
     plan_tile((int)blockIdx.x);
-    big4_issue_scales(plan, 0, 0);
+    big4_issue_scales(plan, 0, 0);  // K >= 512: the first block is a whole one
     big4_issue_codes(plan, 0, 0);
     big4_issue_codes(plan, 1, 1);
     big4_issue_codes(plan, 2, 2);
@@ -831,10 +844,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     lks = ks;
                 }
             }
-            big4_step<0, sizeof(OutT) == 2, FIRST>(plan, smem_bytes, lks, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
-            big4_step<1, sizeof(OutT) == 2>(plan, smem_bytes, lks + 1, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
-            big4_step<2, sizeof(OutT) == 2>(plan, smem_bytes, lks + 2, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
-            big4_step<3, sizeof(OutT) == 2>(plan, smem_bytes, lks + 3, par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+            const int lbase = lks + 4 <= nk_real ? lks : nk_real - 4;    // a short last block: the row's final four steps
+            const int first_live = ks + 4 > nk_real ? muted : 0;         // this block's steps below it are muted
+            const auto sw = [&](int q) { return q < first_live ? 0 : 16; };
+            big4_step<0, sizeof(OutT) == 2, FIRST>(plan, smem_bytes, lbase, lbase * 4, sw(0), par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+            big4_step<1, sizeof(OutT) == 2>(plan, smem_bytes, lbase + 1, 0, sw(1), par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+            big4_step<2, sizeof(OutT) == 2>(plan, smem_bytes, lbase + 2, 0, sw(2), par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+            big4_step<3, sizeof(OutT) == 2>(plan, smem_bytes, lbase + 3, 0, sw(3), par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
             par ^= 1;
         };
         block4(0, std::true_type{});
@@ -985,9 +1001,15 @@ hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const 
     const int at = a_layout == LAYOUT_TILED, bt = b_layout == LAYOUT_TILED;
     const bool big_ok = gemm_supports_tiled(M, N, K);
     if ((at || bt) && !big_ok) return hipErrorInvalidValue;
-    if (big_ok && K % 512 == 0 && (reinterpret_cast<uintptr_t>(a_scales) & 15) == 0 && (reinterpret_cast<uintptr_t>(b_scales) & 15) == 0) {
+    // The persistent kernel walks K in blocks of four steps: K % 512 == 0 directly (scale rows are then 16-byte aligned
+    // like their base), other multiples of 128 padded with zero-scale steps when that wastes at most an eighth of the
+    // work (their 16-byte scale requests start at 4-byte aligned addresses)
+    const int64_t nk_real = K / kBK, nk_pad = (nk_real + 3) & ~(int64_t)3;
+    const bool persistent_ok = K % 512 == 0 ? ((reinterpret_cast<uintptr_t>(a_scales) | reinterpret_cast<uintptr_t>(b_scales)) & 15) == 0
+                                            : (nk_real >= 4 && (nk_pad - nk_real) * 8 <= nk_real);
+    if (big_ok && persistent_ok) {
         const int cus = device_cus();
-        int sp = workspace ? choose_splits(M, N, K, cus) : 1;
+        int sp = workspace && K % 512 == 0 ? choose_splits(M, N, K, cus) : 1;  // K ranges are whole blocks of four steps
         if (sp > 1 && ((size_t)sp * M * N * sizeof(float) > workspace_bytes || (reinterpret_cast<uintptr_t>(workspace) & 15))) sp = 1;
         if (sp > 1) {
             // partial sums per K range in fp32 (plain accumulator layout), then one ordered reduction

@@ -624,14 +624,14 @@ struct TransposedJob {
 };
 
 // ---- packed MXFP4 in, transposed + rotated + re-quantized out --------------------------------------------
-// in: codes [R, C/2], scales [R, C/32]; out: the [C, R] tensor quantized along R.  A wave owns 128 rows by 128
-// columns: lane l reads, for the 32 rows of row group l / 16, the four code bytes (eight columns c) at byte column
-// 4 (l % 16) straight from global memory as dwords -- a wave load is four contiguous 64-byte row segments -- plus the
-// rows' E8M0 byte of its column group.  It then handles its eight columns two at a time: the hardware FP4
-// de-quantizing convert turns byte p of each dword into two floats, which gives two groups of 32 along r in registers.
-// A workgroup stacks its four waves along r (512 rows), so that a column's scale bytes leave as one 16-byte piece;
-// codes leave through LDS as whole 64-byte row pieces (tiled output: eight contiguous 1 KiB tiles per wave).
-constexpr int kRqR = 512, kRqC = 128;
+// in: codes [R, C/2], scales [R, C/32]; out: the [C, R] tensor quantized along R.  A wave owns 128 rows by 64
+// columns: lane l reads, for the 32 rows of row group l / 16, the two code bytes (four columns c) at byte column
+// 2 (l % 16) straight from global memory -- a wave load is four contiguous 32-byte row segments, two rows share a
+// register -- plus the rows' E8M0 byte of its column group.  It then handles its four columns two at a time: the
+// hardware FP4 de-quantizing convert turns one byte of each row into two floats, which gives two groups of 32 along r
+// in registers.  A workgroup stacks its four waves along r (512 rows), so that a column's scale bytes leave as one
+// 16-byte piece; codes leave through LDS as whole 64-byte row pieces (tiled output: four contiguous 1 KiB tiles per wave).
+constexpr int kRqR = 512, kRqC = 64;
 
 template <int VAL_DTYPE, int MODE, bool DENSE = false>
 struct RequantJob {
@@ -656,27 +656,30 @@ struct RequantJob {
           grid_r((unsigned)((R_ + kRqR - 1) / kRqR)),
           blocks((unsigned)(((R_ + kRqR - 1) / kRqR) * ((C_ + kRqC - 1) / kRqC))) {}
 
-    // columns 2 P and 2 P + 1 of the lane's eight: de-quantize byte P of the 32 row dwords, rotate, quantize, stage
+    // columns 2 P and 2 P + 1 of the lane's four: de-quantize byte P of the 32 rows, rotate, quantize, stage
     template <int P>
-    __device__ __forceinline__ void column_pair(const uint32_t (&cw)[32], const float (&sc)[32], const DenseFrag& frag, bool active,
-                                                int64_t ca, int64_t rbase, int co, int rg, int wave, uint4* ocodes,
+    __device__ __forceinline__ void column_pair(const uint32_t (&cw)[16], const float (&sc)[32], const DenseFrag& frag, bool active,
+                                                int64_t ca, int64_t rbase, int cq, int rg, int wave, uint4* ocodes,
                                                 uint8_t* oscales) const {
         using T = typename std::conditional<VAL_DTYPE == BF16, uint16_t, float>::type;
         float v[2][32];
 #pragma unroll
-        for (int i = 0; i < 32; ++i) {
-            const v2f pr = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(cw[i], sc[i], P);
-            float a = pr.x, b = pr.y;
-            if (post != 1.0f) {  // absmax-coded input: value = code * 2^k * post, held in val_dtype
-                a *= post;
-                b *= post;
-                if constexpr (VAL_DTYPE == BF16) {
-                    a = bf16_to_f32(f32_to_bf16(a));
-                    b = bf16_to_f32(f32_to_bf16(b));
+        for (int i = 0; i < 32; i += 2) {
+            // cw[i / 2]: bytes 0, 1 = row i, bytes 2, 3 = row i + 1
+            const v2f pr0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(cw[i >> 1], sc[i], P);
+            const v2f pr1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(cw[i >> 1], sc[i + 1], 2 + P);
+            v[0][i] = pr0.x; v[1][i] = pr0.y;
+            v[0][i + 1] = pr1.x; v[1][i + 1] = pr1.y;
+        }
+        if (post != 1.0f) {  // absmax-coded input: value = code * 2^k * post, held in val_dtype
+#pragma unroll
+            for (int gq = 0; gq < 2; ++gq)
+#pragma unroll
+                for (int i = 0; i < 32; ++i) {
+                    float a = v[gq][i] * post;
+                    if constexpr (VAL_DTYPE == BF16) a = bf16_to_f32(f32_to_bf16(a));
+                    v[gq][i] = a;
                 }
-            }
-            v[0][i] = a;
-            v[1][i] = b;
         }
         if constexpr (DENSE) {  // the matrix instruction needs the whole wave, lanes outside the tensor included
             dense_rotate(v[0], frag);
@@ -690,7 +693,7 @@ struct RequantJob {
             if constexpr (!DENSE) rotate_group(v[gq], c, sign_word);
             quantize_group_regs<MODE, false>(v[gq], seed, gi, res);
             if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res);
-            const int cl = 8 * co + 2 * P + gq;
+            const int cl = 4 * cq + 2 * P + gq;
             ocodes[cl * 4 + rg] = make_uint4(res.w[0], res.w[1], res.w[2], res.w[3]);
             oscales[cl * 16 + wave * 4 + rg] = (uint8_t)res.scale_byte;
         }
@@ -705,47 +708,48 @@ struct RequantJob {
         const int64_t r0 = (int64_t)(bid - bc * grid_r) * kRqR, c0 = (int64_t)bc * kRqC;
         const int64_t in_code_pitch = C / 2, in_scale_pitch = C / 32;
         const int64_t rw = r0 + wave * 128;          // this wave's first row
-        const int rg = lane >> 4, co = lane & 15;    // row group within the wave, column octet
+        const int rg = lane >> 4, cq = lane & 15;    // row group within the wave, column quad
         const int64_t rbase = rw + 32 * rg;
-        const int64_t ca = c0 + 8 * co;              // this lane's first column
+        const int64_t ca = c0 + 4 * cq;              // this lane's first column
         const bool active = rbase < R && ca < C;     // R % 32 == 0 and C % 32 == 0: all of a lane's groups or none
-        uint32_t cw[32];
+        uint32_t cw[16];
         float sc[32];
         if (active) {
             // Uniform row pointers (scalar unit) + the lane's 32-bit byte offset: no per-lane 64-bit address math.
             // Tiled input: rows are 64 bytes apart inside a 16-row block, blocks (C / 128) KiB apart.
             const int64_t blk = (C / 128) * 1024;
-            const uint8_t* cu = tiled_in ? codes_in + tiled_code_offset(rw, c0 / 128, C / 128) : codes_in + rw * in_code_pitch + c0 / 2;
-            const uint32_t lane_off = (uint32_t)((tiled_in ? 2 * rg * blk : 32 * rg * in_code_pitch) + 4 * co);
+            const uint8_t* cu = tiled_in ? codes_in + tiled_code_offset(rw, c0 / 128, C / 128) + (c0 & 127) / 2
+                                         : codes_in + rw * in_code_pitch + c0 / 2;
+            const uint32_t lane_off = (uint32_t)((tiled_in ? 2 * rg * blk : 32 * rg * in_code_pitch) + 2 * cq);
             const int64_t row_step = tiled_in ? 64 : in_code_pitch;                 // next row of a 16-row block
             const int64_t block_step = tiled_in ? blk - 16 * 64 : 0;                // extra hop into the next block
             const uint8_t* su = scales_in + rw * in_scale_pitch + c0 / 32;
-            const uint32_t slane_off = (uint32_t)(32 * rg * in_scale_pitch + (co >> 2));
+            const uint32_t slane_off = (uint32_t)(32 * rg * in_scale_pitch + (cq >> 3));
 #pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                cw[i] = *reinterpret_cast<const uint32_t*>(cu + i * row_step + (i >> 4) * block_step + lane_off);
-                sc[i] = u2f((uint32_t)(su + i * in_scale_pitch)[slane_off] << 23);
+            for (int i = 0; i < 32; i += 2) {
+                const uint32_t lo = *reinterpret_cast<const uint16_t*>(cu + i * row_step + (i >> 4) * block_step + lane_off);
+                const uint32_t hi = *reinterpret_cast<const uint16_t*>(cu + (i + 1) * row_step + (i >> 4) * block_step + lane_off);
+                cw[i >> 1] = lo | (hi << 16);
             }
+#pragma unroll
+            for (int i = 0; i < 32; ++i) sc[i] = u2f((uint32_t)(su + i * in_scale_pitch)[slane_off] << 23);
         } else {
 #pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                cw[i] = 0u;
-                sc[i] = 1.0f;
-            }
+            for (int i = 0; i < 16; ++i) cw[i] = 0u;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) sc[i] = 1.0f;
         }
         DenseFrag frag;
         if constexpr (DENSE) load_dense_frag(matrix, VAL_DTYPE, frag);
         uint4* ocodes = ocodes_all[wave];
         uint8_t* oscales = reinterpret_cast<uint8_t*>(oscales_all);
-        column_pair<0>(cw, sc, frag, active, ca, rbase, co, rg, wave, ocodes, oscales);
-        column_pair<1>(cw, sc, frag, active, ca, rbase, co, rg, wave, ocodes, oscales);
-        column_pair<2>(cw, sc, frag, active, ca, rbase, co, rg, wave, ocodes, oscales);
-        column_pair<3>(cw, sc, frag, active, ca, rbase, co, rg, wave, ocodes, oscales);
+        column_pair<0>(cw, sc, frag, active, ca, rbase, cq, rg, wave, ocodes, oscales);
+        column_pair<1>(cw, sc, frag, active, ca, rbase, cq, rg, wave, ocodes, oscales);
         __syncthreads();
         const int64_t code_pitch = R / 2, scale_pitch = R / 32;
-        // codes: each wave writes its own 128 x 64-byte tile
+        // codes: each wave writes its own 64 x 64-byte tile
 #pragma unroll
-        for (int it = 0; it < 8; ++it) {
+        for (int it = 0; it < 4; ++it) {
             const int idx = it * 64 + lane, cl = idx >> 2, part = idx & 3;
             if (c0 + cl < C && rw + part * 32 < R) {
                 const int64_t off = tiled_out ? tiled_code_offset(c0 + cl, rw / 128, R / 128) + part * 16

@@ -85,12 +85,16 @@ def _torch_dequant(codes, scales):
 
 # Shapes the 256x256-tile kernels serve: a single tile, fewer tiles than CUs, more tiles than CUs (each
 # workgroup walks several tiles, with an odd and an even number of scale blocks per tile), and K that is a
-# multiple of 128 but not of 512 (per-step scale loads).
+# multiple of 128 but not of 512 (per-step scale loads on the one-tile-per-workgroup kernel, or padding steps on the
+# persistent one).
 @pytest.mark.parametrize("M,N,K_", [(256, 256, 512), (512, 768, 1024), (4352, 4352, 512), (4608, 4352, 1024),
                                     (768, 512, 1536), (512, 256, 640), (4352, 4608, 384), (8192, 4096, 2048),
                                     # tiles hanging over the edge of M and/or N (extents multiples of 64, not of 256)
                                     (320, 256, 512), (256, 448, 640), (640, 1920, 640), (1728, 640, 1024), (4416, 4160, 512),
                                     (320, 320, 128),
+                                    # K a multiple of 128 that the persistent kernel pads to whole blocks of four steps with
+                                    # zero-scale steps: three, two and one real steps in the last block; one tile and many
+                                    (512, 768, 1920), (4352, 4608, 3840), (320, 256, 3712), (768, 512, 2944), (4608, 4352, 1920),
                                     # few output tiles, long K: cut into K ranges (split-K) when scratch is offered
                                     (512, 256, 8192), (320, 640, 16384), (1920, 640, 4096)])
 @pytest.mark.parametrize("exact", [True, False])
@@ -122,7 +126,7 @@ def test_gemm_tile_kernels(oracle, K, M, N, K_, exact):
 
 
 @pytest.mark.parametrize("M,N,K_", [(256, 256, 512), (768, 512, 1536), (512, 256, 640), (4352, 4608, 1024), (640, 1920, 640),
-                                    (1728, 448, 1024)])
+                                    (1728, 448, 1024), (512, 768, 1920), (640, 384, 3712), (4352, 512, 3840)])
 @pytest.mark.parametrize("a_tiled,b_tiled", [(True, True), (True, False), (False, True)])
 def test_gemm_tiled_operands_match_rowmajor(K, M, N, K_, a_tiled, b_tiled):
     print(f"case gemm tiled {M}x{N}x{K_} a={a_tiled} b={b_tiled}", flush=True)
