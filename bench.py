@@ -299,6 +299,29 @@ def gemm_operand_content(x, w, dy, rounds=3):
     return {k: {"ms": round(sorted(v)[len(v) // 2], 4), "TFLOPs": round(flops / sorted(v)[len(v) // 2] / 1e9, 1)} for k, v in out.items()}
 
 
+def mfma_only_ceiling(x, w, iters=400, rounds=3):
+    """The FP4 matrix instruction alone (no loads, no epilogue) on the bytes of the forward product's real operands, on
+    uniformly random bytes and on zero bytes: what the chip sustains for this instruction at its power limit, which is
+    the ceiling the product's own rate is to be read against."""
+    from quartet_amd import kernels as K
+    xc, _, _, _ = K.quantize_mxfp4(x, 32, None, K.QM_QUEST_RTN, tiled=True)
+    wc, _, _, _ = K.quantize_mxfp4(w, 32, None, K.QM_QUEST_RTN, tiled=True)
+    real = torch.cat([xc.flatten()[: 8 << 20], wc.flatten()[: 8 << 20]]).contiguous()
+    cases = {"quest_rtn_codes_of_the_forward_operands": real,
+             "uniform_random_bytes": torch.randint(0, 256, (16 << 20,), dtype=torch.uint8, device=x.device),
+             "zero_bytes": torch.zeros(16 << 20, dtype=torch.uint8, device=x.device)}
+    out = {}
+    for _ in range(rounds):
+        for name, buf in cases.items():
+            n = [0]
+
+            def run():
+                n[0] = K.mfma_only(buf, iters)
+            ms = time_kernel(run, reps=10, warmup=2, graph=False)
+            out.setdefault(name, []).append(2.0 * 32 * 32 * 64 * n[0] / ms / 1e9)
+    return {k: round(sorted(v)[len(v) // 2], 1) for k, v in out.items()}
+
+
 def llama_step(args, device):
     """Whole-model step of a Llama configuration with every block linear on the Quartet path: bf16 autocast around
     forward and backward, cross-entropy on random ids, AdamW (fp32 state) for the ~800 M configuration."""
@@ -610,6 +633,11 @@ def main():
                                        "achieved": qk["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                        "frac": round(qk["GBps"] / PEAK_HBM_GBS, 4), "traffic": traffic, "traffic_source": source,
                                        "avg_launch_ms": qk["ms"]}
+    if not args.no_breakdown:
+        ceil = mfma_only_ceiling(x.detach(), w)
+        result["mfma_only_TFLOPs"] = ceil
+        result["roofline"]["frac_of_mfma_only_rate_on_real_operands"] = round(
+            result["roofline"]["achieved"] / ceil["quest_rtn_codes_of_the_forward_operands"], 4)
     if not args.no_extra and not args.no_breakdown and out_f == OUT_F:
         del layer
         result["out11008"] = out11008_block(device, args)

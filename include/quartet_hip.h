@@ -145,6 +145,17 @@ int qm_gemm_mxfp4_tn_noalloc(const uint8_t* a_codes, const uint8_t* a_scales, co
                              int c_dtype, int a_layout, int b_layout, void* stream);
 
 /*
+ * Measurement aid, no counterpart in the reference: the block-scaled FP4 matrix instruction of the product above in a
+ * loop without memory traffic, on operand bytes taken from `operands` (one workgroup of four waves per CU, each wave
+ * 16 instructions of 32 x 32 x 64 per iteration).  The rate it reaches on the bytes of real operands is the ceiling
+ * the chip's power limit leaves for qm_gemm_mxfp4_tn; bench.py reports both.  Returns the number of matrix
+ * instructions issued (each 2 * 32 * 32 * 64 flop), or a negative value on rejected arguments / launch failure.
+ *   operands: at least 32 KiB per CU, 16-byte aligned; sink: at least 1 KiB per CU (receives checksums).
+ */
+int64_t qm_diag_mfma_only(const uint8_t* operands, size_t operand_bytes, float* sink, size_t sink_bytes, int iters,
+                          void* stream);
+
+/*
  * out = ((g * mask).view(-1, hd)) @ H^T: the straight-through backward of the forward quantizer,
  * QuestMXFP4QuantizerFn.backward (src/models/quantization/quantizers/mxfp4.py:143-146); with
  * maskbits == NULL it is AlbertTsengQuantizerFn.backward (mxfp4.py:31-34).

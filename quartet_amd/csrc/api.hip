@@ -168,6 +168,16 @@ int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint
                     "qm_gemm_mxfp4_tn");
 }
 
+int64_t qm_diag_mfma_only(const uint8_t* operands, size_t operand_bytes, float* sink, size_t sink_bytes, int iters, void* stream) {
+    const int blocks = qm::mfma_only_blocks();
+    if (!operands || !sink || iters < 0 || operand_bytes < (size_t)blocks * 32768 || sink_bytes < (size_t)blocks * 1024 ||
+        !aligned(operands, 16) || !aligned(sink, 4))
+        return fail(QM_ERR_INVALID, "qm_diag_mfma_only: needs %zu bytes of operands (16-byte aligned) and %zu bytes of sink",
+                    (size_t)blocks * 32768, (size_t)blocks * 1024);
+    if (int rc = from_hip(qm::mfma_only(operands, sink, iters, reinterpret_cast<hipStream_t>(stream)), "qm_diag_mfma_only")) return -(int64_t)(rc > 0 ? rc : -rc);
+    return (int64_t)blocks * 4 * (int64_t)iters * 16;
+}
+
 size_t qm_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0 || K % 32) return 0;
     return qm::gemm_workspace_bytes(M, N, K);

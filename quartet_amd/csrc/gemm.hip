@@ -894,6 +894,48 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     }
 }
 
+// Measurement aid: the block-scaled FP4 matrix instruction alone, on operand bytes taken from `operands`, with no
+// memory traffic inside the loop.  What a wave of the GEMM does between its loads: 16 products per iteration on a 4 x 4
+// grid of 32 x 32 accumulator blocks.  The rate this reaches on real operand bytes is the chip's ceiling for the
+// product at its power limit (the clock it sustains depends on how much the operand bits toggle).
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mfma_only_kernel(const uint4* __restrict__ operands,
+                                                                                                    float* __restrict__ sink, int iters) {
+    const int tid = threadIdx.x;
+    uint4 a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        a[i] = operands[((size_t)blockIdx.x * 8 + i) * 256 + tid];
+        b[i] = operands[((size_t)blockIdx.x * 8 + 4 + i) * 256 + tid];
+    }
+    v16f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+    const int sc = 0x7f7f7f7f;  // scale 2^0
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const v8i av = v8i{(int)a[i].x, (int)a[i].y, (int)a[i].z, (int)a[i].w, 0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const v8i bv = v8i{(int)b[j].x, (int)b[j].y, (int)b[j].z, (int)b[j].w, 0, 0, 0, 0};
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[i][j], 4, 4, 0, sc, 0, sc);
+            }
+        }
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) sum += acc[i][j][e];
+    sink[(size_t)blockIdx.x * 256 + tid] = sum;
+}
+
 int device_cus() {
     static int cached = 0;  // one GPU model per process
     if (cached > 0) return cached;
@@ -979,6 +1021,13 @@ hipError_t launch_gemm(const uint8_t* a_codes, const uint8_t* a_scales, const ui
 }
 
 }  // namespace
+
+// one workgroup (four waves, one per SIMD) per CU; reads blocks * 32 KiB of operands, writes blocks * 256 floats
+int mfma_only_blocks() { return device_cus(); }
+hipError_t mfma_only(const uint8_t* operands, float* sink, int iters, hipStream_t stream) {
+    mfma_only_kernel<<<dim3((unsigned)device_cus()), dim3(256), 0, stream>>>(reinterpret_cast<const uint4*>(operands), sink, iters);
+    return hipGetLastError();
+}
 
 // Shapes the 256x256-tile kernels serve (they also read tiled operands): extents multiples of 64 and at least one
 // full tile wide, K a multiple of 128; tiles hanging over the edge of M or N compute on clamped rows and store nothing there.

@@ -178,6 +178,18 @@ def gemm_mxfp4_tn_noalloc(a_codes, a_scales, b_codes, b_scales, alpha, out):
     return out
 
 
+def mfma_only(operand_bytes, iters):
+    """Measurement aid: `iters` iterations of the FP4 matrix instruction alone on every CU, fed with bytes of
+    `operand_bytes` (uint8, at least 32 KiB per CU).  Returns the number of 32 x 32 x 64 instructions issued."""
+    _require_cuda(operand_bytes)
+    assert operand_bytes.dtype == torch.uint8 and operand_bytes.is_contiguous()
+    sink = torch.empty(1 << 18, dtype=torch.float32, device=operand_bytes.device)
+    n = _lib.lib().qm_diag_mfma_only(_ptr(operand_bytes), operand_bytes.numel(), _ptr(sink), sink.numel() * 4, iters, _stream())
+    if n < 0:
+        _lib.check(int(n), "qm_diag_mfma_only")
+    return n
+
+
 def masked_hadamard_bwd(g, hadamard_dim=32, scale_dtype=torch.bfloat16, sign_bits=None, maskbits=None, out_dtype=None,
                         out=None):
     """g [R,C] -> ((g*mask).view(-1,hd) @ H^T) as [R,C] of out_dtype (default g.dtype); `out` may be pre-allocated."""

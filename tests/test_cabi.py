@@ -15,7 +15,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def declared_functions():
     text = open(os.path.join(ROOT, "include", "quartet_hip.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return set(re.findall(r"^\s*(?:const\s+char\s*\*|int|size_t)\s+(qm_\w+)\s*\(", text, flags=re.M))
+    return set(re.findall(r"^\s*(?:const\s+char\s*\*|int|int64_t|size_t)\s+(qm_\w+)\s*\(", text, flags=re.M))
 
 
 def test_library_exports_every_declared_function():
