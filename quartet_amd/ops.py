@@ -26,7 +26,7 @@ matrix scaled by ``hd^-1/2`` with negated columns, which is what every quantizer
 import torch
 
 from . import kernels as K
-from .quantizers.mxfp4 import _fresh_seed, remember_host_value, sylvester_sign_bits
+from .quantizers.mxfp4 import _fresh_seed, register_host_value, remember_host_value, sylvester_sign_bits
 
 ALPHA_FWD = 1.0
 ALPHA_BWD = K.FOUR_THIRDS * K.FOUR_THIRDS
@@ -46,6 +46,22 @@ def rotation_sign_bits(hadamard_matrix):
 
 def _host_scalar(t):
     return remember_host_value("scalar", t, lambda: float(t.detach().reshape(-1)[0].item()))
+
+
+_constants = {}
+
+
+def constant_alpha(value, device):
+    """A one-element tensor holding `value` on `device`, created once and remembered together with its host value: the
+    operators that take an ``alpha`` tensor then need no device-to-host copy (a copy would synchronise the stream on
+    every call and is not allowed while a HIP graph is being captured)."""
+    key = (float(value), torch.device(device))
+    t = _constants.get(key)
+    if t is None:
+        t = torch.full((1,), float(value), device=device)
+        _constants[key] = t
+    register_host_value("scalar", t, float(value))
+    return t
 
 
 def _rows(x):
@@ -162,15 +178,15 @@ def packed_forward(x2, weight, forward_matrix):
     """x [T,I], W [O,I] -> (y bf16 [T,O], packed operands kept for backward)."""
     xq, xs, xm = fusedQuantizeMx_op(x2, forward_matrix, True)
     wq, ws, wm = fusedQuantizeMx_op(weight, forward_matrix, True)
-    y = matmul_mxf4_bf16_tn_op(xq, wq, xs, ws, torch.full((1,), ALPHA_FWD, device=x2.device))
+    y = matmul_mxf4_bf16_tn_op(xq, wq, xs, ws, constant_alpha(ALPHA_FWD, x2.device))
     return y, (xq, xs, xm, wq, ws, wm)
 
 
 def packed_backward(e2, packed, forward_matrix, backward_matrix):
     """e [T,O] and the operands kept by packed_forward -> (grad x bf16 [T,I], grad W bf16 [O,I])."""
     xq, xs, xm, wq, ws, wm = packed
-    one = torch.ones(1, device=e2.device)
-    alpha = torch.full((1,), ALPHA_BWD, device=e2.device)
+    one = constant_alpha(1.0, e2.device)
+    alpha = constant_alpha(ALPHA_BWD, e2.device)
     eq, es = fusedQuantizeMxAbsMax_op(e2, backward_matrix, True)
     wtq, wts = backward_qt_bf16_op(wq, ws, backward_matrix, one)
     gx = maskedHadamardBwd_op(matmul_mxf4_bf16_tn_op(eq, wtq, es, wts, alpha), xm, forward_matrix)

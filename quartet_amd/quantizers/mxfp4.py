@@ -66,6 +66,14 @@ def remember_host_value(kind, t, make):
     return value
 
 
+def register_host_value(kind, t, value):
+    """Record a host-side value of tensor `t` that the caller already knows, so that remember_host_value finds it
+    without a device-to-host copy."""
+    if len(_host_cache) >= _HOST_CACHE_LIMIT:
+        _host_cache.clear()
+    _host_cache[(kind, id(t))] = (weakref.ref(t), t._version, value)
+
+
 def sylvester_sign_bits(matrix):
     """Bit mask of the negated columns if `matrix` is ``hd^-1/2 * Sylvester * diag(+-1)`` (hd 32, 64 or 128, the
     scale rounded to the matrix's dtype), else None: a dense rotation."""
