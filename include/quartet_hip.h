@@ -154,6 +154,14 @@ int qm_gemm_mxfp4_tn_noalloc(const uint8_t* a_codes, const uint8_t* a_scales, co
  */
 int64_t qm_diag_mfma_only(const uint8_t* operands, size_t operand_bytes, float* sink, size_t sink_bytes, int iters,
                           void* stream);
+/*
+ * Measurement aid, no counterpart in the reference: hands the library `count` pairs of hipEvent_t (HOST arrays of
+ * handles created with timing enabled).  Each of the next `count` launches of the product's persistent tile kernel
+ * -- from qm_gemm_mxfp4_tn or from inside qm_linear_forward / qm_linear_backward -- takes one pair, and the runtime
+ * stamps it with that kernel's own begin and end, so hipEventElapsedTime(start, stop) is the kernel's duration as a
+ * profiler's kernel trace shows it, inside whatever sequence of kernels it runs.  count == 0 withdraws unused pairs.
+ */
+int qm_diag_time_gemm_launches(void* const* start_events, void* const* stop_events, int count);
 
 /*
  * out = ((g * mask).view(-1, hd)) @ H^T: the straight-through backward of the forward quantizer,

@@ -168,6 +168,15 @@ int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint
                     "qm_gemm_mxfp4_tn");
 }
 
+int qm_diag_time_gemm_launches(void* const* start_events, void* const* stop_events, int count) {
+    if (count < 0 || (count > 0 && (!start_events || !stop_events)))
+        return fail(QM_ERR_INVALID, "qm_diag_time_gemm_launches: %d event pairs, null arrays", count);
+    for (int i = 0; i < count; ++i)
+        if (!start_events[i] || !stop_events[i]) return fail(QM_ERR_INVALID, "qm_diag_time_gemm_launches: null event at %d", i);
+    qm::gemm_time_next_launches(start_events, stop_events, count);
+    return 0;
+}
+
 int64_t qm_diag_mfma_only(const uint8_t* operands, size_t operand_bytes, float* sink, size_t sink_bytes, int iters, void* stream) {
     const int blocks = qm::mfma_only_blocks();
     if (!operands || !sink || iters < 0 || operand_bytes < (size_t)blocks * 32768 || sink_bytes < (size_t)blocks * 1024 ||

@@ -122,6 +122,8 @@ hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const 
                          const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
                          int a_layout, int b_layout, void* workspace, size_t workspace_bytes, hipStream_t stream);
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+// measurement aid: attach these event pairs to the next `count` launches of the persistent product kernel
+void gemm_time_next_launches(void* const* start_events, void* const* stop_events, int count);
 // measurement aid: the FP4 matrix instruction alone (see gemm.hip)
 int mfma_only_blocks();
 hipError_t mfma_only(const uint8_t* operands, float* sink, int iters, hipStream_t stream);

@@ -178,6 +178,26 @@ def gemm_mxfp4_tn_noalloc(a_codes, a_scales, b_codes, b_scales, alpha, out):
     return out
 
 
+def time_gemm_launches(n):
+    """Measurement aid: the next `n` launches of the product's persistent tile kernel (stand-alone or inside the
+    whole-layer calls) are stamped with their own begin and end.  Returns a function that, after a synchronisation,
+    gives their durations in milliseconds."""
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+    for e in starts + stops:
+        e.record()   # creates the underlying event; the launch re-records it
+    arr = ctypes.c_void_p * n
+    a = arr(*[e.cuda_event for e in starts])
+    b = arr(*[e.cuda_event for e in stops])
+    _lib.check(_lib.lib().qm_diag_time_gemm_launches(a, b, n), "qm_diag_time_gemm_launches")
+
+    def durations():
+        torch.cuda.synchronize()
+        _lib.lib().qm_diag_time_gemm_launches(None, None, 0)
+        return [s.elapsed_time(t) for s, t in zip(starts, stops)]
+    return durations
+
+
 def mfma_only(operand_bytes, iters):
     """Measurement aid: `iters` iterations of the FP4 matrix instruction alone on every CU, fed with bytes of
     `operand_bytes` (uint8, at least 32 KiB per CU).  Returns the number of 32 x 32 x 64 instructions issued."""
