@@ -176,6 +176,53 @@ def in_step_gemm_times(step, iters=60, warmup=5):
     return {n: round(sum(d[i::3]) / iters, 4) for i, n in enumerate(names)}
 
 
+def in_step_gemm_ms_by_difference(x, w, dy, steps=10, rounds=5):
+    """Mean duration of the three products inside the layer step, from two HIP graphs timed with events: the step's
+    eleven kernels launched one by one in the layer's order (`steps` times), and the same sequence without the three
+    products.  The difference of the two replays is what the step pays for its products where they actually run --
+    between quantizer kernels -- with no event or host time inside the measured interval."""
+    from quartet_amd import kernels as K
+    tl, signs = True, 0x5A5AA5A5
+
+    def one_step(full):
+        def product(ac, as_, bc, bs, alpha):
+            return K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha, torch.bfloat16, a_tiled=tl, b_tiled=tl) if full else None
+        xc, xs, xm, _ = K.quantize_mxfp4(x, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)
+        wc, ws, wm, _ = K.quantize_mxfp4(w, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)
+        product(xc, xs, wc, ws, 1.0)
+        ec, es, _, _ = K.quantize_mxfp4(dy, 32, signs, K.QM_ABSMAX_SR, seed=1, tiled=tl)
+        etc, ets, _, _ = K.quantize_mxfp4(dy, 32, signs, K.QM_ABSMAX_SR, transposed_in=True, seed=2, tiled=tl)
+        wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=3, tiled_in=tl, tiled_out=tl)
+        xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=4, tiled_in=tl, tiled_out=tl)
+        gxq = product(ec, es, wtc, wts, K.FOUR_THIRDS ** 2)
+        gwq = product(etc, ets, xtc, xts, K.FOUR_THIRDS ** 2)
+        K.masked_hadamard_bwd(gxq if full else x, 32, torch.bfloat16, None, xm)
+        K.masked_hadamard_bwd(gwq if full else w, 32, torch.bfloat16, None, wm)
+
+    graphs = {}
+    for full in (True, False):
+        one_step(full)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(steps):
+                one_step(full)
+        g.replay()
+        graphs[full] = g
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    times = {True: [], False: []}
+    for _ in range(rounds):
+        for full in (True, False):
+            torch.cuda.synchronize()
+            start.record()
+            graphs[full].replay()
+            stop.record()
+            stop.synchronize()
+            times[full].append(start.elapsed_time(stop) / steps)
+    med = {k: sorted(v)[len(v) // 2] for k, v in times.items()}
+    return {"ms": (med[True] - med[False]) / 3.0, "step_graph_ms": round(med[True], 4), "step_graph_without_products_ms": round(med[False], 4)}
+
+
 def quantizer_sweep(device):
     """Quantizer-only throughput (HBM-cold) on [rows x 4096] bf16 with 0.1 % entries at +-1e3, for the three
     production modes and Hadamard blocks 32/64/128."""
@@ -637,13 +684,16 @@ def main():
         result["kernels"] = kb
         # the three GEMMs of a step (fwd, dgrad, wgrad) run the same kernel on the same flop count: the roofline
         # entry is their mean, which is what a profiler's per-kernel average over the run reports
-        # the three GEMMs of a step (fwd, dgrad, wgrad) run the same kernel on the same flop count: the roofline entry is
-        # their mean, each timed as an unbroken chain of its own launches (graph replay, HIP events around the chain).
-        # Such a chain holds the chip at its power limit throughout and is the slowest setting for this kernel: inside
-        # the layer step, where quantizer kernels run in between, a profiler's kernel trace shows the same launches 5-10 %
-        # shorter.  `in_step_ms` times them there with event pairs the library attaches to each launch; an event pair
-        # costs the dispatcher a few microseconds of its own, which that figure includes.
-        gemm_ms, gemm_tf = gemm_summary(kb, T_TOKENS, out_f)
+        # The three GEMMs of a step (fwd, dgrad, wgrad) run the same kernel on the same flop count: the roofline entry is
+        # their mean duration inside the step, where they run between quantizer kernels (in_step_gemm_ms_by_difference),
+        # which is what a profiler's per-kernel average over the step loop shows.  `back_to_back` times each of the three
+        # as an unbroken chain of its own launches: that holds the chip at its power limit throughout and is the slowest
+        # setting for this kernel (5-10 % longer).  `in_step_stamped_ms` are readings of event pairs the library attaches
+        # to each launch in the production path; a pair's own dispatch adds a few microseconds to each.
+        chain_ms, chain_tf = gemm_summary(kb, T_TOKENS, out_f)
+        diff = in_step_gemm_ms_by_difference(x.detach(), w, dy)
+        gemm_ms = diff.pop("ms")
+        gemm_tf = 2.0 * T_TOKENS * IN_F * out_f / gemm_ms / 1e9
         x.requires_grad_(True)
         ist = in_step_gemm_times(make_step(layer, x, dy))
         x.requires_grad_(False)
@@ -651,7 +701,10 @@ def main():
         result["roofline"] = {"bound": "mfma", "kernel": f"gemm_mxfp4_tn ({T_TOKENS}x{out_f}x{IN_F}, {T_TOKENS}x{IN_F}x{out_f}, {out_f}x{IN_F}x{T_TOKENS})",
                               "achieved": round(gemm_tf, 1), "peak": PEAK_FP4_TFLOPS, "unit": "TFLOP/s",
                               "frac": round(gemm_tf / PEAK_FP4_TFLOPS, 4), "traffic": traffic, "traffic_source": source,
-                              "avg_launch_ms": round(gemm_ms, 4), "in_step_ms": ist}
+                              "avg_launch_ms": round(gemm_ms, 4), "how": {"what": "mean of the step's three products, timed inside the step", **diff},
+                              "back_to_back": {"avg_launch_ms": round(chain_ms, 4), "TFLOPs": round(chain_tf, 1),
+                                               "frac": round(chain_tf / PEAK_FP4_TFLOPS, 4)},
+                              "in_step_stamped_ms": ist}
         qk = kb["quantize_x_quest_rtn_mask"]
         traffic, source = _traffic_entry(prof, "quantize_x_quest_rtn_mask_alone")
         result["roofline_quantize"] = {"bound": "hbm", "kernel": f"quantize_rowmajor (quest RTN + mask, {T_TOKENS}x{IN_F} bf16)",
