@@ -55,6 +55,8 @@ def constant_alpha(value, device):
     """A one-element tensor holding `value` on `device`, created once and remembered together with its host value: the
     operators that take an ``alpha`` tensor then need no device-to-host copy (a copy would synchronise the stream on
     every call and is not allowed while a HIP graph is being captured)."""
+    if torch.compiler.is_compiling():   # under tracing the tensor is a graph constant; the operator reads it at run time
+        return torch.full((1,), float(value), device=device)
     key = (float(value), torch.device(device))
     t = _constants.get(key)
     if t is None:
