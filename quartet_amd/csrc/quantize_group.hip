@@ -460,22 +460,34 @@ void launch_rowmajor_g32(int mode, const void* x, int64_t rows, int64_t cols, bo
 
 // ---- Hadamard blocks 64 and 128, row-major ---------------------------------------------------------------
 // Same one-group-per-lane layout; a Hadamard chunk is HD/32 consecutive lanes (a lane pair or a quad).  The
-// five in-register stages are followed by the stride-32 (and stride-64) stages across the lanes of the chunk:
-// the lower lane of a butterfly gets a + b, the upper one a - b = partner + (-own), one sign flip and one
-// DPP-fed add per element.  The column sign word differs per lane of the chunk.
+// five in-register stages are followed by the stride-32 (and stride-64) stages across the lanes of the chunk, one
+// DPP-fed multiply-add per element: own + partner in the lower lane of a butterfly, own - partner in the upper one.
+// The upper lane's exact value is partner - own = -(own - partner): rounding is symmetric, so the negation commutes
+// with it, and it is folded into the column sign applied at the end (a lane's values are negated once per stage in
+// which it is the upper lane).  The column signs differ per lane of the chunk; they are applied as lane masks held in
+// scalar registers (bit l of mask j: negate element j in lane l), one select per element.
 template <int CTRL>
-__device__ __forceinline__ void cross_lane_stage(float (&v)[32], bool upper) {
-    const uint32_t flip = upper ? 0x80000000u : 0u;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) {
-        const float partner = u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(v[i]), CTRL, 0xf, 0xf, false));
-        v[i] = partner + u2f(f2u(v[i]) ^ flip);
-    }
+__device__ __forceinline__ void cross_lane_stage(float (&v)[32], float s) {
+    // s = +1 in the lower lane, -1 in the upper one.  An instruction reads its own destination register from the
+    // partner lane; the leading s_nop keeps the two wait states a DPP read needs after a vector write to that register
+    // (the compiler does not look into assembly statements).
+#define QM_X(N) "v_fmac_f32_dpp %" #N ", %" #N ", %16 quad_perm:[%17,%18,%19,%20] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+#define QM_STAGE16(B)                                                                                                   \
+    asm volatile("s_nop 1\n\t" QM_X(0) QM_X(1) QM_X(2) QM_X(3) QM_X(4) QM_X(5) QM_X(6) QM_X(7) QM_X(8) QM_X(9) QM_X(10) QM_X(11)  \
+                 QM_X(12) QM_X(13) QM_X(14) QM_X(15)                                                                     \
+                 : "+v"(v[(B)]), "+v"(v[(B) + 1]), "+v"(v[(B) + 2]), "+v"(v[(B) + 3]), "+v"(v[(B) + 4]), "+v"(v[(B) + 5]),  \
+                   "+v"(v[(B) + 6]), "+v"(v[(B) + 7]), "+v"(v[(B) + 8]), "+v"(v[(B) + 9]), "+v"(v[(B) + 10]),             \
+                   "+v"(v[(B) + 11]), "+v"(v[(B) + 12]), "+v"(v[(B) + 13]), "+v"(v[(B) + 14]), "+v"(v[(B) + 15])          \
+                 : "v"(s), "n"(CTRL & 3), "n"((CTRL >> 2) & 3), "n"((CTRL >> 4) & 3), "n"((CTRL >> 6) & 3))
+    QM_STAGE16(0);
+    QM_STAGE16(16);
+#undef QM_STAGE16
+#undef QM_X
 }
 
 template <typename T, int MODE, bool WANT_MASK, int HD>
 __global__ __launch_bounds__(256) void quantize_rowmajor_wide_kernel(const T* __restrict__ x, int64_t n_groups, float c,
-                                                                     SignBits sb, uint64_t seed, GroupOut out) {
+                                                                     SignBits sf, uint64_t seed, GroupOut out) {
     static_assert(HD == 64 || HD == 128, "lane pairs or quads");
     const int64_t gi = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (gi >= n_groups) return;  // n_groups is a multiple of HD/32: the lanes of a chunk leave together
@@ -483,16 +495,20 @@ __global__ __launch_bounds__(256) void quantize_rowmajor_wide_kernel(const T* __
     load_group<T>(x + gi * 32, v);
     butterfly32(v);
     const int part = (int)threadIdx.x & (HD / 32 - 1);
-    cross_lane_stage<0xB1>(v, (part & 1) != 0);                           // quad_perm [1,0,3,2]: stride 32
-    if constexpr (HD == 128) cross_lane_stage<0x4E>(v, (part & 2) != 0);  // quad_perm [2,3,0,1]: stride 64
-    uint32_t sw = sb.w[0];
-    if (part == 1) sw = sb.w[1];
-    if constexpr (HD == 128) {
-        if (part == 2) sw = sb.w[2];
-        if (part == 3) sw = sb.w[3];
-    }
+    cross_lane_stage<0xB1>(v, (part & 1) ? -1.0f : 1.0f);                           // quad_perm [1,0,3,2]: stride 32
+    if constexpr (HD == 128) cross_lane_stage<0x4E>(v, (part & 2) ? -1.0f : 1.0f);  // quad_perm [2,3,0,1]: stride 64
+    // sf holds, per element j, a field of HD/32 bits: bit p = negate element j in the chunk's lane p (column sign
+    // xor the stage negations above).  field * 0x5555... (or 0x1111...) spreads it over the wave's chunks.
+    constexpr int P = HD / 32;
+    constexpr uint32_t kUnit = P == 2 ? 0x55555555u : 0x11111111u;
 #pragma unroll
-    for (int j = 0; j < 32; ++j) v[j] = u2f(f2u(v[j] * c) ^ ((sw << (31 - j)) & 0x80000000u));
+    for (int j = 0; j < 32; ++j) {
+        const uint32_t field = (sf.w[(j * P) >> 5] >> ((j * P) & 31)) & ((1u << P) - 1u);  // wave-uniform: scalar registers
+        const uint32_t half = field * kUnit;
+        const uint64_t m = ((uint64_t)half << 32) | half;
+        const float scaled = v[j] * c;
+        asm("v_cndmask_b32_e64 %0, %1, -%1, %2" : "=v"(v[j]) : "v"(scaled), "s"(m));
+    }
     GroupCodes o;
     quantize_group_regs<MODE, WANT_MASK>(v, seed, gi, o);
     out.codes[gi] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
@@ -501,17 +517,32 @@ __global__ __launch_bounds__(256) void quantize_rowmajor_wide_kernel(const T* __
     if (out.dequant) store_dequant<T>(reinterpret_cast<T*>(out.dequant) + gi * 32, o);
 }
 
+// Per-element negation fields of the wide kernel: bit p of field j = column sign of rotated element 32 p + j, xor 1 for
+// the lanes of a chunk whose index has an odd number of set bits (their values come out of the cross-lane stages negated).
+template <int HD>
+SignBits wide_sign_fields(const SignBits& sb) {
+    constexpr int P = HD / 32;
+    SignBits sf{{0u, 0u, 0u, 0u}};
+    for (int j = 0; j < 32; ++j) {
+        uint32_t field = 0u;
+        for (int p = 0; p < P; ++p) field |= (((sb.w[p] >> j) & 1u) ^ (uint32_t)(__builtin_popcount((unsigned)p) & 1)) << p;
+        sf.w[(j * P) >> 5] |= field << ((j * P) & 31);
+    }
+    return sf;
+}
+
 template <typename T, bool WANT_MASK, int HD>
 void launch_rowmajor_wide(int mode, const void* x, int64_t n, float c, const SignBits& sb, uint64_t seed,
                           const GroupOut& out, hipStream_t stream) {
     const T* xp = reinterpret_cast<const T*>(x);
     const int64_t n_groups = n / 32;
+    const SignBits sf = wide_sign_fields<HD>(sb);
     dim3 grid((unsigned)((n_groups + 255) / 256)), block(256);
     switch (mode) {
-        case QUEST_RTN: quantize_rowmajor_wide_kernel<T, QUEST_RTN, WANT_MASK, HD><<<grid, block, 0, stream>>>(xp, n_groups, c, sb, seed, out); break;
-        case ABSMAX_RTN: quantize_rowmajor_wide_kernel<T, ABSMAX_RTN, WANT_MASK, HD><<<grid, block, 0, stream>>>(xp, n_groups, c, sb, seed, out); break;
-        case ABSMAX_SR: quantize_rowmajor_wide_kernel<T, ABSMAX_SR, WANT_MASK, HD><<<grid, block, 0, stream>>>(xp, n_groups, c, sb, seed, out); break;
-        default: quantize_rowmajor_wide_kernel<T, QUEST_SR, WANT_MASK, HD><<<grid, block, 0, stream>>>(xp, n_groups, c, sb, seed, out); break;
+        case QUEST_RTN: quantize_rowmajor_wide_kernel<T, QUEST_RTN, WANT_MASK, HD><<<grid, block, 0, stream>>>(xp, n_groups, c, sf, seed, out); break;
+        case ABSMAX_RTN: quantize_rowmajor_wide_kernel<T, ABSMAX_RTN, WANT_MASK, HD><<<grid, block, 0, stream>>>(xp, n_groups, c, sf, seed, out); break;
+        case ABSMAX_SR: quantize_rowmajor_wide_kernel<T, ABSMAX_SR, WANT_MASK, HD><<<grid, block, 0, stream>>>(xp, n_groups, c, sf, seed, out); break;
+        default: quantize_rowmajor_wide_kernel<T, QUEST_SR, WANT_MASK, HD><<<grid, block, 0, stream>>>(xp, n_groups, c, sf, seed, out); break;
     }
 }
 
