@@ -468,29 +468,37 @@ def _traffic_entry(prof, key):
                                                          "fetch_bytes": k["fetch_bytes"], "write_bytes": k["write_bytes"]}
 
 
-def counters_to_json(fetch_dir, write_dir):
+def counters_to_json(fetch_dir, write_dir, sq_dir=None):
     """Turn the CSV output of the two byte-counter runs
 
         rocprofv3 --pmc FETCH_SIZE -d <fetch_dir> -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-breakdown --calibration-copy
         rocprofv3 --pmc WRITE_SIZE -d <write_dir> -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-breakdown --calibration-copy
 
     into profiles/hbm_traffic.json.  The calibration copy (the largest copyBuffer dispatch: 256 MiB read, 256 MiB
-    written) fixes how many bytes one counter unit stands for."""
+    written) fixes how many bytes one counter unit stands for.  With a third directory, the output of
+
+        rocprofv3 --pmc SQ_WAVES SQ_INSTS_VALU ... -d <sq_dir> -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-breakdown
+
+    adds each kernel's vector instructions per wave (one wave instruction serves 64 lanes; in the quantizers a lane owns
+    one group of 32 values per launch, so the figure is also the instructions per group)."""
     import collections
     import csv
     import glob
     import re
     import subprocess
 
-    def read(d):
+    def read(d, counter=None):
         files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
         if not files:
             sys.exit(f"no *counter_collection.csv under {d}")
         agg = collections.defaultdict(list)
         for r in csv.DictReader(open(files[0])):
-            agg[re.sub(r"\(anonymous namespace\)::", "", r["Kernel_Name"])].append(float(r["Counter_Value"]))
+            if counter is None or r["Counter_Name"] == counter:
+                agg[re.sub(r"\(anonymous namespace\)::", "", r["Kernel_Name"])].append(float(r["Counter_Value"]))
         return agg
     fetch, write = read(fetch_dir), read(write_dir)
+    valu = read(sq_dir, "SQ_INSTS_VALU") if sq_dir else {}
+    waves = read(sq_dir, "SQ_WAVES") if sq_dir else {}
     copy_bytes = 256 << 20
 
     def unit(agg):
@@ -509,6 +517,10 @@ def counters_to_json(fetch_dir, write_dir):
         w = [v for k, vs in write.items() if match(k) for v in vs]
         if f and w:
             out[name] = {"fetch_bytes": round(sum(f) / len(f) * fu), "write_bytes": round(sum(w) / len(w) * wu), "dispatches": len(f)}
+            vi = [v for k, vs in valu.items() if match(k) for v in vs]
+            wv = [v for k, vs in waves.items() if match(k) for v in vs]
+            if vi and wv:
+                out[name]["valu_instr_per_wave"] = round(sum(vi) / sum(wv), 1)
     head = subprocess.run(["git", "-C", ROOT, "rev-parse", "HEAD"], capture_output=True, text=True).stdout.strip()
     dirty = subprocess.run(["git", "-C", ROOT, "status", "--porcelain", "--", "quartet_amd/csrc"], capture_output=True, text=True).stdout.strip()
     prof = {"what": "HBM-side bytes per launch (mean over the dispatches of a 2-step run) of the isolated linear, tokens 8192 x in 4096 x out 4096",
@@ -516,7 +528,8 @@ def counters_to_json(fetch_dir, write_dir):
             "calibration": {"copy_bytes": copy_bytes, "bytes_per_fetch_unit": round(fu, 2), "bytes_per_write_unit": round(wu, 2)},
             "commands": ["rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof_fetch -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-breakdown --calibration-copy",
                          "rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof_write -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-breakdown --calibration-copy",
-                         "python3 bench.py --counters-to-json gpurun_out/prof_fetch gpurun_out/prof_write"],
+                         "rocprofv3 --pmc SQ_WAVES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_ACTIVE_INST_VALU SQ_WAIT_INST_ANY SQ_INSTS_VMEM_RD SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_MFMA -d gpurun_out/prof_sq -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-breakdown",
+                         "python3 bench.py --counters-to-json gpurun_out/prof_fetch gpurun_out/prof_write gpurun_out/prof_sq"],
             "kernels": out}
     with open(TRAFFIC_PROFILE, "w") as f:
         json.dump(prof, f, indent=1)
@@ -583,6 +596,71 @@ def out11008_block(device, args):
             "gemm_mean": {"ms": round(gemm_ms, 4), "TFLOPs": round(gemm_tf, 1), "frac_of_peak": round(gemm_tf / PEAK_FP4_TFLOPS, 4)}}
 
 
+def reference_shapes(device):
+    """The two layer shapes the reference's notebook reports latencies for (notebooks/benchmark_mxfp4.ipynb: 32768 tokens,
+    4096 -> 4096 and 1024 -> 1024, forward and forward + backward, there on another vendor's consumer GPU), timed here
+    for this layer and for a plain bf16 linear layer on the same GPU, with the notebook's method in spirit: warm-up, then
+    the median of repeated synchronised blocks."""
+    import quartet_amd as q
+    out = {}
+    for tokens, n in ((32768, 4096), (32768, 1024)):
+        g = torch.Generator().manual_seed(n)
+        x = torch.randn(tokens, n, generator=g).to(torch.bfloat16).to(device).requires_grad_(True)
+        dy = (1e-3 * torch.randn(tokens, n, generator=g)).to(torch.bfloat16).to(device)
+        layers = {
+            "quartet": q.QuantizedLinear(
+                n, n, bias=False,
+                weight_quantizer=q.QUANTIZER_CLASSES["QuestMXFP4Quantizer"](hadamard_dim=32),
+                activation_quantizer=q.QUANTIZER_CLASSES["QuestMXFP4Quantizer"](hadamard_dim=32),
+                gradient_quantizer=q.QUANTIZER_CLASSES["AlbertTsengQuantizer"](hadamard_dim=32, stochastic=True, rerotate="signs"),
+                backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]()).to(device=device, dtype=torch.bfloat16),
+            "bf16": torch.nn.Linear(n, n, bias=False).to(device=device, dtype=torch.bfloat16),
+        }
+        row = {}
+        for name, layer in layers.items():
+            def fwd():
+                with torch.no_grad(), torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+                    layer(x)
+
+            def fwd_bwd():
+                with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+                    y = layer(x)
+                y.backward(dy)
+                x.grad = None
+                layer.weight.grad = None
+            for label, fn in (("fwd_ms", fwd), ("fwd_bwd_ms", fwd_bwd)):
+                _, st = time_layer_steps(fn, 10, 3, sustain_s=0.2)
+                row[f"{name}_{label}"] = st["ms_per_step_median"]
+        row["speedup_fwd"] = round(row["bf16_fwd_ms"] / row["quartet_fwd_ms"], 2)
+        row["speedup_fwd_bwd"] = round(row["bf16_fwd_bwd_ms"] / row["quartet_fwd_bwd_ms"], 2)
+        row["quartet_fwd_bwd_TFLOPs"] = round(6.0 * tokens * n * n / row["quartet_fwd_bwd_ms"] / 1e9, 1)
+        out[f"{tokens}x{n}x{n}"] = row
+        del x, dy, layers
+    return out
+
+
+def quantizer_bounds(prof, x):
+    """What else bounds the forward quantizer at this size: its vector-instruction floor (instructions per group from the
+    tracked counter profile: a lane owns one group, an instruction occupies its SIMD for four cycles) and what two plain
+    library kernels reach on the same tensor with the same timing method (a copy; a sum over four column blocks, which
+    reads everything and writes a quarter, about the quantizer's byte mix)."""
+    out = {}
+    k = (prof or {}).get("kernels", {}).get("quantize_x_quest_rtn_mask_alone", {})
+    if "valu_instr_per_wave" in k:
+        groups = x.numel() // 32
+        lanes = torch.cuda.get_device_properties(x.device).multi_processor_count * 4 * 64
+        out["valu_instr_per_group"] = k["valu_instr_per_wave"]
+        out["valu_floor_ms_at_2400MHz"] = round(k["valu_instr_per_wave"] * 4 * groups / lanes / 2.4e9 * 1e3, 4)
+    rows, cols = x.shape
+    dst = torch.empty_like(x)
+    quarter = torch.empty(rows, cols // 4, device=x.device, dtype=x.dtype)
+    ms_copy = time_kernel_cold(lambda a: (lambda: dst.copy_(a)), [x], reps=8, warmup=1)
+    ms_sum = time_kernel_cold(lambda a: (lambda: torch.sum(a.view(rows, 4, cols // 4), dim=1, out=quarter)), [x], reps=8, warmup=1)
+    out["library_kernels_same_tensor"] = {"copy_GBps": round(x.numel() * 4 / ms_copy / 1e6, 1),
+                                          "sum_of_four_column_blocks_GBps": round(x.numel() * 2.5 / ms_sum / 1e6, 1)}
+    return out
+
+
 def quantizer_sizes_block(device):
     """Quantizer-only configuration in brief: for each tensor size, the slowest and fastest of the nine (mode x Hadamard
     block) cells, HBM-cold."""
@@ -611,7 +689,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed steps before the timed ones (default 100 for the isolated layer, about 35 ms, and 3 for the model steps: the first steps after an idle period run "
+                         "at a clock the chip does not hold; the `sustained` block shows the first timed block beside the median)")
     ap.add_argument("--out-features", type=int, default=OUT_F,
                     help="out features of the isolated layer: 4096 (default, the shape the metric is quoted on) or 11008")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -629,18 +709,26 @@ def main():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a known-traffic kernel for scaling profiler byte counters) and one "
                          "forward quantizer launch on its own")
-    ap.add_argument("--counters-to-json", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
-                    help="no GPU work: summarise the CSV output of the two byte-counter runs into profiles/hbm_traffic.json")
+    ap.add_argument("--counters-to-json", nargs="+", metavar="DIR",
+                    help="no GPU work: summarise the CSV output of the two byte-counter runs (FETCH_DIR WRITE_DIR) and, if given, "
+                         "of the shader-sequencer counter run (SQ_DIR) into profiles/hbm_traffic.json")
     ap.add_argument("--quantizer-sweep", action="store_true",
                     help="also time the quantizer alone on [rows x 4096] for rows 4096/16384/65536, three modes, hd 32/64/128")
     ap.add_argument("--gemm-operand-content", action="store_true",
                     help="also time the forward GEMM on operands of different content (real codes, random, constant): shows the power limit")
+    ap.add_argument("--reference-shapes", action="store_true",
+                    help="also time the layer (and a bf16 linear layer, for the ratio) at the two shapes the reference's notebook "
+                         "reports: 32768 tokens x 4096 x 4096 and x 1024 x 1024, forward and forward + backward")
     ap.add_argument("--library-gemm", action="store_true",
                     help="also time the vendor library's MXFP4 product (torch._scaled_mm) on the forward GEMM's shape, for context")
     args = ap.parse_args()
     if args.counters_to_json:
+        if len(args.counters_to_json) not in (2, 3):
+            sys.exit("--counters-to-json FETCH_DIR WRITE_DIR [SQ_DIR]")
         counters_to_json(*args.counters_to_json)
         return
+    if args.warmup is None:
+        args.warmup = 100 if args.workload == "linear" else 3
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)")
     if not torch.cuda.is_available():
@@ -710,7 +798,7 @@ def main():
         result["roofline_quantize"] = {"bound": "hbm", "kernel": f"quantize_rowmajor (quest RTN + mask, {T_TOKENS}x{IN_F} bf16)",
                                        "achieved": qk["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                        "frac": round(qk["GBps"] / PEAK_HBM_GBS, 4), "traffic": traffic, "traffic_source": source,
-                                       "avg_launch_ms": qk["ms"]}
+                                       "avg_launch_ms": qk["ms"], **quantizer_bounds(prof, x.detach())}
     if not args.no_breakdown:
         ceil = mfma_only_ceiling(x.detach(), w)
         result["mfma_only_TFLOPs"] = ceil
@@ -722,6 +810,8 @@ def main():
         result["quantizer_sizes"] = quantizer_sizes_block(device)
     if args.quantizer_sweep:
         result["quantizer_sweep"] = quantizer_sweep(device)
+    if args.reference_shapes:
+        result["reference_shapes"] = reference_shapes(device)
     if args.library_gemm:
         result["library_gemm"] = library_gemm(device)
     if args.gemm_operand_content:
