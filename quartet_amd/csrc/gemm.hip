@@ -233,13 +233,21 @@ typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 // acc element e of a 32x32 tile is row 8*(e/4) + 4*half + e%4, column lane%32: per store instruction the
 // two half-waves each write one 64-byte (bf16) row segment.  (Making a lane's 4 values contiguous along n by
 // swapping the MFMA operand roles was measured slower: 64 scattered 8-byte pieces per instruction.)
-template <typename OutT>
+// One accumulator register into a vector register, in program order: left to itself the compiler copies ten blocks of
+// sixteen ahead of the first pass, and the 160 registers that takes push values the K loop needs out to scratch memory,
+// whose reloads then wait for every operand load in flight (loads return in order).
+__device__ __forceinline__ float acc_read(float a) {
+    float v;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    return v;
+}
+template <typename OutT, bool IN_ORDER = false>
 __device__ __forceinline__ void store_tile(const v16f& t, float alpha, OutT* __restrict__ c, int64_t row0, int64_t col,
                                            int64_t N, int half) {
 #pragma unroll
     for (int e = 0; e < 16; e += 2) {
         const int64_t r = row0 + 8 * (e / 4) + 4 * half + (e & 3);
-        const float v0 = t[e] * alpha, v1 = t[e + 1] * alpha;
+        const float v0 = (IN_ORDER ? acc_read(t[e]) : t[e]) * alpha, v1 = (IN_ORDER ? acc_read(t[e + 1]) : t[e + 1]) * alpha;
         if constexpr (sizeof(OutT) == 2) {
             // v_cvt_pk_bf16_f32: round-to-nearest-even, two values per instruction
             const v2bf p = __builtin_convertvector(v2f{v0, v1}, v2bf);
@@ -700,7 +708,9 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
                                                    uint8_t* smem_bytes, int rows_valid, int cols_valid) {
     // The opaque copy keeps the address arithmetic below inside the (rarely executed) epilogue instead of being
     // hoisted out of the K loop, where it would hold dozens of registers across the MFMA schedule.
-    int lane = lane_in;
+    // the lane index straight from the hardware, so that no copy of it has to stay alive through the K loop
+    (void)lane_in;
+    int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     asm volatile("" : "+v"(lane));
     const int lrow = lane & 31, half = lane >> 5;
     uint8_t* region = smem_bytes + kEpiAreaOff + wave * kEpiWaveBytes;
@@ -720,8 +730,9 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
 #pragma unroll
                 for (int b = 0; b < 4; ++b) {
                     const v16f& t = acc[i][2 * jp + jj];
-                    const v2bf p0 = __builtin_convertvector(v2f{t[4 * b] * alpha, t[4 * b + 1] * alpha}, v2bf);
-                    const v2bf p1 = __builtin_convertvector(v2f{t[4 * b + 2] * alpha, t[4 * b + 3] * alpha}, v2bf);
+                    const float t0 = acc_read(t[4 * b]), t1 = acc_read(t[4 * b + 1]), t2 = acc_read(t[4 * b + 2]), t3 = acc_read(t[4 * b + 3]);
+                    const v2bf p0 = __builtin_convertvector(v2f{t0 * alpha, t1 * alpha}, v2bf);
+                    const v2bf p1 = __builtin_convertvector(v2f{t2 * alpha, t3 * alpha}, v2bf);
                     *reinterpret_cast<uint2*>(wr + (((jj * 4 + b) * 16) ^ wsw)) =
                         make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
                 }
@@ -734,6 +745,9 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
                 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
                 __builtin_nontemporal_store(u4v{v.x, v.y, v.z, v.w}, reinterpret_cast<u4v*>(out + r8 * pitch8 + jp * 128));
             }
+            // keeps the passes apart: a scheduler that reads many passes' accumulators into vector registers ahead of time
+            // pushes the K loop's live values out to scratch memory, and their reloads wait for every operand load in flight
+            __builtin_amdgcn_sched_barrier(0);
         }
         out += 4 * pitch8;
     }
@@ -751,7 +765,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     uint8_t* smem_bytes = reinterpret_cast<uint8_t*>(smem);
     const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)smem;
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    // wave-uniform by construction; saying so keeps everything derived from it (tile corners, edge tests, the epilogue's
+    // base addresses) in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     const int lrow = lane & 31, half = lane >> 5;
     const int tiles_m = (M + kBigM - 1) / kBigM, tiles_n = (N + kBigN - 1) / kBigN, total = tiles_m * tiles_n;
@@ -797,7 +814,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             plan.voff_b[i] = plan.lane_codes_b + (uint32_t)i * step16;
         }
     }
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int wave_u = wave;
     int load_tm, load_tn, load_split;  // work item the load stream is in
     auto plan_tile = [&](int item) {
         const int t = item / splits;
@@ -871,7 +888,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                     if (i * 32 < rows_valid && j * 32 < cols_valid)
-                        store_tile<OutT>(acc[i][j], a_eff, dst, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
+                        store_tile<OutT, true>(acc[i][j], a_eff, dst, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
         }
     }
     // direct-to-LDS loads must not outlive the workgroup's LDS allocation
