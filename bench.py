@@ -477,7 +477,7 @@ def counters_to_json(fetch_dir, write_dir, sq_dir=None):
     into profiles/hbm_traffic.json.  The calibration copy (the largest copyBuffer dispatch: 256 MiB read, 256 MiB
     written) fixes how many bytes one counter unit stands for.  With a third directory, the output of
 
-        rocprofv3 --pmc SQ_WAVES SQ_INSTS_VALU ... -d <sq_dir> -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-breakdown
+        rocprofv3 --pmc SQ_WAVES SQ_INSTS_VALU ... -d <sq_dir> -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-breakdown --calibration-copy
 
     adds each kernel's vector instructions per wave (one wave instruction serves 64 lanes; in the quantizers a lane owns
     one group of 32 values per launch, so the figure is also the instructions per group)."""
@@ -528,7 +528,7 @@ def counters_to_json(fetch_dir, write_dir, sq_dir=None):
             "calibration": {"copy_bytes": copy_bytes, "bytes_per_fetch_unit": round(fu, 2), "bytes_per_write_unit": round(wu, 2)},
             "commands": ["rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof_fetch -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-breakdown --calibration-copy",
                          "rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof_write -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-breakdown --calibration-copy",
-                         "rocprofv3 --pmc SQ_WAVES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_ACTIVE_INST_VALU SQ_WAIT_INST_ANY SQ_INSTS_VMEM_RD SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_MFMA -d gpurun_out/prof_sq -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-breakdown",
+                         "rocprofv3 --pmc SQ_WAVES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_ACTIVE_INST_VALU SQ_WAIT_INST_ANY SQ_INSTS_VMEM_RD SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_MFMA -d gpurun_out/prof_sq -o bench --output-format csv -- python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --no-breakdown --calibration-copy",
                          "python3 bench.py --counters-to-json gpurun_out/prof_fetch gpurun_out/prof_write gpurun_out/prof_sq"],
             "kernels": out}
     with open(TRAFFIC_PROFILE, "w") as f:
