@@ -81,6 +81,7 @@ struct HadamardBwdJob {
             v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
         }
         const uint32_t keep = maskbits ? (uint32_t)maskbits[octet] : 0xffu;
+        job_requests_issued();
         const int j0 = lic * 8;
         const uint32_t sign8 = (sb.w[j0 >> 5] >> (j0 & 31)) & 0xffu;
 #pragma unroll

@@ -333,10 +333,12 @@ template <typename T, int MODE, bool WANT_MASK>
 __global__ __launch_bounds__(256) void quantize_rowmajor_g32_kernel(const T* __restrict__ x, int64_t n_groups, float c,
                                                                     uint32_t sign_word, uint64_t seed, GroupOut out,
                                                                     int rotate) {
+    job_starts();
     const int64_t gi = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (gi >= n_groups) return;
     float v[32];
     load_group<T>(x + gi * 32, v);
+    job_requests_issued();
     finish_group<T, MODE, WANT_MASK>(v, gi, gi, c, sign_word, seed, out, rotate != 0);
 }
 
@@ -419,9 +421,11 @@ struct RowmajorTiledJob {
         const int64_t ci = (int64_t)rb * 16 * groups + ((g >> 2) * 64 + rin * 4 + (g & 3));
         float v[32];
         load_group<T>(x + gi * 32, v);
+        job_requests_issued();
         rotate_group(v, c, sign_word);
         GroupCodes o;
         quantize_group_regs<MODE, WANT_MASK>(v, seed, gi, o);
+        job_stores_next();
         out.codes[ci] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
         // quad_perm broadcasts of lanes 1, 2, 3 of each quad
         const uint32_t s1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)o.scale_byte, 0x55, 0xf, 0xf, false);
@@ -489,10 +493,12 @@ template <typename T, int MODE, bool WANT_MASK, int HD>
 __global__ __launch_bounds__(256) void quantize_rowmajor_wide_kernel(const T* __restrict__ x, int64_t n_groups, float c,
                                                                      SignBits sf, uint64_t seed, GroupOut out) {
     static_assert(HD == 64 || HD == 128, "lane pairs or quads");
+    job_starts();
     const int64_t gi = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (gi >= n_groups) return;  // n_groups is a multiple of HD/32: the lanes of a chunk leave together
     float v[32];
     load_group<T>(x + gi * 32, v);
+    job_requests_issued();
     butterfly32(v);
     const int part = (int)threadIdx.x & (HD / 32 - 1);
     cross_lane_stage<0xB1>(v, (part & 1) ? -1.0f : 1.0f);                           // quad_perm [1,0,3,2]: stride 32
@@ -511,6 +517,7 @@ __global__ __launch_bounds__(256) void quantize_rowmajor_wide_kernel(const T* __
     }
     GroupCodes o;
     quantize_group_regs<MODE, WANT_MASK>(v, seed, gi, o);
+    job_stores_next();
     out.codes[gi] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
     out.scales[gi] = (uint8_t)o.scale_byte;
     if constexpr (WANT_MASK) out.maskbits[gi] = o.keep;
@@ -612,6 +619,7 @@ struct TransposedJob {
 #pragma unroll
                 for (int i = 0; i < 32; ++i) v[gq][i] = 0.0f;
         }
+        job_requests_issued();
         if constexpr (DENSE) {  // the matrix instruction needs the whole wave, lanes outside the tensor included
             DenseFrag frag;
             load_dense_frag(matrix, sizeof(T) == 2 ? BF16 : F32, frag);
@@ -770,6 +778,7 @@ struct RequantJob {
 #pragma unroll
             for (int i = 0; i < 32; ++i) sc[i] = 1.0f;
         }
+        job_requests_issued();
         DenseFrag frag;
         if constexpr (DENSE) load_dense_frag(matrix, VAL_DTYPE, frag);
         uint4* ocodes = ocodes_all[wave];
