@@ -226,6 +226,21 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                        int w_val_dtype, int mid_dtype, int x_scale_dtype, int w_scale_dtype, void* workspace,
                        size_t workspace_bytes, void* gx, void* gw, int gw_dtype, int codes_layout, int gx_rotated,
                        const float* g_matrix, void* stream);
+/*
+ * qm_linear_backward for callers that replay the step from a captured HIP graph.  It has no counterpart in the reference
+ * (whose stochastic rounding draws a fresh host seed per call, mxfp4_triton.py:196-199, which a captured graph would
+ * freeze).  seed_base: NULL (then exactly qm_linear_backward), or a DEVICE pointer, 8-byte aligned, to one 64-bit value
+ * that the four gradient quantizations read when they run and add to their seed: a graph that also contains a kernel
+ * incrementing that value draws fresh random streams on every replay.  With the value v the results equal those of
+ * qm_linear_backward with seeds[i] + v.  Needs the layout the layer's production path uses (QM_LAYOUT_TILED, Hadamard
+ * blocks 32, T, I, O multiples of 128, g_matrix == NULL); the sign words stay host values.
+ */
+int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, int64_t O, const void* packed_x,
+                              const void* packed_w, int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w,
+                              int hd_g, const uint32_t* signs_g, int g_mode, const uint64_t* seeds, int x_val_dtype,
+                              int w_val_dtype, int mid_dtype, int x_scale_dtype, int w_scale_dtype, void* workspace,
+                              size_t workspace_bytes, void* gx, void* gw, int gw_dtype, int codes_layout, int gx_rotated,
+                              const float* g_matrix, const uint64_t* seed_base, void* stream);
 
 /*
  * Producers fused into the activation quantizer.  The tensor the model would hand to a quantized linear is computed

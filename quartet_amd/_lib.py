@@ -32,6 +32,7 @@ EXPORTS = (
     "qm_linear_backward_workspace_bytes",
     "qm_linear_forward",
     "qm_linear_backward",
+    "qm_linear_backward_seeded",
     "qm_rmsnorm_quantize_mxfp4",
     "qm_swiglu_quantize_mxfp4",
     "qm_rmsnorm_backward_workspace_bytes",
@@ -112,6 +113,8 @@ def lib():
     L.qm_linear_backward.restype = i32
     L.qm_linear_backward.argtypes = [vp, i32, i64, i64, i64, vp, vp, i32, vp, i32, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32,
                                      vp, sz, vp, vp, i32, i32, i32, vp, vp]
+    L.qm_linear_backward_seeded.restype = i32
+    L.qm_linear_backward_seeded.argtypes = L.qm_linear_backward.argtypes[:-1] + [vp, vp]
     _lib = L
     return L
 

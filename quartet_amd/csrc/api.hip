@@ -44,7 +44,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 10; }
+int qm_version(void) { return 11; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -386,7 +386,21 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                        int g_mode, const uint64_t* seeds, int x_val_dtype, int w_val_dtype, int mid_dtype, int x_scale_dtype,
                        int w_scale_dtype, void* workspace, size_t workspace_bytes, void* gx, void* gw, int gw_dtype,
                        int codes_layout, int gx_rotated, const float* g_matrix, void* stream) {
+    return qm_linear_backward_seeded(e, e_dtype, T, I, O, packed_x, packed_w, hd_x, signs_x, hd_w, signs_w, hd_g, signs_g, g_mode, seeds,
+                                     x_val_dtype, w_val_dtype, mid_dtype, x_scale_dtype, w_scale_dtype, workspace, workspace_bytes, gx,
+                                     gw, gw_dtype, codes_layout, gx_rotated, g_matrix, nullptr, stream);
+}
+
+int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, int64_t O, const void* packed_x,
+                              const void* packed_w, int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, int hd_g,
+                              const uint32_t* signs_g, int g_mode, const uint64_t* seeds, int x_val_dtype, int w_val_dtype,
+                              int mid_dtype, int x_scale_dtype, int w_scale_dtype, void* workspace, size_t workspace_bytes, void* gx,
+                              void* gw, int gw_dtype, int codes_layout, int gx_rotated, const float* g_matrix,
+                              const uint64_t* seed_base, void* stream) {
     if (T < 0 || I < 0 || O < 0) return fail(QM_ERR_INVALID, "qm_linear_backward: negative extent");
+    if (seed_base && (!aligned(seed_base, 8) || g_matrix || !pair_launches(codes_layout, T, I, O, hd_x, hd_w, hd_g)))
+        return fail(QM_ERR_INVALID, "qm_linear_backward_seeded: a device seed base needs the tiled layout with Hadamard blocks 32, "
+                                    "T, I, O multiples of 128, no dense rotation, and an 8-byte aligned pointer");
     if (T == 0 || O == 0 || I == 0) return 0;
     if (g_mode != QM_ABSMAX_RTN && g_mode != QM_ABSMAX_SR)
         return fail(QM_ERR_INVALID, "qm_linear_backward: gradient mode must be QM_ABSMAX_RTN or QM_ABSMAX_SR");
@@ -458,11 +472,11 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
         // seven launches: Q(e) with Q(e^T), Q(Q(W)^T) with Q(Q(x)^T), the two products, the two inverse rotations
         const uint32_t sg = signs_g ? signs_g[0] : 0u;
         rc = from_hip(qm::quantize_both_orientations_hd32_tiled(e, e_dtype, T, O, sg, g_mode, seeds[0], seeds[2], k + wl.ec, k + wl.es,
-                                                                k + wl.etc, k + wl.ets, hs), "qm_linear_backward");
+                                                                k + wl.etc, k + wl.ets, seed_base, hs), "qm_linear_backward");
         if (rc) return rc;
         const qm::RequantArgs rw{pw + lw.c, pw + lw.s, O, I, w_val_dtype, seeds[1], k + wl.wtc, k + wl.wts};
         const qm::RequantArgs rx{px + lx.c, px + lx.s, T, I, x_val_dtype, seeds[3], k + wl.xtc, k + wl.xts};
-        rc = from_hip(qm::requantize_transposed_hd32_tiled_pair(rx, rw, sg, g_mode, hs), "qm_linear_backward");
+        rc = from_hip(qm::requantize_transposed_hd32_tiled_pair(rx, rw, sg, g_mode, seed_base, hs), "qm_linear_backward");
         if (rc) return rc;
         rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, gx_product, mid_dtype, codes_layout,
                               codes_layout, gws, wl.gemm_ws_bytes, stream);
@@ -476,6 +490,7 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                                                           w_scale_dtype, signs_w ? signs_w[0] : 0u,
                                                           pw + lw.m, gw, mid_dtype, gw_dtype, hs), "qm_linear_backward");
     }
+    if (seed_base) return fail(QM_ERR_INVALID, "qm_linear_backward_seeded: null, misaligned or ill-typed tensors");
     rc = qm_quantize_mxfp4(e, e_dtype, T, O, hd_g, signs_g, g_mode, 0, nullptr, seeds[0], k + wl.ec, k + wl.es, nullptr, nullptr,
                            codes_layout, stream);
     if (rc) return rc;

@@ -86,9 +86,10 @@ hipError_t quantize_rowmajor_hd32_tiled_pair(const RowmajorArgs& a, const Rowmaj
 hipError_t quantize_both_orientations_hd32_tiled(const void* e, int dtype, int64_t T, int64_t O, uint32_t sign_word, int mode,
                                                  uint64_t seed_rows, uint64_t seed_transposed, uint8_t* codes_rows,
                                                  uint8_t* scales_rows, uint8_t* codes_transposed, uint8_t* scales_transposed,
-                                                 hipStream_t stream);
+                                                 const uint64_t* seed_base, hipStream_t stream);
+// seed_base: null, or device memory holding a value the kernels add to every seed when they run
 hipError_t requantize_transposed_hd32_tiled_pair(const RequantArgs& a, const RequantArgs& b, uint32_t sign_word, int mode,
-                                                 hipStream_t stream);
+                                                 const uint64_t* seed_base, hipStream_t stream);
 hipError_t masked_hadamard_bwd_hd32_pair(const void* ga, int64_t na, int scale_dtype_a, uint32_t sign_a, const uint8_t* mask_a, void* out_a,
                                          const void* gb, int64_t nb, int scale_dtype_b, uint32_t sign_b, const uint8_t* mask_b, void* out_b,
                                          int dtype, int out_dtype_b, hipStream_t stream);

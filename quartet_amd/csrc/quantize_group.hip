@@ -401,6 +401,7 @@ struct RowmajorTiledJob {
     float c;
     uint32_t sign_word;
     uint64_t seed;
+    const uint64_t* seed_base = nullptr;  // device memory, or null: a value the kernel adds to `seed` when it runs
     GroupOut out;
     unsigned blocks;
 
@@ -424,7 +425,7 @@ struct RowmajorTiledJob {
         job_requests_issued();
         rotate_group(v, c, sign_word);
         GroupCodes o;
-        quantize_group_regs<MODE, WANT_MASK>(v, seed, gi, o);
+        quantize_group_regs<MODE, WANT_MASK>(v, seed_base ? seed + *seed_base : seed, gi, o);
         job_stores_next();
         out.codes[ci] = make_uint4(o.w[0], o.w[1], o.w[2], o.w[3]);
         // quad_perm broadcasts of lanes 1, 2, 3 of each quad
@@ -573,6 +574,7 @@ struct TransposedJob {
     float c;
     uint32_t sign_word;
     uint64_t seed;
+    const uint64_t* seed_base = nullptr;  // device memory, or null: a value the kernel adds to `seed` when it runs
     uint8_t* codes;
     uint8_t* scales;
     void* dequant;
@@ -632,7 +634,7 @@ struct TransposedJob {
                 const int64_t gi = (qa + gq) * (P / 32) + pbase / 32;
                 GroupCodes res;
                 if constexpr (!DENSE) rotate_group(v[gq], c, sign_word);
-                quantize_group_regs<MODE, false>(v[gq], seed, gi, res);
+                quantize_group_regs<MODE, false>(v[gq], seed_base ? seed + *seed_base : seed, gi, res);
                 if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res);
                 ocodes[(lane * GPL + gq) * 4 + wave] = make_uint4(res.w[0], res.w[1], res.w[2], res.w[3]);
                 reinterpret_cast<uint8_t*>(oscales)[(lane * GPL + gq) * 4 + wave] = (uint8_t)res.scale_byte;
@@ -680,6 +682,7 @@ struct RequantJob {
     float post, c;
     uint32_t sign_word;
     uint64_t seed;
+    const uint64_t* seed_base = nullptr;  // device memory, or null: a value the kernel adds to `seed` when it runs
     uint8_t* codes;
     uint8_t* scales;
     void* dequant;
@@ -730,7 +733,7 @@ struct RequantJob {
             const int64_t gi = (ca + 2 * P + gq) * (R / 32) + rbase / 32;
             GroupCodes res;
             if constexpr (!DENSE) rotate_group(v[gq], c, sign_word);
-            quantize_group_regs<MODE, false>(v[gq], seed, gi, res);
+            quantize_group_regs<MODE, false>(v[gq], seed_base ? seed + *seed_base : seed, gi, res);
             if (dequant) store_dequant<T>(reinterpret_cast<T*>(dequant) + gi * 32, res);
             const int cl = 4 * cq + 2 * P + gq;
             ocodes[cl * 4 + rg] = make_uint4(res.w[0], res.w[1], res.w[2], res.w[3]);
@@ -1210,15 +1213,17 @@ hipError_t quantize_rowmajor_hd32_tiled_pair(const RowmajorArgs& a, const Rowmaj
 hipError_t quantize_both_orientations_hd32_tiled(const void* e, int dtype, int64_t T, int64_t O, uint32_t sign_word, int mode,
                                                  uint64_t seed_rows, uint64_t seed_transposed, uint8_t* codes_rows,
                                                  uint8_t* scales_rows, uint8_t* codes_transposed, uint8_t* scales_transposed,
-                                                 hipStream_t stream) {
+                                                 const uint64_t* seed_base, hipStream_t stream) {
     const GroupOut orow{reinterpret_cast<uint4*>(codes_rows), scales_rows, nullptr, nullptr};
     const float c = hadamard_scale(32, dtype);
     with_elem_type(dtype, [&](auto t) {
         with_absmax_mode(mode, [&](auto m) {
             using T_ = decltype(t);
             constexpr int M = decltype(m)::value;
-            launch_job_pair(TransposedJob<T_, M>(e, T, O, c, sign_word, seed_transposed, codes_transposed, scales_transposed, nullptr, true),
-                            RowmajorTiledJob<T_, M, false>(e, T, O, c, sign_word, seed_rows, orow), stream);
+            TransposedJob<T_, M> jt(e, T, O, c, sign_word, seed_transposed, codes_transposed, scales_transposed, nullptr, true);
+            RowmajorTiledJob<T_, M, false> jr(e, T, O, c, sign_word, seed_rows, orow);
+            jt.seed_base = jr.seed_base = seed_base;
+            launch_job_pair(jt, jr, stream);
         });
     });
     return hipGetLastError();
@@ -1226,7 +1231,7 @@ hipError_t quantize_both_orientations_hd32_tiled(const void* e, int dtype, int64
 
 // transpose + rotate + re-quantize two packed tensors (tiled codes in and out), e.g. Q(W) and Q(x) of a layer
 hipError_t requantize_transposed_hd32_tiled_pair(const RequantArgs& a, const RequantArgs& b, uint32_t sign_word, int mode,
-                                                 hipStream_t stream) {
+                                                 const uint64_t* seed_base, hipStream_t stream) {
     const float ca = hadamard_scale(32, a.val_dtype), cb = hadamard_scale(32, b.val_dtype);
     const auto with_val = [](int dt, auto&& f) {
         if (dt == BF16) f(std::integral_constant<int, BF16>{});
@@ -1236,8 +1241,10 @@ hipError_t requantize_transposed_hd32_tiled_pair(const RequantArgs& a, const Req
         with_val(b.val_dtype, [&](auto vb) {
             with_absmax_mode(mode, [&](auto m) {
                 constexpr int M = decltype(m)::value;
-                launch_job_pair(RequantJob<decltype(va)::value, M>(a.codes_in, a.scales_in, a.R, a.C, 1.0f, ca, sign_word, a.seed, a.codes, a.scales, nullptr, true, true),
-                                RequantJob<decltype(vb)::value, M>(b.codes_in, b.scales_in, b.R, b.C, 1.0f, cb, sign_word, b.seed, b.codes, b.scales, nullptr, true, true), stream);
+                RequantJob<decltype(va)::value, M> ja(a.codes_in, a.scales_in, a.R, a.C, 1.0f, ca, sign_word, a.seed, a.codes, a.scales, nullptr, true, true);
+                RequantJob<decltype(vb)::value, M> jb(b.codes_in, b.scales_in, b.R, b.C, 1.0f, cb, sign_word, b.seed, b.codes, b.scales, nullptr, true, true);
+                ja.seed_base = jb.seed_base = seed_base;
+                launch_job_pair(ja, jb, stream);
             });
         });
     });

@@ -371,12 +371,17 @@ def rope_merge_qkv_grad(dq, dk, dv, table, n_embd, head_dim, seq_len, out_dtype)
 
 
 def linear_backward(e2, packed_x, packed_w, T, I, O, hd_x, signs_x, hd_w, signs_w, hd_g, signs_g, mode, seeds, x_val_dtype,
-                    w_val_dtype, mid_dtype, x_scale_dtype, w_scale_dtype, tiled, gx_rotated=False, gw_dtype=None, g_matrix=None):
+                    w_val_dtype, mid_dtype, x_scale_dtype, w_scale_dtype, tiled, gx_rotated=False, gw_dtype=None, g_matrix=None,
+                    seed_base=None):
     """Whole backward pass in one foreign call: e [T,O] -> (gx [T,I], gw [O,I]) of mid_dtype.  With `gx_rotated`, gx is
     still in the rotated basis of the activation quantizer: its masked inverse rotation is left to the kernel that
     consumes gx (rmsnorm_backward / swiglu_backward with `maskbits`).  `gw_dtype` = float32 with a bf16 mid_dtype returns
-    gw as the bf16-rounded values widened to fp32 (the cast autograd would apply for an fp32 weight) in the same pass."""
-    _require_cuda(e2, packed_x, packed_w)
+    gw as the bf16-rounded values widened to fp32 (the cast autograd would apply for an fp32 weight) in the same pass.
+    `seed_base`: a one-element int64 tensor on the GPU whose value the gradient quantizers add to their seeds when they
+    run (a step replayed from a captured graph draws fresh random streams if the graph also increments it)."""
+    _require_cuda(e2, packed_x, packed_w, seed_base)
+    if seed_base is not None:
+        assert seed_base.dtype == torch.int64 and seed_base.numel() >= 1 and seed_base.is_contiguous()
     assert e2.is_contiguous() and e2.shape == (T, O)
     L = _lib.lib()
     mid = _dtype_code(mid_dtype)
@@ -385,10 +390,10 @@ def linear_backward(e2, packed_x, packed_w, T, I, O, hd_x, signs_x, hd_w, signs_
     gx = torch.empty((T, I), dtype=mid_dtype, device=e2.device)
     gw_dtype = mid_dtype if gw_dtype is None or mid_dtype != torch.bfloat16 else gw_dtype
     gw = torch.empty((O, I), dtype=gw_dtype, device=e2.device)
-    rc = L.qm_linear_backward(_ptr(e2), _dtype_code(e2.dtype), T, I, O, _ptr(packed_x), _ptr(packed_w), hd_x, sign_words(signs_x),
-                              hd_w, sign_words(signs_w), hd_g, sign_words(signs_g), mode, (ctypes.c_uint64 * 4)(*seeds),
-                              _dtype_code(x_val_dtype), _dtype_code(w_val_dtype), mid, _dtype_code(x_scale_dtype),
-                              _dtype_code(w_scale_dtype), _ptr(work), nbytes, _ptr(gx), _ptr(gw), _dtype_code(gw_dtype), _layout(tiled),
-                              int(gx_rotated), _ptr(g_matrix), _stream())
+    rc = L.qm_linear_backward_seeded(_ptr(e2), _dtype_code(e2.dtype), T, I, O, _ptr(packed_x), _ptr(packed_w), hd_x,
+                                     sign_words(signs_x), hd_w, sign_words(signs_w), hd_g, sign_words(signs_g), mode,
+                                     (ctypes.c_uint64 * 4)(*seeds), _dtype_code(x_val_dtype), _dtype_code(w_val_dtype), mid,
+                                     _dtype_code(x_scale_dtype), _dtype_code(w_scale_dtype), _ptr(work), nbytes, _ptr(gx), _ptr(gw),
+                                     _dtype_code(gw_dtype), _layout(tiled), int(gx_rotated), _ptr(g_matrix), _ptr(seed_base), _stream())
     _lib.check(rc, "qm_linear_backward")
     return gx, gw

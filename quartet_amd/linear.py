@@ -16,6 +16,23 @@ from .quantizers import QUANTIZER_CLASSES, AlbertTsengQuantizer, NoQuantizer, Qu
 from .quantizers.mxfp4 import _autocast_bf16, _fresh_seed
 
 
+_SEED_BASE = None
+
+
+def set_device_seed_base(tensor):
+    """A one-element int64 tensor on the GPU (or None to switch this off) whose value the gradient quantizers of every
+    packed-path layer add to their seeds when their kernels run.  The reference draws a fresh host seed per stochastic
+    quantization (mxfp4_triton.py:196-199); a training step replayed from a captured HIP graph would repeat the seeds
+    drawn at capture time, so capture the step with a seed base set and let the graph increment the tensor (any
+    in-place add recorded in the graph): every replay then rounds with fresh random streams.  The sign flips drawn at
+    capture time stay as they are.  Applies to layers on the tiled layout (tokens, in- and out-features multiples of
+    128, Hadamard blocks 32, no dense rotation); others ignore it."""
+    global _SEED_BASE
+    if tensor is not None and not (tensor.is_cuda and tensor.dtype == torch.int64 and tensor.numel() >= 1):
+        raise ValueError("the seed base must be an int64 tensor on the GPU")
+    _SEED_BASE = tensor
+
+
 def _use_tiled_codes(T, I, O, a_q, w_q, g_q):
     """Tiled code bytes (16 rows x 128 elements contiguous) when every operand of the three products qualifies: all
     three extents multiples of 128 and at least 256, Hadamard block 32 throughout; row-major codes otherwise."""
@@ -63,7 +80,8 @@ def _backward_packed(ctx, e, packed_x, packed_w, gx_rotated=False):
     sd_w = torch.bfloat16 if low else ctx.w_dtype
     gx, gw = K.linear_backward(e2, packed_x, packed_w, T, I, O, a_hd, a_signs, w_hd, w_signs, hd, signs, mode, seeds, ctx.x_dtype,
                                ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled, gx_rotated,
-                               ctx.w_dtype if ctx.w_dtype in (torch.float32, torch.bfloat16) else None, g_matrix)
+                               ctx.w_dtype if ctx.w_dtype in (torch.float32, torch.bfloat16) else None, g_matrix,
+                               _SEED_BASE if (ctx.tiled and g_matrix is None and g_q.stochastic) else None)
     if gx_rotated:
         return gx, gw, (K.packed_mask_bits(packed_x, T, I), a_signs, sd_x)
     return gx, gw
