@@ -135,3 +135,23 @@ def test_captured_layer_step_draws_fresh_streams_with_a_seed_base():
     finally:
         lin._fresh_seed = old
         q.set_device_seed_base(None)
+
+
+def test_sign_flips_of_the_gradient_rotation_cancel_in_both_products():
+    """Why a captured step needs no device-side sign words: the gradient quantizer's sign flips (re_randomize("signs"),
+    mxfp4.py:53-60) multiply both operands of each backward product along the contracted index, and the absmax
+    quantizers are odd, so gx and gw do not depend on them, bit for bit."""
+    from quartet_amd import kernels as K
+    dev = torch.device("cuda:0")
+    T, I, O = 512, 384, 640
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(T, I, generator=g).bfloat16().to(dev)
+    w = (0.02 * torch.randn(O, I, generator=g)).to(dev)
+    e = (1e-3 * torch.randn(T, O, generator=g)).bfloat16().to(dev)
+    _, px, pw = K.linear_forward(x, w, 32, None, 32, None, torch.bfloat16, True)
+    for mode in (K.QM_ABSMAX_SR, K.QM_ABSMAX_RTN):
+        outs = [K.linear_backward(e, px, pw, T, I, O, 32, None, 32, None, 32, sg, mode, (31, 32, 33, 34), x.dtype, w.dtype,
+                                  torch.bfloat16, torch.bfloat16, torch.bfloat16, True, False, torch.float32)
+                for sg in (0, 0x0F0F3C3C, 0xFFFFFFFF, 0x80000001)]
+        for o in outs[1:]:
+            assert torch.equal(o[0], outs[0][0]) and torch.equal(o[1], outs[0][1])

@@ -434,3 +434,35 @@ def test_notebook_error_bands(oracle):
     gwq = oracle.gemm_tn(et["codes"], et["scales"], xt["codes"], xt["scales"], a_post=d, b_post=d)
     gw = oracle.masked_hadamard_bwd(gwq.astype(np.float32), 32, oracle.BF16, None, qw["mask"])
     assert 6e-2 < err(gw.astype(np.float64), ef.T @ xf) < 15e-2
+
+
+def test_sign_flips_of_the_rotation_only_flip_code_signs(oracle):
+    """re_randomize("signs") multiplies the rotation's columns by +-1 (mxfp4.py:53-60).  The quantizers are odd functions
+    The absmax quantizers are odd functions (the scale and the rounding brackets work on magnitudes,
+    mxfp4_triton.py:57-121), so a flipped column changes nothing but the sign bit of its non-zero codes: the two products
+    of the backward pass, which rotate both operands with the same flipped matrix along the contracted index
+    (backward.py:64-85), are bit-for-bit independent of the flips.  (The quest scale is not: its standard deviation
+    is taken about the group's mean, mxfp4_triton.py:52-54.)"""
+    o = oracle
+    rng = np.random.default_rng(11)
+    x = o.bf16_bits_to_f32(o.f32_to_bf16_bits(rng.standard_normal((64, 256)).astype(np.float32)))
+    xb = o.f32_to_bf16_bits(x)
+    sa = rng.integers(0, 2, 32) * 2 - 1
+    sb = rng.integers(0, 2, 32) * 2 - 1
+    flipped = np.tile(sa != sb, 256 // 32)                       # per column of the rotated tensor
+    for mode in (o.ABSMAX_RTN, o.ABSMAX_SR):
+        a = o.quantize(xb, 32, signs=sa, mode=mode, seed=5)
+        b = o.quantize(xb, 32, signs=sb, mode=mode, seed=5)
+        assert np.array_equal(a["scales"], b["scales"])
+        na, nb = o.unpack_codes(a["codes"]), o.unpack_codes(b["codes"])
+        assert np.array_equal(na & 7, nb & 7)
+        nonzero = (na & 7) != 0
+        assert np.array_equal(((na ^ nb) >> 3)[nonzero], np.broadcast_to(flipped, na.shape)[nonzero].astype(na.dtype))
+    # both operands of a product flipped alike: the product does not move
+    w = o.f32_to_bf16_bits(rng.standard_normal((96, 256)).astype(np.float32))
+    prods = []
+    for s in (sa, sb):
+        qa = o.quantize(xb, 32, signs=s, mode=o.ABSMAX_SR, seed=7)
+        qb = o.quantize(w, 32, signs=s, mode=o.ABSMAX_SR, seed=8)
+        prods.append(o.gemm_tn(qa["codes"], qa["scales"], qb["codes"], qb["scales"]))
+    assert np.array_equal(prods[0], prods[1])
