@@ -362,6 +362,40 @@ def gemm_operand_content(x, w, dy, rounds=3):
     return {k: {"ms": round(sorted(v)[len(v) // 2], 4), "TFLOPs": round(flops / sorted(v)[len(v) // 2] / 1e9, 1)} for k, v in out.items()}
 
 
+def gemm_tile_phases(x, w, launches=5):
+    """Where a tile's time goes in the forward product: the persistent kernel's stamping instantiation records the shader
+    clock around every tile's K loop and epilogue (thread 0 of each workgroup).  No matrix instruction runs during an
+    epilogue, so its share of a tile is the share of the launch the matrix pipe idles for at the tile boundaries."""
+    import statistics
+    from quartet_amd import kernels as K
+    xc, xs, _, _ = K.quantize_mxfp4(x, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=True)
+    wc, ws, _, _ = K.quantize_mxfp4(w, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=True)
+    for _ in range(40):   # the state the chip is in during the step: clocks settled under this kernel
+        K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.bfloat16, a_tiled=True, b_tiled=True)
+    ksteps = x.shape[1] // 128
+    k_loop, epi, span = [], [], []
+    for _ in range(launches):
+        _, st = K.gemm_tile_phases(xc, xs, wc, ws, 1.0, a_tiled=True, b_tiled=True)
+        st = st.tolist()
+        for row in st:
+            start = row[1]
+            for i in range(2, len(row) - 1, 2):
+                if row[i] == 0:
+                    break
+                k_loop.append(row[i] - start)
+                epi.append(row[i + 1] - row[i])
+                start = row[i + 1]
+        span.append(max(max(r) - r[0] for r in st))   # per workgroup: the XCDs' counters are not aligned with each other
+    kl, ep = statistics.median(k_loop), statistics.median(epi)
+    return {"what": "shader-clock stamps of the forward product's kernel, medians over every tile of %d launches" % launches,
+            "tiles_per_workgroup": len(k_loop) // max(1, launches * len(st)),
+            "k_loop_cycles": int(kl), "cycles_per_k_step": round(kl / ksteps, 1), "epilogue_cycles": int(ep),
+            "epilogue_share_of_tile": round(ep / (kl + ep), 4),
+            "k_loop_matrix_pipe_duty": round(32 * 32 * ksteps / kl, 4),   # 32 instructions of 32 cycles per K step per SIMD
+            "longest_workgroup_cycles": int(statistics.median(span)),
+            "matrix_pipe_duty_of_the_launch": round(32 * 32 * ksteps * (len(k_loop) / max(1, launches * len(st))) / statistics.median(span), 4)}
+
+
 def mfma_only_ceiling(x, w, iters=400, rounds=3):
     """The FP4 matrix instruction alone (no loads, no epilogue) on the bytes of the forward product's real operands, on
     uniformly random bytes and on zero bytes: what the chip sustains for this instruction at its power limit, which is
@@ -800,6 +834,7 @@ def main():
                                        "frac": round(qk["GBps"] / PEAK_HBM_GBS, 4), "traffic": traffic, "traffic_source": source,
                                        "avg_launch_ms": qk["ms"], **quantizer_bounds(prof, x.detach())}
     if not args.no_breakdown:
+        result["roofline"]["tile_phases"] = gemm_tile_phases(x.detach(), w)
         ceil = mfma_only_ceiling(x.detach(), w)
         result["mfma_only_TFLOPs"] = ceil
         result["roofline"]["frac_of_mfma_only_rate_on_real_operands"] = round(

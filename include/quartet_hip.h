@@ -162,6 +162,20 @@ int64_t qm_diag_mfma_only(const uint8_t* operands, size_t operand_bytes, float* 
  * profiler's kernel trace shows it, inside whatever sequence of kernels it runs.  count == 0 withdraws unused pairs.
  */
 int qm_diag_time_gemm_launches(void* const* start_events, void* const* stop_events, int count);
+/*
+ * Measurement aid, no counterpart in the reference: one launch of an instantiation of the product's persistent tile kernel
+ * (bf16 output, arguments as qm_gemm_mxfp4_tn) that also records the shader clock, per workgroup, at its entry, at the
+ * start of its tile loop, and after every tile's K loop and epilogue (up to 15 tiles): QM_DIAG_PHASE_STAMPS 64-bit values
+ * per workgroup into `stamps` (DEVICE memory, stamps_bytes >= workgroups * QM_DIAG_PHASE_STAMPS * 8; one workgroup per
+ * CU or per tile, whichever is fewer).  Where the time of a tile goes -- K steps against the epilogue, during which no
+ * matrix instruction runs -- is read from the differences; bench.py --gemm-phases prints them.  c receives the product.
+ * Serves M, N multiples of 64 and >= 256, K % 512 == 0.  Returns the number of workgroups launched, or a negative
+ * status.  Synchronises with the host once (it sets a device-side pointer before the launch).
+ */
+#define QM_DIAG_PHASE_STAMPS 32
+int qm_diag_gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
+                             int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout, uint64_t* stamps,
+                             size_t stamps_bytes, void* stream);
 
 /*
  * out = ((g * mask).view(-1, hd)) @ H^T: the straight-through backward of the forward quantizer,

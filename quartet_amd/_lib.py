@@ -25,6 +25,7 @@ EXPORTS = (
     "qm_gemm_workspace_bytes",
     "qm_diag_mfma_only",
     "qm_diag_time_gemm_launches",
+    "qm_diag_gemm_tile_phases",
     "qm_gemm_noalloc_scratch_bytes",
     "qm_gemm_mxfp4_tn_noalloc",
     "qm_packed_operand_bytes",
@@ -75,6 +76,8 @@ def lib():
     L.qm_gemm_mxfp4_tn.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, i32, vp, ctypes.c_size_t, vp]
     L.qm_diag_time_gemm_launches.restype = i32
     L.qm_diag_time_gemm_launches.argtypes = [vp, vp, i32]
+    L.qm_diag_gemm_tile_phases.restype = i32
+    L.qm_diag_gemm_tile_phases.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, vp, ctypes.c_size_t, vp]
     L.qm_diag_mfma_only.restype = i64
     L.qm_diag_mfma_only.argtypes = [vp, ctypes.c_size_t, vp, ctypes.c_size_t, i32, vp]
     L.qm_gemm_workspace_bytes.restype = ctypes.c_size_t

@@ -44,7 +44,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 11; }
+int qm_version(void) { return 12; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -175,6 +175,23 @@ int qm_diag_time_gemm_launches(void* const* start_events, void* const* stop_even
         if (!start_events[i] || !stop_events[i]) return fail(QM_ERR_INVALID, "qm_diag_time_gemm_launches: null event at %d", i);
     qm::gemm_time_next_launches(start_events, stop_events, count);
     return 0;
+}
+
+int qm_diag_gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
+                             int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout, uint64_t* stamps,
+                             size_t stamps_bytes, void* stream) {
+    if (!a_codes || !a_scales || !b_codes || !b_scales || !c || !stamps || !aligned(a_codes, 16) || !aligned(b_codes, 16) ||
+        !aligned(c, 16) || !aligned(stamps, 8) || !valid_layout(a_layout) || !valid_layout(b_layout))
+        return fail(QM_ERR_INVALID, "qm_diag_gemm_tile_phases: null, misaligned or ill-typed arguments");
+    int grid = 0;
+    const hipError_t e = qm::gemm_tile_phases(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, a_layout, b_layout,
+                                              reinterpret_cast<unsigned long long*>(stamps), stamps_bytes, &grid,
+                                              reinterpret_cast<hipStream_t>(stream));
+    if (e == hipErrorInvalidValue && grid == 0)
+        return fail(QM_ERR_INVALID, "qm_diag_gemm_tile_phases: serves M, N multiples of 64 and >= 256, K %% 512 == 0, 16-byte aligned scales, "
+                                    "and needs %d 64-bit values per workgroup in stamps", qm::gemm_phase_stamps_per_group());
+    if (int rc = from_hip(e, "qm_diag_gemm_tile_phases")) return rc > 0 ? -rc : rc;
+    return grid;
 }
 
 int64_t qm_diag_mfma_only(const uint8_t* operands, size_t operand_bytes, float* sink, size_t sink_bytes, int iters, void* stream) {

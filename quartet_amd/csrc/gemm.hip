@@ -753,10 +753,21 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
     }
 }
 
+// Measurement aid (the STAMP instantiation of the kernel below): the shader clock at a workgroup's entry, at the start of
+// its tile loop, and after every tile's K loop and epilogue, kPhaseStamps values per workgroup at *g_phase_stamps.
+constexpr int kPhaseStamps = 32;  // entry, loop start, then (K loop end, epilogue end) of up to 15 tiles
+__device__ unsigned long long* g_phase_stamps;
+__device__ __forceinline__ unsigned long long shader_clock() {
+    unsigned long long t;
+    // the counter arrives like a scalar load: without the wait the registers it lands in may be reused before it does
+    asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t));
+    return t;
+}
+
 // Persistent: the grid is one workgroup per CU (or fewer); each workgroup walks tiles bid, bid + grid, ... as one
 // flat stream of K steps.  The loads that refill a freed ring stage simply continue into the next tile, so the
 // pipeline never drains between tiles and the epilogue runs while the next tile's first four stages arrive.
-template <typename OutT>
+template <typename OutT, bool STAMP = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mxfp4_tn_big4_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ b_codes,
     const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c, int a_tiled,
@@ -766,6 +777,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)smem;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
+    [[maybe_unused]] int stamps_taken = 0;
+    const auto stamp = [&]() {
+        if constexpr (STAMP) {
+            const unsigned long long now = shader_clock();
+            if (tid == 0 && stamps_taken < kPhaseStamps) g_phase_stamps[(size_t)blockIdx.x * kPhaseStamps + stamps_taken] = now;
+            ++stamps_taken;
+        }
+    };
+    stamp();
     // wave-uniform by construction; saying so keeps everything derived from it (tile corners, edge tests, the epilogue's
     // base addresses) in scalar registers
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -847,6 +867,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     big_read_sub(smem_bytes, a_off0, b_off0, st.f0);
 
     int par = 0;
+    stamp();
     for (int t = (int)blockIdx.x; t < total_items; t += stride) {
         v16f acc[4][4];
         const int64_t m0 = (int64_t)load_tm * kBigM, n0 = (int64_t)load_tn * kBigN;  // the load stream is still in item t
@@ -877,6 +898,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         };
         block4(0, std::true_type{});
         for (int ks = 4; ks < nk; ks += 4) block4(ks, std::false_type{});
+        stamp();
         if constexpr (sizeof(OutT) == 2) {
             big4_epilogue_bf16(acc, alpha, reinterpret_cast<uint16_t*>(c), m0, n0, N, wm, wn, wave, lane, smem_bytes,
                                rows_valid, cols_valid);
@@ -890,6 +912,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     if (i * 32 < rows_valid && j * 32 < cols_valid)
                         store_tile<OutT, true>(acc[i][j], a_eff, dst, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
         }
+        stamp();
     }
     // direct-to-LDS loads must not outlive the workgroup's LDS allocation
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
@@ -1065,6 +1088,32 @@ hipError_t launch_gemm(const uint8_t* a_codes, const uint8_t* a_scales, const ui
 }
 
 }  // namespace
+
+// one launch of the persistent kernel's stamping instantiation (bf16 output, no K ranges); returns its grid size, 0 on
+// shapes that kernel does not serve.  stamps: device memory for grid * kPhaseStamps 64-bit values.
+int gemm_phase_stamps_per_group() { return kPhaseStamps; }
+hipError_t gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
+                            int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout,
+                            unsigned long long* stamps, size_t stamps_bytes, int* grid_out, hipStream_t stream) {
+    *grid_out = 0;
+    if (!gemm_supports_tiled(M, N, K) || K % 512 || ((reinterpret_cast<uintptr_t>(a_scales) | reinterpret_cast<uintptr_t>(b_scales)) & 15))
+        return hipErrorInvalidValue;
+    auto kern = gemm_mxfp4_tn_big4_kernel<uint16_t, true>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kBig4SmemBytes);
+    if (e != hipSuccess) return e;
+    const int64_t items = ((M + kBigM - 1) / kBigM) * ((N + kBigN - 1) / kBigN);
+    const int cus = device_cus();
+    int64_t g = items < cus ? items : cus;
+    if (g > 8) g -= g % 8;
+    if (stamps_bytes < (size_t)g * kPhaseStamps * sizeof(unsigned long long)) return hipErrorInvalidValue;
+    e = hipMemcpyToSymbol(HIP_SYMBOL(g_phase_stamps), &stamps, sizeof(stamps), 0, hipMemcpyHostToDevice);
+    if (e != hipSuccess) return e;
+    kern<<<dim3((unsigned)g), dim3(256), kBig4SmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
+                                                                  reinterpret_cast<uint16_t*>(c), a_layout == LAYOUT_TILED,
+                                                                  b_layout == LAYOUT_TILED, 1);
+    *grid_out = (int)g;
+    return hipGetLastError();
+}
 
 void gemm_time_next_launches(void* const* start_events, void* const* stop_events, int count) {
     std::lock_guard<std::mutex> lock(g_timing_mutex);

@@ -125,6 +125,11 @@ hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const 
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 // measurement aid: attach these event pairs to the next `count` launches of the persistent product kernel
 void gemm_time_next_launches(void* const* start_events, void* const* stop_events, int count);
+// measurement aid: one launch of the persistent kernel that records the shader clock around every tile's K loop and epilogue
+int gemm_phase_stamps_per_group();
+hipError_t gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
+                            int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout,
+                            unsigned long long* stamps, size_t stamps_bytes, int* grid_out, hipStream_t stream);
 // measurement aid: the FP4 matrix instruction alone (see gemm.hip)
 int mfma_only_blocks();
 hipError_t mfma_only(const uint8_t* operands, float* sink, int iters, hipStream_t stream);

@@ -198,6 +198,28 @@ def time_gemm_launches(n):
     return durations
 
 
+PHASE_STAMPS = 32   # QM_DIAG_PHASE_STAMPS
+
+
+def gemm_tile_phases(a_codes, a_scales, b_codes, b_scales, alpha=1.0, a_tiled=False, b_tiled=False):
+    """Measurement aid: one launch of the persistent tile kernel's stamping instantiation.  Returns (c [M,N] bf16,
+    stamps int64 [workgroups, 32] on the host): per workgroup the shader clock at entry, at the start of its tile loop,
+    then after the K loop and after the epilogue of each of its tiles (unused slots are zero)."""
+    _require_cuda(a_codes, a_scales, b_codes, b_scales)
+    M, K = a_codes.shape[0], a_codes.shape[1] * 2
+    N = b_codes.shape[0]
+    assert b_codes.shape[1] * 2 == K
+    c = torch.empty((M, N), dtype=torch.bfloat16, device=a_codes.device)
+    stamps = torch.zeros((1024, PHASE_STAMPS), dtype=torch.int64, device=a_codes.device)
+    groups = _lib.lib().qm_diag_gemm_tile_phases(_ptr(a_codes), _ptr(a_scales), _ptr(b_codes), _ptr(b_scales), M, N, K, alpha,
+                                                 _ptr(c), _layout(a_tiled), _layout(b_tiled), _ptr(stamps),
+                                                 stamps.numel() * 8, _stream())
+    if groups < 0:
+        _lib.check(int(groups), "qm_diag_gemm_tile_phases")
+    torch.cuda.synchronize()
+    return c, stamps[:groups].cpu()
+
+
 def mfma_only(operand_bytes, iters):
     """Measurement aid: `iters` iterations of the FP4 matrix instruction alone on every CU, fed with bytes of
     `operand_bytes` (uint8, at least 32 KiB per CU).  Returns the number of 32 x 32 x 64 instructions issued."""

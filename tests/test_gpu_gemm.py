@@ -191,3 +191,35 @@ def test_measurement_aids_leave_results_alone(K):
     n = K.mfma_only(buf, 10)
     torch.cuda.synchronize()
     assert n > 0 and n % (4 * 10 * 16) == 0
+
+
+def test_tile_phase_stamps_of_the_persistent_kernel():
+    """The measurement instantiation of the persistent tile kernel (qm_diag_gemm_tile_phases) computes the same product,
+    bit for bit, and its per-workgroup stamps are ordered: entry <= loop start < K loop end < epilogue end < ... for as
+    many tiles as the workgroup walked; together the workgroups walked every tile once."""
+    from quartet_amd import kernels as K, _lib
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(17)
+    M, N, Kd = 2048, 2816, 1024    # 8 x 11 tiles: fewer tiles than CUs, then one per workgroup
+    for M, N in ((2048, 2816), (8192, 4096)):
+        ac = torch.randint(0, 256, (M, Kd // 2), generator=g, dtype=torch.uint8).to(dev)
+        as_ = torch.randint(118, 130, (M, Kd // 32), generator=g, dtype=torch.uint8).to(dev)
+        bc = torch.randint(0, 256, (N, Kd // 2), generator=g, dtype=torch.uint8).to(dev)
+        bs = torch.randint(118, 130, (N, Kd // 32), generator=g, dtype=torch.uint8).to(dev)
+        want = K.gemm_mxfp4_tn(ac, as_, bc, bs, 1.5, torch.bfloat16, split_k=False)
+        got, stamps = K.gemm_tile_phases(ac, as_, bc, bs, 1.5)
+        assert torch.equal(got, want)
+        tiles = 0
+        for row in stamps.tolist():
+            assert 0 < row[0] <= row[1]
+            prev = row[1]
+            for i in range(2, K.PHASE_STAMPS - 1, 2):
+                if row[i] == 0:
+                    assert row[i + 1] == 0
+                    break
+                assert prev < row[i] < row[i + 1]
+                prev = row[i + 1]
+                tiles += 1
+        assert tiles == (M // 256) * (N // 256)
+    with pytest.raises(_lib.QuartetHipError):   # K % 512 != 0: not served
+        K.gemm_tile_phases(ac[:, :320].contiguous(), as_[:, :20].contiguous(), bc[:, :320].contiguous(), bs[:, :20].contiguous())
