@@ -160,22 +160,6 @@ def kernel_breakdown(x, w, dy, only_gemms=False):
     return out
 
 
-def in_step_gemm_times(step, iters=60, warmup=5):
-    """Durations of the three products as they run inside the layer step (the production path, `step` = one forward +
-    backward): the library attaches a HIP event pair to each launch of the product kernel, recorded by the runtime
-    directly around the kernel on the stream it runs on, so no host time falls inside.  The pair's own dispatch adds a
-    few microseconds to each reading."""
-    from quartet_amd import kernels as K
-    for _ in range(warmup):
-        step()
-    durations = K.time_gemm_launches(3 * iters)
-    for _ in range(iters):
-        step()
-    d = durations()
-    names = ("gemm_fwd", "gemm_dgrad", "gemm_wgrad")
-    return {n: round(sum(d[i::3]) / iters, 4) for i, n in enumerate(names)}
-
-
 def in_step_gemm_ms_by_difference(x, w, dy, steps=10, rounds=5):
     """Mean duration of the three products inside the layer step, from two HIP graphs timed with events: the step's
     eleven kernels launched one by one in the layer's order (`steps` times), and the same sequence without the three
@@ -419,14 +403,14 @@ def mfma_only_ceiling(x, w, iters=400, rounds=3):
     return {k: round(sorted(v)[len(v) // 2], 1) for k, v in out.items()}
 
 
-def llama_step(args, device):
+def run_llama(workload, device, unquantized=False, sdpa="auto", warmup=3, steps=5):
     """Whole-model step of a Llama configuration with every block linear on the Quartet path: bf16 autocast around
     forward and backward, cross-entropy on random ids, AdamW (fp32 state) for the ~800 M configuration."""
     from quartet_amd import llama as L
     torch.manual_seed(0)
-    over = L.unquantized() if args.unquantized else {}
-    over["sdpa_backend"] = args.sdpa
-    if args.workload == "llama30m":
+    over = L.unquantized() if unquantized else {}
+    over["sdpa_backend"] = sdpa
+    if workload == "llama30m":
         cfg, batch, seq, opt_step = L.llama_30m(**over), 64, 512, False
     else:
         cfg, batch, seq, opt_step = L.llama_800m(**over), 16, 2048, True
@@ -445,28 +429,69 @@ def llama_step(args, device):
         model.zero_grad(set_to_none=True)
         return loss
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     torch.cuda.reset_peak_memory_stats()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         loss = step()
     torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    ms = (time.perf_counter() - t0) / steps * 1e3
     peak_gib = torch.cuda.max_memory_allocated() / 2 ** 30
     lin = sum(m.weight.numel() for _, m in model.block_linears())
     tokens = batch * seq
-    flops = 6.0 * tokens * lin
+    out = {"ms_per_step": round(ms, 3), "tokens_per_s": round(tokens / (ms * 1e-3), 1), "final_loss": round(float(loss.detach()), 4),
+           "peak_allocated_GiB": round(peak_gib, 2), "block_linear_flops": 6.0 * tokens * lin, "tokens": tokens,
+           "what": f"{cfg.n_layer} layers, d {cfg.n_embd}, {batch}x{seq} tokens, {'fwd+bwd+AdamW' if opt_step else 'fwd+bwd'}"}
+    del model, opt
+    torch.cuda.empty_cache()
+    return out
+
+
+def llama_step(args, device):
+    r = run_llama(args.workload, device, args.unquantized, args.sdpa, args.warmup, args.steps)
+    flops = r.pop("block_linear_flops")
+    ms = r["ms_per_step"]
     return {"metric": "Quartet linear fwd+bwd TFLOPS (MXFP4 MFMA) + Hadamard/quantize HBM GB/s",
             "value": round(flops / (ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-            "warmup": args.warmup, "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak",
+            "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "bf16" if args.unquantized else "mxfp4", "data": "synthetic",
-            "config": {"workload": f"{args.workload}{' (unquantized bf16 linears)' if args.unquantized else ''} whole-model step ({cfg.n_layer} layers, d {cfg.n_embd}, {batch}x{seq} tokens, "
-                                   f"{'fwd+bwd+AdamW' if opt_step else 'fwd+bwd'}); value counts the block linears' 6*tokens*params "
-                                   f"flops only ({flops / 1e12:.2f} TFLOP) over the whole step time"},
-            "tokens_per_s": round(tokens / (ms * 1e-3), 1), "final_loss": round(float(loss.detach()), 4),
-            "peak_allocated_GiB": round(peak_gib, 2)}
+            "config": {"workload": f"{args.workload}{' (unquantized bf16 linears)' if args.unquantized else ''} whole-model step ({r['what']}); "
+                                   f"value counts the block linears' 6*tokens*params flops only ({flops / 1e12:.2f} TFLOP) over the whole step time"},
+            "tokens_per_s": r["tokens_per_s"], "final_loss": r["final_loss"], "peak_allocated_GiB": r["peak_allocated_GiB"]}
+
+
+def llama_blocks(device):
+    """The two whole-model configurations in brief: 2 warm-up + 3 timed steps each, the Quartet model and the same model
+    with plain bf16 linears beside it."""
+    out = {}
+    for name in ("llama30m", "llama800m"):
+        row = {}
+        for label, unq in (("quartet", False), ("bf16_linears", True)):
+            r = run_llama(name, device, unquantized=unq, warmup=2, steps=3)
+            row["what"] = r["what"]
+            row[label] = {"ms_per_step": r["ms_per_step"], "tokens_per_s": r["tokens_per_s"], "peak_allocated_GiB": r["peak_allocated_GiB"]}
+        row["speedup_over_bf16_linears"] = round(row["bf16_linears"]["ms_per_step"] / row["quartet"]["ms_per_step"], 3)
+        out[name] = row
+    return out
+
+
+def k1536_block(device):
+    """The short-K product of the ~800 M model's attention projection (32768 tokens x 4608 out x 1536 in): chain timing
+    and the tile-phase stamps, on quest codes of Gaussian operands."""
+    from quartet_amd import kernels as K
+    M, N, Kd = 32768, 4608, 1536
+    g = torch.Generator(device=device).manual_seed(1536)
+    x = torch.randn(M, Kd, generator=g, device=device).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, Kd, generator=g, device=device)).to(torch.bfloat16)
+    xc, xs, _, _ = K.quantize_mxfp4(x, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=True)
+    wc, ws, _, _ = K.quantize_mxfp4(w, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=True)
+    ms = sorted(time_kernel(lambda: K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.bfloat16, a_tiled=True, b_tiled=True), reps=20)
+                for _ in range(3))[1]
+    tf = 2.0 * M * N * Kd / ms / 1e9
+    return {"shape": [M, N, Kd], "ms": round(ms, 4), "TFLOPs": round(tf, 1), "frac_of_peak": round(tf / PEAK_FP4_TFLOPS, 4),
+            "how": "median of three replays of a 20-launch graph", "tile_phases": gemm_tile_phases(x, w, launches=3)}
 
 
 def _csrc_sha16():
@@ -731,7 +756,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
     ap.add_argument("--no-extra", action="store_true",
-                    help="skip the brief out=11008 and quantizer-size blocks the default run appends")
+                    help="skip the blocks the default run appends: out=11008, the K=1536 product, quantizer sizes, the reference's notebook shapes, the two Llama steps")
     ap.add_argument("--workload", default="linear", choices=["linear", "llama30m", "llama800m"],
                     help="linear (default): the isolated 8192x4096x4096 layer the metric is quoted on; llama30m / llama800m: "
                          "whole-model fwd+bwd(+AdamW) step of the 30 M / ~800 M Llama configurations, reported in the same unit "
@@ -786,9 +811,16 @@ def main():
         K.quantize_mxfp4(x.detach(), 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=True)
         torch.cuda.synchronize()
         del src, dst
+    flops = 6.0 * T_TOKENS * IN_F * out_f
+    kb = None
+    if not args.no_breakdown:
+        # the per-kernel timings run first: the headline figure below is then taken on a chip that has been busy for a
+        # few seconds, as during training, instead of on one that has just left idle clocks
+        x.requires_grad_(False)
+        kb = kernel_breakdown(x.detach(), w, dy)
+        x.requires_grad_(True)
     ms_per_step, sustained = time_layer_steps(make_step(layer, x, dy), args.steps, args.warmup,
                                               sustain_s=0.0 if args.calibration_copy else 1.0)
-    flops = 6.0 * T_TOKENS * IN_F * out_f
     result = {
         "metric": "Quartet linear fwd+bwd TFLOPS (MXFP4 MFMA) + Hadamard/quantize HBM GB/s",
         "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2),
@@ -797,36 +829,29 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "mxfp4", "data": "synthetic",
         "config": {"workload": f"isolated Quartet linear fwd+dgrad+wgrad, tokens {T_TOKENS} x in {IN_F} x out {out_f}, "
                                "bf16 X/W/dY, quest-RTN forward, absmax-SR backward, Hadamard 32"},
+        "order": "per-kernel timings, then warm-up + timed steps (value), then the remaining blocks",
         "sustained": {**sustained, "TFLOPs_median": round(flops / sustained["ms_per_step_median"] / 1e9, 1)},
     }
     prof = traffic_profile() if out_f == OUT_F else None
     if not args.no_breakdown:
         x.requires_grad_(False)
-        kb = kernel_breakdown(x.detach(), w, dy)
         result["kernels"] = kb
-        # the three GEMMs of a step (fwd, dgrad, wgrad) run the same kernel on the same flop count: the roofline
-        # entry is their mean, which is what a profiler's per-kernel average over the run reports
         # The three GEMMs of a step (fwd, dgrad, wgrad) run the same kernel on the same flop count: the roofline entry is
         # their mean duration inside the step, where they run between quantizer kernels (in_step_gemm_ms_by_difference),
         # which is what a profiler's per-kernel average over the step loop shows.  `back_to_back` times each of the three
         # as an unbroken chain of its own launches: that holds the chip at its power limit throughout and is the slowest
-        # setting for this kernel (5-10 % longer).  `in_step_stamped_ms` are readings of event pairs the library attaches
-        # to each launch in the production path; a pair's own dispatch adds a few microseconds to each.
+        # setting for this kernel (5-10 % longer).
         chain_ms, chain_tf = gemm_summary(kb, T_TOKENS, out_f)
         diff = in_step_gemm_ms_by_difference(x.detach(), w, dy)
         gemm_ms = diff.pop("ms")
         gemm_tf = 2.0 * T_TOKENS * IN_F * out_f / gemm_ms / 1e9
-        x.requires_grad_(True)
-        ist = in_step_gemm_times(make_step(layer, x, dy))
-        x.requires_grad_(False)
         traffic, source = _traffic_entry(prof, "gemm_mxfp4_tn")
         result["roofline"] = {"bound": "mfma", "kernel": f"gemm_mxfp4_tn ({T_TOKENS}x{out_f}x{IN_F}, {T_TOKENS}x{IN_F}x{out_f}, {out_f}x{IN_F}x{T_TOKENS})",
                               "achieved": round(gemm_tf, 1), "peak": PEAK_FP4_TFLOPS, "unit": "TFLOP/s",
                               "frac": round(gemm_tf / PEAK_FP4_TFLOPS, 4), "traffic": traffic, "traffic_source": source,
                               "avg_launch_ms": round(gemm_ms, 4), "how": {"what": "mean of the step's three products, timed inside the step", **diff},
                               "back_to_back": {"avg_launch_ms": round(chain_ms, 4), "TFLOPs": round(chain_tf, 1),
-                                               "frac": round(chain_tf / PEAK_FP4_TFLOPS, 4)},
-                              "in_step_stamped_ms": ist}
+                                               "frac": round(chain_tf / PEAK_FP4_TFLOPS, 4)}}
         qk = kb["quantize_x_quest_rtn_mask"]
         traffic, source = _traffic_entry(prof, "quantize_x_quest_rtn_mask_alone")
         result["roofline_quantize"] = {"bound": "hbm", "kernel": f"quantize_rowmajor (quest RTN + mask, {T_TOKENS}x{IN_F} bf16)",
@@ -842,10 +867,16 @@ def main():
     if not args.no_extra and not args.no_breakdown and out_f == OUT_F:
         del layer
         result["out11008"] = out11008_block(device, args)
+        result["k1536"] = k1536_block(device)
         result["quantizer_sizes"] = quantizer_sizes_block(device)
+        result["reference_shapes"] = reference_shapes(device)
+        del x, w, dy
+        torch.cuda.empty_cache()
+        result["llama"] = llama_blocks(device)
+        x, w, dy = make_inputs(device, out_f=out_f)
     if args.quantizer_sweep:
         result["quantizer_sweep"] = quantizer_sweep(device)
-    if args.reference_shapes:
+    if args.reference_shapes and "reference_shapes" not in result:
         result["reference_shapes"] = reference_shapes(device)
     if args.library_gemm:
         result["library_gemm"] = library_gemm(device)

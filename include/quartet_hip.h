@@ -136,10 +136,16 @@ int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint
  * device array built into the library (QM_GEMM_NOALLOC_SCRATCH_BYTES per GPU, held until the process ends) instead.
  * A shape whose partial sums need more is rejected with QM_ERR_INVALID.  Nothing in the array has to start at zero
  * (every partial sum that is read has been written by the same call), but every call on a GPU uses that GPU's one
- * array: calls that overlap on one GPU (two streams, two threads) race.  Allocates nothing, frees nothing.
+ * array: calls that overlap on one GPU (two streams, two threads) race.  Allocates nothing, frees nothing --
+ * with one proviso about the HIP runtime: the device address of the array is looked up on a device's first use, and
+ * that lookup is when the runtime places this library's device image (the array included) in that GPU's memory.
+ * qm_gemm_noalloc_prepare() performs the lookup for the current device and nothing else: call it once per device,
+ * outside any stream capture, before the first call that must not allocate (a first qm_gemm_mxfp4_tn_noalloc call
+ * without it does the lookup itself).  Every later call on that device touches no allocator of any kind.
  */
 #define QM_GEMM_NOALLOC_SCRATCH_BYTES ((size_t)64 << 20)
 size_t qm_gemm_noalloc_scratch_bytes(void);
+int qm_gemm_noalloc_prepare(void);
 int qm_gemm_mxfp4_tn_noalloc(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                              const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c,
                              int c_dtype, int a_layout, int b_layout, void* stream);
@@ -155,14 +161,6 @@ int qm_gemm_mxfp4_tn_noalloc(const uint8_t* a_codes, const uint8_t* a_scales, co
 int64_t qm_diag_mfma_only(const uint8_t* operands, size_t operand_bytes, float* sink, size_t sink_bytes, int iters,
                           void* stream);
 /*
- * Measurement aid, no counterpart in the reference: hands the library `count` pairs of hipEvent_t (HOST arrays of
- * handles created with timing enabled).  Each of the next `count` launches of the product's persistent tile kernel
- * -- from qm_gemm_mxfp4_tn or from inside qm_linear_forward / qm_linear_backward -- takes one pair, and the runtime
- * stamps it with that kernel's own begin and end, so hipEventElapsedTime(start, stop) is the kernel's duration as a
- * profiler's kernel trace shows it, inside whatever sequence of kernels it runs.  count == 0 withdraws unused pairs.
- */
-int qm_diag_time_gemm_launches(void* const* start_events, void* const* stop_events, int count);
-/*
  * Measurement aid, no counterpart in the reference: one launch of an instantiation of the product's persistent tile kernel
  * (bf16 output, arguments as qm_gemm_mxfp4_tn) that also records the shader clock, per workgroup, at its entry, at the
  * start of its tile loop, and after every tile's K loop and epilogue (up to 15 tiles): QM_DIAG_PHASE_STAMPS 64-bit values
@@ -170,7 +168,7 @@ int qm_diag_time_gemm_launches(void* const* start_events, void* const* stop_even
  * CU or per tile, whichever is fewer).  Where the time of a tile goes -- K steps against the epilogue, during which no
  * matrix instruction runs -- is read from the differences; bench.py --gemm-phases prints them.  c receives the product.
  * Serves M, N multiples of 64 and >= 256, K % 512 == 0.  Returns the number of workgroups launched, or a negative
- * status.  Synchronises with the host once (it sets a device-side pointer before the launch).
+ * status.
  */
 #define QM_DIAG_PHASE_STAMPS 32
 int qm_diag_gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,

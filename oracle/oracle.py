@@ -48,10 +48,13 @@ def lib():
         L.qo_hadamard_scale.restype = f32
         L.qo_hadamard_scale.argtypes = [i32, i32]
         L.qo_philox4x32_10.argtypes = [vp, vp, vp]
-        L.qo_philox_uniform16.restype = f32
-        L.qo_philox_uniform16.argtypes = [u64, u64]
-        L.qo_philox_uniform16_fill.argtypes = [u64, i64, vp]
-        L.qo_philox_uniform16_at.argtypes = [u64, i64, vp, vp]
+        L.qo_philox4x32_7.argtypes = [vp, vp, vp]
+        L.qo_philox_field22.restype = ctypes.c_uint32
+        L.qo_philox_field22.argtypes = [u64, u64]
+        L.qo_philox_uniform.restype = f32
+        L.qo_philox_uniform.argtypes = [u64, u64]
+        L.qo_philox_uniform_fill.argtypes = [u64, i64, vp]
+        L.qo_philox_uniform_at.argtypes = [u64, i64, vp, vp]
         L.qo_quantize.restype = i32
         L.qo_quantize.argtypes = [vp, i32, i64, i64, i32, vp, i32, i32, vp, u64, vp, vp, vp, vp, vp]
         L.qo_quantize_dense.restype = i32
@@ -131,25 +134,32 @@ def hadamard_scale(hd, dtype):
 # ---------------------------------------------------------------------------------------------
 # ctypes wrappers around the canonical C oracle
 # ---------------------------------------------------------------------------------------------
-def philox4x32_10(ctr, key):
+def philox4x32(ctr, key, rounds=7):
+    """Philox4x32 with 7 rounds (what the stochastic-rounding stream uses) or 10."""
     c = np.asarray(ctr, dtype=np.uint32)
     k = np.asarray(key, dtype=np.uint32)
     o = np.zeros(4, dtype=np.uint32)
-    lib().qo_philox4x32_10(_ptr(c), _ptr(k), _ptr(o))
+    {7: lib().qo_philox4x32_7, 10: lib().qo_philox4x32_10}[rounds](_ptr(c), _ptr(k), _ptr(o))
     return o
 
 
-def philox_uniform16(seed, n):
+def philox_field22(seed, o):
+    """The 22-bit random field of the element at flat offset o."""
+    return int(lib().qo_philox_field22(seed, o))
+
+
+def philox_uniform(seed, n):
+    """The stream's uniforms of flat element offsets 0..n-1."""
     u = np.empty(n, dtype=np.float32)
-    lib().qo_philox_uniform16_fill(seed, n, _ptr(u))
+    lib().qo_philox_uniform_fill(seed, n, _ptr(u))
     return u
 
 
-def philox_uniform16_at(seed, offsets):
+def philox_uniform_at(seed, offsets):
     """The stream's uniforms at the given flat element offsets (any shape of int64), same shape back."""
     off = np.ascontiguousarray(offsets, dtype=np.int64)
     u = np.empty(off.shape, dtype=np.float32)
-    lib().qo_philox_uniform16_at(seed, off.size, _ptr(off), _ptr(u))
+    lib().qo_philox_uniform_at(seed, off.size, _ptr(off), _ptr(u))
     return u
 
 

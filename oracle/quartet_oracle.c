@@ -23,7 +23,7 @@
  *
  * Parity pins (see tests/): Sylvester matrix vs scipy.linalg.hadamard; order-independent
  * integer fixtures worked out by hand; exhaustive RTN table over all bf16 patterns against the
- * seven strict thresholds; SR bracket/probability grids and unbiasedness; Philox4x32-10
+ * seven strict thresholds; SR bracket/probability grids and unbiasedness; Philox4x32-7 and -10
  * Random123 known-answer vectors; an independent numpy matmul-form restatement (oracle.py);
  * the notebook's recorded error bands.
  */
@@ -76,11 +76,11 @@ static inline int sign_is_negative(const uint32_t* sign_bits, int j) {
     return sign_bits ? (int)((sign_bits[j >> 5] >> (j & 31)) & 1u) : 0;
 }
 
-/* ---- Philox4x32-10 (Salmon et al., Random123) ---------------------------------------- */
-void qo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+/* ---- Philox4x32 (Salmon et al., Random123): the 10-round form and the 7-round form the stream uses ------ */
+static void philox4x32(const uint32_t ctr[4], const uint32_t key[2], int rounds, uint32_t out[4]) {
     uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3];
     uint32_t k0 = key[0], k1 = key[1];
-    for (int r = 0; r < 10; ++r) {
+    for (int r = 0; r < rounds; ++r) {
         uint64_t p0 = (uint64_t)0xD2511F53u * c0;
         uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
         uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
@@ -93,38 +93,44 @@ void qo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out
     }
     out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
 }
+void qo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) { philox4x32(ctr, key, 10, out); }
+void qo_philox4x32_7(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) { philox4x32(ctr, key, 7, out); }
 
 /*
  * Uniform for the element at flat offset o of the tensor being quantized (the role of
- * tl.rand(seed, offsets), mxfp4_triton.py:124).  One Philox4x32-10 call serves sixteen
- * consecutive elements: counter = (o/16 low, o/16 high, 0, 0), key = (seed low, seed high);
- * element o takes 16 random bits r16: byte (o%4) of word (o%16)/4 as the high half and the next byte
- * of the same word (byte (o+1)%4) as the low half.  Every element's r16 is uniform over 65536
- * values; neighbours inside a word share one byte, which correlates their rounding decisions by
- * less than 2^-8.  The uniform is the largest float below (r16 + 1/2) / 65536 + 2^-22, so that
- * "u < p" holds exactly when floor(p * 2^22) > r16 * 2^6 + 2^5: a comparison at 22 fractional
- * bits, which is what gfx950's stochastic-rounding convert evaluates, centred in the r16-th of
- * 65536 equal bins.  E[round up] differs from p by at most 2^-17 (mxfp4_triton.py:124 draws a
- * 24-bit uniform).
+ * tl.rand(seed, offsets), mxfp4_triton.py:124; the reference's own Philox stream is not reproduced, the
+ * contract is equality under identical uniforms).  One Philox4x32-7 call (the fewest rounds Random123
+ * publishes as passing its test batteries, and known-answer vectors for) serves sixteen consecutive
+ * elements: counter = (o/16 low, o/16 high, 0, 0), key = (seed low, seed high).  Element o reads word
+ * (o%16)/4 of the call rotated left by 8 * (o%4) bits and takes its top 22 bits as the field f: every
+ * element of a word has its own most significant byte, the bytes below it are shared with the word's
+ * other three elements at lower significance, which correlates two of their rounding decisions by less
+ * than 2^-8.  The uniform is the largest float below (2^22 - f) / 2^22, so that "u < p" holds exactly
+ * when floor(p * 2^22) + f >= 2^22: gfx950's stochastic-rounding convert evaluates this very carry out
+ * of a 22-bit addition.  P[round up] = floor(p * 2^22) / 2^22, below p by less than 2^-22.
  */
-float qo_philox_uniform16(uint64_t seed, uint64_t o) {
+uint32_t qo_philox_field22(uint64_t seed, uint64_t o) {
     uint32_t ctr[4] = {(uint32_t)(o >> 4), (uint32_t)((o >> 4) >> 32), 0u, 0u};
     uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
     uint32_t w[4];
-    qo_philox4x32_10(ctr, key, w);
+    philox4x32(ctr, key, 7, w);
     uint32_t word = w[(o & 15) >> 2];
-    uint32_t r16 = (((word >> (8 * (o & 3))) & 0xffu) << 8) | ((word >> (8 * ((o + 1) & 3))) & 0xffu);
-    float bound = (float)(64u * r16 + 33u) * (1.0f / 4194304.0f); /* exact: 22 significant bits */
+    unsigned s = 8u * (unsigned)(o & 3);
+    uint32_t rot = s ? ((word << s) | (word >> (32u - s))) : word;
+    return rot >> 10;
+}
+float qo_philox_uniform(uint64_t seed, uint64_t o) {
+    float bound = (float)(4194304u - qo_philox_field22(seed, o)) * (1.0f / 4194304.0f); /* exact: at most 23 significant bits */
     return bits_to_f32(f32_to_bits(bound) - 1u);
 }
 
-void qo_philox_uniform16_fill(uint64_t seed, int64_t n, float* u) {
-    for (int64_t o = 0; o < n; ++o) u[o] = qo_philox_uniform16(seed, (uint64_t)o);
+void qo_philox_uniform_fill(uint64_t seed, int64_t n, float* u) {
+    for (int64_t o = 0; o < n; ++o) u[o] = qo_philox_uniform(seed, (uint64_t)o);
 }
 
 /* the uniforms of n arbitrary flat offsets (a sample of rows of a large tensor) */
-void qo_philox_uniform16_at(uint64_t seed, int64_t n, const int64_t* offsets, float* u) {
-    for (int64_t i = 0; i < n; ++i) u[i] = qo_philox_uniform16(seed, (uint64_t)offsets[i]);
+void qo_philox_uniform_at(uint64_t seed, int64_t n, const int64_t* offsets, float* u) {
+    for (int64_t i = 0; i < n; ++i) u[i] = qo_philox_uniform(seed, (uint64_t)offsets[i]);
 }
 
 /* ---- rotation --------------------------------------------------------------------- */
@@ -295,7 +301,7 @@ static void quantize_row(float* row, int64_t r, int64_t cols, int hd, float c,
         int sr = (mode == QO_ABSMAX_SR || mode == QO_QUEST_SR);
         if (sr) {
             for (int i = 0; i < 32; ++i)
-                ug[i] = u ? u[r * cols + j0 + i] : qo_philox_uniform16(seed, (uint64_t)(r * cols + j0 + i));
+                ug[i] = u ? u[r * cols + j0 + i] : qo_philox_uniform(seed, (uint64_t)(r * cols + j0 + i));
         }
         quantize_group(row + j0, mode, ug, code, &e8, keep, deq);
         scales[r * (cols / 32) + j0 / 32] = e8;

@@ -24,10 +24,10 @@ EXPORTS = (
     "qm_dequantize_mxfp4",
     "qm_gemm_workspace_bytes",
     "qm_diag_mfma_only",
-    "qm_diag_time_gemm_launches",
     "qm_diag_gemm_tile_phases",
     "qm_gemm_noalloc_scratch_bytes",
     "qm_gemm_mxfp4_tn_noalloc",
+    "qm_gemm_noalloc_prepare",
     "qm_packed_operand_bytes",
     "qm_packed_operand_offsets",
     "qm_linear_backward_workspace_bytes",
@@ -74,8 +74,6 @@ def lib():
     L.qm_requantize_transposed_mxfp4_dense.argtypes = [vp, vp, i64, i64, f32, i32, vp, i32, u64, vp, vp, vp, i32, i32, vp]
     L.qm_gemm_mxfp4_tn.restype = i32
     L.qm_gemm_mxfp4_tn.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, i32, vp, ctypes.c_size_t, vp]
-    L.qm_diag_time_gemm_launches.restype = i32
-    L.qm_diag_time_gemm_launches.argtypes = [vp, vp, i32]
     L.qm_diag_gemm_tile_phases.restype = i32
     L.qm_diag_gemm_tile_phases.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, vp, ctypes.c_size_t, vp]
     L.qm_diag_mfma_only.restype = i64
@@ -84,6 +82,8 @@ def lib():
     L.qm_gemm_workspace_bytes.argtypes = [i64, i64, i64]
     L.qm_gemm_noalloc_scratch_bytes.restype = ctypes.c_size_t
     L.qm_gemm_noalloc_scratch_bytes.argtypes = []
+    L.qm_gemm_noalloc_prepare.restype = i32
+    L.qm_gemm_noalloc_prepare.argtypes = []
     L.qm_gemm_mxfp4_tn_noalloc.restype = i32
     L.qm_gemm_mxfp4_tn_noalloc.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, i32, vp]
     L.qm_masked_hadamard_bwd.restype = i32

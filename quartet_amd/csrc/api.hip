@@ -168,15 +168,6 @@ int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint
                     "qm_gemm_mxfp4_tn");
 }
 
-int qm_diag_time_gemm_launches(void* const* start_events, void* const* stop_events, int count) {
-    if (count < 0 || (count > 0 && (!start_events || !stop_events)))
-        return fail(QM_ERR_INVALID, "qm_diag_time_gemm_launches: %d event pairs, null arrays", count);
-    for (int i = 0; i < count; ++i)
-        if (!start_events[i] || !stop_events[i]) return fail(QM_ERR_INVALID, "qm_diag_time_gemm_launches: null event at %d", i);
-    qm::gemm_time_next_launches(start_events, stop_events, count);
-    return 0;
-}
-
 int qm_diag_gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
                              int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout, uint64_t* stamps,
                              size_t stamps_bytes, void* stream) {
@@ -244,6 +235,11 @@ extern "C" {
 
 size_t qm_gemm_noalloc_scratch_bytes(void) { return kNoAllocScratchBytes; }
 
+int qm_gemm_noalloc_prepare(void) {
+    void* ws = nullptr;
+    return scratch_of_current_device(&ws);
+}
+
 int qm_gemm_mxfp4_tn_noalloc(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
                              int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype, int a_layout, int b_layout,
                              void* stream) {
@@ -256,11 +252,11 @@ int qm_gemm_mxfp4_tn_noalloc(const uint8_t* a_codes, const uint8_t* a_scales, co
         return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn_noalloc: this shape's split-K partial sums need %zu bytes, the built-in scratch "
                                     "holds %zu (M=%lld N=%lld K=%lld); use qm_gemm_mxfp4_tn with a caller-provided workspace",
                     need, kNoAllocScratchBytes, (long long)M, (long long)N, (long long)K);
+    // resolved on every path, so that the first call on a device is the only one that can make the runtime load this
+    // library's device image (qm_gemm_noalloc_prepare() does the same ahead of time)
     void* ws = nullptr;
-    if (need) {
-        if (int rc = scratch_of_current_device(&ws)) return rc;
-    }
-    return qm_gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, c_dtype, a_layout, b_layout, ws, need, stream);
+    if (int rc = scratch_of_current_device(&ws)) return rc;
+    return qm_gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, c_dtype, a_layout, b_layout, need ? ws : nullptr, need, stream);
 }
 
 int qm_masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t cols, int hadamard_dim, int scale_dtype,

@@ -29,10 +29,9 @@
 #include <hip/hip_ext.h>
 #include <stdint.h>
 
-#include <mutex>
+#include <atomic>
 #include <type_traits>
 #include <utility>
-#include <vector>
 
 #include "qm_kernels.h"
 #include "qm_math.h"
@@ -754,9 +753,9 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
 }
 
 // Measurement aid (the STAMP instantiation of the kernel below): the shader clock at a workgroup's entry, at the start of
-// its tile loop, and after every tile's K loop and epilogue, kPhaseStamps values per workgroup at *g_phase_stamps.
+// its tile loop, and after every tile's K loop and epilogue, kPhaseStamps values per workgroup at the kernel's `stamps`
+// argument (which the production instantiation never reads).
 constexpr int kPhaseStamps = 32;  // entry, loop start, then (K loop end, epilogue end) of up to 15 tiles
-__device__ unsigned long long* g_phase_stamps;
 __device__ __forceinline__ unsigned long long shader_clock() {
     unsigned long long t;
     // the counter arrives like a scalar load: without the wait the registers it lands in may be reused before it does
@@ -771,7 +770,7 @@ template <typename OutT, bool STAMP = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mxfp4_tn_big4_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ b_codes,
     const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c, int a_tiled,
-    int b_tiled, int splits) {
+    int b_tiled, int splits, [[maybe_unused]] unsigned long long* __restrict__ stamps) {
     extern __shared__ uint32_t smem[];
     uint8_t* smem_bytes = reinterpret_cast<uint8_t*>(smem);
     const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)smem;
@@ -781,7 +780,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const auto stamp = [&]() {
         if constexpr (STAMP) {
             const unsigned long long now = shader_clock();
-            if (tid == 0 && stamps_taken < kPhaseStamps) g_phase_stamps[(size_t)blockIdx.x * kPhaseStamps + stamps_taken] = now;
+            if (tid == 0 && stamps_taken < kPhaseStamps) stamps[(size_t)blockIdx.x * kPhaseStamps + stamps_taken] = now;
             ++stamps_taken;
         }
     };
@@ -981,19 +980,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     sink[(size_t)blockIdx.x * 256 + tid] = sum;
 }
 
-// Measurement aid: event pairs handed over by gemm_time_next_launches() are attached, one pair per launch, to the next
-// launches of the persistent kernel; the runtime stamps them with the kernel's begin and end, so their elapsed time is
-// the kernel's duration wherever in a sequence of other kernels it runs (no launch pause, no host time inside).
-std::mutex g_timing_mutex;
-std::vector<std::pair<hipEvent_t, hipEvent_t>> g_timing_events;
-size_t g_timing_next = 0;
-bool next_timing_events(hipEvent_t& a, hipEvent_t& b) {
-    std::lock_guard<std::mutex> lock(g_timing_mutex);
-    if (g_timing_next >= g_timing_events.size()) return false;
-    a = g_timing_events[g_timing_next].first;
-    b = g_timing_events[g_timing_next].second;
-    ++g_timing_next;
-    return true;
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per kernel and device instead of on every launch
+constexpr int kMaxDevices = 64;
+template <typename Kern>
+hipError_t allow_dynamic_lds(Kern kern, int bytes, std::atomic<bool> (&done)[kMaxDevices]) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < kMaxDevices && done[dev].load(std::memory_order_acquire)) return hipSuccess;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && dev >= 0 && dev < kMaxDevices) done[dev].store(true, std::memory_order_release);
+    return e;
 }
 
 int device_cus() {
@@ -1031,22 +1028,16 @@ hipError_t launch_big4(const uint8_t* a_codes, const uint8_t* a_scales, const ui
                        const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_tiled,
                        int b_tiled, int splits, int cus, hipStream_t stream) {
     auto kern = gemm_mxfp4_tn_big4_kernel<OutT>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kBig4SmemBytes);
+    static std::atomic<bool> lds_allowed[kMaxDevices];
+    hipError_t e = allow_dynamic_lds(kern, kBig4SmemBytes, lds_allowed);
     if (e != hipSuccess) return e;
     const int64_t items = ((M + kBigM - 1) / kBigM) * ((N + kBigN - 1) / kBigN) * splits;
     // one workgroup per CU, and a grid that is a multiple of 8 so that item t and t + grid land on the same XCD
     int64_t g = items < cus ? items : cus;
     if (g > 8) g -= g % 8;
     dim3 grid((unsigned)g), block(256);
-    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
-    if (next_timing_events(ev_start, ev_stop)) {
-        // measurement aid: the runtime stamps these events with the kernel's own begin and end
-        hipExtLaunchKernelGGL(kern, grid, block, kBig4SmemBytes, stream, ev_start, ev_stop, 0, a_codes, a_scales, b_codes, b_scales,
-                              (int)M, (int)N, (int)K, alpha, reinterpret_cast<OutT*>(c), a_tiled, b_tiled, splits);
-        return hipGetLastError();
-    }
     kern<<<grid, block, kBig4SmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
-                                                  reinterpret_cast<OutT*>(c), a_tiled, b_tiled, splits);
+                                                  reinterpret_cast<OutT*>(c), a_tiled, b_tiled, splits, nullptr);
     return hipGetLastError();
 }
 
@@ -1055,7 +1046,8 @@ hipError_t launch_big(const uint8_t* a_codes, const uint8_t* a_scales, const uin
                       const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_tiled,
                       int b_tiled, hipStream_t stream) {
     auto kern = gemm_mxfp4_tn_big_kernel<OutT>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kBigSmemBytes);
+    static std::atomic<bool> lds_allowed[kMaxDevices];
+    hipError_t e = allow_dynamic_lds(kern, kBigSmemBytes, lds_allowed);
     if (e != hipSuccess) return e;
     dim3 grid((unsigned)(((M + kBigM - 1) / kBigM) * ((N + kBigN - 1) / kBigN))), block(256);
     kern<<<grid, block, kBigSmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
@@ -1072,14 +1064,16 @@ hipError_t launch_gemm(const uint8_t* a_codes, const uint8_t* a_scales, const ui
     if (c_dtype == BF16) {
         auto kern = gemm_mxfp4_tn_kernel<BM, BN, WM, WN, uint16_t>;
         if (smem > 48 * 1024) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+            static std::atomic<bool> lds_allowed[kMaxDevices];
+            hipError_t e = allow_dynamic_lds(kern, smem, lds_allowed);
             if (e != hipSuccess) return e;
         }
         kern<<<grid, block, smem, stream>>>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, reinterpret_cast<uint16_t*>(c));
     } else {
         auto kern = gemm_mxfp4_tn_kernel<BM, BN, WM, WN, float>;
         if (smem > 48 * 1024) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+            static std::atomic<bool> lds_allowed[kMaxDevices];
+            hipError_t e = allow_dynamic_lds(kern, smem, lds_allowed);
             if (e != hipSuccess) return e;
         }
         kern<<<grid, block, smem, stream>>>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, reinterpret_cast<float*>(c));
@@ -1106,21 +1100,11 @@ hipError_t gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, con
     int64_t g = items < cus ? items : cus;
     if (g > 8) g -= g % 8;
     if (stamps_bytes < (size_t)g * kPhaseStamps * sizeof(unsigned long long)) return hipErrorInvalidValue;
-    e = hipMemcpyToSymbol(HIP_SYMBOL(g_phase_stamps), &stamps, sizeof(stamps), 0, hipMemcpyHostToDevice);
-    if (e != hipSuccess) return e;
     kern<<<dim3((unsigned)g), dim3(256), kBig4SmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
                                                                   reinterpret_cast<uint16_t*>(c), a_layout == LAYOUT_TILED,
-                                                                  b_layout == LAYOUT_TILED, 1);
+                                                                  b_layout == LAYOUT_TILED, 1, stamps);
     *grid_out = (int)g;
     return hipGetLastError();
-}
-
-void gemm_time_next_launches(void* const* start_events, void* const* stop_events, int count) {
-    std::lock_guard<std::mutex> lock(g_timing_mutex);
-    g_timing_events.clear();
-    g_timing_next = 0;
-    for (int i = 0; i < count; ++i)
-        g_timing_events.emplace_back(reinterpret_cast<hipEvent_t>(start_events[i]), reinterpret_cast<hipEvent_t>(stop_events[i]));
 }
 
 // one workgroup (four waves, one per SIMD) per CU; reads blocks * 32 KiB of operands, writes blocks * 256 floats

@@ -123,8 +123,6 @@ hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const 
                          const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
                          int a_layout, int b_layout, void* workspace, size_t workspace_bytes, hipStream_t stream);
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
-// measurement aid: attach these event pairs to the next `count` launches of the persistent product kernel
-void gemm_time_next_launches(void* const* start_events, void* const* stop_events, int count);
 // measurement aid: one launch of the persistent kernel that records the shader clock around every tile's K loop and epilogue
 int gemm_phase_stamps_per_group();
 hipError_t gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,

@@ -130,13 +130,14 @@ QM_HD float exp_fixed(float z) {
 // x / (1 + e^-x), the form torch.nn.functional.silu evaluates (src/models/llama.py:113 of the reference calls it)
 QM_HD float silu_fixed(float x) { return x / (1.0f + exp_fixed(-x)); }
 
-// ---- Philox4x32-10 ----------------------------------------------------------------------
+// ---- Philox4x32-7 (Random123; the fewest rounds it publishes as passing its test batteries) ------------------
 struct Philox4 {
     uint32_t w[4];
 };
-QM_HD Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1) {
+template <int ROUNDS>
+QM_HD Philox4 philox4x32(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1) {
 #pragma unroll
-    for (int r = 0; r < 10; ++r) {
+    for (int r = 0; r < ROUNDS; ++r) {
         // one 32x32->64 multiply each (v_mad_u64_u32 on the GPU)
         const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
         const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
@@ -149,21 +150,20 @@ QM_HD Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, 
     o.w[0] = c0; o.w[1] = c1; o.w[2] = c2; o.w[3] = c3;
     return o;
 }
-// Random bits of element `o` (flat offset in the tensor being quantized): one Philox call per sixteen
-// consecutive elements, counter = o/16; element j of the sixteen takes byte j%4 of word j/4 as the high half
-// and byte (j+1)%4 of the same word as the low half of its 16 random bits (uniform over 65536 values per
-// element; neighbours inside a word share one byte).  Its uniform is the largest float below
-// (r16 * 2^6 + 2^5 + 1) * 2^-22: "u < p" is then exactly the 22-bit comparison
-// floor(p * 2^22) > r16 * 2^6 + 2^5 that the hardware convert performs, centred in the r16-th of 65536 bins.
-QM_HD uint32_t philox_r16(const Philox4& p, int j) {
-    const uint32_t w = p.w[j >> 2];
-    return (((w >> (8 * (j & 3))) & 0xffu) << 8) | ((w >> (8 * ((j + 1) & 3))) & 0xffu);
-}
-QM_HD float uniform_from_r16(uint32_t r16) {
-    return u2f(f2u((float)(64u * r16 + 33u) * (1.0f / 4194304.0f)) - 1u);
+constexpr int kPhiloxRounds = 7;
+// Random bits of element `o` (flat offset in the tensor being quantized): one Philox call per sixteen consecutive
+// elements, counter = o/16.  Element j of the sixteen reads word j/4 rotated left by 8 * (j%4) bits and takes its top 22
+// bits as the field f: each element of a word has its own most significant byte and shares the bytes below with the
+// word's other elements at lower significance.  Its uniform is the largest float below (2^22 - f) * 2^-22: "u < p" is
+// then exactly "floor(p * 2^22) + f carries out of 22 bits", which is what the hardware's stochastic-rounding convert
+// evaluates with f as its random field.
+QM_HD uint32_t rotl32(uint32_t w, int s) { return s ? ((w << s) | (w >> (32 - s))) : w; }
+QM_HD uint32_t philox_field22(const Philox4& p, int j) { return rotl32(p.w[j >> 2], 8 * (j & 3)) >> 10; }
+QM_HD float uniform_from_field22(uint32_t f) {
+    return u2f(f2u((float)(4194304u - f) * (1.0f / 4194304.0f)) - 1u);
 }
 QM_HD Philox4 philox_for_hexadecad(uint64_t seed, uint64_t block16) {
-    return philox4x32_10((uint32_t)block16, (uint32_t)(block16 >> 32), 0u, 0u, (uint32_t)seed, (uint32_t)(seed >> 32));
+    return philox4x32<kPhiloxRounds>((uint32_t)block16, (uint32_t)(block16 >> 32), 0u, 0u, (uint32_t)seed, (uint32_t)(seed >> 32));
 }
 
 }  // namespace qm

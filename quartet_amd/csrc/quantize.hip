@@ -221,7 +221,7 @@ __device__ __forceinline__ void process_octet(float (&v)[8], int lane_in_chunk, 
             // sixteen elements share one Philox call: the two octets of a pair compute it twice
             Philox4 ph = philox_for_hexadecad(seed, (uint64_t)(octet >> 1));
 #pragma unroll
-            for (int i = 0; i < 8; ++i) uu[i] = uniform_from_r16(philox_r16(ph, (int)(octet & 1) * 8 + i));
+            for (int i = 0; i < 8; ++i) uu[i] = uniform_from_field22(philox_field22(ph, (int)(octet & 1) * 8 + i));
         }
     }
     OctetResult r;

@@ -15,9 +15,9 @@
 //            (b - 1) | 1 moves every tie just below itself and nothing else across a boundary.
 //       SR   v_cvt_scalef32_sr_pk_fp4_f32 rounds up iff floor(p * 2^22) + R >= 2^22 with p the position
 //            inside the bracket and R = bits 31..10 of the random operand for the pair's first element,
-//            bits 30..9 for its second (measured).  With R = 2^22 - 1 - r16 2^6 - 2^5 this is "u < p" for
-//            the uniform the Philox stream defines (qm_math.h), bit for bit.  Each element gets its
-//            own 16 random bits (two converts per pair, merged with one mask).
+//            bits 30..9 for its second (measured).  With R = the element's 22-bit field of the Philox stream this is
+//            "u < p" for the uniform that stream defines (qm_math.h), bit for bit.  Each element gets its
+//            own field (two converts per pair, merged with one mask).
 //     The reference's sign rule "negative unless t > 0" makes +0 negative: adding -2^-149 first turns
 //     both zeros into a negative denormal and changes no other value's code.
 // Outputs are one 16-byte code store, one scale byte and one mask dword per lane, all contiguous across
@@ -174,15 +174,15 @@ __device__ __forceinline__ void quantize_group_regs(const float (&g)[32], uint64
 #define QM_RTN_PAIR(B)                                                                                   \
     w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, tie_nudge(t[wi * 8 + 2 * (B)] + kNegTiny),           \
                                                  tie_nudge(t[wi * 8 + 2 * (B) + 1] + kNegTiny), hw_scale, (B));
-    // element j of a Philox call (16 elements): r16 = byte j%4 (high) and byte (j+1)%4 (low) of word j/4.  r for the
-    // pair's first element carries ~r16 in bits 31..16 above the constant 0x7fff (R = 2^22 - 1 - r16 2^6 - 2^5 in bits
-    // 31..10); the second element reads bits 30..9, i.e. the same pattern shifted right by one.  v_perm_b32 builds the
-    // pattern: selector bytes pick {~high byte, ~low byte, 0x7f, 0xff}.
+    // element j of a Philox call (16 elements): its random field is the top 22 bits of word j/4 rotated left by
+    // 8 * (j%4).  The convert reads the field of a pair's first element from bits 31..10 of its random operand and that of
+    // the second from bits 30..9, so the even element's operand is the word rotated by 0 or 16 bits and the odd element's
+    // the word rotated by 7 or 23 (one more bit to the right): one v_alignbit_b32 each, none for a word's first element.
 #define QM_SR_PAIR(B, J0)                                                                                 \
     {                                                                                                     \
-        const uint32_t nw = ~ph.w[(J0) >> 2];                                                             \
-        const uint32_t r_even = __builtin_amdgcn_perm(nw, 0x7f7f7f7fu, 0x000000ffu | ((4u + ((J0) & 3)) << 24) | ((4u + (((J0) + 1) & 3)) << 16));        \
-        const uint32_t r_odd = __builtin_amdgcn_perm(nw, 0x7f7f7f7fu, 0x000000ffu | ((4u + (((J0) + 1) & 3)) << 24) | ((4u + (((J0) + 2) & 3)) << 16)) >> 1;  \
+        const uint32_t pw = ph.w[(J0) >> 2];                                                              \
+        const uint32_t r_even = ((J0) & 3) == 0 ? pw : __builtin_amdgcn_alignbit(pw, pw, 16);             \
+        const uint32_t r_odd = __builtin_amdgcn_alignbit(pw, pw, ((J0) & 3) == 0 ? 25 : 9);               \
         const v2f pr = {t[wi * 8 + 2 * (B)] + kNegTiny, t[wi * 8 + 2 * (B) + 1] + kNegTiny};              \
         sr_convert_pair<(B)>(even, pr, r_even, hw_scale);                                                 \
         sr_convert_pair<(B)>(odd, pr, r_odd, hw_scale);                                                   \

@@ -164,6 +164,19 @@ def gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, alpha=1.0, out_dtype=tor
     return c
 
 
+_noalloc_prepared = set()
+
+
+def gemm_noalloc_prepare():
+    """Look up the current device's copy of the library's built-in scratch array (once per device; the one step of the
+    allocation-free product that may make the HIP runtime place the library's device image in GPU memory).  Must not
+    run under stream capture."""
+    dev = torch.cuda.current_device()
+    if dev not in _noalloc_prepared:
+        _lib.check(_lib.lib().qm_gemm_noalloc_prepare(), "qm_gemm_noalloc_prepare")
+        _noalloc_prepared.add(dev)
+
+
 def gemm_mxfp4_tn_noalloc(a_codes, a_scales, b_codes, b_scales, alpha, out):
     """The same product through the library's allocation-free entry point: `out` [M,N] (bf16 or fp32) is written in
     place and split-K partial sums go to the library's built-in device scratch.  Row-major code bytes."""
@@ -171,31 +184,13 @@ def gemm_mxfp4_tn_noalloc(a_codes, a_scales, b_codes, b_scales, alpha, out):
     M, K = a_codes.shape[0], a_codes.shape[1] * 2
     N = b_codes.shape[0]
     assert out.shape == (M, N) and out.is_contiguous() and b_codes.shape[1] * 2 == K
+    with torch.cuda.device(out.device):
+        gemm_noalloc_prepare()
     rc = _lib.lib().qm_gemm_mxfp4_tn_noalloc(_ptr(a_codes), _ptr(a_scales), _ptr(b_codes), _ptr(b_scales), M, N, K, alpha,
                                              _ptr(out), _dtype_code(out.dtype), QM_LAYOUT_ROWMAJOR, QM_LAYOUT_ROWMAJOR,
                                              _stream())
     _lib.check(rc, "qm_gemm_mxfp4_tn_noalloc")
     return out
-
-
-def time_gemm_launches(n):
-    """Measurement aid: the next `n` launches of the product's persistent tile kernel (stand-alone or inside the
-    whole-layer calls) are stamped with their own begin and end.  Returns a function that, after a synchronisation,
-    gives their durations in milliseconds."""
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
-    stops = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
-    for e in starts + stops:
-        e.record()   # creates the underlying event; the launch re-records it
-    arr = ctypes.c_void_p * n
-    a = arr(*[e.cuda_event for e in starts])
-    b = arr(*[e.cuda_event for e in stops])
-    _lib.check(_lib.lib().qm_diag_time_gemm_launches(a, b, n), "qm_diag_time_gemm_launches")
-
-    def durations():
-        torch.cuda.synchronize()
-        _lib.lib().qm_diag_time_gemm_launches(None, None, 0)
-        return [s.elapsed_time(t) for s, t in zip(starts, stops)]
-    return durations
 
 
 PHASE_STAMPS = 32   # QM_DIAG_PHASE_STAMPS

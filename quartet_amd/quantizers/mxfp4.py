@@ -189,14 +189,21 @@ def _unpack_mask(maskbits, shape):
 
 
 class DenseRotationQuantizerFn(torch.autograd.Function):
-    """Either quantizer with a dense 32 x 32 rotation: the kernel rotates every group of 32 on the matrix pipe and
-    quantizes it; straight-through backward ``(g * mask) @ matrix^T`` (mxfp4.py:30-34,143-146)."""
+    """Either quantizer with a dense rotation: for a 32 x 32 matrix the kernel rotates every group of 32 on the matrix
+    pipe and quantizes it, a 64 x 64 or 128 x 128 matrix is applied as a library product first; straight-through backward ``(g * mask) @ matrix^T`` (mxfp4.py:30-34,143-146)."""
 
     @staticmethod
     def forward(ctx, x, matrix, mode, want_mask, post_scale):
         stochastic = mode in (K.QM_ABSMAX_SR, K.QM_QUEST_SR)
-        _, _, maskbits, deq = K.quantize_mxfp4_dense(_as_2d(x, 32), matrix, mode, seed=_fresh_seed() if stochastic else 0,
-                                                     want_mask=want_mask, want_dequant=True)
+        seed = _fresh_seed() if stochastic else 0
+        if matrix.shape[0] == 32:
+            _, _, maskbits, deq = K.quantize_mxfp4_dense(_as_2d(x, 32), matrix, mode, seed=seed, want_mask=want_mask,
+                                                         want_dequant=True)
+        else:
+            # a dense matrix over 64 or 128 values: library product in fp32, then the kernel quantizes the rotated groups
+            # of 32 as they are (what mxfp4_forward_kernel_wrapper does for such a matrix)
+            _, _, maskbits, deq = K.quantize_mxfp4(_rotate_dense(x, matrix), 1, None, mode, seed=seed, want_mask=want_mask,
+                                                   want_dequant=True)
         if post_scale != 1.0:
             deq *= post_scale
         ctx.save_for_backward(matrix, maskbits) if want_mask else ctx.save_for_backward(matrix)

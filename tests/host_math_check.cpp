@@ -77,37 +77,58 @@ int main() {
     }
     if (rtn_code(1e9f) != 7 || sr_code(7.5f, 0.f) != 7) fail("saturation", 0);
 
-    // the uniform of 16 random bits turns "u < p" into the integer comparison floor(p 2^22) > r16 2^6 + 2^5
-    for (uint32_t r16 = 0; r16 < 65536; ++r16) {
-        const float u = uniform_from_r16(r16);
-        const uint32_t R = r16 * 64u + 32u;
-        for (int d = -2; d <= 2; ++d) {
-            const uint32_t k = R + (uint32_t)d;  // p = k 2^-22, exact in fp32
-            const float p = (float)k * (1.0f / 4194304.0f);
-            if ((u < p) != (k > R)) fail("uniform_from_r16", r16);
-            const float p_half = ((float)k + 0.5f) * (1.0f / 4194304.0f);  // p with bits below 2^-22
-            if ((u < p_half) != (k > R)) fail("uniform_from_r16 (sub-grid p)", r16);
+    // the uniform of a 22-bit field f turns "u < p" into the carry out of floor(p 2^22) + f: every value of the top 16 bits
+    // with the extreme and a few mixed low parts, p on and next to the boundary
+    for (uint32_t hi = 0; hi < 65536; ++hi) {
+        const uint32_t lows[5] = {0u, 1u, 32u, 62u, 63u};
+        for (int li = 0; li < 5; ++li) {
+            const uint32_t f = (hi << 6) | lows[li];
+            const float u = uniform_from_field22(f);
+            if (!(u > 0.0f && u < 1.0f)) fail("uniform_from_field22 range", f);
+            const uint32_t boundary = 4194304u - f;  // smallest k with k + f >= 2^22
+            for (int d = -2; d <= 2; ++d) {
+                const int64_t k64 = (int64_t)boundary + d;
+                if (k64 < 0 || k64 > 4194304) continue;
+                const uint32_t k = (uint32_t)k64;  // p = k 2^-22, exact in fp32
+                const float p = (float)k * (1.0f / 4194304.0f);
+                if ((u < p) != (k + f >= 4194304u)) fail("uniform_from_field22", f);
+                if (k < 4194304u) {
+                    const float p_half = ((float)k + 0.5f) * (1.0f / 4194304.0f);  // p with bits below 2^-22
+                    if ((u < p_half) != (k + f >= 4194304u)) fail("uniform_from_field22 (sub-grid p)", f);
+                }
+            }
         }
     }
-    // an element's 16 bits: its own byte of the word above the next byte of the same word
+    // an element's field: its word rotated left by a byte per position, top 22 bits
     {
         Philox4 ph;
         ph.w[0] = 0x04030201u; ph.w[1] = 0x08070605u; ph.w[2] = 0x0c0b0a09u; ph.w[3] = 0x100f0e0du;
         for (int j = 0; j < 16; ++j) {
-            const uint32_t own = (uint32_t)j + 1u, next = (uint32_t)((j & ~3) + ((j + 1) & 3)) + 1u;
-            if (philox_r16(ph, j) != ((own << 8) | next)) fail("philox_r16", (uint32_t)j);
+            const uint32_t base = (uint32_t)(j & ~3) + 1u;  // value of the word's lowest byte
+            uint32_t bytes[4];                               // most significant first after the rotation
+            for (int i = 0; i < 4; ++i) bytes[i] = base + (uint32_t)((3 - (j & 3) - i + 8) & 3);
+            const uint32_t rot = (bytes[0] << 24) | (bytes[1] << 16) | (bytes[2] << 8) | bytes[3];
+            if (philox_field22(ph, j) != (rot >> 10)) fail("philox_field22", (uint32_t)j);
         }
     }
 
-    // Philox4x32-10 known-answer vectors (Random123)
+    // Philox4x32 known-answer vectors (Random123): 7 rounds, which the stream uses, and 10
     {
-        const Philox4 a = philox4x32_10(0, 0, 0, 0, 0, 0);
+        const Philox4 a = philox4x32<10>(0, 0, 0, 0, 0, 0);
         const uint32_t wa[4] = {0x6627e8d5u, 0xe169c58du, 0xbc57ac4cu, 0x9b00dbd8u};
-        const Philox4 b = philox4x32_10(0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu);
+        const Philox4 b = philox4x32<10>(0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu);
         const uint32_t wb[4] = {0x408f276du, 0x41c83b0eu, 0xa20bc7c6u, 0x6d5451fdu};
+        const Philox4 c = philox4x32<7>(0, 0, 0, 0, 0, 0);
+        const uint32_t wc[4] = {0x5f6fb709u, 0x0d893f64u, 0x4f121f81u, 0x4f730a48u};
+        const Philox4 d = philox4x32<7>(0x243f6a88u, 0x85a308d3u, 0x13198a2eu, 0x03707344u, 0xa4093822u, 0x299f31d0u);
+        const uint32_t wd[4] = {0x4dfccabau, 0x190a87f0u, 0xc47362bau, 0xb6b5242au};
+        const Philox4 e = philox_for_hexadecad(0, 0);
         for (int i = 0; i < 4; ++i) {
-            if (a.w[i] != wa[i]) fail("philox zeros", (uint32_t)i);
-            if (b.w[i] != wb[i]) fail("philox ones", (uint32_t)i);
+            if (a.w[i] != wa[i]) fail("philox-10 zeros", (uint32_t)i);
+            if (b.w[i] != wb[i]) fail("philox-10 ones", (uint32_t)i);
+            if (c.w[i] != wc[i]) fail("philox-7 zeros", (uint32_t)i);
+            if (d.w[i] != wd[i]) fail("philox-7 pi", (uint32_t)i);
+            if (e.w[i] != wc[i]) fail("the stream's call is the 7-round form", (uint32_t)i);
         }
     }
 

@@ -112,7 +112,7 @@ def test_quantizer_sweep_sampled_rows_match_oracle(oracle, K, rows, hd, mode):
     u = None
     if mode == "absmax_sr":
         offsets = idx.numpy().astype(np.int64)[:, None] * cols + np.arange(cols, dtype=np.int64)[None, :]
-        u = oracle.philox_uniform16_at(kseed, offsets)
+        u = oracle.philox_uniform_at(kseed, offsets)
     ref = oracle.quantize(to_oracle(xd[idx.to(dev)]), hd, signs=sv, mode=omode, want_mask=want_mask, u=u)
     assert np.array_equal(_rows(scales, idx.to(dev)), ref["scales"])
     assert np.array_equal(_rows(codes, idx.to(dev)), ref["codes"])

@@ -169,9 +169,9 @@ def test_split_k_is_offered_and_reproducible(K):
     assert rel < 1e-6, rel
 
 
-def test_measurement_aids_leave_results_alone(K):
-    """The two measurement aids: event pairs attached to the product kernel's launches give positive durations and do
-    not change what the product computes; the matrix-instruction loop reports how many instructions it issued."""
+def test_matrix_instruction_loop_reports_its_instruction_count(K):
+    """The matrix-instruction loop (a measurement aid) reports how many instructions it issued, and leaves the product's
+    results alone."""
     dev = torch.device("cuda:0")
     g = torch.Generator(device="cpu").manual_seed(5)
     M, N, K_ = 512, 768, 1024
@@ -180,17 +180,12 @@ def test_measurement_aids_leave_results_alone(K):
     as_ = torch.randint(120, 130, (M, K_ // 32), generator=g, dtype=torch.uint8).to(dev)
     bs = torch.randint(120, 130, (N, K_ // 32), generator=g, dtype=torch.uint8).to(dev)
     plain = K.gemm_mxfp4_tn(ac, as_, bc, bs, 1.0, torch.bfloat16)
-    durations = K.time_gemm_launches(3)
-    timed = [K.gemm_mxfp4_tn(ac, as_, bc, bs, 1.0, torch.bfloat16) for _ in range(2)]
-    d = durations()          # the third pair was never used and is withdrawn
-    assert all(torch.equal(t, plain) for t in timed)
-    assert 0.0 < d[0] < 50.0 and 0.0 < d[1] < 50.0
-    after = K.gemm_mxfp4_tn(ac, as_, bc, bs, 1.0, torch.bfloat16)   # no pairs left: an ordinary launch
-    assert torch.equal(after, plain)
     buf = torch.randint(0, 256, (16 << 20,), generator=g, dtype=torch.uint8).to(dev)
     n = K.mfma_only(buf, 10)
     torch.cuda.synchronize()
     assert n > 0 and n % (4 * 10 * 16) == 0
+    after = K.gemm_mxfp4_tn(ac, as_, bc, bs, 1.0, torch.bfloat16)
+    assert torch.equal(after, plain)
 
 
 def test_tile_phase_stamps_of_the_persistent_kernel():

@@ -217,6 +217,40 @@ def test_dense_rotation_quantizers_against_oracle(oracle, q, cls_name, mode_name
     assert float((x.grad.float() - gref).norm() / gref.norm()) < 1e-2   # the module's product runs in bf16
 
 
+@pytest.mark.parametrize("hd", [64, 128])
+@pytest.mark.parametrize("cls_name,mode_name", [("QuestMXFP4Quantizer", "QUEST_RTN"), ("AlbertTsengQuantizer", "ABSMAX_SR")])
+def test_dense_rotation_over_wider_blocks(oracle, q, hd, cls_name, mode_name):
+    """rerotate="O32" with hadamard_dim 64 / 128: the module holds an [hd, hd] orthogonal matrix (mxfp4.py:61-64), applies
+    it as an fp32 product and hands the rotated rows to the kernel as they are.  Forward equals the oracle's quantizer on
+    the same rotated tensor bit for bit; backward is the (masked) product with the transposed matrix."""
+    print(f"case dense rotation hd={hd} {cls_name}", flush=True)
+    import random
+    from tests.util import from_oracle_bf16
+    dev = "cuda:0"
+    torch.manual_seed(21)
+    quant = getattr(q, cls_name)(hadamard_dim=hd, rerotate="O32")
+    quant.re_randomize()
+    assert quant.is_dense and quant._dense.shape == (hd, hd)
+    x = make_input(40, 256, torch.bfloat16, seed=22).to(dev).requires_grad_(True)
+    random.seed(9)
+    y = quant(x)
+    R = quant.hadamard_matrix
+    assert R.shape == (hd, hd) and R.dtype == torch.bfloat16
+    rotated = (x.detach().reshape(-1, hd).float() @ R.float()).view(40, 256)
+    random.seed(9)
+    seed = random.getrandbits(63) if "SR" in mode_name else 0
+    want = oracle.quantize(to_oracle(rotated), hd=1, mode=getattr(oracle, mode_name), seed=seed, want_mask=True, want_dequant=True)
+    ref = torch.from_numpy(want["dequant"]).to(torch.bfloat16)      # de-quantized values are exact in bf16
+    assert y.dtype == torch.bfloat16 and torch.equal(y.detach().cpu(), ref)
+    g = make_input(40, 256, torch.bfloat16, seed=23).to(dev)
+    y.backward(g)
+    gm = g.float()
+    if cls_name == "QuestMXFP4Quantizer":
+        gm = gm * torch.from_numpy(np.unpackbits(want["mask"], axis=1, bitorder="little")).to(dev).float()
+    gref = (gm.reshape(-1, hd) @ R.float().T).view(40, 256)
+    assert float((x.grad.float() - gref).norm() / gref.norm()) < 1e-2   # the module's product runs in bf16
+
+
 def test_layer_with_dense_gradient_rotation(oracle, q):
     """The production configuration with rerotate="O32" on the gradient quantizer stays on the packed FP4 path (the
     four gradient quantizations rotate by the dense matrix on the matrix pipe): the step must equal the oracle pipeline

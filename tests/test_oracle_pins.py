@@ -135,52 +135,93 @@ def test_division_by_four_thirds_is_ieee(oracle):
 
 # ---- Philox ---------------------------------------------------------------------------------
 def test_philox_known_answer_vectors(oracle):
-    # Random123 kat_vectors, philox4x32-10
+    # Random123 kat_vectors: philox4x32 with 7 rounds (what the stream uses) and with 10
     kat = [
-        ([0] * 4, [0, 0], [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]),
-        ([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2, [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]),
-        ([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0],
+        (7, [0] * 4, [0, 0], [0x5F6FB709, 0x0D893F64, 0x4F121F81, 0x4F730A48]),
+        (7, [0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2, [0x5207DDC2, 0x45165E59, 0x4D8EE751, 0x8C52F662]),
+        (7, [0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0],
+         [0x4DFCCABA, 0x190A87F0, 0xC47362BA, 0xB6B5242A]),
+        (10, [0] * 4, [0, 0], [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]),
+        (10, [0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2, [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]),
+        (10, [0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0],
          [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]),
     ]
-    for ctr, key, out in kat:
-        assert oracle.philox4x32_10(ctr, key).tolist() == out
+    for rounds, ctr, key, out in kat:
+        assert oracle.philox4x32(ctr, key, rounds).tolist() == out
 
 
-def test_philox_uniform16_mapping(oracle):
-    # u(r16) = largest float below (r16 * 2^6 + 2^5 + 1) / 2^22; r16 = a byte of a Philox word above the next byte of
-    # the same word; 16 elements per call
+def _rotl32(w, s):
+    return ((w << s) | (w >> (32 - s))) & 0xFFFFFFFF if s else w
+
+
+def test_philox_uniform_mapping(oracle):
+    # element j of a call: f = top 22 bits of word j/4 rotated left by 8 (j%4); u(f) = largest float below (2^22 - f) / 2^22
     seed = 0x1234_5678_9ABC
-    u = oracle.philox_uniform16(seed, 64)
+    u = oracle.philox_uniform(seed, 64)
     for blk in range(4):
-        w = oracle.philox4x32_10([blk, 0, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
+        w = oracle.philox4x32([blk, 0, 0, 0], [seed & 0xFFFFFFFF, seed >> 32], 7)
         want = []
-        for word in w.tolist():
+        for wi, word in enumerate(w.tolist()):
             for b in range(4):
-                r16 = (((word >> (8 * b)) & 0xFF) << 8) | ((word >> (8 * ((b + 1) % 4))) & 0xFF)
-                bound = np.float32((64 * r16 + 33) / 4194304.0)
-                assert float(bound) == (64 * r16 + 33) / 4194304.0  # exactly representable
+                f = _rotl32(word, 8 * b) >> 10
+                assert f == oracle.philox_field22(seed, 16 * blk + 4 * wi + b)
+                bound = np.float32((4194304 - f) / 4194304.0)
+                assert float(bound) == (4194304 - f) / 4194304.0  # exactly representable
                 want.append(float(np.nextafter(bound, np.float32(0))))
         assert u[16 * blk:16 * blk + 16].tolist() == want
     off = np.array([[5, 1 << 20], [(1 << 33) + 7, 63]], dtype=np.int64)
-    at = oracle.philox_uniform16_at(seed, off)
+    at = oracle.philox_uniform_at(seed, off)
     assert at.shape == off.shape and at[0, 0] == u[5] and at[1, 1] == u[63]
-    w = oracle.philox4x32_10([((1 << 33) + 7) >> 4 & 0xFFFFFFFF, ((1 << 33) + 7) >> 36, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
-    word = int(w[1])   # element 7 of its call: word 1, byte 3 above byte 0
-    r16 = ((word >> 24) << 8) | (word & 0xFF)
-    assert at[1, 0] == np.nextafter(np.float32((64 * r16 + 33) / 4194304.0), np.float32(0))
-    big = oracle.philox_uniform16(7, 1 << 16)
-    assert 0 <= big.min() and big.max() < 1 and abs(big.mean() - 0.5) < 5e-3
-    # "u < p" is the 22-bit comparison "floor(p * 2^22) > r16 * 2^6 + 2^5" for every float p in [0, 1]
+    w = oracle.philox4x32([((1 << 33) + 7) >> 4 & 0xFFFFFFFF, ((1 << 33) + 7) >> 36, 0, 0], [seed & 0xFFFFFFFF, seed >> 32], 7)
+    f = _rotl32(int(w[1]), 24) >> 10   # element 7 of its call: word 1 rotated by three bytes
+    assert at[1, 0] == np.nextafter(np.float32((4194304 - f) / 4194304.0), np.float32(0))
+    big = oracle.philox_uniform(7, 1 << 16)
+    assert 0 < big.min() and big.max() < 1 and abs(big.mean() - 0.5) < 5e-3
+    # "u < p" is the carry out of the 22-bit addition "floor(p * 2^22) + f" for every float p in [0, 1]
     rng = np.random.default_rng(0)
-    r16 = rng.integers(0, 65536, 20000)
-    bound = ((64 * r16 + 33) / 4194304.0).astype(np.float32)
+    f = rng.integers(0, 1 << 22, 20000)
+    f[:4] = [0, 1, (1 << 22) - 1, (1 << 22) - 2]
+    bound = ((4194304 - f) / 4194304.0).astype(np.float32)
     uu = np.nextafter(bound, np.float32(0))
     p = np.concatenate([rng.random(10000, dtype=np.float32), bound[:5000], uu[:2500], np.nextafter(bound[:2500], np.float32(2))])
-    assert np.array_equal(uu < p, np.floor(p.astype(np.float64) * 4194304.0) > 64 * r16 + 32)
-    # centred bins: averaged over r16 the round-up probability of p is p to within 2^-17, also for p below 1/512
-    allu = np.nextafter(((64 * np.arange(65536) + 33) / 4194304.0).astype(np.float32), np.float32(0))
-    for pv in (1e-4, 1 / 700, 0.1, 0.37, 0.5, 0.93, 1 - 1e-4):
-        assert abs(np.mean(allu < np.float32(pv)) - float(np.float32(pv))) <= 2.0 ** -17 + 1e-12
+    p[:4] = [0.0, 1.0, 2.0 ** -22, 1.0 - 2.0 ** -22]
+    assert np.array_equal(uu < p, np.floor(p.astype(np.float64) * 4194304.0).astype(np.int64) + f >= 1 << 22)
+    # averaged over every field value the round-up probability of p is floor(p 2^22) / 2^22: below p by less than 2^-22
+    for pv in (1e-6, 1e-4, 1 / 700, 0.1, 0.37, 0.5, 0.93, 1 - 1e-4):
+        k = int(np.floor(np.float64(np.float32(pv)) * 4194304.0))
+        # fields f with k + f >= 2^22 are f >= 2^22 - k: exactly k of the 2^22 values
+        assert 0 <= float(np.float32(pv)) - k / 4194304.0 < 2.0 ** -22
+
+
+def test_philox_stream_statistics(oracle):
+    """The 22-bit fields of the stream: uniform in their top byte (chi-square over 256 bins), in a 12-bit slice crossing
+    the boundary between an element's own byte and the byte it shares (4096 bins), serially uncorrelated at lags 1..4 and
+    16 (neighbours inside a word share bytes at different significance; neighbours across calls share nothing), and
+    jointly uniform for the pair (element, next element) on a 16 x 16 grid of their top nibbles."""
+    n = 1 << 19
+    u = oracle.philox_uniform(0xC0FFEE1234, n).astype(np.float64)
+    f = np.round((1.0 - u) * 4194304.0).astype(np.int64) - 1     # u sits just below (2^22 - f) / 2^22
+    f = np.clip(f, 0, (1 << 22) - 1)
+    assert f.min() >= 0 and f.max() < 1 << 22
+
+    def chi2(counts):
+        e = counts.sum() / counts.size
+        return float(((counts - e) ** 2 / e).sum()), counts.size - 1
+    for name, vals, bins in (("top byte", f >> 14, 256), ("bits 17..6", (f >> 6) & 0xFFF, 4096), ("low byte", f & 0xFF, 256)):
+        stat, dof = chi2(np.bincount(vals, minlength=bins).astype(np.float64))
+        assert abs(stat - dof) < 6.0 * np.sqrt(2.0 * dof), (name, stat, dof)     # six sigma of a chi-square
+    x = u - u.mean()
+    for lag in (1, 2, 3, 4, 16, 17):
+        r = float((x[:-lag] * x[lag:]).mean() / x.var())
+        assert abs(r) < 5.0 / np.sqrt(n), (lag, r)
+    joint = np.bincount(((f[:-1] >> 18) << 4) | (f[1:] >> 18), minlength=256).astype(np.float64)
+    stat, dof = chi2(joint)
+    assert abs(stat - dof) < 6.0 * np.sqrt(2.0 * dof), ("pairs", stat)
+    # rounding decisions of neighbours at the same threshold: the covariance of 1[u_i < p] and 1[u_(i+1) < p]
+    for pv in (0.01, 0.3, 0.5, 0.77):
+        d = (u < pv).astype(np.float64)
+        cov = float(((d[:-1] - pv) * (d[1:] - pv)).mean())
+        assert abs(cov) < 5.0 * pv * (1 - pv) / np.sqrt(n) + 2.0 ** -8 * pv * (1 - pv), (pv, cov)
 
 
 def test_stochastic_rounding_is_unbiased_over_seeds(oracle):

@@ -27,10 +27,14 @@ def test_noalloc_product_matches_the_allocating_entry_point(out_dtype):
         ac, as_, bc, bs = _operands(M, N, Kd, 100 + call, dev)
         want = K.gemm_mxfp4_tn(ac, as_, bc, bs, 16.0 / 9.0, out_dtype)     # allocates its split-K workspace
         out = torch.full((M, N), float("nan"), dtype=out_dtype, device=dev)
-        before = torch.cuda.memory_allocated()
+        K.gemm_noalloc_prepare()      # the one step that may load the library's device image; a no-op from then on
+        torch.cuda.synchronize()
+        # free device memory as the driver reports it (hipMemGetInfo): it sees allocations of the library and of the HIP
+        # runtime as well, which torch's own allocator statistics would not
+        before, before_torch = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
         K.gemm_mxfp4_tn_noalloc(ac, as_, bc, bs, 16.0 / 9.0, out)
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.mem_get_info()[0] == before and torch.cuda.memory_allocated() == before_torch
         assert torch.equal(out, want), f"call {call}: {(out.float() - want.float()).abs().max()}"
     # a shape without a split goes through as well (no scratch used)
     M, N, Kd = 512, 512, 512
@@ -38,6 +42,34 @@ def test_noalloc_product_matches_the_allocating_entry_point(out_dtype):
     ac, as_, bc, bs = _operands(M, N, Kd, 7, dev)
     out = torch.empty((M, N), dtype=out_dtype, device=dev)
     assert torch.equal(K.gemm_mxfp4_tn_noalloc(ac, as_, bc, bs, 1.0, out), K.gemm_mxfp4_tn(ac, as_, bc, bs, 1.0, out_dtype))
+
+
+def test_noalloc_product_under_graph_capture():
+    """A split-K product captured into a HIP graph through the allocation-free entry point: every replay, with eager work
+    and synchronisations in between, gives the bits of the eager allocating call on the operands then in place."""
+    from quartet_amd import _lib, kernels as K
+    dev = torch.device("cuda:0")
+    M, N, Kd = 512, 768, 8192
+    assert _lib.lib().qm_gemm_workspace_bytes(M, N, Kd) > 0
+    ac, as_, bc, bs = _operands(M, N, Kd, 300, dev)
+    out = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    K.gemm_noalloc_prepare()
+    K.gemm_mxfp4_tn_noalloc(ac, as_, bc, bs, 1.0, out)        # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        K.gemm_mxfp4_tn_noalloc(ac, as_, bc, bs, 1.0, out)
+    for replay in range(3):
+        print(f"case noalloc gemm graph replay={replay}", flush=True)
+        fresh = _operands(M, N, Kd, 310 + replay, dev)        # new operand bytes in the captured buffers
+        for dst, src in zip((ac, as_, bc, bs), fresh):
+            dst.copy_(src)
+        want = K.gemm_mxfp4_tn(ac, as_, bc, bs, 1.0, torch.bfloat16)   # eager work between the replays (uses the stream)
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {replay}"
 
 
 def test_noalloc_product_rejects_what_does_not_fit():
