@@ -115,8 +115,9 @@ int qm_requantize_transposed_mxfp4_dense(const uint8_t* codes_in, const uint8_t*
  * Replaces F.linear / einsum on de-quantized operands (src/models/quantization/backward.py:62,
  * 71-75, 79-83) and matmul_mxf4_bf16_tn of notebooks/benchmark_mxfp4.ipynb.  K % 32 == 0.
  * alpha carries the per-operand constants of absmax coding (fl32(4/3) each).
- * Alignment: a_codes, b_codes and c 16 bytes (the tile kernels store c in 16-byte pieces), scales 4 bytes;
- * QM_ERR_UNALIGNED otherwise.
+ * Alignment: a_codes and b_codes 16 bytes, scales 4 bytes; c 16 bytes for the shapes the tile kernels serve (M, N
+ * multiples of 64 and >= 256, K % 128 == 0: they store c in 16-byte pieces), 4 bytes otherwise; QM_ERR_UNALIGNED
+ * if not.
  * a_layout / b_layout: layouts of a_codes / b_codes; QM_LAYOUT_TILED needs M and N multiples of 64 and
  * at least 256, and K % 128 == 0 (the shapes the 256x256-tile kernels serve).
  * workspace: optional scratch (NULL, 0 for none).  With qm_gemm_workspace_bytes(M, N, K) > 0 bytes of it, 16-byte

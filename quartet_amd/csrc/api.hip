@@ -44,7 +44,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 12; }
+int qm_version(void) { return 13; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -158,8 +158,11 @@ int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint
     if (M < 0 || N < 0 || K < 0 || K % 32) return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn: need K %% 32 == 0 (M=%lld N=%lld K=%lld)", (long long)M, (long long)N, (long long)K);
     if (M == 0 || N == 0) return 0;
     if (!c || (K > 0 && (!a_codes || !a_scales || !b_codes || !b_scales))) return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn: null tensor");
-    if (!aligned(a_codes, 16) || !aligned(b_codes, 16) || !aligned(a_scales, 4) || !aligned(b_scales, 4) || !aligned(c, 16))
-        return fail(QM_ERR_UNALIGNED, "qm_gemm_mxfp4_tn: codes and c need 16-byte, scales 4-byte alignment");
+    // the 256 x 256 tile kernels store c in 16-byte pieces; the generic kernel (any M, N) stores single elements
+    const uintptr_t c_align = qm::gemm_supports_tiled(M, N, K) ? 16 : 4;
+    if (!aligned(a_codes, 16) || !aligned(b_codes, 16) || !aligned(a_scales, 4) || !aligned(b_scales, 4) || !aligned(c, c_align))
+        return fail(QM_ERR_UNALIGNED, "qm_gemm_mxfp4_tn: codes need 16-byte, scales 4-byte alignment, c 16-byte (4-byte for shapes "
+                                      "outside the tile kernels: M or N not a multiple of 64 or below 256, K %% 128 != 0)");
     if ((a_layout == QM_LAYOUT_TILED || b_layout == QM_LAYOUT_TILED) && !qm::gemm_supports_tiled(M, N, K))
         return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn: tiled operands need M, N multiples of 64 and >= 256, K %% 128 == 0 (M=%lld N=%lld K=%lld)",
                     (long long)M, (long long)N, (long long)K);

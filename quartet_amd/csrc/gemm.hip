@@ -240,6 +240,10 @@ __device__ __forceinline__ float acc_read(float a) {
     asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
     return v;
 }
+// The hazard recogniser does not look inside assembly statements: a matrix instruction's result may be read by a vector
+// instruction only a number of wait states after it issued (19 for the sixteen-pass forms).  Every epilogue that reads
+// accumulators through acc_read() starts with this, whatever the scheduler has put between the last product and it.
+__device__ __forceinline__ void acc_settle() { asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory"); }
 template <typename OutT, bool IN_ORDER = false>
 __device__ __forceinline__ void store_tile(const v16f& t, float alpha, OutT* __restrict__ c, int64_t row0, int64_t col,
                                            int64_t N, int half) {
@@ -719,6 +723,7 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
     const uint8_t* rd = region + rsub * 128 + ((chunk ^ rsub) * 16);  // rows rsub + 8k share rsub's swizzle
     const int64_t pitch8 = N * 16;                                   // eight rows of bf16
     uint8_t* out = reinterpret_cast<uint8_t*>(c + (m0 + wm * 128 + rsub) * N + n0 + wn * 128) + chunk * 16;
+    acc_settle();
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
@@ -904,6 +909,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         } else {
             OutT* dst = splits > 1 ? c + (int64_t)cur_split * M * N : c;
             const float a_eff = splits > 1 ? 1.0f : alpha;
+            acc_settle();
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll

@@ -10,6 +10,7 @@ quantizer modules and library GEMMs, as the reference does."""
 import torch
 import torch.nn as nn
 
+from . import _lib
 from . import kernels as K
 from .backward import BACKWARD_SCHEMES, EW_EtX_Scheme, QEQWtt_QEtQXtt_Scheme  # noqa: F401
 from .quantizers import QUANTIZER_CLASSES, AlbertTsengQuantizer, NoQuantizer, QuestMXFP4Quantizer  # noqa: F401
@@ -26,7 +27,8 @@ def set_device_seed_base(tensor):
     drawn at capture time, so capture the step with a seed base set and let the graph increment the tensor (any
     in-place add recorded in the graph): every replay then rounds with fresh random streams.  The sign flips drawn at
     capture time stay as they are.  Applies to layers on the tiled layout (tokens, in- and out-features multiples of
-    128, Hadamard blocks 32, no dense rotation); others ignore it."""
+    128, Hadamard blocks 32, no dense rotation); a stochastic layer outside it raises while a seed base is set, since
+    its replays would repeat their random streams."""
     global _SEED_BASE
     if tensor is not None and not (tensor.is_cuda and tensor.dtype == torch.int64 and tensor.numel() >= 1):
         raise ValueError("the seed base must be an int64 tensor on the GPU")
@@ -78,6 +80,14 @@ def _backward_packed(ctx, e, packed_x, packed_w, gx_rotated=False):
     mid_dtype = torch.bfloat16 if low else e2.dtype
     sd_x = torch.bfloat16 if low else ctx.x_dtype
     sd_w = torch.bfloat16 if low else ctx.w_dtype
+    if _SEED_BASE is not None and g_q.stochastic and not (ctx.tiled and g_matrix is None):
+        # the device seed base is read by the pair launches of the tiled layout only: on any other path a captured replay
+        # would silently repeat this launch's random streams
+        raise _lib.QuartetHipError(
+            f"a device seed base is set (set_device_seed_base), but this layer (tokens {T}, in {I}, out {O}"
+            f"{', dense gradient rotation' if g_matrix is not None else ''}) does not run on the tiled layout, whose kernels are the "
+            "only ones that read it (every extent a multiple of 128 and >= 256, Hadamard blocks 32, no dense rotation); "
+            "clear the seed base or change the layer")
     gx, gw = K.linear_backward(e2, packed_x, packed_w, T, I, O, a_hd, a_signs, w_hd, w_signs, hd, signs, mode, seeds, ctx.x_dtype,
                                ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled, gx_rotated,
                                ctx.w_dtype if ctx.w_dtype in (torch.float32, torch.bfloat16) else None, g_matrix,

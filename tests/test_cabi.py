@@ -29,7 +29,7 @@ def test_library_exports_every_declared_function():
 
 def test_host_only_entry_points():
     L = _lib.lib()
-    assert L.qm_version() == 12
+    assert L.qm_version() == 13
     T, I, O = 256, 128, 384
     off = (ctypes.c_size_t * 3)()
     for rows, cols in ((T, I), (O, I)):
@@ -60,7 +60,9 @@ def test_host_only_entry_points():
     (lambda L: L.qm_requantize_transposed_mxfp4(None, None, 30, 64, 1.0, 0, 32, None, 2, None, 0, None, None, None, 0, 0, None), b"hadamard_dim"),
     (lambda L: L.qm_gemm_mxfp4_tn(None, None, None, None, 64, 64, 48, 1.0, None, 0, 0, 0, None, 0, None), b"qm_gemm_mxfp4_tn"),
     # an output offset by 4 bytes: the tile kernels store 16-byte pieces, so the call is refused before any launch
-    (lambda L: L.qm_gemm_mxfp4_tn(0x1000, 0x2000, 0x3000, 0x4000, 256, 256, 128, 1.0, 0x5004, 0, 0, 0, None, 0, None), b"c need 16-byte"),
+    (lambda L: L.qm_gemm_mxfp4_tn(0x1000, 0x2000, 0x3000, 0x4000, 256, 256, 128, 1.0, 0x5004, 0, 0, 0, None, 0, None), b"c 16-byte"),
+    # a shape of the generic kernel stores single elements: c misaligned for 4 bytes is refused, 4-byte aligned c is not
+    (lambda L: L.qm_gemm_mxfp4_tn(0x1000, 0x2000, 0x3000, 0x4000, 96, 256, 128, 1.0, 0x5002, 0, 0, 0, None, 0, None), b"c 16-byte (4-byte"),
     (lambda L: L.qm_quantize_mxfp4_dense(None, 0, 4, 40, None, 1, 0, 0, None, None, None, None, 0, None), b"multiple of 32"),
     (lambda L: L.qm_quantize_mxfp4_dense(None, 0, 4, 64, None, 1, 0, 0, None, None, None, None, 0, None), b"non-null"),
     (lambda L: L.qm_quantize_mxfp4_dense(0x1000, 0, 64, 64, 0x2000, 1, 1, 0, 0x3000, 0x4000, None, None, 0, None), b"transposed input needs"),

@@ -137,6 +137,26 @@ def test_captured_layer_step_draws_fresh_streams_with_a_seed_base():
         q.set_device_seed_base(None)
 
 
+def test_seed_base_refuses_layers_that_would_ignore_it():
+    """With a device seed base set, a stochastic layer whose shape keeps it off the tiled layout must fail loudly: its
+    kernels take host seeds only, so a captured replay would repeat their random streams."""
+    import quartet_amd as q
+    from quartet_amd import _lib
+    dev = torch.device("cuda:0")
+    layer = q.QuantizedLinear(96, 160, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(), activation_quantizer=q.QuestMXFP4Quantizer(),
+                              gradient_quantizer=q.AlbertTsengQuantizer(stochastic=True, rerotate="signs"),
+                              backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]()).to(dev, torch.bfloat16)
+    x = torch.randn(64, 96, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    q.set_device_seed_base(torch.zeros(1, dtype=torch.int64, device=dev))
+    try:
+        with pytest.raises(_lib.QuartetHipError, match="seed base"):
+            layer(x).sum().backward()
+    finally:
+        q.set_device_seed_base(None)
+    layer(x).sum().backward()      # without a seed base the same layer runs
+    assert torch.isfinite(x.grad.float()).all()
+
+
 def test_sign_flips_of_the_gradient_rotation_cancel_in_both_products():
     """Why a captured step needs no device-side sign words: the gradient quantizer's sign flips (re_randomize("signs"),
     mxfp4.py:53-60) multiply both operands of each backward product along the contracted index, and the absmax
