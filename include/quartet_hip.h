@@ -131,6 +131,20 @@ int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint
                      void* stream);
 
 /*
+ * c[M, N] = alpha * A @ B with A packed MXFP4 (row-major codes [M, K/2], E8M0 scales [M, K/32]) and B plain bf16
+ * [K, N] row-major: the two gradient products of the scheme that quantizes only the error signal,
+ * QEW_QEtXFn.backward (src/models/quantization/backward.py:31-43): grad_x = Q(e) @ w with A = Q(e) [T, O], B = w [O, I],
+ * and grad_w = Q(e^T) @ x with A = Q(e^T) [O, T], B = x [T, I] -- the saved operands exactly as they lie in memory, no
+ * transposed copy, no de-quantized tensor (the reference multiplies a de-quantized bf16 copy of Q(e) with a library GEMM).
+ * Codes are decoded to bf16 in registers (exact), products accumulate in fp32.  alpha carries the quantizer's
+ * post-scale (fl32(4/3) for the absmax modes).  c_dtype QM_BF16 or QM_F32.  A scale byte of 0 reads as zero (not
+ * 2^-127).  Needs K % 64 == 0 and N % 8 == 0 (QM_ERR_INVALID otherwise); a_codes, b, c 16-byte and a_scales 2-byte
+ * aligned.
+ */
+int qm_gemm_mxfp4_bf16_nn(const uint8_t* a_codes, const uint8_t* a_scales, const void* b, int64_t M, int64_t N, int64_t K,
+                          float alpha, void* c, int c_dtype, void* stream);
+
+/*
  * qm_gemm_mxfp4_tn for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses that forbid
  * hipMalloc).  It has no counterpart in the reference.  Same arguments and the same results, bit for bit, as
  * qm_gemm_mxfp4_tn offered qm_gemm_workspace_bytes(M, N, K) bytes of workspace; the split-K partial sums live in a

@@ -25,6 +25,7 @@ EXPORTS = (
     "qm_gemm_workspace_bytes",
     "qm_diag_mfma_only",
     "qm_diag_gemm_tile_phases",
+    "qm_gemm_mxfp4_bf16_nn",
     "qm_gemm_noalloc_scratch_bytes",
     "qm_gemm_mxfp4_tn_noalloc",
     "qm_gemm_noalloc_prepare",
@@ -82,6 +83,8 @@ def lib():
     L.qm_gemm_workspace_bytes.argtypes = [i64, i64, i64]
     L.qm_gemm_noalloc_scratch_bytes.restype = ctypes.c_size_t
     L.qm_gemm_noalloc_scratch_bytes.argtypes = []
+    L.qm_gemm_mxfp4_bf16_nn.restype = i32
+    L.qm_gemm_mxfp4_bf16_nn.argtypes = [vp, vp, vp, i64, i64, i64, f32, vp, i32, vp]
     L.qm_gemm_noalloc_prepare.restype = i32
     L.qm_gemm_noalloc_prepare.argtypes = []
     L.qm_gemm_mxfp4_tn_noalloc.restype = i32

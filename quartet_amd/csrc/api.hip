@@ -198,6 +198,21 @@ int64_t qm_diag_mfma_only(const uint8_t* operands, size_t operand_bytes, float* 
     return (int64_t)blocks * 4 * (int64_t)iters * 16;
 }
 
+int qm_gemm_mxfp4_bf16_nn(const uint8_t* a_codes, const uint8_t* a_scales, const void* b, int64_t M, int64_t N, int64_t K,
+                          float alpha, void* c, int c_dtype, void* stream) {
+    if (!valid_dtype(c_dtype)) return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_bf16_nn: c_dtype %d", c_dtype);
+    if (M < 0 || N < 0 || K < 0) return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_bf16_nn: negative extent");
+    if (M == 0 || N == 0) return 0;
+    if (!qm::gemm_fp4_bf16_nn_supported(M, N, K))
+        return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_bf16_nn: need K a positive multiple of 64 and N a multiple of 8 (M=%lld N=%lld K=%lld)",
+                    (long long)M, (long long)N, (long long)K);
+    if (!a_codes || !a_scales || !b || !c) return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_bf16_nn: null tensor");
+    if (!aligned(a_codes, 16) || !aligned(a_scales, 2) || !aligned(b, 16) || !aligned(c, 16))
+        return fail(QM_ERR_UNALIGNED, "qm_gemm_mxfp4_bf16_nn: a_codes, b and c need 16-byte, a_scales 2-byte alignment");
+    return from_hip(qm::gemm_fp4_bf16_nn(a_codes, a_scales, b, M, N, K, alpha, c, c_dtype, reinterpret_cast<hipStream_t>(stream)),
+                    "qm_gemm_mxfp4_bf16_nn");
+}
+
 size_t qm_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0 || K % 32) return 0;
     return qm::gemm_workspace_bytes(M, N, K);

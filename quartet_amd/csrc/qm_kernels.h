@@ -123,6 +123,10 @@ hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const 
                          const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
                          int a_layout, int b_layout, void* workspace, size_t workspace_bytes, hipStream_t stream);
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+// C = alpha * A (packed MXFP4 [M, K]) x B (bf16 [K, N] row-major): K % 64 == 0, N % 8 == 0
+bool gemm_fp4_bf16_nn_supported(int64_t M, int64_t N, int64_t K);
+hipError_t gemm_fp4_bf16_nn(const uint8_t* a_codes, const uint8_t* a_scales, const void* b, int64_t M, int64_t N, int64_t K,
+                            float alpha, void* c, int c_dtype, hipStream_t stream);
 // measurement aid: one launch of the persistent kernel that records the shader clock around every tile's K loop and epilogue
 int gemm_phase_stamps_per_group();
 hipError_t gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,

@@ -164,6 +164,24 @@ def gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, alpha=1.0, out_dtype=tor
     return c
 
 
+def gemm_mxfp4_bf16_nn_supported(M, N, K):
+    return K > 0 and K % 64 == 0 and N % 8 == 0 and M > 0 and N > 0
+
+
+def gemm_mxfp4_bf16_nn(a_codes, a_scales, b, alpha=1.0, out_dtype=torch.bfloat16):
+    """[M,K/2],[M,K/32] packed MXFP4 (row-major) x b [K,N] bf16 row-major -> alpha * A @ b as [M,N] of out_dtype."""
+    _require_cuda(a_codes, a_scales, b)
+    M, K = a_codes.shape[0], a_codes.shape[1] * 2
+    if b.dtype != torch.bfloat16 or b.dim() != 2 or b.shape[0] != K or not b.is_contiguous():
+        raise _lib.QuartetHipError(f"gemm_mxfp4_bf16_nn: b must be a contiguous bf16 [{K}, N] tensor, got {tuple(b.shape)} {b.dtype}")
+    N = b.shape[1]
+    c = torch.empty((M, N), dtype=out_dtype, device=a_codes.device)
+    rc = _lib.lib().qm_gemm_mxfp4_bf16_nn(_ptr(a_codes), _ptr(a_scales), _ptr(b), M, N, K, alpha, _ptr(c), _dtype_code(out_dtype),
+                                          _stream())
+    _lib.check(rc, "qm_gemm_mxfp4_bf16_nn")
+    return c
+
+
 _noalloc_prepared = set()
 
 

@@ -218,3 +218,71 @@ def test_tile_phase_stamps_of_the_persistent_kernel():
         assert tiles == (M // 256) * (N // 256)
     with pytest.raises(_lib.QuartetHipError):   # K % 512 != 0: not served
         K.gemm_tile_phases(ac[:, :320].contiguous(), as_[:, :20].contiguous(), bc[:, :320].contiguous(), bs[:, :20].contiguous())
+
+
+# ---- MXFP4 x bf16 "NN" product (the scheme that quantizes only the error signal) -----------------------------------
+def _nn_reference(oracle, ac, as_, b, alpha):
+    """float64 product of the de-quantized codes with the bf16 operand: the reference's `Q(e) @ w` without any rounding."""
+    a = oracle.dequantize(ac, as_).astype(np.float64)
+    return alpha * (a @ b.float().numpy().astype(np.float64))
+
+
+@pytest.mark.parametrize("M,N,K_", [(128, 128, 64), (256, 384, 512), (96, 200, 192), (1000, 72, 1728), (640, 1728, 2048)])
+def test_fp4_bf16_product_against_fp64_matmul(oracle, K, M, N, K_):
+    """A packed (absmax codes of a small-valued tensor, like an error signal), B bf16 [K, N] as it lies in memory."""
+    print(f"case fp4 x bf16 product {M}x{N}x{K_}", flush=True)
+    dev = torch.device("cuda:0")
+    ac, as_ = _quant(oracle, M, K_, oracle.ABSMAX_RTN, 11, scale=1e-3)
+    b = make_input(K_, N, torch.bfloat16, seed=12, scale=0.02)
+    d = float(oracle.FOUR_THIRDS)
+    want = _nn_reference(oracle, ac, as_, b, d)
+    act, ast, bt = torch.from_numpy(ac).to(dev), torch.from_numpy(as_).to(dev), b.to(dev)
+    got32 = K.gemm_mxfp4_bf16_nn(act, ast, bt, alpha=d, out_dtype=torch.float32)
+    got16 = K.gemm_mxfp4_bf16_nn(act, ast, bt, alpha=d, out_dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    rel = np.linalg.norm(got32.cpu().numpy().astype(np.float64) - want) / np.linalg.norm(want)
+    assert rel <= 1e-5, rel          # exact decode, exact bf16 products, fp32 accumulation
+    assert torch.equal(got16.cpu(), got32.cpu().to(torch.bfloat16))
+
+
+def test_fp4_bf16_product_bit_exact_when_sums_are_exact(oracle, K):
+    """Random code bytes with one common scale against small integers: every partial sum is a multiple of 1/2 below 2^24,
+    so the fp32 result must equal the float64 product whatever order the contraction index is walked in."""
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(3)
+    M, N, K_ = 192, 136, 448
+    ac = rng.integers(0, 256, (M, K_ // 2), dtype=np.uint8)
+    as_ = np.full((M, K_ // 32), 127, dtype=np.uint8)
+    b = torch.from_numpy(rng.integers(-8, 9, (K_, N)).astype(np.float32)).to(torch.bfloat16)
+    want = _nn_reference(oracle, ac, as_, b, 1.0)
+    got = K.gemm_mxfp4_bf16_nn(torch.from_numpy(ac).to(dev), torch.from_numpy(as_).to(dev), b.to(dev), 1.0, torch.float32)
+    assert np.array_equal(got.cpu().numpy().astype(np.float64), want)
+
+
+def test_fp4_bf16_product_selects_rows_and_columns(oracle, K):
+    """One +1.0 per row of A at a known k (every k of a K step occurs, per-group scales differ) returns row k of B times
+    the group's scale: pins the order in which lanes, matrix instructions and the transposing LDS read walk k."""
+    dev = torch.device("cuda:0")
+    M, N, K_ = 256, 128, 128
+    ac = np.zeros((M, K_ // 2), dtype=np.uint8)
+    as_ = (120 + (np.arange(M)[:, None] + np.arange(K_ // 32)[None, :]) % 12).astype(np.uint8)
+    ks = [(m * 5 + 3) % K_ for m in range(M)]
+    assert set(ks) == set(range(K_))
+    for m, k in enumerate(ks):
+        ac[m, k // 2] = 0x2 << (4 * (k & 1))
+    b = make_input(K_, N, torch.bfloat16, seed=5, scale=1.0, outlier_frac=0)
+    got = K.gemm_mxfp4_bf16_nn(torch.from_numpy(ac).to(dev), torch.from_numpy(as_).to(dev), b.to(dev), 1.0, torch.float32)
+    bf = b.float().numpy()
+    want = np.stack([bf[k] * np.float32(2.0) ** (int(as_[m, k // 32]) - 127) for m, k in enumerate(ks)])
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+def test_fp4_bf16_product_rejects_what_it_does_not_serve(K):
+    from quartet_amd import _lib
+    dev = torch.device("cuda:0")
+    a = torch.zeros(64, 48, dtype=torch.uint8, device=dev)      # K = 96: not a multiple of 64
+    s = torch.zeros(64, 3, dtype=torch.uint8, device=dev)
+    with pytest.raises(_lib.QuartetHipError, match="multiple of 64"):
+        K.gemm_mxfp4_bf16_nn(a, s, torch.zeros(96, 64, dtype=torch.bfloat16, device=dev))
+    with pytest.raises(_lib.QuartetHipError, match="bf16"):
+        K.gemm_mxfp4_bf16_nn(a, s, torch.zeros(96, 64, dtype=torch.float32, device=dev))

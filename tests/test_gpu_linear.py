@@ -460,3 +460,57 @@ def test_error_only_scheme_under_autocast(oracle, q):
     gw_ref = from_oracle_bf16(oracle.masked_hadamard_bwd(to_oracle(gwq), 32, oracle.BF16, None, qw["mask"])).double().numpy()
     assert rel(xd.grad.float().cpu(), gx_ref) < 1e-2
     assert rel(layer.weight.grad.float().cpu(), gw_ref) < 1e-2
+
+
+@pytest.mark.parametrize("cls_name,stochastic", [("AlbertTsengQuantizer", True), ("AlbertTsengQuantizer", False),
+                                                 ("AlignedAlbertTsengQuantizer", False), ("QuestMXFP4Quantizer", False)])
+def test_error_only_scheme_on_packed_codes(oracle, q, cls_name, stochastic, monkeypatch):
+    """Scheme "Q(E)W_Q(Et)X" with bf16 products (autocast): grad_x = Q(e) w and grad_w = Q(e^T) x run on the packed codes
+    of Q(e) in the FP4 x bf16 kernel (both products, counted), with the saved operands as they lie in memory.  Checked
+    against the oracle's de-quantized Q(e), Q(e^T) (same seeds) times the bf16 operands in float64; the only rounding
+    beyond fp32 accumulation is the bf16 output (2^-9 per element)."""
+    print(f"case packed error-only scheme {cls_name} stochastic={stochastic}", flush=True)
+    from quartet_amd import kernels as K
+    dev = "cuda:0"
+    T, I, O = 384, 200, 192
+    kw = {"stochastic": stochastic} if cls_name == "AlbertTsengQuantizer" else {}
+    g_q = getattr(q, cls_name)(**kw)
+    layer = q.QuantizedLinear(I, O, bias=False, gradient_quantizer=g_q, backward_scheme=q.BACKWARD_SCHEMES["Q(E)W_Q(Et)X"]()).to(dev)
+    calls = []
+    real = K.gemm_mxfp4_bf16_nn
+    monkeypatch.setattr(K, "gemm_mxfp4_bf16_nn", lambda *a, **k: (calls.append(a[2].shape), real(*a, **k))[1])
+    x = make_input(T, I, torch.bfloat16, 51, outlier_frac=0.0)
+    dy = make_input(T, O, torch.bfloat16, 52, outlier_frac=0.0, scale=1e-3)
+    xd = x.to(dev).requires_grad_(True)
+    random.seed(91)
+    with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+        y = layer(xd)
+        y.backward(dy.to(dev))
+    torch.cuda.synchronize()
+    assert calls == [(O, I), (T, I)]
+    random.seed(91)
+    seeds = [random.getrandbits(63) for _ in range(2)] if stochastic else [0, 0]
+    mode = {"QuestMXFP4Quantizer": oracle.QUEST_RTN}.get(cls_name, oracle.ABSMAX_SR if stochastic else oracle.ABSMAX_RTN)
+    post = 1.009276 if cls_name == "AlignedAlbertTsengQuantizer" else 1.0
+    qe = oracle.quantize(to_oracle(dy), 32, mode=mode, seed=seeds[0])
+    qet = oracle.quantize(to_oracle(dy), 32, mode=mode, transposed_in=True, seed=seeds[1])
+    d = 1.0 if mode == oracle.QUEST_RTN else float(oracle.FOUR_THIRDS)
+    w16 = layer.weight.detach().to(torch.bfloat16).double().cpu().numpy()
+    gx_ref = post * oracle.dequantize(qe["codes"], qe["scales"], d).astype(np.float64) @ w16
+    gw_ref = post * oracle.dequantize(qet["codes"], qet["scales"], d).astype(np.float64) @ x.double().numpy()
+    assert xd.grad.shape == (T, I) and layer.weight.grad.shape == (O, I)
+    assert rel(xd.grad.float().cpu(), gx_ref) < 3e-3
+    assert rel(layer.weight.grad.float().cpu(), gw_ref) < 3e-3
+
+
+def test_error_only_scheme_keeps_the_library_path_for_fp32_products(q, monkeypatch):
+    """Without autocast on fp32 tensors the reference's products are fp32 library GEMMs: the packed kernel (bf16 operand)
+    must not be used."""
+    from quartet_amd import kernels as K
+    monkeypatch.setattr(K, "gemm_mxfp4_bf16_nn", lambda *a, **k: pytest.fail("packed product used for fp32 operands"))
+    dev = "cuda:0"
+    layer = q.QuantizedLinear(128, 64, bias=False, gradient_quantizer=q.AlbertTsengQuantizer(stochastic=False),
+                              backward_scheme=q.BACKWARD_SCHEMES["Q(E)W_Q(Et)X"]()).to(dev)
+    x = torch.randn(64, 128, device=dev, requires_grad=True)
+    layer(x).sum().backward()
+    assert torch.isfinite(x.grad).all() and torch.isfinite(layer.weight.grad).all()
