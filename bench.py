@@ -698,6 +698,41 @@ def reference_shapes(device):
     return out
 
 
+def error_only_scheme_block(device):
+    """The two gradient products of scheme "Q(E)W_Q(Et)X" at 8192 x 4096 x 4096: this build's FP4 x bf16 kernel on the
+    packed Q(e) / Q(e^T) against the module path the reference takes (de-quantized bf16 Q(e), a transposed copy of e, two
+    library bf16 GEMMs), quantizer launches included on both sides."""
+    from quartet_amd import kernels as K
+    T, I, O = T_TOKENS, IN_F, OUT_F
+    g = torch.Generator(device=device).manual_seed(7)
+    e = (1e-3 * torch.randn(T, O, generator=g, device=device)).to(torch.bfloat16)
+    w = (0.02 * torch.randn(O, I, generator=g, device=device)).to(torch.bfloat16)
+    x = torch.randn(T, I, generator=g, device=device).to(torch.bfloat16)
+    d = K.FOUR_THIRDS
+
+    def packed():
+        ec, es, _, _ = K.quantize_mxfp4(e, 32, None, K.QM_ABSMAX_SR, seed=1)
+        K.gemm_mxfp4_bf16_nn(ec, es, w, d)
+        etc, ets, _, _ = K.quantize_mxfp4(e, 32, None, K.QM_ABSMAX_SR, transposed_in=True, seed=2)
+        K.gemm_mxfp4_bf16_nn(etc, ets, x, d)
+
+    def module_path():
+        K.quantize_mxfp4(e, 32, None, K.QM_ABSMAX_SR, seed=1, want_dequant=True)[3] @ w
+        K.quantize_mxfp4(e.T.contiguous(), 32, None, K.QM_ABSMAX_SR, seed=2, want_dequant=True)[3] @ x
+    ec, es, _, _ = K.quantize_mxfp4(e, 32, None, K.QM_ABSMAX_SR, seed=1)
+    etc, ets, _, _ = K.quantize_mxfp4(e, 32, None, K.QM_ABSMAX_SR, transposed_in=True, seed=2)
+    fl = 2.0 * T * I * O
+    out = {"shape": [T, I, O]}
+    for name, fn in (("packed_ms", packed), ("module_path_ms", module_path),
+                     ("product_grad_x_ms", lambda: K.gemm_mxfp4_bf16_nn(ec, es, w, d)),
+                     ("product_grad_w_ms", lambda: K.gemm_mxfp4_bf16_nn(etc, ets, x, d))):
+        out[name] = round(sorted(time_kernel(fn, reps=10) for _ in range(3))[1], 4)
+    out["product_grad_x_TFLOPs"] = round(fl / out["product_grad_x_ms"] / 1e9, 1)
+    out["product_grad_w_TFLOPs"] = round(fl / out["product_grad_w_ms"] / 1e9, 1)
+    out["speedup_over_module_path"] = round(out["module_path_ms"] / out["packed_ms"], 3)
+    return out
+
+
 def quantizer_bounds(prof, x):
     """What else bounds the forward quantizer at this size: its vector-instruction floor (instructions per group from the
     tracked counter profile: a lane owns one group, an instruction occupies its SIMD for four cycles) and what two plain
@@ -870,6 +905,7 @@ def main():
         result["k1536"] = k1536_block(device)
         result["quantizer_sizes"] = quantizer_sizes_block(device)
         result["reference_shapes"] = reference_shapes(device)
+        result["error_only_scheme"] = error_only_scheme_block(device)
         del x, w, dy
         torch.cuda.empty_cache()
         result["llama"] = llama_blocks(device)

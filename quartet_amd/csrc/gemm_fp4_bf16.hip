@@ -31,6 +31,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+#include <type_traits>
+
 #include "qm_kernels.h"
 #include "qm_math.h"
 
@@ -216,6 +219,217 @@ __global__ __launch_bounds__(256, 2) void gemm_fp4_bf16_nn_kernel(const uint8_t*
     }
 }
 
+
+// ---- large-tile variant: 256 x 256 per workgroup, one wave per SIMD owning 128 x 128 ---------------------------------
+// For products with at least one full tile in each direction.  Four waves x (4 x 4 blocks of 32 x 32) = 256 accumulator
+// registers; per K step of 64 a wave issues 64 matrix instructions against 4 code reads, 32 transposing reads and 64
+// decode instructions, so LDS and the vector ALU stay well below the matrix pipe's time.  Operands go global -> LDS
+// directly (global_load_lds_dwordx4) into a ring of three stages, requested two K steps ahead; the B swizzle is applied
+// on the global-address side of those loads.  Scale bytes go global -> registers directly (one 16-bit load per row block
+// and step: a lane keeps the two E8M0 bytes of its row's step and picks its half's).  One barrier per K step.
+constexpr int kBM = 256, kBN = 256;
+constexpr int kBigA = kBM * (kTK / 2);       // 8 KiB of codes per stage: [256 rows][32 bytes]
+constexpr int kBigB = kTK * kBN * 2;         // 32 KiB: [64 k][512 bytes]
+constexpr int kBigStage = kBigA + kBigB;
+constexpr int kBigStages = 3;
+constexpr int kBigSmem = kBigStages * kBigStage;   // 120 KiB
+constexpr int kBigLoads = 14;                // VMEM instructions per wave per K step: 2 (A) + 8 (B) + 4 (scales)
+
+// global -> LDS without passing through registers; issued from assembly so that the compiler's wait-count insertion
+// does not treat every later LDS read as depending on it (the kernel waits explicitly for the stage it is about to read).
+// LDS destination = lds_base (wave-uniform, through M0) + lane * 16.
+__device__ __forceinline__ void dma_b128(const uint8_t* base, uint32_t lane_off, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(lds_base) : "memory");
+}
+__device__ __forceinline__ void dma_b128_v(const uint8_t* gsrc, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gsrc), "s"(lds_base) : "memory");
+}
+__device__ __forceinline__ uint32_t load_u16_async(const uint8_t* base, uint32_t lane_off) {
+    uint32_t v;
+    asm volatile("global_load_ushort %0, %1, %2" : "=v"(v) : "v"(lane_off), "s"(base) : "memory");
+    return v;
+}
+constexpr int vmcnt_only(int n) { return 0x0f70 | (n & 0xf) | ((n >> 4) << 14); }
+
+template <typename OutT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_fp4_bf16_nn_big_kernel(
+    const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint16_t* __restrict__ b, int M, int N, int K,
+    float alpha, OutT* __restrict__ c) {
+    extern __shared__ uint8_t smem_nn[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem_nn;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lrow = lane & 31, half = lane >> 5;
+    int tm, tn;
+    tile_of_block_nn((int)blockIdx.x, (M + kBM - 1) / kBM, (N + kBN - 1) / kBN, tm, tn);
+    const int64_t m0 = (int64_t)tm * kBM, n0 = (int64_t)tn * kBN;
+    const int64_t code_pitch = K / 2, groups = K / 32;
+    const int nk = K / kTK;
+
+    // ---- what this wave requests per K step ---------------------------------------------------------------------------
+    // A codes: two wave-loads of 32 rows x 32 bytes (rows wave*64 + 32 v + lane/2, 16-byte half lane%2); rows beyond M
+    // read the last row, their results are dropped
+    const uint8_t* a_src[2];
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {
+        int64_t row = m0 + wave * 64 + 32 * v + (lane >> 1);
+        row = row < M ? row : (int64_t)M - 1;
+        a_src[v] = a_codes + row * code_pitch + (lane & 1) * 16;
+    }
+    // B: eight wave-loads of 2 rows x 512 bytes (rows wave*16 + 2 u + lane/32).  LDS slot lane%32 of a row holds the
+    // logical 16-byte piece (lane%32) ^ 4 (row & 3); row & 3 = 2 (u & 1) + lane/32.  Pieces beyond N read the row's last
+    // piece instead (their columns are dropped).
+    const int last_piece = (int)((N - n0 + 7) / 8) - 1;   // N % 8 == 0
+    uint32_t b_lane[2];
+#pragma unroll
+    for (int par = 0; par < 2; ++par) {
+        int piece = (lane & 31) ^ (4 * (2 * par + (lane >> 5)));
+        piece = piece < last_piece ? piece : last_piece;
+        b_lane[par] = (uint32_t)((lane >> 5) * N * 2 + piece * 16);
+    }
+    const uint8_t* b_base = reinterpret_cast<const uint8_t*>(b + (int64_t)(wave * 16) * N + n0);   // + (ks * 64 + 2 u) rows
+    const int64_t b_row_bytes = (int64_t)N * 2;
+    // scales: per row block i the two bytes of row wm*128 + i*32 + lrow at step ks
+    uint32_t s_lane[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int64_t row = m0 + wm * 128 + i * 32 + lrow;
+        row = row < M ? row : (int64_t)M - 1;
+        s_lane[i] = (uint32_t)(row * groups);
+    }
+    const uint32_t lds_a = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + wave * 2048));
+    const uint32_t lds_b = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + kBigA + wave * 8192));
+
+    uint32_t sc[kBigStages][4] = {};
+    auto issue = [&](int ks, int stage, uint32_t (&scs)[4]) {
+        const int kk = ks < nk ? ks : nk - 1;   // past the end: a harmless repeat of the last step into a free stage
+        const uint32_t sa = lds_a + stage * kBigStage, sb = lds_b + stage * kBigStage;
+        dma_b128_v(a_src[0] + (int64_t)kk * 32, sa);
+        dma_b128_v(a_src[1] + (int64_t)kk * 32, sa + 1024);
+        const uint8_t* bs = b_base + (int64_t)kk * kTK * b_row_bytes;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) dma_b128(bs + (int64_t)(2 * u) * b_row_bytes, b_lane[u & 1], sb + u * 1024);
+        const uint8_t* ss = a_scales + (int64_t)kk * 2;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) scs[i] = load_u16_async(ss, s_lane[i]);
+    };
+
+    // ---- LDS -> registers: per-lane offsets ---------------------------------------------------------------------------
+    const int a_off = (wm * 128 + lrow) * 32 + half * 16;                 // + i * 1024
+    const int r16 = lane & 15, nh = (lane >> 4) & 1;
+    const int b_krow = 32 * half + (r16 >> 2);                            // + 8 s + 4 rd
+    const int b_swz = 4 * ((r16 >> 2) & 3);
+    int b_off[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int byte = (wn * 128 + j * 32 + 16 * nh + 4 * (r16 & 3)) * 2;
+        b_off[j] = kBigA + b_krow * 512 + (((byte >> 4) ^ b_swz) << 4) + (byte & 15);
+    }
+
+    v16f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    auto compute = [&](int stage, uint32_t (&scs)[4]) {
+        const uint8_t* st = smem_nn + stage * kBigStage;
+        uint4 codes[4];
+        float scale[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            codes[i] = *reinterpret_cast<const uint4*>(st + a_off + i * 1024);
+            scale[i] = u2f(__builtin_amdgcn_ubfe(scs[i], (uint32_t)(8 * half), 8u) << 23);   // E8M0 -> 2^(byte - 127); byte 0 reads as 0
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            v8bf bf[4], af[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                typedef v4s __attribute__((address_space(3))) * lds_v4s;
+                typedef short v8s __attribute__((ext_vector_type(8)));
+                const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(st + b_off[j] + (8 * s) * 512));
+                const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(st + b_off[j] + (8 * s + 4) * 512));
+                bf[j] = __builtin_bit_cast(v8bf, v8s{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t w = s == 0 ? codes[i].x : (s == 1 ? codes[i].y : (s == 2 ? codes[i].z : codes[i].w));
+                const v2bf p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale[i], 0);
+                const v2bf p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale[i], 1);
+                const v2bf p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale[i], 2);
+                const v2bf p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale[i], 3);
+                af[i] = v8bf{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[j], af[i], acc[i][j], 0, 0, 0);
+        }
+    };
+
+    // One K step: wait for this wave's share of the stage (WAIT = how many younger loads may still be in flight: the 14
+    // of the step after it), barrier (every wave's share has landed, and every wave has finished reading the stage about
+    // to be refilled), request step ks + 2 into the stage freed by step ks - 1, then compute.
+    // The scale loads write their registers when they land, not when they issue: a register whose value the compiler
+    // considers dead would be handed to something else and then overwritten by the late load.  So the steps after the
+    // main loop request nothing, and the final wait names every scale register.
+    auto step = [&](int ks, auto stage_c, auto issue_c, auto wait_c) {
+        constexpr int S = decltype(stage_c)::value;
+        constexpr int WAIT = decltype(wait_c)::value;
+        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(sc[S][0]), "+v"(sc[S][1]), "+v"(sc[S][2]), "+v"(sc[S][3]) : "n"(WAIT) : "memory");
+        __syncthreads();
+        if constexpr (decltype(issue_c)::value) issue(ks + 2, (S + 2) % kBigStages, sc[(S + 2) % kBigStages]);
+        compute(S, sc[S]);
+    };
+    using std::integral_constant;
+    issue(0, 0, sc[0]);
+    issue(1, 1, sc[1]);
+    int ks = 0;
+    for (; ks + 3 <= nk; ks += 3) {
+        step(ks, integral_constant<int, 0>{}, std::true_type{}, integral_constant<int, kBigLoads>{});
+        step(ks + 1, integral_constant<int, 1>{}, std::true_type{}, integral_constant<int, kBigLoads>{});
+        step(ks + 2, integral_constant<int, 2>{}, std::true_type{}, integral_constant<int, kBigLoads>{});
+    }
+    // two sets of loads are in flight here (steps ks and ks + 1, real or repeats)
+    if (ks < nk) step(ks, integral_constant<int, 0>{}, std::false_type{}, integral_constant<int, kBigLoads>{});
+    if (ks + 1 < nk) step(ks + 1, integral_constant<int, 1>{}, std::false_type{}, integral_constant<int, 0>{});
+    // direct-to-LDS loads must not outlive the workgroup's LDS allocation, nor scale loads their registers
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(sc[0][0]), "+v"(sc[0][1]), "+v"(sc[0][2]), "+v"(sc[0][3]), "+v"(sc[1][0]), "+v"(sc[1][1]), "+v"(sc[1][2]),
+                   "+v"(sc[1][3]), "+v"(sc[2][0]), "+v"(sc[2][1]), "+v"(sc[2][2]), "+v"(sc[2][3])
+                 :
+                 : "memory");
+
+    // epilogue: element e of block (i, j) is n = 8 (e/4) + 4 half + e%4 of the block, row m = lrow
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int64_t row = m0 + wm * 128 + i * 32 + lrow;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                const int64_t col = n0 + wn * 128 + j * 32 + 8 * qd + 4 * half;
+                if (row >= M || col >= N) continue;   // N % 4 == 0: the quad is inside or outside as a whole
+                const float v0 = acc[i][j][4 * qd] * alpha, v1 = acc[i][j][4 * qd + 1] * alpha;
+                const float v2 = acc[i][j][4 * qd + 2] * alpha, v3 = acc[i][j][4 * qd + 3] * alpha;
+                if constexpr (sizeof(OutT) == 2) {
+                    const v2bf p0 = __builtin_convertvector(v2f{v0, v1}, v2bf);
+                    const v2bf p1 = __builtin_convertvector(v2f{v2, v3}, v2bf);
+                    *reinterpret_cast<uint2*>(c + row * N + col) =
+                        make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
+                } else {
+                    *reinterpret_cast<float4*>(c + row * N + col) = make_float4(v0, v1, v2, v3);
+                }
+            }
+    }
+}
+
 }  // namespace
 
 bool gemm_fp4_bf16_nn_supported(int64_t M, int64_t N, int64_t K) {
@@ -227,6 +441,32 @@ hipError_t gemm_fp4_bf16_nn(const uint8_t* a_codes, const uint8_t* a_scales, con
                             float alpha, void* c, int c_dtype, hipStream_t stream) {
     if (M == 0 || N == 0) return hipSuccess;
     if (!gemm_fp4_bf16_nn_supported(M, N, K)) return hipErrorInvalidValue;
+    if (M >= kBM && N >= kBN) {
+        // at least one full 256 x 256 tile in each direction: the large-tile kernel
+        dim3 grid((unsigned)(((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN))), block(256);
+        static std::atomic<bool> allowed16[64], allowed32[64];
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        auto allow = [&](auto kern, std::atomic<bool>(&done)[64]) -> hipError_t {
+            if (dev >= 0 && dev < 64 && done[dev].load(std::memory_order_acquire)) return hipSuccess;
+            hipError_t r = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kBigSmem);
+            if (r == hipSuccess && dev >= 0 && dev < 64) done[dev].store(true, std::memory_order_release);
+            return r;
+        };
+        if (c_dtype == BF16) {
+            auto kern = gemm_fp4_bf16_nn_big_kernel<uint16_t>;
+            if ((e = allow(kern, allowed16)) != hipSuccess) return e;
+            kern<<<grid, block, kBigSmem, stream>>>(a_codes, a_scales, static_cast<const uint16_t*>(b), (int)M, (int)N, (int)K, alpha,
+                                                    static_cast<uint16_t*>(c));
+        } else {
+            auto kern = gemm_fp4_bf16_nn_big_kernel<float>;
+            if ((e = allow(kern, allowed32)) != hipSuccess) return e;
+            kern<<<grid, block, kBigSmem, stream>>>(a_codes, a_scales, static_cast<const uint16_t*>(b), (int)M, (int)N, (int)K, alpha,
+                                                    static_cast<float*>(c));
+        }
+        return hipGetLastError();
+    }
     dim3 grid((unsigned)(((M + kTM - 1) / kTM) * ((N + kTN - 1) / kTN))), block(256);
     if (c_dtype == BF16)
         gemm_fp4_bf16_nn_kernel<uint16_t><<<grid, block, kSmem, stream>>>(a_codes, a_scales, static_cast<const uint16_t*>(b), (int)M,

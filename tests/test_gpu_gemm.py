@@ -245,12 +245,14 @@ def test_fp4_bf16_product_against_fp64_matmul(oracle, K, M, N, K_):
     assert torch.equal(got16.cpu(), got32.cpu().to(torch.bfloat16))
 
 
-def test_fp4_bf16_product_bit_exact_when_sums_are_exact(oracle, K):
+@pytest.mark.parametrize("M,N,K_", [(192, 136, 448), (320, 264, 448), (512, 512, 64), (260, 256, 320)])
+def test_fp4_bf16_product_bit_exact_when_sums_are_exact(oracle, K, M, N, K_):
     """Random code bytes with one common scale against small integers: every partial sum is a multiple of 1/2 below 2^24,
-    so the fp32 result must equal the float64 product whatever order the contraction index is walked in."""
+    so the fp32 result must equal the float64 product whatever order the contraction index is walked in.  Shapes of the
+    128 x 128 kernel and of the 256 x 256 kernel (with tiles hanging over both edges, one to five K steps)."""
+    print(f"case fp4 x bf16 exact sums {M}x{N}x{K_}", flush=True)
     dev = torch.device("cuda:0")
     rng = np.random.default_rng(3)
-    M, N, K_ = 192, 136, 448
     ac = rng.integers(0, 256, (M, K_ // 2), dtype=np.uint8)
     as_ = np.full((M, K_ // 32), 127, dtype=np.uint8)
     b = torch.from_numpy(rng.integers(-8, 9, (K_, N)).astype(np.float32)).to(torch.bfloat16)
@@ -259,11 +261,13 @@ def test_fp4_bf16_product_bit_exact_when_sums_are_exact(oracle, K):
     assert np.array_equal(got.cpu().numpy().astype(np.float64), want)
 
 
-def test_fp4_bf16_product_selects_rows_and_columns(oracle, K):
+@pytest.mark.parametrize("M,N,K_", [(256, 128, 128), (512, 264, 256)])
+def test_fp4_bf16_product_selects_rows_and_columns(oracle, K, M, N, K_):
     """One +1.0 per row of A at a known k (every k of a K step occurs, per-group scales differ) returns row k of B times
-    the group's scale: pins the order in which lanes, matrix instructions and the transposing LDS read walk k."""
+    the group's scale: pins the order in which lanes, matrix instructions and the transposing LDS read walk k (both
+    kernels)."""
+    print(f"case fp4 x bf16 selection {M}x{N}x{K_}", flush=True)
     dev = torch.device("cuda:0")
-    M, N, K_ = 256, 128, 128
     ac = np.zeros((M, K_ // 2), dtype=np.uint8)
     as_ = (120 + (np.arange(M)[:, None] + np.arange(K_ // 32)[None, :]) % 12).astype(np.uint8)
     ks = [(m * 5 + 3) % K_ for m in range(M)]
