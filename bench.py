@@ -698,6 +698,34 @@ def reference_shapes(device):
     return out
 
 
+def gemm_shapes(device):
+    """The forward and grad-input products of every block linear of the two Llama configurations (32768 tokens), as chains
+    of launches on quest codes of Gaussian operands: duration, TFLOP/s, and the rate at which the bf16 output leaves --
+    with a short contraction a product is bound by writing its result, not by the matrix pipe."""
+    from quartet_amd import kernels as K
+    T = 32768
+    models = {"llama30m": [(640, 1920), (640, 640), (640, 3456), (1728, 640)],
+              "llama800m": [(1536, 4608), (1536, 1536), (1536, 8192), (4096, 1536)]}
+    out = {}
+    for name, linears in models.items():
+        rows = []
+        for I, O in linears:
+            for what, (M, N, Kd) in (("fwd", (T, O, I)), ("dgrad", (T, I, O))):
+                g = torch.Generator(device=device).manual_seed(M + N + Kd)
+                tiled = all(d % 128 == 0 and d >= 256 for d in (M, N, Kd))
+                a = torch.randn(M, Kd, generator=g, device=device).to(torch.bfloat16)
+                b = torch.randn(N, Kd, generator=g, device=device).to(torch.bfloat16)
+                ac, as_, _, _ = K.quantize_mxfp4(a, 32, None, K.QM_QUEST_RTN, tiled=tiled)
+                bc, bs, _, _ = K.quantize_mxfp4(b, 32, None, K.QM_QUEST_RTN, tiled=tiled)
+                del a, b
+                ms = sorted(time_kernel(lambda: K.gemm_mxfp4_tn(ac, as_, bc, bs, 1.0, torch.bfloat16, a_tiled=tiled, b_tiled=tiled),
+                                        reps=20) for _ in range(3))[1]
+                rows.append({"linear": f"{I}->{O}", "product": what, "shape": [M, N, Kd], "ms": round(ms, 4),
+                             "TFLOPs": round(2.0 * M * N * Kd / ms / 1e9, 1), "output_GBps": round(M * N * 2 / ms / 1e6, 1)})
+        out[name] = rows
+    return out
+
+
 def error_only_scheme_block(device):
     """The two gradient products of scheme "Q(E)W_Q(Et)X" at 8192 x 4096 x 4096: this build's FP4 x bf16 kernel on the
     packed Q(e) / Q(e^T) against the module path the reference takes (de-quantized bf16 Q(e), a transposed copy of e, two
@@ -813,6 +841,8 @@ def main():
     ap.add_argument("--reference-shapes", action="store_true",
                     help="also time the layer (and a bf16 linear layer, for the ratio) at the two shapes the reference's notebook "
                          "reports: 32768 tokens x 4096 x 4096 and x 1024 x 1024, forward and forward + backward")
+    ap.add_argument("--gemm-shapes", action="store_true",
+                    help="also time the forward and grad-input products of every block linear of the two Llama configurations")
     ap.add_argument("--library-gemm", action="store_true",
                     help="also time the vendor library's MXFP4 product (torch._scaled_mm) on the forward GEMM's shape, for context")
     args = ap.parse_args()
@@ -914,6 +944,8 @@ def main():
         result["quantizer_sweep"] = quantizer_sweep(device)
     if args.reference_shapes and "reference_shapes" not in result:
         result["reference_shapes"] = reference_shapes(device)
+    if args.gemm_shapes:
+        result["gemm_shapes"] = gemm_shapes(device)
     if args.library_gemm:
         result["library_gemm"] = library_gemm(device)
     if args.gemm_operand_content:

@@ -15,12 +15,12 @@
 // instruction needs.
 //
 // Three kernels, picked by shape in gemm_mxfp4_tn() at the end of the file:
-//   gemm_mxfp4_tn_big4_kernel  M, N multiples of 64 and >= 256, K % 512 == 0, or another multiple of 128 whose last block
-//                              of four K steps repeats (muted) at most a third as many steps as K has.  Persistent, 256x256
-//                              macro tile, 4 waves x 128x128, operands global -> LDS directly into a 4-stage ring,
-//                              scales in blocks of four K steps, row-major or tiled code bytes, optional split-K.
-//   gemm_mxfp4_tn_big_kernel   same tile for the remaining K % 128 == 0 (short K): one workgroup per tile, scales per
-//                              K step.
+//   gemm_mxfp4_tn_big4_kernel  M, N multiples of 64 and >= 256, K > 768 and K % 512 == 0, or another multiple of 128 whose
+//                              last block of four K steps repeats (muted) at most a third as many steps as K has.
+//                              Persistent, 256x256 macro tile, 4 waves x 128x128, operands global -> LDS directly into a
+//                              4-stage ring, scales in blocks of four K steps, row-major or tiled code bytes, optional split-K.
+//   gemm_mxfp4_tn_duo_kernel   same M, N, K % 128 == 0 and K <= 768: 256x128 tiles, two workgroups per CU hiding each
+//                              other's tile boundaries, scales per K step.
 //   gemm_mxfp4_tn_kernel       any M, N and K % 32 == 0: 128x128 macro tile, 4 waves x 64x64, operands staged
 //                              global -> registers -> LDS (rows padded from 64 to 80 bytes so the 16-byte fragment
 //                              reads of 16 consecutive rows hit 64 distinct banks), double buffered.
@@ -266,12 +266,7 @@ __device__ __forceinline__ void store_tile(const v16f& t, float alpha, OutT* __r
 
 constexpr int kBigM = 256, kBigN = 256;
 constexpr int kStages = 4;
-constexpr int kStageBytes = (kBigM + kBigN) * kRowBytes + (kBigM + kBigN) * 4;  // 32 KiB codes + 2 KiB scales
 constexpr int kBOff = kBigM * kRowBytes;
-constexpr int kSAOff = (kBigM + kBigN) * kRowBytes;
-constexpr int kSBOff = kSAOff + kBigM * 4;
-constexpr int kBigSmemBytes = kStages * kStageBytes;
-constexpr int kLoadsPerStep = 10;  // VMEM instructions per wave per K step
 
 // Tile order: workgroup ids are dealt round-robin to the 8 XCDs by the hardware; give each XCD a
 // contiguous run of tiles in an order that walks 4-row groups column by column, so the tiles that
@@ -290,43 +285,19 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
     tn = r / gm;
 }
 
-struct BigLoadPlan {
-    const uint8_t* a;   // this lane's A source for wave-load 0 at K step 0 (+ j * 16 rows, + ks * 64 bytes)
-    const uint8_t* b;
-    const uint8_t* sa;  // this lane's A scale dword source at K step 0 (+ ks * 4 bytes)
-    const uint8_t* sb;
-    int64_t row16_bytes;   // 16 rows of codes
-    int kstep_a, kstep_b;  // bytes from one K step to the next in this lane's source: 64 row-major, 1024 tiled
-    uint32_t lds_codes;    // wave-uniform LDS byte address of this wave's first A wave-load in stage 0
-    uint32_t lds_scales;   // likewise for its A scale wave-load
-};
-
 // global -> LDS without passing through registers.  Written as inline assembly on purpose: the
 // compiler's wait-count insertion treats every LDS read as possibly aliasing an outstanding
 // global_load_lds and would drain all loads (vmcnt(0)) before each fragment read, which defeats the
 // prefetch ring; the kernel waits explicitly for the one tile it is about to read instead.
 // LDS destination = lds_base (wave-uniform, via M0) + lane * size.
-__device__ __forceinline__ void load_lds_b128(const uint8_t* gsrc, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gsrc), "s"(lds_base));
-}
-// same, addressed as uniform 64-bit base (SGPR pair) + per-lane 32-bit byte offset: no 64-bit VGPR address math
+// addressed as uniform 64-bit base (SGPR pair) + per-lane 32-bit byte offset: no 64-bit VGPR address math
 __device__ __forceinline__ void load_lds_b128_s(const uint8_t* base, uint32_t lane_off, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(lds_base));
 }
+// s_waitcnt immediate that waits for the vector-memory counter only
+constexpr int vmcnt_imm(int n) { return 0x0f70 | (n & 0xf) | ((n >> 4) << 14); }
 __device__ __forceinline__ void load_lds_b32(const uint8_t* gsrc, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gsrc), "s"(lds_base));
-}
-
-// issue the ten loads of K step ks into ring stage `stage`
-__device__ __forceinline__ void big_issue_loads(const BigLoadPlan& p, int stage, int ks) {
-    const uint32_t base = p.lds_codes + stage * kStageBytes;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        load_lds_b128(p.a + j * p.row16_bytes + ks * p.kstep_a, base + j * 1024);
-        load_lds_b128(p.b + j * p.row16_bytes + ks * p.kstep_b, base + kBOff + j * 1024);
-    }
-    load_lds_b32(p.sa + ks * 4, p.lds_scales + stage * kStageBytes);
-    load_lds_b32(p.sb + ks * 4, p.lds_scales + stage * kStageBytes + (kSBOff - kSAOff));
 }
 
 struct SubFrags {
@@ -340,14 +311,6 @@ __device__ __forceinline__ void big_read_sub(const uint8_t* __restrict__ stage, 
         f.a[i] = *reinterpret_cast<const uint4*>(stage + a_off + i * 32 * kRowBytes);
         f.b[i] = *reinterpret_cast<const uint4*>(stage + kBOff + b_off + i * 32 * kRowBytes);
     }
-}
-
-// Scales in LDS: per operand, dword [(row / 128) * 32 + row % 32][(row / 32) % 4] is the row's four E8M0
-// bytes of this K step, so one 16-byte read fetches the scale dwords of a lane's four tiles.
-__device__ __forceinline__ void big_read_scales(const uint8_t* __restrict__ stage, int a_off, int b_off, uint4& sa4,
-                                                uint4& sb4) {
-    sa4 = *reinterpret_cast<const uint4*>(stage + kSAOff + a_off);
-    sb4 = *reinterpret_cast<const uint4*>(stage + kSBOff + b_off);
 }
 
 // SWAP = false: A rows become result rows.  SWAP = true: B's rows (n) are fed as the MFMA's first operand and
@@ -378,54 +341,6 @@ __device__ __forceinline__ void big_mfma_sub(const SubFrags& f, const uint32_t (
     }
 }
 
-// Epilogue of the 256x256 kernels.  fp32: direct stores (acc element e of tile (i,j) is row 8*(e/4)+4*half+e%4,
-// column lane%32).  bf16 (SWAP layout: element e is n = 8*(e/4)+4*half+e%4 of m = lane%32): each wave packs its
-// 128x128 block into its own LDS region (rows of 256 bytes, pitch 272 so the 8-byte writes of 32 consecutive
-// rows spread over the banks), then writes it out as 16-byte pieces, four full 256-byte row segments per
-// instruction.  The LDS used is the operand ring, free once every wave has passed the final barrier.
-constexpr int kEpiPitch = 272;
-// rows_valid / cols_valid: how many of the wave's 128 rows / columns lie inside the matrix (multiples of 64, may be
-// <= 0 for a wave that hangs over the edge of M or N entirely); everything beyond is computed on clamped operand
-// rows and dropped here.
-template <typename OutT>
-__device__ __forceinline__ void big_epilogue(v16f (&acc)[4][4], float alpha, OutT* __restrict__ c, int64_t m0, int64_t n0,
-                                             int64_t N, int wm, int wn, int wave, int lane, uint8_t* smem_bytes,
-                                             int rows_valid, int cols_valid) {
-    const int lrow = lane & 31, half = lane >> 5;
-    if constexpr (sizeof(OutT) == 4) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (i * 32 < rows_valid && j * 32 < cols_valid)
-                    store_tile<OutT>(acc[i][j], alpha, c, m0 + wm * 128 + i * 32, n0 + wn * 128 + j * 32 + lrow, N, half);
-    } else {
-        uint8_t* region = smem_bytes + wave * (128 * kEpiPitch);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    const v16f& t = acc[i][j];
-                    const v2bf p0 = __builtin_convertvector(v2f{t[4 * b] * alpha, t[4 * b + 1] * alpha}, v2bf);
-                    const v2bf p1 = __builtin_convertvector(v2f{t[4 * b + 2] * alpha, t[4 * b + 3] * alpha}, v2bf);
-                    *reinterpret_cast<uint2*>(region + (i * 32 + lrow) * kEpiPitch + (j * 32 + 8 * b + 4 * half) * 2) =
-                        make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
-                }
-        // the region is private to the wave: its own writes are ordered before its own reads
-        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-        const int chunk = lane & 15, rsub = lane >> 4;
-        uint8_t* cbase = reinterpret_cast<uint8_t*>(c + (m0 + wm * 128) * N + n0 + wn * 128) + chunk * 16;
-#pragma unroll 8
-        for (int r4 = 0; r4 < 32; ++r4) {
-            const int row = r4 * 4 + rsub;
-            const uint4 v = *reinterpret_cast<const uint4*>(region + row * kEpiPitch + chunk * 16);
-            if (r4 * 4 < rows_valid && chunk * 8 < cols_valid) *reinterpret_cast<uint4*>(cbase + (int64_t)row * N * 2) = v;
-        }
-    }
-}
-
 // one MFMA, then one memory instruction of the given class, n times: keeps the matrix pipe fed while the
 // wave issues its LDS / VMEM instructions
 #define QM_SCHED_PAIR(mask, n)                                   \
@@ -434,129 +349,229 @@ __device__ __forceinline__ void big_epilogue(v16f (&acc)[4][4], float alpha, Out
         __builtin_amdgcn_sched_group_barrier((mask), 1, 0);      \
     }
 
-// Pipeline, K step ks (tile ks lives in ring stage ks % 4); one barrier per step:
-//   phase 1: read sub-step-1 fragments of tile ks | 16 MFMAs on its sub-step-0 fragments (in registers);
-//   wait until this wave's loads of tile ks+1 have landed, barrier (tile ks+1 visible to all, stage ks%4 free);
-//   phase 2: request tile ks+4 into stage ks%4; read scales and sub-step-0 fragments of tile ks+1 |
-//            16 MFMAs on sub-step 1 of tile ks (in the K % 512 kernel below the requests and reads are dealt out
-//            two each per four MFMAs: a wave that issues its eight requests in one clump stalls behind the others').
+// ---- two workgroups per CU: 256 x 128 tiles for short contractions -------------------------------------------------
+// With a short K the tile boundary dominates: the 256 x 256 kernels spend about 7.5 k cycles per tile converting, staging
+// and storing the result while no matrix instruction runs, against 1.3 k cycles per K step.  Here a workgroup owns a
+// 256 x 128 tile with four waves of 128 x 64 (128 accumulator registers, at most 256 registers per wave), so a SIMD holds
+// one wave of each of two workgroups: while one of them waits at its barrier, requests operands, or converts and stores
+// its tile, the other's matrix instructions keep the pipe busy.  The price is 1.5 x the operand traffic per flop (LDS
+// fragment reads and global -> LDS bytes), which is why long contractions stay on the 256 x 256 kernel.
+// Three-stage ring per workgroup (3 x 25.5 KiB: codes of 256 + 128 rows and one scale dword per row and K step); the
+// ring doubles as the epilogue's staging area, so nothing is prefetched across tiles -- the neighbour workgroup covers
+// the gap.  Persistent: the grid is two workgroups per CU.  M, N multiples of 64, M >= 256, N >= 128, K % 128 == 0.
+constexpr int kDuoM = 256, kDuoN = 128, kDuoStages = 3;
+constexpr int kDuoBOff = kDuoM * kRowBytes;                                   // 16 KiB of A codes
+constexpr int kDuoSAOff = (kDuoM + kDuoN) * kRowBytes;                        // 24 KiB of codes
+constexpr int kDuoSBOff = kDuoSAOff + kDuoM * 4;
+constexpr int kDuoStageBytes = kDuoSBOff + kDuoN * 4;                         // 25.5 KiB
+constexpr int kDuoSmemBytes = kDuoStages * kDuoStageBytes;                    // 76.5 KiB
+constexpr int kDuoEpiPitch = 144;   // bytes per staged row of 64 bf16: 128 rows x 144 B = 18 KiB per wave
+#ifndef QM_DUO_MAX_K
+#define QM_DUO_MAX_K 768
+#endif
+constexpr int kDuoMaxK = QM_DUO_MAX_K;  // longest contraction served by this kernel
+constexpr int kDuoLoads = 8;        // VMEM instructions per wave per K step: 4 (A) + 2 (B) + 2 (scales)
+static_assert(4 * 128 * kDuoEpiPitch <= kDuoSmemBytes, "the epilogue stages through the operand ring");
+
+struct DuoFrags {
+    uint4 a[4], b[2];
+};
+struct DuoPlan {
+    const uint8_t* a;   // uniform: this wave's 64 A rows of the tile, K step 0
+    const uint8_t* b;   // uniform: this wave's 32 B rows
+    const uint8_t* sa;  // this lane's A scale dword source at K step 0 (+ ks * 4 bytes)
+    const uint8_t* sb;
+    int64_t row16_bytes;
+    uint32_t lane_codes_a, lane_codes_b;
+    int kstep_a, kstep_b;
+    uint32_t lds_a, lds_b, lds_sa, lds_sb;  // wave-uniform LDS addresses (stage 0)
+};
+__device__ __forceinline__ void duo_issue(const DuoPlan& p, int stage, int ks) {
+    const uint32_t off = (uint32_t)stage * kDuoStageBytes;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) load_lds_b128_s(p.a + j * p.row16_bytes + ks * p.kstep_a, p.lane_codes_a, p.lds_a + off + j * 1024);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) load_lds_b128_s(p.b + j * p.row16_bytes + ks * p.kstep_b, p.lane_codes_b, p.lds_b + off + j * 1024);
+    load_lds_b32(p.sa + ks * 4, p.lds_sa + off);
+    load_lds_b32(p.sb + ks * 4, p.lds_sb + off);
+}
+__device__ __forceinline__ void duo_read_sub(const uint8_t* __restrict__ stage, int a_off, int b_off, DuoFrags& f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f.a[i] = *reinterpret_cast<const uint4*>(stage + a_off + i * 32 * kRowBytes);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) f.b[j] = *reinterpret_cast<const uint4*>(stage + b_off + j * 32 * kRowBytes);
+}
+template <int SUB, bool SWAP, bool ZERO>
+__device__ __forceinline__ void duo_mfma_sub(const DuoFrags& f, const uint32_t (&sca)[4], const uint32_t (&scb)[2], v16f (&acc)[4][2]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const v8i av = v8i{(int)f.a[i].x, (int)f.a[i].y, (int)f.a[i].z, (int)f.a[i].w, 0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const v8i bv = v8i{(int)f.b[j].x, (int)f.b[j].y, (int)f.b[j].z, (int)f.b[j].w, 0, 0, 0, 0};
+            v16f cin;
+            if constexpr (ZERO) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) cin[e] = 0.0f;
+            } else {
+                cin = acc[i][j];
+            }
+            if constexpr (SWAP)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, cin, 4, 4, SUB, (int)scb[j], SUB, (int)sca[i]);
+            else
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, cin, 4, 4, SUB, (int)sca[i], SUB, (int)scb[j]);
+        }
+    }
+}
+
 template <typename OutT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mxfp4_tn_big_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_mxfp4_tn_duo_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ b_codes,
-    const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c, int a_tiled,
-    int b_tiled) {
+    const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c, int a_tiled, int b_tiled) {
     extern __shared__ uint32_t smem[];
     uint8_t* smem_bytes = reinterpret_cast<uint8_t*>(smem);
     const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)smem;
+    constexpr bool SWAP = sizeof(OutT) == 2;
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     const int lrow = lane & 31, half = lane >> 5;
-    int tm, tn;
-    tile_of_block((int)blockIdx.x, (M + kBigM - 1) / kBigM, (N + kBigN - 1) / kBigN, tm, tn);
-    const int64_t m0 = (int64_t)tm * kBigM, n0 = (int64_t)tn * kBigN;
+    const int tiles_m = (M + kDuoM - 1) / kDuoM, tiles_n = (N + kDuoN - 1) / kDuoN, total = tiles_m * tiles_n;
     const int code_pitch = K / 2, groups = K / 32;
     const int nk = K / kBK;
-
-    BigLoadPlan plan;
-    {
-        // codes: wave-load j of wave w fills LDS rows (w*4+j)*16 .. +15; lane l -> row + l/4, slot l%4
-        const int row = wave * 64 + (lane >> 2);
-        const int cv = (lane & 3) ^ ((row >> 2) & 3);
-        // tiled codes: the wave-load's 16 rows x 64 bytes are one 1 KiB tile; same (row, swizzled slot) pick inside it
-        const int trow = wave * 64;  // first row of this wave's four wave-loads
-        const int tile_off = (lane >> 2) * 64 + cv * 16;
-        // M and N are multiples of 64: a wave's 64-row share of a panel is inside the matrix or outside it as a whole;
-        // an outside share reads the matrix's last 64 rows instead (its products are dropped by the epilogue)
-        const int64_t ma = m0 + trow < M ? m0 + trow : (int64_t)M - 64;
-        const int64_t nb = n0 + trow < N ? n0 + trow : (int64_t)N - 64;
-        plan.a = a_tiled ? a_codes + ma * code_pitch + tile_off : a_codes + (ma + (lane >> 2)) * code_pitch + cv * 16;
-        plan.b = b_tiled ? b_codes + nb * code_pitch + tile_off : b_codes + (nb + (lane >> 2)) * code_pitch + cv * 16;
-        plan.kstep_a = a_tiled ? 1024 : kRowBytes;
-        plan.kstep_b = b_tiled ? 1024 : kRowBytes;
-        plan.row16_bytes = (int64_t)16 * code_pitch;
-        // scales: LDS dword p = wave*64 + lane holds operand row (p>>7)*128 + (p&3)*32 + ((p>>2)&31)
-        const int p = wave * 64 + lane;
-        const int srow = (p >> 7) * 128 + (p & 3) * 32 + ((p >> 2) & 31);
-        plan.sa = a_scales + (m0 + srow < M ? m0 + srow : (int64_t)M - 1) * groups;
-        plan.sb = b_scales + (n0 + srow < N ? n0 + srow : (int64_t)N - 1) * groups;
-        plan.lds_codes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + wave * 4096));
-        plan.lds_scales = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + kSAOff + wave * 256));
-    }
-
-    v16f acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
     const int swz = (lrow >> 2) & 3;
     const int a_off0 = (wm * 128 + lrow) * kRowBytes + (((2 * half) ^ swz) * 16);
     const int a_off1 = (wm * 128 + lrow) * kRowBytes + (((2 * half + 1) ^ swz) * 16);
-    const int b_off0 = (wn * 128 + lrow) * kRowBytes + (((2 * half) ^ swz) * 16);
-    const int b_off1 = (wn * 128 + lrow) * kRowBytes + (((2 * half + 1) ^ swz) * 16);
-    const int a_sc_off = (wm * 32 + lrow) * 16, b_sc_off = (wn * 32 + lrow) * 16;
+    const int b_off0 = kDuoBOff + (wn * 64 + lrow) * kRowBytes + (((2 * half) ^ swz) * 16);
+    const int b_off1 = kDuoBOff + (wn * 64 + lrow) * kRowBytes + (((2 * half + 1) ^ swz) * 16);
+    // scales in LDS: A dword p holds row (p >> 7) * 128 + (p & 3) * 32 + ((p >> 2) & 31), so one 16-byte read fetches the
+    // scale dwords of a lane's four A tiles; B dword p holds row (p >> 6) * 64 + (p & 1) * 32 + ((p >> 1) & 31): one 8-byte read
+    const int a_sc_off = kDuoSAOff + (wm * 32 + lrow) * 16;
+    const int b_sc_off = kDuoSBOff + (wn * 32 + lrow) * 8;
     const int sh = 16 * half;
 
-    // prologue: request the first four tiles, wait for tile 0
-#pragma unroll
-    for (int t = 0; t < kStages; ++t)
-        if (t < nk) big_issue_loads(plan, t, t);
-    if (nk >= kStages) __builtin_amdgcn_s_waitcnt(0x0f70 | (3 * kLoadsPerStep & 0xf) | (((3 * kLoadsPerStep) >> 4) << 14));
-    else __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-    __syncthreads();
-    SubFrags f0, f1;
-    uint4 sa4, sb4;
-    big_read_sub(smem_bytes, a_off0, b_off0, f0);
-    big_read_scales(smem_bytes, a_sc_off, b_sc_off, sa4, sb4);
-
-    int ks = 0;
-    // steady state: tiles up to ks+4 exist; no conditionals inside the scheduling regions
-    for (; ks + kStages < nk; ++ks) {
-        const uint8_t* cur = smem_bytes + (ks & 3) * kStageBytes;
-        const uint8_t* nxt = smem_bytes + ((ks + 1) & 3) * kStageBytes;
-        const uint32_t sca[4] = {sa4.x >> sh, sa4.y >> sh, sa4.z >> sh, sa4.w >> sh};
-        const uint32_t scb[4] = {sb4.x >> sh, sb4.y >> sh, sb4.z >> sh, sb4.w >> sh};
-        big_read_sub(cur, a_off1, b_off1, f1);
-        big_mfma_sub<0, sizeof(OutT) == 2>(f0, sca, scb, acc);
-        QM_SCHED_PAIR(0x100, 8)
-        __builtin_amdgcn_sched_barrier(0);
-        // this wave's loads of tile ks+1 are older than those of tiles ks+2, ks+3: allow 20 outstanding
-        __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * kLoadsPerStep & 0xf) | (((2 * kLoadsPerStep) >> 4) << 14));
-        __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
-        big_read_scales(nxt, a_sc_off, b_sc_off, sa4, sb4);
-        big_read_sub(nxt, a_off0, b_off0, f0);
-        big_issue_loads(plan, ks & 3, ks + kStages);
-        big_mfma_sub<1, sizeof(OutT) == 2>(f1, sca, scb, acc);
-        QM_SCHED_PAIR(0x100, 10)
-        __builtin_amdgcn_sched_barrier(0);
+    DuoPlan plan;
+    plan.row16_bytes = (int64_t)16 * code_pitch;
+    {
+        const int prow = lane >> 2;
+        const int pcv = (lane & 3) ^ ((prow >> 2) & 3);
+        const uint32_t rowmajor_off = (uint32_t)(prow * code_pitch + pcv * 16);
+        const uint32_t tiled_off = (uint32_t)(prow * 64 + pcv * 16);
+        plan.lane_codes_a = a_tiled ? tiled_off : rowmajor_off;
+        plan.lane_codes_b = b_tiled ? tiled_off : rowmajor_off;
+        plan.kstep_a = a_tiled ? 1024 : kRowBytes;
+        plan.kstep_b = b_tiled ? 1024 : kRowBytes;
+        plan.lds_a = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + wave * 4096));
+        plan.lds_b = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + kDuoBOff + wave * 2048));
+        plan.lds_sa = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + kDuoSAOff + wave * 256));
+        // 128 B scale dwords: waves 2 and 3 repeat the requests of waves 0 and 1 (same bytes to the same place), which
+        // keeps every wave's count of outstanding loads the same
+        plan.lds_sb = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + kDuoSBOff + (wave & 1) * 256));
     }
-    // drain: the last (up to four) tiles, nothing left to request
-    for (; ks < nk; ++ks) {
-        const uint8_t* cur = smem_bytes + (ks & 3) * kStageBytes;
-        const uint8_t* nxt = smem_bytes + ((ks + 1) & 3) * kStageBytes;
-        const bool has_next = ks + 1 < nk;
-        const uint32_t sca[4] = {sa4.x >> sh, sa4.y >> sh, sa4.z >> sh, sa4.w >> sh};
-        const uint32_t scb[4] = {sb4.x >> sh, sb4.y >> sh, sb4.z >> sh, sb4.w >> sh};
-        big_read_sub(cur, a_off1, b_off1, f1);
-        big_mfma_sub<0, sizeof(OutT) == 2>(f0, sca, scb, acc);
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): everything requested has landed
-        __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
-        if (has_next) {
-            big_read_scales(nxt, a_sc_off, b_sc_off, sa4, sb4);
-            big_read_sub(nxt, a_off0, b_off0, f0);
+    // operand rows behind the scale dwords this lane requests
+    const int pa = wave * 64 + lane, pb = (wave & 1) * 64 + lane;
+    const int srow_a = (pa >> 7) * 128 + (pa & 3) * 32 + ((pa >> 2) & 31);
+    const int srow_b = (pb >> 6) * 64 + (pb & 1) * 32 + ((pb >> 1) & 31);
+
+    for (int t = (int)blockIdx.x; t < total; t += (int)gridDim.x) {
+        int tm, tn;
+        tile_of_block(t, tiles_m, tiles_n, tm, tn);
+        const int64_t m0 = (int64_t)tm * kDuoM, n0 = (int64_t)tn * kDuoN;
+        {
+            // M and N are multiples of 64 (32 for a wave's share of B): a wave's share of a panel lies inside the matrix or
+            // outside it as a whole; an outside share reads the matrix's last rows instead (its products are dropped below)
+            int64_t ma = m0 + wave * 64, nb = n0 + wave * 32;
+            ma = ma < M ? ma : (int64_t)M - 64;
+            nb = nb < N ? nb : (int64_t)N - 32;
+            plan.a = a_codes + ma * code_pitch;
+            plan.b = b_codes + nb * code_pitch;
+            plan.sa = a_scales + (m0 + srow_a < M ? m0 + srow_a : (int64_t)M - 1) * groups;
+            plan.sb = b_scales + (n0 + srow_b < N ? n0 + srow_b : (int64_t)N - 1) * groups;
         }
-        big_mfma_sub<1, sizeof(OutT) == 2>(f1, sca, scb, acc);
-    }
+        const int rows_valid = (int)(M - m0) - wm * 128, cols_valid = (int)(N - n0) - wn * 64;
 
-    __syncthreads();  // every wave has finished reading the operand ring: it becomes the epilogue stage
-    big_epilogue<OutT>(acc, alpha, c, m0, n0, N, wm, wn, wave, lane, smem_bytes, (int)(M - m0) - wm * 128,
-                       (int)(N - n0) - wn * 128);
+        duo_issue(plan, 0, 0);
+        duo_issue(plan, 1, nk > 1 ? 1 : 0);
+        duo_issue(plan, 2, nk > 2 ? 2 : nk - 1);
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(2 * kDuoLoads));  // step 0 is in; steps 1, 2 may be pending
+        __syncthreads();
+        DuoFrags f0, f1;
+        uint4 sa4 = *reinterpret_cast<const uint4*>(smem_bytes + a_sc_off);
+        uint2 sb2 = *reinterpret_cast<const uint2*>(smem_bytes + b_sc_off);
+        duo_read_sub(smem_bytes, a_off0, b_off0, f0);
+
+        v16f acc[4][2];
+        int stage = 0;
+        // one K step: `stage` is the ring slot it consumes and then refills with step s + 3
+        auto step = [&](auto first_tag, int s) {
+            constexpr bool FIRST = decltype(first_tag)::value;
+            const int nstage = stage == kDuoStages - 1 ? 0 : stage + 1;
+            const uint8_t* cur = smem_bytes + stage * kDuoStageBytes;
+            const uint8_t* nxt = smem_bytes + nstage * kDuoStageBytes;
+            const uint32_t sca[4] = {__builtin_amdgcn_ubfe(sa4.x, (uint32_t)sh, 16u), __builtin_amdgcn_ubfe(sa4.y, (uint32_t)sh, 16u),
+                                     __builtin_amdgcn_ubfe(sa4.z, (uint32_t)sh, 16u), __builtin_amdgcn_ubfe(sa4.w, (uint32_t)sh, 16u)};
+            const uint32_t scb[2] = {__builtin_amdgcn_ubfe(sb2.x, (uint32_t)sh, 16u), __builtin_amdgcn_ubfe(sb2.y, (uint32_t)sh, 16u)};
+            duo_read_sub(cur, a_off1, b_off1, f1);
+            duo_mfma_sub<0, SWAP, FIRST>(f0, sca, scb, acc);
+            QM_SCHED_PAIR(0x100, 6)
+            __builtin_amdgcn_sched_barrier(0);
+            // younger than the loads of step s + 1: those of step s + 2
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(kDuoLoads));
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            // past the end: a repeat nobody reads keeps the counts of outstanding loads uniform
+            duo_issue(plan, stage, s + 3 < nk ? s + 3 : nk - 1);
+            sa4 = *reinterpret_cast<const uint4*>(nxt + a_sc_off);
+            sb2 = *reinterpret_cast<const uint2*>(nxt + b_sc_off);
+            duo_read_sub(nxt, a_off0, b_off0, f0);
+            duo_mfma_sub<1, SWAP, false>(f1, sca, scb, acc);
+            QM_SCHED_PAIR(0x100, 6)
+            __builtin_amdgcn_sched_barrier(0);
+            stage = nstage;
+        };
+        step(std::true_type{}, 0);
+        for (int ks = 1; ks < nk; ++ks) step(std::false_type{}, ks);
+        // every request has landed and every wave has read its last fragments: the ring becomes the staging area
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        __syncthreads();
+        if constexpr (SWAP) {
+            uint8_t* region = smem_bytes + wave * (128 * kDuoEpiPitch);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        const v16f& v = acc[i][j];
+                        const v2bf p0 = __builtin_convertvector(v2f{v[4 * b] * alpha, v[4 * b + 1] * alpha}, v2bf);
+                        const v2bf p1 = __builtin_convertvector(v2f{v[4 * b + 2] * alpha, v[4 * b + 3] * alpha}, v2bf);
+                        *reinterpret_cast<uint2*>(region + (i * 32 + lrow) * kDuoEpiPitch + (j * 32 + 8 * b + 4 * half) * 2) =
+                            make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
+                    }
+            // the region is private to the wave; LDS operations of one wave complete in order
+            const int chunk = lane & 7, rsub = lane >> 3;
+            uint8_t* out = reinterpret_cast<uint8_t*>(reinterpret_cast<uint16_t*>(c) + (m0 + wm * 128 + rsub) * N + n0 + wn * 64) + chunk * 16;
+            const int64_t pitch8 = (int64_t)N * 16;  // eight rows of bf16
+            if (cols_valid > 0) {
+#pragma unroll
+                for (int r8 = 0; r8 < 16; ++r8) {
+                    const uint4 v = *reinterpret_cast<const uint4*>(region + (r8 * 8 + rsub) * kDuoEpiPitch + chunk * 16);
+                    typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+                    if (r8 * 8 < rows_valid) __builtin_nontemporal_store(u4v{v.x, v.y, v.z, v.w}, reinterpret_cast<u4v*>(out + r8 * pitch8));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    if (i * 32 < rows_valid && j * 32 < cols_valid)
+                        store_tile<OutT>(acc[i][j], alpha, c, m0 + wm * 128 + i * 32, n0 + wn * 64 + j * 32 + lrow, N, half);
+        }
+        __syncthreads();  // the staging area is the next tile's ring
+    }
 }
 
 // ---- persistent variant: scales travel in blocks of four K steps ------------------------------------
@@ -629,7 +644,6 @@ __device__ __forceinline__ uint32_t pick(const uint4& v) {
     return Q == 0 ? v.x : (Q == 1 ? v.y : (Q == 2 ? v.z : v.w));
 }
 
-constexpr int vmcnt_imm(int n) { return 0x0f70 | (n & 0xf) | ((n >> 4) << 14); }
 
 struct Big4State {
     SubFrags f0, f1;
@@ -1048,16 +1062,18 @@ hipError_t launch_big4(const uint8_t* a_codes, const uint8_t* a_scales, const ui
 }
 
 template <typename OutT>
-hipError_t launch_big(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
-                      const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_tiled,
-                      int b_tiled, hipStream_t stream) {
-    auto kern = gemm_mxfp4_tn_big_kernel<OutT>;
+hipError_t launch_duo(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
+                      int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_tiled, int b_tiled, int cus, hipStream_t stream) {
+    auto kern = gemm_mxfp4_tn_duo_kernel<OutT>;
     static std::atomic<bool> lds_allowed[kMaxDevices];
-    hipError_t e = allow_dynamic_lds(kern, kBigSmemBytes, lds_allowed);
+    hipError_t e = allow_dynamic_lds(kern, kDuoSmemBytes, lds_allowed);
     if (e != hipSuccess) return e;
-    dim3 grid((unsigned)(((M + kBigM - 1) / kBigM) * ((N + kBigN - 1) / kBigN))), block(256);
-    kern<<<grid, block, kBigSmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
-                                                 reinterpret_cast<OutT*>(c), a_tiled, b_tiled);
+    const int64_t tiles = ((M + kDuoM - 1) / kDuoM) * ((N + kDuoN - 1) / kDuoN);
+    // two workgroups per CU, and a grid that is a multiple of 8 so that tile t and t + grid land on the same XCD
+    int64_t g = tiles < 2 * cus ? tiles : 2 * cus;
+    if (g > 8) g -= g % 8;
+    kern<<<dim3((unsigned)g), dim3(256), kDuoSmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
+                                                                  reinterpret_cast<OutT*>(c), a_tiled, b_tiled);
     return hipGetLastError();
 }
 
@@ -1129,7 +1145,7 @@ bool gemm_supports_tiled(int64_t M, int64_t N, int64_t K) {
 
 // bytes of scratch with which gemm_mxfp4_tn cuts this shape into K ranges (0: it would not)
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    if (!gemm_supports_tiled(M, N, K) || K % 512) return 0;
+    if (!gemm_supports_tiled(M, N, K) || K % 512 || K <= kDuoMaxK) return 0;
     const int sp = choose_splits(M, N, K, device_cus());
     return sp > 1 ? (size_t)sp * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
@@ -1143,11 +1159,20 @@ hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const 
     if ((at || bt) && !big_ok) return hipErrorInvalidValue;
     // The persistent kernel walks K in blocks of four steps: K % 512 == 0 directly (scale rows are then 16-byte aligned
     // like their base), other multiples of 128 with up to three muted steps in the last block when those are at most a
-    // third of the real ones (measured: K = 1152 and 1664 gain 3-5 % over the one-tile-per-workgroup kernel, K = 640
-    // gains nothing); their 16-byte scale requests start at 4-byte aligned addresses
+    // third of the real ones (K = 1152 and 1664 gain 3-5 % over a kernel without muted steps); their 16-byte scale
+    // requests start at 4-byte aligned addresses.  Every multiple of 128 above 768 qualifies; up to 768 the contraction is
+    // so short that the tile boundary dominates and the two-workgroups-per-CU kernel is faster (measured at 32768 tokens:
+    // 640 x 640 15 against 23 us, 3456 x 640 70 against 82 us; at K = 1536 it is 13-25 % slower than the persistent kernel).
     const int64_t nk_real = K / kBK, nk_pad = (nk_real + 3) & ~(int64_t)3;
     const bool persistent_ok = K % 512 == 0 ? ((reinterpret_cast<uintptr_t>(a_scales) | reinterpret_cast<uintptr_t>(b_scales)) & 15) == 0
                                             : (nk_real >= 4 && (nk_pad - nk_real) * 3 <= nk_real);
+    if (big_ok && (K <= kDuoMaxK || !persistent_ok)) {
+        // short contraction: two 256 x 128 workgroups per CU hide each other's tile boundaries (also the fallback for scale
+        // arrays that are not 16-byte aligned, which the persistent kernel's 16-byte scale requests need when K % 512 == 0)
+        const int cus = device_cus();
+        if (c_dtype == BF16) return launch_duo<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, cus, stream);
+        return launch_duo<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, cus, stream);
+    }
     if (big_ok && persistent_ok) {
         const int cus = device_cus();
         int sp = workspace && K % 512 == 0 ? choose_splits(M, N, K, cus) : 1;  // K ranges are whole blocks of four steps
@@ -1166,10 +1191,6 @@ hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const 
         }
         if (c_dtype == BF16) return launch_big4<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, 1, cus, stream);
         return launch_big4<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, 1, cus, stream);
-    }
-    if (big_ok) {
-        if (c_dtype == BF16) return launch_big<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, stream);
-        return launch_big<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, stream);
     }
     return launch_gemm<128, 128, 64, 64>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, c_dtype, stream);
 }

@@ -170,16 +170,20 @@ def test_transposed_and_requantize_column_slices(oracle, K, data):
         assert np.array_equal(to_oracle(xts[c0:c0 + 32]), ref["scales"]), c0
 
 
-def _random_operand(K, rows, cols, seed, mode, dev):
-    """A packed [rows, cols] operand (tiled codes) quantized from seeded Gaussian data generated on the GPU."""
+def _random_operand(K, rows, cols, seed, mode, dev, tiled=True):
+    """A packed [rows, cols] operand (tiled codes unless told otherwise) quantized from seeded Gaussian data generated on
+    the GPU."""
     gd = torch.Generator(device=dev).manual_seed(seed)
     t = torch.randn(rows, cols, generator=gd, device=dev).to(torch.bfloat16)
-    codes, scales, _, _ = K.quantize_mxfp4(t, 32, None, mode, tiled=True, seed=seed)
+    codes, scales, _, _ = K.quantize_mxfp4(t, 32, None, mode, tiled=tiled, seed=seed)
     return codes, scales
 
 
 # the three products of the isolated layer at out = 4096 and out = 11008 (forward, grad-input, grad-weight: M x N x K)
 GEMM_SHAPES = [(T, 4096, I), (4096, I, T), (T, 11008, I), (T, I, 11008), (11008, I, T)]
+# forward / grad-input products of the two Llama configurations (32768 tokens): short contractions on the 256 x 128
+# kernel (K = 640 and 1536, with N = 1728 hanging over a tile edge), K = 1728 (not a multiple of 128) on the generic one
+GEMM_SHAPES += [(32768, 3456, 640), (32768, 1728, 640), (32768, 640, 1728), (32768, 4608, 1536), (32768, 640, 1920)]
 
 
 @pytest.mark.parametrize("M,N,Kdim", GEMM_SHAPES)
@@ -193,23 +197,25 @@ def test_gemm_rows_and_sample(oracle, K, M, N, Kdim):
     absmax = Kdim == T
     mode = K.QM_ABSMAX_RTN if absmax else K.QM_QUEST_RTN
     post = float(oracle.FOUR_THIRDS) if absmax else 1.0
-    ac, as_ = _random_operand(K, M, Kdim, 100 + M, mode, dev)
-    bc, bs = _random_operand(K, N, Kdim, 200 + N, mode, dev)
+    tl = Kdim % 128 == 0 and N % 128 == 0    # what the tiled layout needs
+    ac, as_ = _random_operand(K, M, Kdim, 100 + M, mode, dev, tl)
+    bc, bs = _random_operand(K, N, Kdim, 200 + N, mode, dev, tl)
     alpha = post * post
-    y = K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha, torch.float32, a_tiled=True, b_tiled=True)
-    y16 = K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha, torch.bfloat16, a_tiled=True, b_tiled=True)
+    y = K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha, torch.float32, a_tiled=tl, b_tiled=tl)
+    y16 = K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha, torch.bfloat16, a_tiled=tl, b_tiled=tl)
     assert torch.equal(y16, y.to(torch.bfloat16))
-    ar = K.untile_codes(ac)
+    ar = K.untile_codes(ac) if tl else ac
     if _lib.lib().qm_gemm_workspace_bytes(M, N, Kdim) == 0:
         # a 256-row panel alone (one tile row, same K order inside every tile): bitwise the same rows
         r0 = (M // 2 // 256) * 256
-        sub = K.gemm_mxfp4_tn(K.tile_codes(ar[r0:r0 + 256].contiguous()), as_[r0:r0 + 256].contiguous(), bc, bs, alpha,
-                              torch.float32, a_tiled=True, b_tiled=True, split_k=False)
+        a_sub = ar[r0:r0 + 256].contiguous()
+        sub = K.gemm_mxfp4_tn(K.tile_codes(a_sub) if tl else a_sub, as_[r0:r0 + 256].contiguous(), bc, bs, alpha,
+                              torch.float32, a_tiled=tl, b_tiled=tl, split_k=False)
         assert torch.equal(sub, y[r0:r0 + 256])
     # sampled rows (first, last and random ones) against the float64 product of the de-quantized operands
     idx = torch.cat([torch.tensor([0, M - 1]), torch.randint(0, M, (46,), generator=g)]).to(dev)
     A = oracle.dequantize(to_oracle(ar[idx]), to_oracle(as_[idx]), post).astype(np.float64)
-    B = oracle.dequantize(to_oracle(K.untile_codes(bc)), to_oracle(bs), post).astype(np.float64)
+    B = oracle.dequantize(to_oracle(K.untile_codes(bc) if tl else bc), to_oracle(bs), post).astype(np.float64)
     want = A @ B.T
     got = y[idx].cpu().numpy().astype(np.float64)
     rel = np.linalg.norm(got - want) / np.linalg.norm(want)

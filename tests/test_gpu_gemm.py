@@ -83,15 +83,15 @@ def _torch_dequant(codes, scales):
     return v * s
 
 
-# Shapes the 256x256-tile kernels serve: a single tile, fewer tiles than CUs, more tiles than CUs (each
-# workgroup walks several tiles, with an odd and an even number of scale blocks per tile), and K that is a
-# multiple of 128 but not of 512 (per-step scale loads on the one-tile-per-workgroup kernel, or padding steps on the
-# persistent one).
+# Shapes the tile kernels serve: a single tile, fewer tiles than CUs, more tiles than CUs (each workgroup walks several
+# tiles, with an odd and an even number of scale blocks per tile), K that is a multiple of 128 but not of 512 (padding steps
+# on the persistent 256x256 kernel), and K up to 768 (one to six K steps on the 256x128 kernel that runs two workgroups per
+# CU, scale dwords per K step).
 @pytest.mark.parametrize("M,N,K_", [(256, 256, 512), (512, 768, 1024), (4352, 4352, 512), (4608, 4352, 1024),
                                     (768, 512, 1536), (512, 256, 640), (4352, 4608, 384), (8192, 4096, 2048),
                                     # tiles hanging over the edge of M and/or N (extents multiples of 64, not of 256)
                                     (320, 256, 512), (256, 448, 640), (640, 1920, 640), (1728, 640, 1024), (4416, 4160, 512),
-                                    (320, 320, 128),
+                                    (320, 320, 128), (512, 384, 256), (4352, 4480, 768), (256, 128 + 64, 640),
                                     # K a multiple of 128 that the persistent kernel pads to whole blocks of four steps with
                                     # zero-scale steps: three, two and one real steps in the last block; one tile and many
                                     (512, 768, 1920), (4352, 4608, 3840), (320, 256, 3712), (768, 512, 2944), (4608, 4352, 1920),
@@ -145,6 +145,33 @@ def test_gemm_tiled_operands_match_rowmajor(K, M, N, K_, a_tiled, b_tiled):
     # same kernel, same summation order: the layout only changes where the operand bytes are fetched from
     assert torch.equal(got, want)
     assert torch.equal(got16, want.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("tiled", [False, True])
+def test_gemm_scale_arrays_off_16_byte_alignment(K, tiled):
+    """K % 512 == 0 with scale arrays that are 4-byte but not 16-byte aligned: the persistent kernel's 16-byte scale
+    requests cannot serve them, the 256x128 kernel (4-byte scale requests, any K % 128 == 0) takes over -- same result,
+    row-major or tiled codes."""
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(77)
+    M, N, K_ = 512, 384, 1024
+    ac = torch.randint(0, 256, (M, K_ // 2), generator=g, dtype=torch.uint8).to(dev)
+    bc = torch.randint(0, 256, (N, K_ // 2), generator=g, dtype=torch.uint8).to(dev)
+    as_ = torch.randint(118, 132, (M, K_ // 32), generator=g, dtype=torch.uint8).to(dev)
+    bs = torch.randint(120, 136, (N, K_ // 32), generator=g, dtype=torch.uint8).to(dev)
+    want = K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha=1.0, out_dtype=torch.float32)
+
+    def shifted(t):
+        buf = torch.empty(t.numel() + 4, dtype=torch.uint8, device=dev)
+        view = buf[4:].view(t.shape)
+        view.copy_(t)
+        assert view.data_ptr() % 16 == 4
+        return view
+    a_in, b_in = (K.tile_codes(ac), K.tile_codes(bc)) if tiled else (ac, bc)
+    got = K.gemm_mxfp4_tn(a_in, shifted(as_), b_in, shifted(bs), alpha=1.0, out_dtype=torch.float32, a_tiled=tiled, b_tiled=tiled)
+    # another kernel, another order of the partial sums: equal to fp32 rounding, not bit for bit
+    rel = float((got.double() - want.double()).norm() / want.double().norm())
+    assert rel <= 1e-6, rel
 
 
 def test_split_k_is_offered_and_reproducible(K):
