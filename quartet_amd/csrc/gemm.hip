@@ -789,7 +789,7 @@ template <typename OutT, bool STAMP = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mxfp4_tn_big4_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ b_codes,
     const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c, int a_tiled,
-    int b_tiled, int splits, [[maybe_unused]] unsigned long long* __restrict__ stamps) {
+    int b_tiled, int splits, int late, [[maybe_unused]] unsigned long long* __restrict__ stamps) {
     extern __shared__ uint32_t smem[];
     uint8_t* smem_bytes = reinterpret_cast<uint8_t*>(smem);
     const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)smem;
@@ -870,6 +870,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         plan.sb = b_scales + n0 * groups + k0 * 4;
     };
 
+    // Short contractions: every other group of eight workgroups (one per XCD) starts `late` x 1024 cycles late -- about the
+    // length of an epilogue -- so that half of an XCD's CUs convert and store their tiles while the other half multiply.
+    // Left alone the CUs can fall into step, and then every tile boundary is a burst of 33 MB of stores during which no CU
+    // multiplies; which of the two states a launch settles in differs from chip to chip and from run to run (measured at
+    // 32768 x 1536 x 1536: 53-57 us in step, 45-46 us out of step; with the late start always the latter).
+    if (((int)blockIdx.x >> 3) & 1)
+        for (int i = 0; i < late; ++i) __builtin_amdgcn_s_sleep(16);
     plan_tile((int)blockIdx.x);
     big4_issue_scales(plan, 0, 0);  // K >= 512: the first block is a whole one
     big4_issue_codes(plan, 0, 0);
@@ -1043,6 +1050,10 @@ int choose_splits(int64_t M, int64_t N, int64_t K, int cus) {
     return best;
 }
 
+// late start (units of 1024 cycles) of every other group of workgroups: contractions of at most sixteen K steps per work
+// item, where the tile boundary is a third or more of a tile; longer ones neither gain nor lose (within 0.7 %)
+int big4_late_start(int64_t K, int splits) { return K / kBK / splits <= 16 ? 6 : 0; }
+
 template <typename OutT>
 hipError_t launch_big4(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                        const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_tiled,
@@ -1057,7 +1068,7 @@ hipError_t launch_big4(const uint8_t* a_codes, const uint8_t* a_scales, const ui
     if (g > 8) g -= g % 8;
     dim3 grid((unsigned)g), block(256);
     kern<<<grid, block, kBig4SmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
-                                                  reinterpret_cast<OutT*>(c), a_tiled, b_tiled, splits, nullptr);
+                                                  reinterpret_cast<OutT*>(c), a_tiled, b_tiled, splits, big4_late_start(K, splits), nullptr);
     return hipGetLastError();
 }
 
@@ -1124,7 +1135,7 @@ hipError_t gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, con
     if (stamps_bytes < (size_t)g * kPhaseStamps * sizeof(unsigned long long)) return hipErrorInvalidValue;
     kern<<<dim3((unsigned)g), dim3(256), kBig4SmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
                                                                   reinterpret_cast<uint16_t*>(c), a_layout == LAYOUT_TILED,
-                                                                  b_layout == LAYOUT_TILED, 1, stamps);
+                                                                  b_layout == LAYOUT_TILED, 1, big4_late_start(K, 1), stamps);
     *grid_out = (int)g;
     return hipGetLastError();
 }
