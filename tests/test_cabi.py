@@ -63,6 +63,12 @@ def test_host_only_entry_points():
     (lambda L: L.qm_gemm_mxfp4_tn(0x1000, 0x2000, 0x3000, 0x4000, 256, 256, 128, 1.0, 0x5004, 0, 0, 0, None, 0, None), b"c 16-byte"),
     # a shape of the generic kernel stores single elements: c misaligned for 4 bytes is refused, 4-byte aligned c is not
     (lambda L: L.qm_gemm_mxfp4_tn(0x1000, 0x2000, 0x3000, 0x4000, 96, 256, 128, 1.0, 0x5002, 0, 0, 0, None, 0, None), b"c 16-byte (4-byte"),
+    # the FP4 x bf16 product: contraction a multiple of 64, N a multiple of 8, tensors non-null and aligned
+    (lambda L: L.qm_gemm_mxfp4_bf16_nn(None, None, None, 64, 64, 96, 1.0, None, 0, None), b"multiple of 64"),
+    (lambda L: L.qm_gemm_mxfp4_bf16_nn(None, None, None, 64, 60, 128, 1.0, None, 0, None), b"multiple of 8"),
+    (lambda L: L.qm_gemm_mxfp4_bf16_nn(None, None, None, 64, 64, 128, 1.0, None, 0, None), b"null tensor"),
+    (lambda L: L.qm_gemm_mxfp4_bf16_nn(0x1000, 0x2000, 0x3008, 64, 64, 128, 1.0, 0x4000, 0, None), b"16-byte"),
+    (lambda L: L.qm_gemm_mxfp4_bf16_nn(0x1000, 0x2000, 0x3000, 64, 64, 128, 1.0, 0x4000, 9, None), b"c_dtype"),
     (lambda L: L.qm_quantize_mxfp4_dense(None, 0, 4, 40, None, 1, 0, 0, None, None, None, None, 0, None), b"multiple of 32"),
     (lambda L: L.qm_quantize_mxfp4_dense(None, 0, 4, 64, None, 1, 0, 0, None, None, None, None, 0, None), b"non-null"),
     (lambda L: L.qm_quantize_mxfp4_dense(0x1000, 0, 64, 64, 0x2000, 1, 1, 0, 0x3000, 0x4000, None, None, 0, None), b"transposed input needs"),
@@ -96,6 +102,7 @@ def test_empty_shapes_are_accepted_without_touching_pointers():
     L = _lib.lib()
     assert L.qm_quantize_mxfp4(None, 0, 0, 64, 32, None, 0, 0, None, 0, None, None, None, None, 0, None) == 0
     assert L.qm_gemm_mxfp4_tn(None, None, None, None, 0, 64, 64, 1.0, None, 0, 0, 0, None, 0, None) == 0
+    assert L.qm_gemm_mxfp4_bf16_nn(None, None, None, 0, 64, 64, 1.0, None, 0, None) == 0
     assert L.qm_linear_forward(None, 0, None, 0, 0, 64, 64, 32, None, 32, None, None, 0, None, 0, 0, None, 0, 0, None) == 0
     assert L.qm_rmsnorm_quantize_mxfp4(None, 0, None, 0, None, None, 1e-5, 0, 64, None, None, 0, None, 0, None) == 0
     assert L.qm_swiglu_quantize_mxfp4(None, 0, 0, 64, None, None, 0, 0, None) == 0
