@@ -40,6 +40,8 @@ enum { QM_QUEST_RTN = 0, QM_ABSMAX_RTN = 1, QM_ABSMAX_SR = 2, QM_QUEST_SR = 3 };
 enum { QM_LAYOUT_ROWMAJOR = 0, QM_LAYOUT_TILED = 1 };
 /* qm_linear_forward: which packed operand buffers already hold their operand on entry */
 enum { QM_W_IS_PACKED = 1, QM_X_IS_PACKED = 2 };
+/* rotated_flags of qm_linear_backward */
+enum { QM_GX_ROTATED = 1, QM_GW_ROTATED = 2 };
 
 #define QM_ERR_INVALID (-1)
 #define QM_ERR_UNALIGNED (-2)
@@ -233,9 +235,11 @@ int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, 
  *   g_matrix          NULL, or a DEVICE pointer to the gradient quantizer's dense rotation ([32][32] fp32, as for
  *                     qm_quantize_mxfp4_dense; AlbertTsengQuantizer with rerotate="O32"): replaces hd_g / signs_g in the
  *                     four gradient quantizations; needs hd_g == 32 and T, I, O multiples of 128
- *   gx_rotated        != 0: gx receives the gradient w.r.t. the activation quantizer's rotated output (the first
+ *   rotated_flags     QM_GX_ROTATED: gx receives the gradient w.r.t. the activation quantizer's rotated output (the first
  *                     product, B3) and its straight-through backward is left to the caller, who folds it into the
- *                     next kernel (maskbits argument of qm_rmsnorm_backward / qm_swiglu_backward); needs hd_x == 32
+ *                     next kernel (maskbits argument of qm_rmsnorm_backward / qm_swiglu_backward) or, for a forward
+ *                     quantizer that holds a dense rotation, applies mask and transposed matrix itself; needs hd_x == 32.
+ *                     QM_GW_ROTATED: the same for gw and the weight quantizer (second product, B6; gw_dtype == mid_dtype)
  * codes_layout applies to every packed tensor inside; QM_LAYOUT_TILED needs T, I, O multiples of 128 and at
  * least 256, and all Hadamard blocks 32.  T, I, O must be multiples of 32 for the backward pass.
  */
@@ -251,7 +255,7 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                        const void* packed_w, int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w,
                        int hd_g, const uint32_t* signs_g, int g_mode, const uint64_t* seeds, int x_val_dtype,
                        int w_val_dtype, int mid_dtype, int x_scale_dtype, int w_scale_dtype, void* workspace,
-                       size_t workspace_bytes, void* gx, void* gw, int gw_dtype, int codes_layout, int gx_rotated,
+                       size_t workspace_bytes, void* gx, void* gw, int gw_dtype, int codes_layout, int rotated_flags,
                        const float* g_matrix, void* stream);
 /*
  * qm_linear_backward for callers that replay the step from a captured HIP graph.  It has no counterpart in the reference
@@ -266,7 +270,7 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
                               const void* packed_w, int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w,
                               int hd_g, const uint32_t* signs_g, int g_mode, const uint64_t* seeds, int x_val_dtype,
                               int w_val_dtype, int mid_dtype, int x_scale_dtype, int w_scale_dtype, void* workspace,
-                              size_t workspace_bytes, void* gx, void* gw, int gw_dtype, int codes_layout, int gx_rotated,
+                              size_t workspace_bytes, void* gx, void* gw, int gw_dtype, int codes_layout, int rotated_flags,
                               const float* g_matrix, const uint64_t* seed_base, void* stream);
 
 /*
@@ -292,7 +296,7 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
  *   gradient of a bf16 `add` of qm_rmsnorm_quantize_mxfp4.
  * qm_swiglu_backward: autograd of silu(up) * gate: g [rows, hidden] -> d_h12 [rows, 2 hidden] of h12's dtype.
  *   Both backward kernels take the gradient either as it is (maskbits == NULL) or still in the rotated basis of the
- *   layer's activation quantizer (qm_linear_backward with gx_rotated): then maskbits [rows, cols/8] (the mask region of
+ *   layer's activation quantizer (qm_linear_backward with QM_GX_ROTATED): then maskbits [rows, cols/8] (the mask region of
  *   the layer's packed_x; 4-byte aligned for qm_rmsnorm_backward), sign_bits and scale_dtype describe that quantizer, and the masked inverse rotation of
  *   qm_masked_hadamard_bwd (same operations, same bits, rounded to the gradient's dtype) is applied on the fly.
  * codes_layout QM_LAYOUT_TILED needs rows % 16 == 0 and cols (hidden) % 128 == 0; cols (hidden) % 32 == 0 always.

@@ -44,7 +44,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 13; }
+int qm_version(void) { return 14; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -416,17 +416,17 @@ int qm_linear_backward(const void* e, int e_dtype, int64_t T, int64_t I, int64_t
                        int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, int hd_g, const uint32_t* signs_g,
                        int g_mode, const uint64_t* seeds, int x_val_dtype, int w_val_dtype, int mid_dtype, int x_scale_dtype,
                        int w_scale_dtype, void* workspace, size_t workspace_bytes, void* gx, void* gw, int gw_dtype,
-                       int codes_layout, int gx_rotated, const float* g_matrix, void* stream) {
+                       int codes_layout, int rotated_flags, const float* g_matrix, void* stream) {
     return qm_linear_backward_seeded(e, e_dtype, T, I, O, packed_x, packed_w, hd_x, signs_x, hd_w, signs_w, hd_g, signs_g, g_mode, seeds,
                                      x_val_dtype, w_val_dtype, mid_dtype, x_scale_dtype, w_scale_dtype, workspace, workspace_bytes, gx,
-                                     gw, gw_dtype, codes_layout, gx_rotated, g_matrix, nullptr, stream);
+                                     gw, gw_dtype, codes_layout, rotated_flags, g_matrix, nullptr, stream);
 }
 
 int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, int64_t O, const void* packed_x,
                               const void* packed_w, int hd_x, const uint32_t* signs_x, int hd_w, const uint32_t* signs_w, int hd_g,
                               const uint32_t* signs_g, int g_mode, const uint64_t* seeds, int x_val_dtype, int w_val_dtype,
                               int mid_dtype, int x_scale_dtype, int w_scale_dtype, void* workspace, size_t workspace_bytes, void* gx,
-                              void* gw, int gw_dtype, int codes_layout, int gx_rotated, const float* g_matrix,
+                              void* gw, int gw_dtype, int codes_layout, int rotated_flags, const float* g_matrix,
                               const uint64_t* seed_base, void* stream) {
     if (T < 0 || I < 0 || O < 0) return fail(QM_ERR_INVALID, "qm_linear_backward: negative extent");
     if (seed_base && (!aligned(seed_base, 8) || g_matrix || !pair_launches(codes_layout, T, I, O, hd_x, hd_w, hd_g)))
@@ -457,11 +457,17 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
     void* gws = wl.gemm_ws_bytes ? k + wl.gemm_ws : nullptr;
     hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
     int rc;
-    // gx_rotated: the caller undoes the activation quantizer's rotation itself (fused into its next kernel); the first
-    // product then lands in gx directly
+    // rotated_flags: bit 0 (QM_GX_ROTATED): the caller undoes the activation quantizer's rotation itself (fused into its
+    // next kernel, or a dense rotation it applies with a library product); the first product then lands in gx directly.
+    // Bit 1 (QM_GW_ROTATED): the same for the weight quantizer's rotation and gw.
+    if (rotated_flags & ~(QM_GX_ROTATED | QM_GW_ROTATED)) return fail(QM_ERR_INVALID, "qm_linear_backward: unknown rotated flags %d", rotated_flags);
+    const bool gx_rotated = rotated_flags & QM_GX_ROTATED, gw_rotated = rotated_flags & QM_GW_ROTATED;
+    if (gw_rotated && gw_dtype != mid_dtype) return fail(QM_ERR_INVALID, "qm_linear_backward: QM_GW_ROTATED needs gw_dtype == mid_dtype");
     void* gx_product = gx_rotated ? gx : static_cast<void*>(k + wl.gxq);
+    void* gw_product = gw_rotated ? gw : static_cast<void*>(k + wl.gwq);
     // B8: gw in gw_dtype; a bf16 result widened to fp32 keeps its bf16 rounding (what converting it afterwards would give)
     const auto rotate_gw = [&]() -> int {
+        if (gw_rotated) return 0;
         if (gw_dtype == mid_dtype)
             return qm_masked_hadamard_bwd(k + wl.gwq, mid_dtype, O, I, hd_w, w_scale_dtype, signs_w, pw + lw.m, gw, mid_dtype, stream);
         if (!valid_hd(hd_w) || I % hd_w || !gw || !aligned(gw, 16) || !valid_dtype(w_scale_dtype))
@@ -488,7 +494,7 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
         rc = qm_requantize_transposed_mxfp4_dense(px + lx.c, px + lx.s, T, I, 1.0f, x_val_dtype, g_matrix, g_mode, seeds[3], k + wl.xtc,
                                                   k + wl.xts, nullptr, codes_layout, codes_layout, stream);
         if (rc) return rc;
-        rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, k + wl.gwq, mid_dtype, codes_layout,
+        rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, gw_product, mid_dtype, codes_layout,
                               codes_layout, gws, wl.gemm_ws_bytes, stream);
         if (rc) return rc;
         if (!gx_rotated) {
@@ -512,10 +518,12 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
         rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, gx_product, mid_dtype, codes_layout,
                               codes_layout, gws, wl.gemm_ws_bytes, stream);
         if (rc) return rc;
-        rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, k + wl.gwq, mid_dtype, codes_layout,
+        rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, gw_product, mid_dtype, codes_layout,
                               codes_layout, gws, wl.gemm_ws_bytes, stream);
         if (rc) return rc;
         if (gx_rotated) return rotate_gw();
+        if (gw_rotated)
+            return qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, px + lx.m, gx, mid_dtype, stream);
         return from_hip(qm::masked_hadamard_bwd_hd32_pair(k + wl.gxq, T * I, x_scale_dtype,
                                                           signs_x ? signs_x[0] : 0u, px + lx.m, gx, k + wl.gwq, O * I,
                                                           w_scale_dtype, signs_w ? signs_w[0] : 0u,
@@ -537,7 +545,7 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
     rc = qm_requantize_transposed_mxfp4(px + lx.c, px + lx.s, T, I, 1.0f, x_val_dtype, hd_g, signs_g, g_mode, nullptr, seeds[3],
                                         k + wl.xtc, k + wl.xts, nullptr, codes_layout, codes_layout, stream);
     if (rc) return rc;
-    rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, k + wl.gwq, mid_dtype, codes_layout,
+    rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, gw_product, mid_dtype, codes_layout,
                           codes_layout, gws, wl.gemm_ws_bytes, stream);
     if (rc) return rc;
     if (!gx_rotated) {

@@ -20,7 +20,8 @@ _KERNEL_DTYPES = (torch.float32, torch.bfloat16)
 
 def _layer_is_fusable(layer, x):
     return (isinstance(layer, QuantizedLinear) and layer._is_production_config(x.numel() // max(x.shape[-1], 1)) and layer.weight.is_cuda
-            and layer.activation_quantizer.hadamard_dim == 32 and layer.weight.dtype in _KERNEL_DTYPES)
+            and layer.activation_quantizer.hadamard_dim == 32 and not layer.activation_quantizer.is_dense
+            and layer.weight.dtype in _KERNEL_DTYPES)
 
 
 class RMSNormLinearFn(torch.autograd.Function):

@@ -279,6 +279,24 @@ def packed_operand_buffer(rows, cols, device):
 QM_W_IS_PACKED, QM_X_IS_PACKED = 1, 2
 
 
+def quantize_dense_into_packed(x2, matrix, tiled):
+    """Quest RTN + clip mask of x2 [rows, cols] under a dense 32 x 32 rotation, written into a fresh packed-operand buffer
+    (what linear_forward fills for a Hadamard rotation): the forward quantizer of a layer whose quantizer holds the matrix
+    of rerotate="O32"."""
+    _require_cuda(x2)
+    assert x2.dim() == 2 and x2.is_contiguous()
+    rows, cols = x2.shape
+    packed = packed_operand_buffer(rows, cols, x2.device)
+    off = (ctypes.c_size_t * 3)()
+    _lib.check(_lib.lib().qm_packed_operand_offsets(rows, cols, off), "qm_packed_operand_offsets")
+    m = _matrix_arg(matrix, x2.device)
+    base = packed.data_ptr()
+    rc = _lib.lib().qm_quantize_mxfp4_dense(_ptr(x2), _dtype_code(x2.dtype), rows, cols, _ptr(m), QM_QUEST_RTN, 0, 0, base + off[0],
+                                            base + off[1], base + off[2], None, _layout(tiled), _stream())
+    _lib.check(rc, "qm_quantize_mxfp4_dense")
+    return packed
+
+
 def linear_forward(x2, w2, hd_x, signs_x, hd_w, signs_w, out_dtype, tiled, packed_w=None, packed_x=None, rows=None):
     """Whole forward pass of a Quartet linear in one foreign call: quantize x [T,I] and w [O,I] (quest RTN + clip
     mask), y = Q(x) Q(w)^T.  Returns (y [T,O], packed_x, packed_w): the byte buffers the backward pass reads.  A
@@ -407,10 +425,11 @@ def rope_merge_qkv_grad(dq, dk, dv, table, n_embd, head_dim, seq_len, out_dtype)
 
 def linear_backward(e2, packed_x, packed_w, T, I, O, hd_x, signs_x, hd_w, signs_w, hd_g, signs_g, mode, seeds, x_val_dtype,
                     w_val_dtype, mid_dtype, x_scale_dtype, w_scale_dtype, tiled, gx_rotated=False, gw_dtype=None, g_matrix=None,
-                    seed_base=None):
+                    seed_base=None, gw_rotated=False):
     """Whole backward pass in one foreign call: e [T,O] -> (gx [T,I], gw [O,I]) of mid_dtype.  With `gx_rotated`, gx is
     still in the rotated basis of the activation quantizer: its masked inverse rotation is left to the kernel that
-    consumes gx (rmsnorm_backward / swiglu_backward with `maskbits`).  `gw_dtype` = float32 with a bf16 mid_dtype returns
+    consumes gx (rmsnorm_backward / swiglu_backward with `maskbits`); with `gw_rotated` likewise gw (mid_dtype) in the
+    weight quantizer's rotated basis.  `gw_dtype` = float32 with a bf16 mid_dtype returns
     gw as the bf16-rounded values widened to fp32 (the cast autograd would apply for an fp32 weight) in the same pass.
     `seed_base`: a one-element int64 tensor on the GPU whose value the gradient quantizers add to their seeds when they
     run (a step replayed from a captured graph draws fresh random streams if the graph also increments it)."""
@@ -423,12 +442,13 @@ def linear_backward(e2, packed_x, packed_w, T, I, O, hd_x, signs_x, hd_w, signs_
     nbytes = L.qm_linear_backward_workspace_bytes(T, I, O, mid)
     work = torch.empty(nbytes, dtype=torch.uint8, device=e2.device)
     gx = torch.empty((T, I), dtype=mid_dtype, device=e2.device)
-    gw_dtype = mid_dtype if gw_dtype is None or mid_dtype != torch.bfloat16 else gw_dtype
+    gw_dtype = mid_dtype if gw_dtype is None or mid_dtype != torch.bfloat16 or gw_rotated else gw_dtype
     gw = torch.empty((O, I), dtype=gw_dtype, device=e2.device)
     rc = L.qm_linear_backward_seeded(_ptr(e2), _dtype_code(e2.dtype), T, I, O, _ptr(packed_x), _ptr(packed_w), hd_x,
                                      sign_words(signs_x), hd_w, sign_words(signs_w), hd_g, sign_words(signs_g), mode,
                                      (ctypes.c_uint64 * 4)(*seeds), _dtype_code(x_val_dtype), _dtype_code(w_val_dtype), mid,
                                      _dtype_code(x_scale_dtype), _dtype_code(w_scale_dtype), _ptr(work), nbytes, _ptr(gx), _ptr(gw),
-                                     _dtype_code(gw_dtype), _layout(tiled), int(gx_rotated), _ptr(g_matrix), _ptr(seed_base), _stream())
+                                     _dtype_code(gw_dtype), _layout(tiled), int(bool(gx_rotated)) | (int(bool(gw_rotated)) << 1), _ptr(g_matrix),
+                                     _ptr(seed_base), _stream())
     _lib.check(rc, "qm_linear_backward")
     return gx, gw

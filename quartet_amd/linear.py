@@ -46,19 +46,39 @@ def _forward_packed(ctx, x2, weight, a_q, w_q, g_q, weight_cache, tiled, out_dty
     """F1 (unless a producer already wrote packed_x), F2 (unless the layer's cache holds Q(W)), F3; records on ctx what
     the backward pass of the products needs.  Returns (y [T, O], packed_x, packed_w)."""
     w2 = weight.contiguous()
+    # a forward quantizer that holds the dense matrix of rerotate="O32": its kernel fills the packed operand here, and the
+    # straight-through backward (clip mask, transposed matrix) is applied to the rotated-basis gradient in _backward_packed
+    # (the matrix cast to the quantized tensor's dtype as the quantizer modules do, mxfp4.py:49,160; fp32 storage for the kernel)
+    x_dense = a_q.dense_matrix(w2.device).to(x_dtype).to(torch.float32) if a_q.is_dense else None
+    w_dense = w_q.dense_matrix(w2.device).to(w2.dtype).to(torch.float32) if w_q.is_dense else None
+    if x_dense is not None and packed_x is None:
+        packed_x, rows, x2 = K.quantize_dense_into_packed(x2, x_dense, tiled), x2.shape[0], None
     # Q(W) of an unchanged weight (the micro-steps of one accumulation) is quantized once and kept by the layer
-    key = (weight.data_ptr(), weight._version, weight.dtype, tuple(weight.shape), w_q.hadamard_dim, w_q.sign_bits, tiled)
+    key = (weight.data_ptr(), weight._version, weight.dtype, tuple(weight.shape), w_q.hadamard_dim, w_q.sign_bits, tiled,
+           None if w_dense is None else w_q._dense_epoch)
     packed_w = weight_cache.get(key) if weight_cache is not None else None
+    if w_dense is not None and packed_w is None:
+        packed_w = K.quantize_dense_into_packed(w2, w_dense, tiled)
     y, packed_x, packed_w = K.linear_forward(x2, w2, a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits,
                                              out_dtype, tiled, packed_w, packed_x, rows)
     if weight_cache is not None:
         weight_cache.put(key, packed_w)
     ctx.g_q = g_q
     ctx.tiled = tiled
+    ctx.dense_fwd = (x_dense, w_dense)
     ctx.fwd = (a_q.hadamard_dim, a_q.sign_bits, w_q.hadamard_dim, w_q.sign_bits)
     ctx.dims = (y.shape[0], weight.shape[1], weight.shape[0])
     ctx.x_dtype, ctx.w_dtype = x_dtype, weight.dtype
     return y, packed_x, packed_w
+
+
+def _dense_rotation_backward(g, maskbits, matrix, scale_dtype):
+    """Straight-through backward of a forward quantizer with a dense rotation (mxfp4.py:143-146 with the matrix of
+    mxfp4.py:61-64): (g * clip mask) @ matrix^T per group of 32, in g's dtype like the module path's product."""
+    from .quantizers.mxfp4 import _unpack_mask
+    g = g * _unpack_mask(maskbits, g.shape).to(g.dtype)
+    m = matrix.to(scale_dtype).to(g.dtype)
+    return (g.reshape(-1, 32) @ m.T).view(g.shape)
 
 
 def _backward_packed(ctx, e, packed_x, packed_w, gx_rotated=False):
@@ -88,12 +108,19 @@ def _backward_packed(ctx, e, packed_x, packed_w, gx_rotated=False):
             f"{', dense gradient rotation' if g_matrix is not None else ''}) does not run on the tiled layout, whose kernels are the "
             "only ones that read it (every extent a multiple of 128 and >= 256, Hadamard blocks 32, no dense rotation); "
             "clear the seed base or change the layer")
+    x_dense, w_dense = ctx.dense_fwd
     gx, gw = K.linear_backward(e2, packed_x, packed_w, T, I, O, a_hd, a_signs, w_hd, w_signs, hd, signs, mode, seeds, ctx.x_dtype,
-                               ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled, gx_rotated,
+                               ctx.w_dtype, mid_dtype, sd_x, sd_w, ctx.tiled, gx_rotated or x_dense is not None,
                                ctx.w_dtype if ctx.w_dtype in (torch.float32, torch.bfloat16) else None, g_matrix,
-                               _SEED_BASE if (ctx.tiled and g_matrix is None and g_q.stochastic) else None)
+                               _SEED_BASE if (ctx.tiled and g_matrix is None and g_q.stochastic) else None,
+                               gw_rotated=w_dense is not None)
+    if w_dense is not None:
+        gw = _dense_rotation_backward(gw, K.packed_mask_bits(packed_w, O, I), w_dense, sd_w)
     if gx_rotated:
+        assert x_dense is None   # the fused producers are not offered layers with a dense forward rotation
         return gx, gw, (K.packed_mask_bits(packed_x, T, I), a_signs, sd_x)
+    if x_dense is not None:
+        gx = _dense_rotation_backward(gx, K.packed_mask_bits(packed_x, T, I), x_dense, sd_x)
     return gx, gw
 
 
@@ -186,10 +213,11 @@ class QuantizedLinear(nn.Linear):
 
     def _is_production_config(self, tokens):
         g_q = self.backward_scheme.g_quantizer
-        # a dense rotation (rerotate="O32") in a forward quantizer, now or after the next re_randomize, needs the generic
-        # path; in the gradient quantizer the packed path serves it when every extent is a multiple of 128 and the
-        # Hadamard block it replaces is 32
-        dense = any(getattr(q_, "is_dense", False) or getattr(q_, "rerotate", None) == "O32"
+        # A dense rotation (rerotate="O32") replaces a Hadamard block of 32 only in the kernels.  In the gradient quantizer
+        # the packed path serves it when every extent is a multiple of 128; in a forward quantizer (the reference's loop
+        # never re-randomises those) the dense quantizer kernel fills the packed operand and the straight-through
+        # backward is a small library product.
+        dense = any(getattr(q_, "is_dense", False) and q_.hadamard_dim != 32
                     for q_ in (self.activation_quantizer, self.weight_quantizer))
         if getattr(g_q, "is_dense", False) or getattr(g_q, "rerotate", None) == "O32":
             dense = dense or g_q.hadamard_dim != 32 or any(d % 128 for d in (tokens, self.in_features, self.out_features))

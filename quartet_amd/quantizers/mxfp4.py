@@ -128,6 +128,7 @@ class _HadamardQuantizer(BaseQuantizer):
         self.sign_bits = 0  # bit j set = column j of H negated
         self._dense = None  # fp32 [hd, hd] orthogonal matrix once re_randomize("O32") has replaced H
         self._dense_dev = None  # its copy on the device of the tensors being quantized
+        self._dense_epoch = 0  # how many times re_randomize has drawn a dense matrix (keys a layer's cache of Q(W))
         self._matrix_dtype = torch.float32
         self._matrix_device = torch.device("cpu")
 
@@ -169,6 +170,7 @@ class _HadamardQuantizer(BaseQuantizer):
             u, _, vh = torch.linalg.svd(torch.randn(self.hadamard_dim, self.hadamard_dim))
             self._dense = (u @ vh).contiguous()
             self._dense_dev = None
+            self._dense_epoch += 1
             self.sign_bits = 0
         elif self.rerotate is None:
             pass

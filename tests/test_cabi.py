@@ -29,7 +29,7 @@ def test_library_exports_every_declared_function():
 
 def test_host_only_entry_points():
     L = _lib.lib()
-    assert L.qm_version() == 13
+    assert L.qm_version() == 14
     T, I, O = 256, 128, 384
     off = (ctypes.c_size_t * 3)()
     for rows, cols in ((T, I), (O, I)):

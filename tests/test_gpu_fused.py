@@ -139,9 +139,10 @@ def production_layer(q, I, O, dtype):
                              backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]()).to(DEV, dtype)
 
 
+@pytest.mark.parametrize("dense_w", [False, True])
 @pytest.mark.parametrize("autocast", [True, False])
 @pytest.mark.parametrize("T,I,O", [(256, 640, 1920), (96, 160, 224)])
-def test_rmsnorm_linear_matches_the_unfused_layer(oracle, q, T, I, O, autocast):
+def test_rmsnorm_linear_matches_the_unfused_layer(oracle, q, T, I, O, autocast, dense_w):
     """The fused layer against the same layer called on the oracle's normalised tensor: identical packed operands, so
     identical outputs and weight gradients; the gradient w.r.t. x against float64 autograd of RMSNorm applied to the
     unfused layer's input gradient."""
@@ -150,6 +151,9 @@ def test_rmsnorm_linear_matches_the_unfused_layer(oracle, q, T, I, O, autocast):
     from quartet_amd.llama import RMSNorm
     torch.manual_seed(0)
     layer = production_layer(q, I, O, torch.float32)
+    if dense_w:   # a weight quantizer holding the dense matrix of rerotate="O32" stays with the fused producer
+        layer.weight_quantizer.rerotate = "O32"
+        layer.weight_quantizer.re_randomize()
     norm = RMSNorm(I, eps=1e-5).to(DEV)
     with torch.no_grad():
         norm.weight.add_(0.1 * torch.randn(I, device=DEV))
@@ -179,13 +183,17 @@ def test_rmsnorm_linear_matches_the_unfused_layer(oracle, q, T, I, O, autocast):
     assert rel(got[3], gd.grad) < 1e-4
 
 
+@pytest.mark.parametrize("dense_w", [False, True])
 @pytest.mark.parametrize("autocast", [True, False])
 @pytest.mark.parametrize("T,I,O", [(256, 1792, 640), (64, 96, 160)])
-def test_swiglu_linear_matches_the_unfused_layer(oracle, q, T, I, O, autocast):
+def test_swiglu_linear_matches_the_unfused_layer(oracle, q, T, I, O, autocast, dense_w):
     print(f"case swiglu_linear T={T} hidden={I} O={O} autocast={autocast}", flush=True)
     from quartet_amd.fused import swiglu_linear
     torch.manual_seed(0)
     layer = production_layer(q, I, O, torch.float32)
+    if dense_w:
+        layer.weight_quantizer.rerotate = "O32"
+        layer.weight_quantizer.re_randomize()
     dtype = torch.bfloat16 if autocast else torch.float32    # w12's output dtype under autocast
     h12 = make_input(T, 2 * I, dtype, seed=6, scale=2.0).to(DEV)
     dy = make_input(T, O, dtype, seed=7, scale=1e-2, outlier_frac=0).to(DEV)
@@ -222,7 +230,12 @@ def test_fallbacks_keep_the_unfused_composition(q):
                              activation_quantizer=q.QuestMXFP4Quantizer(hadamard_dim=64),
                              gradient_quantizer=q.AlbertTsengQuantizer(hadamard_dim=64, stochastic=False),
                              backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]()).to(DEV)
-    for layer, I in ((plain, 64), (wide, 128)):
+    dense_x = q.QuantizedLinear(128, 96, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(),
+                                activation_quantizer=q.QuestMXFP4Quantizer(rerotate="O32"),
+                                gradient_quantizer=q.AlbertTsengQuantizer(stochastic=False),
+                                backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]()).to(DEV)
+    dense_x.activation_quantizer.re_randomize()     # the producers rotate by the Hadamard matrix only
+    for layer, I in ((plain, 64), (wide, 128), (dense_x, 128)):
         norm = RMSNorm(I).to(DEV)
         x = torch.randn(32, I, device=DEV)
         assert torch.equal(rmsnorm_linear(norm, layer, x), layer(norm(x)))

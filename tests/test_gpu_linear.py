@@ -304,6 +304,76 @@ def test_layer_with_dense_gradient_rotation(oracle, q):
         assert 0.03 < errs["O32"][k] < 0.3 and abs(errs["O32"][k] - errs["signs"][k]) < 0.5 * errs["signs"][k]
 
 
+@pytest.mark.parametrize("dense", ["x", "w", "xw"])
+@pytest.mark.parametrize("dtype,shape", [(torch.float32, (384, 256, 160)), (torch.bfloat16, (384, 256, 160)),
+                                         (torch.bfloat16, (256, 512, 256))])
+def test_layer_with_dense_forward_rotation(oracle, q, dense, dtype, shape):
+    """A forward quantizer that holds the dense matrix of rerotate="O32" (mxfp4.py:61-64) keeps the layer on the packed
+    FP4 path: the dense quantizer kernel fills the packed operand, the gradient products run as ever, and the
+    straight-through backward is (g * clip mask) @ matrix^T (mxfp4.py:143-146).  Checked against the oracle pipeline
+    with the matrices the quantizers drew, on the row-major and the tiled operand layout, and against the module path."""
+    print(f"case layer with dense forward rotation of {dense} dtype={dtype} shape={shape}", flush=True)
+    T, I, O = shape
+    x = make_input(T, I, dtype, seed=1, outlier_frac=0.01)
+    w = make_input(O, I, dtype, seed=2, outlier_frac=0, scale=0.02)
+    dy = make_input(T, O, dtype, seed=3, outlier_frac=0, scale=1e-3)
+    layer = production_layer(q, I, O, True, None, dtype)
+    torch.manual_seed(11)
+    mats = {}
+    for name, quantizer in (("x", layer.activation_quantizer), ("w", layer.weight_quantizer)):
+        if name in dense:
+            quantizer.rerotate = "O32"
+            quantizer.re_randomize()
+            assert quantizer.is_dense
+            mats[name] = quantizer._dense.to(dtype).double().numpy()   # the modules cast the matrix to the tensor's dtype
+    assert layer._is_production_config(T)
+    with torch.no_grad():
+        layer.weight.copy_(w.to("cuda:0"))
+
+    def step(packed):
+        layer.use_packed_path = packed
+        layer.weight.grad = None
+        xd = x.to("cuda:0").requires_grad_(True)
+        random.seed(5)
+        y = layer(xd)
+        y.backward(dy.to("cuda:0"))
+        torch.cuda.synchronize()
+        return y.detach().float().cpu().numpy(), xd.grad.float().cpu().numpy(), layer.weight.grad.float().cpu().numpy(), xd.grad.dtype
+
+    y, gx, gw, gdt = step(True)
+    assert gdt == dtype
+    random.seed(5)
+    seeds = [random.getrandbits(63) for _ in range(4)]
+    vd = oracle.BF16 if dtype == torch.bfloat16 else oracle.F32
+    d = float(oracle.FOUR_THIRDS)
+    fwd = lambda t, name: (oracle.quantize(to_oracle(t), mode=oracle.QUEST_RTN, want_mask=True, matrix=mats[name].astype(np.float32))
+                           if name in dense else oracle.quantize(to_oracle(t), 32, mode=oracle.QUEST_RTN, want_mask=True))
+    qx, qw = fwd(x, "x"), fwd(w, "w")
+    y_ref = oracle.gemm_tn(qx["codes"], qx["scales"], qw["codes"], qw["scales"])
+    qe = oracle.quantize(to_oracle(dy), 32, mode=oracle.ABSMAX_SR, seed=seeds[0])
+    qwt = oracle.requantize_transposed(qw["codes"], qw["scales"], val_dtype=vd, hd=32, mode=oracle.ABSMAX_SR, seed=seeds[1])
+    gxq = oracle.gemm_tn(qe["codes"], qe["scales"], qwt["codes"], qwt["scales"], a_post=d, b_post=d)
+    qet = oracle.quantize(to_oracle(dy), 32, mode=oracle.ABSMAX_SR, transposed_in=True, seed=seeds[2])
+    qxt = oracle.requantize_transposed(qx["codes"], qx["scales"], val_dtype=vd, hd=32, mode=oracle.ABSMAX_SR, seed=seeds[3])
+    gwq = oracle.gemm_tn(qet["codes"], qet["scales"], qxt["codes"], qxt["scales"], a_post=d, b_post=d)
+
+    def ste(gq, packed, name):
+        if name not in dense:
+            return oracle.masked_hadamard_bwd(gq.astype(np.float32), 32, vd, None, packed["mask"], out_dtype=oracle.F32)
+        keep = np.unpackbits(packed["mask"], axis=1, bitorder="little").astype(np.float64)
+        return ((gq * keep).reshape(-1, 32) @ mats[name].T).reshape(gq.shape)
+
+    tol_y, tol_g = (1e-5, 1e-5) if dtype == torch.float32 else (3e-3, 6e-3)
+    assert rel(y, y_ref) <= tol_y
+    assert rel(gx, ste(gxq, qx, "x")) <= tol_g
+    assert rel(gw, ste(gwq, qw, "w")) <= tol_g
+    # the module path (quantizer modules, de-quantized tensors, library products) computes the same forward pass; its
+    # backward draws its seeds in another order, so only the size of the difference is checked there
+    y_mod, gx_mod, gw_mod, _ = step(False)
+    assert rel(y_mod, y) <= (1e-5 if dtype == torch.float32 else 6e-3)
+    assert rel(gx_mod, gx) < 1.0 and rel(gw_mod, gw) < 1.0
+
+
 def test_packed_weight_cache_across_micro_steps(q):
     """With the cache on, the second micro-step reuses the packed Q(W) of the first: outputs and gradients are
     bit-identical to a layer that quantizes every time, the buffer saved by an earlier graph survives a weight

@@ -58,8 +58,8 @@ def test_classifier_tells_signed_sylvester_from_everything_else():
 
 
 def test_which_layers_with_a_dense_rotation_stay_on_the_packed_path():
-    """A dense rotation in the gradient quantizer is served by the packed FP4 path when every extent is a multiple of
-    128; in a forward quantizer, or at other shapes, the layer takes the generic path."""
+    """A dense rotation over 32 values is served by the packed FP4 path: in the gradient quantizer when every extent is
+    a multiple of 128, in a forward quantizer at any shape; a dense rotation over a wider block takes the generic path."""
     def make(rr, fwd_rr=None, features=256):
         return q.QuantizedLinear(features, features, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(rerotate=fwd_rr),
                                  activation_quantizer=q.QuestMXFP4Quantizer(),
@@ -69,7 +69,17 @@ def test_which_layers_with_a_dense_rotation_stay_on_the_packed_path():
     assert make("O32")._is_production_config(256)
     assert not make("O32")._is_production_config(160)          # tokens not a multiple of 128
     assert not make("O32", features=64)._is_production_config(256)
-    assert not make("signs", fwd_rr="O32")._is_production_config(256)
+    fwd_dense = make("signs", fwd_rr="O32")
+    assert fwd_dense._is_production_config(256)                  # a Hadamard matrix until re_randomize draws the dense one
+    fwd_dense.weight_quantizer.re_randomize()
+    assert fwd_dense.weight_quantizer.is_dense and fwd_dense._is_production_config(256) and fwd_dense._is_production_config(160)
+    fwd_dense64 = q.QuantizedLinear(256, 256, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(hadamard_dim=64, rerotate="O32"),
+                                    activation_quantizer=q.QuestMXFP4Quantizer(hadamard_dim=64),
+                                    gradient_quantizer=q.AlbertTsengQuantizer(stochastic=True),
+                                    backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]())
+    assert fwd_dense64._is_production_config(256)
+    fwd_dense64.weight_quantizer.re_randomize()
+    assert not fwd_dense64._is_production_config(256)
     dense64 = make("O32")
     dense64.backward_scheme.g_quantizer.hadamard_dim = 64
     assert not dense64._is_production_config(256)
