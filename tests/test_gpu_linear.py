@@ -374,6 +374,40 @@ def test_layer_with_dense_forward_rotation(oracle, q, dense, dtype, shape):
     assert rel(gx_mod, gx) < 1.0 and rel(gw_mod, gw) < 1.0
 
 
+@pytest.mark.parametrize("dense", ["x", "w", "xw"])
+def test_dense_forward_rotation_under_autocast(q, dense):
+    """fp32 master weights under bf16 autocast (the Llama configurations) with dense forward rotations and a deterministic
+    backward: the packed path and the module path (quantizer modules, de-quantized tensors, library products) agree on
+    the output and on both gradients to the bf16 roundings they place differently; gradients keep the parameters' dtypes."""
+    print(f"case dense forward rotation under autocast, dense={dense}", flush=True)
+    T, I, O = 256, 384, 256
+    x = make_input(T, I, torch.float32, seed=1, outlier_frac=0.01)
+    w = make_input(O, I, torch.float32, seed=2, outlier_frac=0, scale=0.02)
+    dy = make_input(T, O, torch.bfloat16, seed=3, outlier_frac=0, scale=1e-3)
+    layer = production_layer(q, I, O, False, None, torch.float32)
+    torch.manual_seed(7)
+    for name, quantizer in (("x", layer.activation_quantizer), ("w", layer.weight_quantizer)):
+        if name in dense:
+            quantizer.rerotate = "O32"
+            quantizer.re_randomize()
+    with torch.no_grad():
+        layer.weight.copy_(w.to("cuda:0"))
+    outs = []
+    for packed in (True, False):
+        layer.use_packed_path = packed
+        layer.weight.grad = None
+        xd = x.to("cuda:0").requires_grad_(True)
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):   # around forward and backward, as the training loop has it
+            y = layer(xd)
+            y.backward(dy.to("cuda:0"))
+        assert y.dtype == torch.bfloat16 and xd.grad.dtype == torch.float32 and layer.weight.grad.dtype == torch.float32
+        outs.append((y.detach().float().cpu().numpy(), xd.grad.cpu().numpy(), layer.weight.grad.cpu().numpy()))
+    layer.use_packed_path = True
+    assert layer._is_production_config(T)
+    for got, want, tol in zip(outs[0], outs[1], (6e-3, 2e-2, 2e-2)):
+        assert rel(got, want) <= tol
+
+
 def test_packed_weight_cache_across_micro_steps(q):
     """With the cache on, the second micro-step reuses the packed Q(W) of the first: outputs and gradients are
     bit-identical to a layer that quantizes every time, the buffer saved by an earlier graph survives a weight
