@@ -19,8 +19,8 @@
 //                              last block of four K steps repeats (muted) at most a third as many steps as K has.
 //                              Persistent, 256x256 macro tile, 4 waves x 128x128, operands global -> LDS directly into a
 //                              4-stage ring, scales in blocks of four K steps, row-major or tiled code bytes, optional split-K.
-//   gemm_mxfp4_tn_duo_kernel   same M, N, K % 128 == 0 and K <= 768: 256x128 tiles, two workgroups per CU hiding each
-//                              other's tile boundaries, scales per K step.
+//   gemm_mxfp4_tn_duo_kernel   same M, N, K % 128 == 0 and K <= 768, or K % 128 == 64 (row-major operands, any K >= 192):
+//                              256x128 tiles, two workgroups per CU hiding each other's tile boundaries, scales per K step.
 //   gemm_mxfp4_tn_kernel       any M, N and K % 32 == 0: 128x128 macro tile, 4 waves x 64x64, operands staged
 //                              global -> registers -> LDS (rows padded from 64 to 80 bytes so the 16-byte fragment
 //                              reads of 16 consecutive rows hit 64 distinct banks), double buffered.
@@ -358,7 +358,8 @@ __device__ __forceinline__ void big_mfma_sub(const SubFrags& f, const uint32_t (
 // fragment reads and global -> LDS bytes), which is why long contractions stay on the 256 x 256 kernel.
 // Three-stage ring per workgroup (3 x 25.5 KiB: codes of 256 + 128 rows and one scale dword per row and K step); the
 // ring doubles as the epilogue's staging area, so nothing is prefetched across tiles -- the neighbour workgroup covers
-// the gap.  Persistent: the grid is two workgroups per CU.  M, N multiples of 64, M >= 256, N >= 128, K % 128 == 0.
+// the gap.  Persistent: the grid is two workgroups per CU.  M, N multiples of 64, M >= 256, N >= 128, K % 128 == 0, or
+// K % 128 == 64 with row-major operands (a final half step, see duo_issue).
 constexpr int kDuoM = 256, kDuoN = 128, kDuoStages = 3;
 constexpr int kDuoBOff = kDuoM * kRowBytes;                                   // 16 KiB of A codes
 constexpr int kDuoSAOff = (kDuoM + kDuoN) * kRowBytes;                        // 24 KiB of codes
@@ -383,17 +384,24 @@ struct DuoPlan {
     const uint8_t* sb;
     int64_t row16_bytes;
     uint32_t lane_codes_a, lane_codes_b;
+    uint32_t half_codes_a, half_codes_b;  // the same for a final half step (K % 128 == 64): the row's last 32 bytes twice
     int kstep_a, kstep_b;
     uint32_t lds_a, lds_b, lds_sa, lds_sb;  // wave-uniform LDS addresses (stage 0)
 };
-__device__ __forceinline__ void duo_issue(const DuoPlan& p, int stage, int ks) {
+// half: the step covers only 64 contraction indices (the last step of a K with K % 128 == 64, row-major operands).  Its
+// lanes request the row's final two 16-byte pieces in place of all four, and the scale dword that ends with the row's last
+// byte (two bytes early), so that no request leaves the row; the consumer shifts that dword down by 16 bits, which puts
+// the two real scale bytes first and zeros (2^-127: products vanish) where the missing half of the step would be.
+__device__ __forceinline__ void duo_issue(const DuoPlan& p, int stage, int ks, bool half) {
     const uint32_t off = (uint32_t)stage * kDuoStageBytes;
+    const uint32_t la = half ? p.half_codes_a : p.lane_codes_a, lb = half ? p.half_codes_b : p.lane_codes_b;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) load_lds_b128_s(p.a + j * p.row16_bytes + ks * p.kstep_a, p.lane_codes_a, p.lds_a + off + j * 1024);
+    for (int j = 0; j < 4; ++j) load_lds_b128_s(p.a + j * p.row16_bytes + ks * p.kstep_a, la, p.lds_a + off + j * 1024);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) load_lds_b128_s(p.b + j * p.row16_bytes + ks * p.kstep_b, p.lane_codes_b, p.lds_b + off + j * 1024);
-    load_lds_b32(p.sa + ks * 4, p.lds_sa + off);
-    load_lds_b32(p.sb + ks * 4, p.lds_sb + off);
+    for (int j = 0; j < 2; ++j) load_lds_b128_s(p.b + j * p.row16_bytes + ks * p.kstep_b, lb, p.lds_b + off + j * 1024);
+    const int sback = half ? 2 : 0;
+    load_lds_b32(p.sa + ks * 4 - sback, p.lds_sa + off);
+    load_lds_b32(p.sb + ks * 4 - sback, p.lds_sb + off);
 }
 __device__ __forceinline__ void duo_read_sub(const uint8_t* __restrict__ stage, int a_off, int b_off, DuoFrags& f) {
 #pragma unroll
@@ -439,7 +447,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int lrow = lane & 31, half = lane >> 5;
     const int tiles_m = (M + kDuoM - 1) / kDuoM, tiles_n = (N + kDuoN - 1) / kDuoN, total = tiles_m * tiles_n;
     const int code_pitch = K / 2, groups = K / 32;
-    const int nk = K / kBK;
+    const int nk = (K + kBK - 1) / kBK;
+    const int half_step = (K % kBK) ? nk - 1 : -1;  // the K step that covers only 64 indices (K % 128 == 64), or none
 
     const int swz = (lrow >> 2) & 3;
     const int a_off0 = (wm * 128 + lrow) * kRowBytes + (((2 * half) ^ swz) * 16);
@@ -461,6 +470,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const uint32_t tiled_off = (uint32_t)(prow * 64 + pcv * 16);
         plan.lane_codes_a = a_tiled ? tiled_off : rowmajor_off;
         plan.lane_codes_b = b_tiled ? tiled_off : rowmajor_off;
+        // a half step exists for row-major operands only: pieces 2 and 3 of the step lie beyond the row, their LDS slots
+        // receive pieces 0 and 1 again (and zero scales)
+        plan.half_codes_a = plan.half_codes_b = (uint32_t)(prow * code_pitch + (pcv & 1) * 16);
         plan.kstep_a = a_tiled ? 1024 : kRowBytes;
         plan.kstep_b = b_tiled ? 1024 : kRowBytes;
         plan.lds_a = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_base + wave * 4096));
@@ -492,14 +504,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         const int rows_valid = (int)(M - m0) - wm * 128, cols_valid = (int)(N - n0) - wn * 64;
 
-        duo_issue(plan, 0, 0);
-        duo_issue(plan, 1, nk > 1 ? 1 : 0);
-        duo_issue(plan, 2, nk > 2 ? 2 : nk - 1);
+        const auto issue = [&](int stage, int ks) { duo_issue(plan, stage, ks, ks == half_step); };
+        // the scale dwords of a half step arrive two bytes early (see duo_issue).  Without a branch: a K step is one basic
+        // block, which is what holds its instruction order in place.
+        const auto settle_scales = [&](uint4& a, uint2& b, int ks) {
+            const uint32_t down = ks == half_step ? 16u : 0u;
+            a.x >>= down; a.y >>= down; a.z >>= down; a.w >>= down;
+            b.x >>= down; b.y >>= down;
+        };
+        issue(0, 0);
+        issue(1, nk > 1 ? 1 : 0);
+        issue(2, nk > 2 ? 2 : nk - 1);
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(2 * kDuoLoads));  // step 0 is in; steps 1, 2 may be pending
         __syncthreads();
         DuoFrags f0, f1;
         uint4 sa4 = *reinterpret_cast<const uint4*>(smem_bytes + a_sc_off);
         uint2 sb2 = *reinterpret_cast<const uint2*>(smem_bytes + b_sc_off);
+        settle_scales(sa4, sb2, 0);
         duo_read_sub(smem_bytes, a_off0, b_off0, f0);
 
         v16f acc[4][2];
@@ -522,9 +543,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             __syncthreads();
             __builtin_amdgcn_sched_barrier(0);
             // past the end: a repeat nobody reads keeps the counts of outstanding loads uniform
-            duo_issue(plan, stage, s + 3 < nk ? s + 3 : nk - 1);
+            issue(stage, s + 3 < nk ? s + 3 : nk - 1);
             sa4 = *reinterpret_cast<const uint4*>(nxt + a_sc_off);
             sb2 = *reinterpret_cast<const uint2*>(nxt + b_sc_off);
+            settle_scales(sa4, sb2, s + 1);
             duo_read_sub(nxt, a_off0, b_off0, f0);
             duo_mfma_sub<1, SWAP, false>(f1, sca, scb, acc);
             QM_SCHED_PAIR(0x100, 6)
@@ -1177,6 +1199,16 @@ hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const 
     const int64_t nk_real = K / kBK, nk_pad = (nk_real + 3) & ~(int64_t)3;
     const bool persistent_ok = K % 512 == 0 ? ((reinterpret_cast<uintptr_t>(a_scales) | reinterpret_cast<uintptr_t>(b_scales)) & 15) == 0
                                             : (nk_real >= 4 && (nk_pad - nk_real) * 3 <= nk_real);
+    // K % 128 == 64 (the 30 M Llama's hidden width 1728): the two-workgroup kernel closes such a contraction with a half
+    // step.  Row-major operands (the tiled layout does not exist for these K); a c that is only 4-byte aligned, which the
+    // interface accepts at these shapes, stays on the generic kernel.
+    const bool half_ok = !at && !bt && K % kBK == 64 && K >= 192 && gemm_supports_tiled(M, N, K - 64) &&
+                         (reinterpret_cast<uintptr_t>(c) & 15) == 0;
+    if (half_ok) {
+        const int cus = device_cus();
+        if (c_dtype == BF16) return launch_duo<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, 0, 0, cus, stream);
+        return launch_duo<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, 0, 0, cus, stream);
+    }
     if (big_ok && (K <= kDuoMaxK || !persistent_ok)) {
         // short contraction: two 256 x 128 workgroups per CU hide each other's tile boundaries (also the fallback for scale
         // arrays that are not 16-byte aligned, which the persistent kernel's 16-byte scale requests need when K % 512 == 0)

@@ -182,7 +182,8 @@ def _random_operand(K, rows, cols, seed, mode, dev, tiled=True):
 # the three products of the isolated layer at out = 4096 and out = 11008 (forward, grad-input, grad-weight: M x N x K)
 GEMM_SHAPES = [(T, 4096, I), (4096, I, T), (T, 11008, I), (T, I, 11008), (11008, I, T)]
 # forward / grad-input products of the two Llama configurations (32768 tokens): short contractions on the 256 x 128
-# kernel (K = 640 and 1536, with N = 1728 hanging over a tile edge), K = 1728 (not a multiple of 128) on the generic one
+# kernel (K = 640, with N = 1728 hanging over a tile edge; K = 1728 = 13.5 steps of 128 closes with a half step), K = 1536 and
+# 1920 on the persistent one
 GEMM_SHAPES += [(32768, 3456, 640), (32768, 1728, 640), (32768, 640, 1728), (32768, 4608, 1536), (32768, 640, 1920)]
 
 

@@ -96,7 +96,10 @@ def _torch_dequant(codes, scales):
                                     # zero-scale steps: three, two and one real steps in the last block; one tile and many
                                     (512, 768, 1920), (4352, 4608, 3840), (320, 256, 3712), (768, 512, 2944), (4608, 4352, 1920),
                                     # few output tiles, long K: cut into K ranges (split-K) when scratch is offered
-                                    (512, 256, 8192), (320, 640, 16384), (1920, 640, 4096)])
+                                    (512, 256, 8192), (320, 640, 16384), (1920, 640, 4096),
+                                    # K % 128 == 64 (row-major operands): a final half step on the 256x128 kernel; one tile,
+                                    # tiles over the edge, one and a half K steps, the 30 M Llama's hidden width
+                                    (256, 256, 192), (512, 384, 1728), (320, 448, 320), (4352, 640, 1728), (1216, 4160, 704)])
 @pytest.mark.parametrize("exact", [True, False])
 def test_gemm_tile_kernels(oracle, K, M, N, K_, exact):
     print(f"case gemm tiles {M}x{N}x{K_} exact={exact}", flush=True)
