@@ -289,15 +289,16 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // compiler's wait-count insertion treats every LDS read as possibly aliasing an outstanding
 // global_load_lds and would drain all loads (vmcnt(0)) before each fragment read, which defeats the
 // prefetch ring; the kernel waits explicitly for the one tile it is about to read instead.
-// LDS destination = lds_base (wave-uniform, via M0) + lane * size.
+// LDS destination = lds_base (wave-uniform, via M0) + lane * size.  The "memory" clobber tells the compiler what it cannot
+// see in the statement: that it writes LDS, so no fragment read may be moved across it (costs nothing measurable).
 // addressed as uniform 64-bit base (SGPR pair) + per-lane 32-bit byte offset: no 64-bit VGPR address math
 __device__ __forceinline__ void load_lds_b128_s(const uint8_t* base, uint32_t lane_off, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(lds_base));
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(lds_base) : "memory");
 }
 // s_waitcnt immediate that waits for the vector-memory counter only
 constexpr int vmcnt_imm(int n) { return 0x0f70 | (n & 0xf) | ((n >> 4) << 14); }
 __device__ __forceinline__ void load_lds_b32(const uint8_t* gsrc, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gsrc), "s"(lds_base));
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gsrc), "s"(lds_base) : "memory");
 }
 
 struct SubFrags {
@@ -648,7 +649,7 @@ __device__ __forceinline__ void set_lds_dma_base(uint32_t lds_base) {
 }
 template <int I>
 __device__ __forceinline__ void load_lds_b128_m0(const uint8_t* base, uint32_t lane_off) {
-    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(lane_off), "s"(base), "i"(I * 1024));
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(lane_off), "s"(base), "i"(I * 1024) : "memory");
 }
 
 struct ScaleRegs {
