@@ -103,8 +103,9 @@ def time_kernel_cold(make_call, inputs, reps=24, warmup=2):
 
 
 def kernel_breakdown(x, w, dy, only_gemms=False):
-    """Per-kernel timings of the eleven launches of one step, with algorithmic bytes / flops.  HBM-bound kernels
-    are timed HBM-cold (see time_kernel_cold) and, for reference, warm on one buffer."""
+    """Per-kernel timings of the launches of one step, with algorithmic bytes / flops ("in_step": false marks a kernel
+    the step does not run at this shape, timed for comparison).  HBM-bound kernels are timed HBM-cold (see
+    time_kernel_cold) and, for reference, warm on one buffer."""
     from quartet_amd import kernels as K
     T, I, O = x.shape[0], x.shape[1], w.shape[0]
     out = {}
@@ -118,6 +119,17 @@ def kernel_breakdown(x, w, dy, only_gemms=False):
     xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=4, tiled_in=tl, tiled_out=tl)
     gxq = K.gemm_mxfp4_tn(ec, es, wtc, wts, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl)
     gwq = K.gemm_mxfp4_tn(etc, ets, xtc, xts, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl)
+    d2 = K.FOUR_THIRDS ** 2
+    # the two gradient products as the layer step runs them at this shape: the masked inverse rotation (B7 / B8) in the epilogue
+    fused = K.gemm_fuses_rotation(es, wts, T, I, O) and K.gemm_fuses_rotation(ets, xts, O, I, T)
+
+    def dgrad():
+        return (K.gemm_mxfp4_tn_rotated(ec, es, wtc, wts, xm, d2, torch.bfloat16, None, a_tiled=tl, b_tiled=tl) if fused
+                else K.gemm_mxfp4_tn(ec, es, wtc, wts, d2, torch.bfloat16, a_tiled=tl, b_tiled=tl))
+
+    def wgrad():
+        return (K.gemm_mxfp4_tn_rotated(etc, ets, xtc, xts, wm, d2, torch.bfloat16, None, a_tiled=tl, b_tiled=tl) if fused
+                else K.gemm_mxfp4_tn(etc, ets, xtc, xts, d2, torch.bfloat16, a_tiled=tl, b_tiled=tl))
 
     def hbm(name, elems, bytes_per_elem, make_call, inputs):
         cold = time_kernel_cold(make_call, inputs)
@@ -129,16 +141,25 @@ def kernel_breakdown(x, w, dy, only_gemms=False):
         ms = time_kernel(fn)
         out[name] = {"ms": round(ms, 4), "TFLOPs": round(2.0 * m * n * k / ms / 1e9, 1), "shape": [m, n, k]}
 
-    if only_gemms:
+    def products():
         mfma("gemm_fwd", T, O, I, lambda: K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
-        mfma("gemm_dgrad", T, I, O, lambda: K.gemm_mxfp4_tn(ec, es, wtc, wts, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
-        mfma("gemm_wgrad", O, I, T, lambda: K.gemm_mxfp4_tn(etc, ets, xtc, xts, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
+        mfma("gemm_dgrad", T, I, O, dgrad)
+        mfma("gemm_wgrad", O, I, T, wgrad)
+        if fused:
+            for k in ("gemm_dgrad", "gemm_wgrad"):
+                out[k]["epilogue"] = "masked inverse rotation (hadamard_bwd) fused"
+            mfma("gemm_dgrad_plain", T, I, O, lambda: K.gemm_mxfp4_tn(ec, es, wtc, wts, d2, torch.bfloat16, a_tiled=tl, b_tiled=tl))
+            mfma("gemm_wgrad_plain", O, I, T, lambda: K.gemm_mxfp4_tn(etc, ets, xtc, xts, d2, torch.bfloat16, a_tiled=tl, b_tiled=tl))
+            for k in ("gemm_dgrad_plain", "gemm_wgrad_plain"):
+                out[k]["in_step"] = False
+
+    if only_gemms:
+        products()
         return out
     hbm("quantize_x_quest_rtn_mask", T * I, 2.65625,
         lambda a: (lambda: K.quantize_mxfp4(a, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)), [x])
     hbm("quantize_w_quest_rtn_mask", O * I, 2.65625,
         lambda a: (lambda: K.quantize_mxfp4(a, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)), [w])
-    mfma("gemm_fwd", T, O, I, lambda: K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
     hbm("quantize_e_absmax_sr", T * O, 2.53125,
         lambda a: (lambda: K.quantize_mxfp4(a, 32, signs, K.QM_ABSMAX_SR, seed=1, tiled=tl)), [dy])
     hbm("quantize_et_absmax_sr_transposed", T * O, 2.53125,
@@ -151,26 +172,34 @@ def kernel_breakdown(x, w, dy, only_gemms=False):
         lambda c, sc: (lambda: K.requantize_transposed_mxfp4(c, sc, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=4,
                                                               tiled_in=tl, tiled_out=tl)),
         [xc, xs])
-    mfma("gemm_dgrad", T, I, O, lambda: K.gemm_mxfp4_tn(ec, es, wtc, wts, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
-    mfma("gemm_wgrad", O, I, T, lambda: K.gemm_mxfp4_tn(etc, ets, xtc, xts, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
+    products()
+    # the stand-alone inverse rotation: in the step only where the products' epilogue does not carry it
     hbm("hadamard_bwd_x", T * I, 4.125,
         lambda g, m: (lambda: K.masked_hadamard_bwd(g, 32, torch.bfloat16, None, m)), [gxq, xm])
     hbm("hadamard_bwd_w", O * I, 4.125,
         lambda g, m: (lambda: K.masked_hadamard_bwd(g, 32, torch.bfloat16, None, m)), [gwq, wm])
+    for k in ("hadamard_bwd_x", "hadamard_bwd_w"):
+        out[k]["in_step"] = not fused
     return out
 
 
-def in_step_gemm_ms_by_difference(x, w, dy, steps=10, rounds=5):
+def in_step_gemm_ms_by_difference(x, w, dy, fused, steps=10, rounds=5):
     """Mean duration of the three products inside the layer step, from two HIP graphs timed with events: the step's
-    eleven kernels launched one by one in the layer's order (`steps` times), and the same sequence without the three
+    kernels launched one by one in the layer's order (`steps` times), and the same sequence without the three
     products.  The difference of the two replays is what the step pays for its products where they actually run --
-    between quantizer kernels -- with no event or host time inside the measured interval."""
+    between quantizer kernels -- with no event or host time inside the measured interval.  `fused`: the two gradient
+    products carry the masked inverse rotation in their epilogue, as the layer runs them where the kernel serves the
+    shape (the step then has no inverse-rotation kernels); otherwise plain products and the two rotation kernels."""
     from quartet_amd import kernels as K
     tl, signs = True, 0x5A5AA5A5
 
     def one_step(full):
-        def product(ac, as_, bc, bs, alpha):
-            return K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha, torch.bfloat16, a_tiled=tl, b_tiled=tl) if full else None
+        def product(ac, as_, bc, bs, alpha, mask=None):
+            if not full:
+                return None
+            if mask is not None and fused:
+                return K.gemm_mxfp4_tn_rotated(ac, as_, bc, bs, mask, alpha, torch.bfloat16, None, a_tiled=tl, b_tiled=tl)
+            return K.gemm_mxfp4_tn(ac, as_, bc, bs, alpha, torch.bfloat16, a_tiled=tl, b_tiled=tl)
         xc, xs, xm, _ = K.quantize_mxfp4(x, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)
         wc, ws, wm, _ = K.quantize_mxfp4(w, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)
         product(xc, xs, wc, ws, 1.0)
@@ -178,10 +207,11 @@ def in_step_gemm_ms_by_difference(x, w, dy, steps=10, rounds=5):
         etc, ets, _, _ = K.quantize_mxfp4(dy, 32, signs, K.QM_ABSMAX_SR, transposed_in=True, seed=2, tiled=tl)
         wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=3, tiled_in=tl, tiled_out=tl)
         xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=4, tiled_in=tl, tiled_out=tl)
-        gxq = product(ec, es, wtc, wts, K.FOUR_THIRDS ** 2)
-        gwq = product(etc, ets, xtc, xts, K.FOUR_THIRDS ** 2)
-        K.masked_hadamard_bwd(gxq if full else x, 32, torch.bfloat16, None, xm)
-        K.masked_hadamard_bwd(gwq if full else w, 32, torch.bfloat16, None, wm)
+        gxq = product(ec, es, wtc, wts, K.FOUR_THIRDS ** 2, xm)
+        gwq = product(etc, ets, xtc, xts, K.FOUR_THIRDS ** 2, wm)
+        if not fused:
+            K.masked_hadamard_bwd(gxq if full else x, 32, torch.bfloat16, None, xm)
+            K.masked_hadamard_bwd(gwq if full else w, 32, torch.bfloat16, None, wm)
 
     graphs = {}
     for full in (True, False):
@@ -357,21 +387,35 @@ def gemm_tile_phases(x, w, launches=5):
     for _ in range(40):   # the state the chip is in during the step: clocks settled under this kernel
         K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.bfloat16, a_tiled=True, b_tiled=True)
     ksteps = x.shape[1] // 128
-    k_loop, epi, span = [], [], []
-    for _ in range(launches):
-        _, st = K.gemm_tile_phases(xc, xs, wc, ws, 1.0, a_tiled=True, b_tiled=True)
-        st = st.tolist()
-        for row in st:
-            start = row[1]
-            for i in range(2, len(row) - 1, 2):
-                if row[i] == 0:
-                    break
-                k_loop.append(row[i] - start)
-                epi.append(row[i + 1] - row[i])
-                start = row[i + 1]
-        span.append(max(max(r) - r[0] for r in st))   # per workgroup: the XCDs' counters are not aligned with each other
+
+    def stamps(maskbits):
+        k_loop, epi, span = [], [], []
+        for _ in range(launches):
+            _, st = K.gemm_tile_phases(xc, xs, wc, ws, 1.0, a_tiled=True, b_tiled=True, maskbits=maskbits)
+            st = st.tolist()
+            for row in st:
+                start = row[1]
+                for i in range(2, len(row) - 1, 2):
+                    if row[i] == 0:
+                        break
+                    k_loop.append(row[i] - start)
+                    epi.append(row[i + 1] - row[i])
+                    start = row[i + 1]
+            span.append(max(max(r) - r[0] for r in st))   # per workgroup: the XCDs' counters are not aligned with each other
+        return k_loop, epi, span, st
+
+    k_loop, epi, span, st = stamps(None)
     kl, ep = statistics.median(k_loop), statistics.median(epi)
-    return {"what": "shader-clock stamps of the forward product's kernel, medians over every tile of %d launches" % launches,
+    # the same launch with the masked inverse rotation in the epilogue (as the step's two gradient products run), on a mask
+    # of the output's shape
+    rot = {}
+    if K.gemm_fuses_rotation(xs, ws, x.shape[0], w.shape[0], x.shape[1]):
+        g = torch.Generator(device=x.device).manual_seed(3)
+        keep = torch.randint(0, 256, (x.shape[0], w.shape[0] // 8), generator=g, dtype=torch.uint8, device=x.device)
+        rk, re_, rs, _ = stamps(keep)
+        rot = {"with_inverse_rotation": {"cycles_per_k_step": round(statistics.median(rk) / ksteps, 1), "epilogue_cycles": int(statistics.median(re_)),
+                                         "longest_workgroup_cycles": int(statistics.median(rs))}}
+    return {"what": "shader-clock stamps of the forward product's kernel, medians over every tile of %d launches" % launches, **rot,
             "tiles_per_workgroup": len(k_loop) // max(1, launches * len(st)),
             "k_loop_cycles": int(kl), "cycles_per_k_step": round(kl / ksteps, 1), "epilogue_cycles": int(ep),
             "epilogue_share_of_tile": round(ep / (kl + ep), 4),
@@ -911,16 +955,28 @@ def main():
         # as an unbroken chain of its own launches: that holds the chip at its power limit throughout and is the slowest
         # setting for this kernel (5-10 % longer).
         chain_ms, chain_tf = gemm_summary(kb, T_TOKENS, out_f)
-        diff = in_step_gemm_ms_by_difference(x.detach(), w, dy)
+        fused = "epilogue" in kb["gemm_dgrad"]
+        diff = in_step_gemm_ms_by_difference(x.detach(), w, dy, fused)
         gemm_ms = diff.pop("ms")
         gemm_tf = 2.0 * T_TOKENS * IN_F * out_f / gemm_ms / 1e9
         traffic, source = _traffic_entry(prof, "gemm_mxfp4_tn")
+        what = "mean of the step's three products, timed inside the step"
+        if fused:
+            what += ("; the two gradient products carry the masked inverse rotation in their epilogue (flops counted: the product's "
+                     "2 M N K only), so the step has no inverse-rotation kernels")
         result["roofline"] = {"bound": "mfma", "kernel": f"gemm_mxfp4_tn ({T_TOKENS}x{out_f}x{IN_F}, {T_TOKENS}x{IN_F}x{out_f}, {out_f}x{IN_F}x{T_TOKENS})",
                               "achieved": round(gemm_tf, 1), "peak": PEAK_FP4_TFLOPS, "unit": "TFLOP/s",
                               "frac": round(gemm_tf / PEAK_FP4_TFLOPS, 4), "traffic": traffic, "traffic_source": source,
-                              "avg_launch_ms": round(gemm_ms, 4), "how": {"what": "mean of the step's three products, timed inside the step", **diff},
+                              "avg_launch_ms": round(gemm_ms, 4), "how": {"what": what, **diff},
                               "back_to_back": {"avg_launch_ms": round(chain_ms, 4), "TFLOPs": round(chain_tf, 1),
                                                "frac": round(chain_tf / PEAK_FP4_TFLOPS, 4)}}
+        if fused:
+            # the same measurement on the composition without the fusion: three plain products and two rotation kernels
+            plain = in_step_gemm_ms_by_difference(x.detach(), w, dy, False)
+            p_ms = plain.pop("ms")
+            p_tf = 2.0 * T_TOKENS * IN_F * out_f / p_ms / 1e9
+            result["roofline"]["plain_products"] = {"avg_launch_ms": round(p_ms, 4), "TFLOPs": round(p_tf, 1), "frac": round(p_tf / PEAK_FP4_TFLOPS, 4),
+                                                    "how": {"what": "three plain products in a step that rotates with kernels of its own", **plain}}
         qk = kb["quantize_x_quest_rtn_mask"]
         traffic, source = _traffic_entry(prof, "quantize_x_quest_rtn_mask_alone")
         result["roofline_quantize"] = {"bound": "hbm", "kernel": f"quantize_rowmajor (quest RTN + mask, {T_TOKENS}x{IN_F} bf16)",

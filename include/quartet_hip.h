@@ -184,13 +184,34 @@ int64_t qm_diag_mfma_only(const uint8_t* operands, size_t operand_bytes, float* 
  * per workgroup into `stamps` (DEVICE memory, stamps_bytes >= workgroups * QM_DIAG_PHASE_STAMPS * 8; one workgroup per
  * CU or per tile, whichever is fewer).  Where the time of a tile goes -- K steps against the epilogue, during which no
  * matrix instruction runs -- is read from the differences; bench.py --gemm-phases prints them.  c receives the product.
+ * maskbits (optional, [M, N/8], 4-byte aligned): stamp the instantiation whose epilogue carries the masked inverse rotation
+ * of qm_gemm_mxfp4_tn_rotated (no sign flips, bf16 scale); c then receives the rotated product.
  * Serves M, N multiples of 64 and >= 256, K % 512 == 0.  Returns the number of workgroups launched, or a negative
  * status.
  */
 #define QM_DIAG_PHASE_STAMPS 32
 int qm_diag_gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
-                             int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout, uint64_t* stamps,
-                             size_t stamps_bytes, void* stream);
+                             int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout,
+                             const uint8_t* maskbits, uint64_t* stamps, size_t stamps_bytes, void* stream);
+
+/*
+ * c = masked inverse rotation of (alpha * A B^T): qm_gemm_mxfp4_tn with a bf16 result followed by qm_masked_hadamard_bwd
+ * (Hadamard block 32 along N, bf16 in and out), the pair a gradient product and the forward quantizer's straight-through
+ * backward form in the layer's backward pass (src/models/quantization/backward.py:62,71-83 feeding
+ * quantizers/mxfp4.py:143-146), as ONE launch: the persistent product kernel rounds its tile to bf16, multiplies it by the
+ * mask and rotates it on the matrix pipe before storing it, so the rotated-basis gradient never travels through memory.
+ * Same values as the two calls except that a group's 32 terms are added in the matrix instruction's order (fp32 sums of
+ * bf16 values: a few results in 10^4 differ in the last bf16 bit).
+ *   maskbits     [M, N/8] clip-mask bits of the forward quantizer (bit n % 8 of byte n / 8), 4-byte aligned; sign_bits,
+ *                scale_dtype as for qm_masked_hadamard_bwd with hadamard_dim 32
+ *   Served shapes: those of the persistent kernel without a cut into K ranges -- qm_gemm_fuses_rotation() tells (M, N
+ *   multiples of 64 and >= 256, K % 128 == 0 and > 768, scale arrays 16-byte aligned when K % 512 == 0, few enough output
+ *   tiles that no workspace would be used); anything else returns QM_ERR_INVALID and the caller makes the two calls.
+ */
+int qm_gemm_fuses_rotation(const uint8_t* a_scales, const uint8_t* b_scales, int64_t M, int64_t N, int64_t K);
+int qm_gemm_mxfp4_tn_rotated(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
+                             int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout,
+                             const uint8_t* maskbits, const uint32_t* sign_bits, int scale_dtype, void* stream);
 
 /*
  * out = ((g * mask).view(-1, hd)) @ H^T: the straight-through backward of the forward quantizer,

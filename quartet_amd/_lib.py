@@ -29,6 +29,8 @@ EXPORTS = (
     "qm_gemm_noalloc_scratch_bytes",
     "qm_gemm_mxfp4_tn_noalloc",
     "qm_gemm_noalloc_prepare",
+    "qm_gemm_fuses_rotation",
+    "qm_gemm_mxfp4_tn_rotated",
     "qm_packed_operand_bytes",
     "qm_packed_operand_offsets",
     "qm_linear_backward_workspace_bytes",
@@ -76,7 +78,7 @@ def lib():
     L.qm_gemm_mxfp4_tn.restype = i32
     L.qm_gemm_mxfp4_tn.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, i32, vp, ctypes.c_size_t, vp]
     L.qm_diag_gemm_tile_phases.restype = i32
-    L.qm_diag_gemm_tile_phases.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, vp, ctypes.c_size_t, vp]
+    L.qm_diag_gemm_tile_phases.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, vp, vp, ctypes.c_size_t, vp]
     L.qm_diag_mfma_only.restype = i64
     L.qm_diag_mfma_only.argtypes = [vp, ctypes.c_size_t, vp, ctypes.c_size_t, i32, vp]
     L.qm_gemm_workspace_bytes.restype = ctypes.c_size_t
@@ -87,6 +89,10 @@ def lib():
     L.qm_gemm_mxfp4_bf16_nn.argtypes = [vp, vp, vp, i64, i64, i64, f32, vp, i32, vp]
     L.qm_gemm_noalloc_prepare.restype = i32
     L.qm_gemm_noalloc_prepare.argtypes = []
+    L.qm_gemm_fuses_rotation.restype = i32
+    L.qm_gemm_fuses_rotation.argtypes = [vp, vp, i64, i64, i64]
+    L.qm_gemm_mxfp4_tn_rotated.restype = i32
+    L.qm_gemm_mxfp4_tn_rotated.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, vp, vp, i32, vp]
     L.qm_gemm_mxfp4_tn_noalloc.restype = i32
     L.qm_gemm_mxfp4_tn_noalloc.argtypes = [vp, vp, vp, vp, i64, i64, i64, f32, vp, i32, i32, i32, vp]
     L.qm_masked_hadamard_bwd.restype = i32

@@ -44,7 +44,7 @@ qm::SignBits make_signs(const uint32_t* sign_bits, int hd) {
 
 extern "C" {
 
-int qm_version(void) { return 14; }
+int qm_version(void) { return 15; }
 
 const char* qm_last_error(void) { return g_last_error; }
 
@@ -172,13 +172,13 @@ int qm_gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint
 }
 
 int qm_diag_gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
-                             int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout, uint64_t* stamps,
-                             size_t stamps_bytes, void* stream) {
+                             int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout,
+                             const uint8_t* maskbits, uint64_t* stamps, size_t stamps_bytes, void* stream) {
     if (!a_codes || !a_scales || !b_codes || !b_scales || !c || !stamps || !aligned(a_codes, 16) || !aligned(b_codes, 16) ||
-        !aligned(c, 16) || !aligned(stamps, 8) || !valid_layout(a_layout) || !valid_layout(b_layout))
+        !aligned(c, 16) || !aligned(stamps, 8) || !aligned(maskbits, 4) || !valid_layout(a_layout) || !valid_layout(b_layout))
         return fail(QM_ERR_INVALID, "qm_diag_gemm_tile_phases: null, misaligned or ill-typed arguments");
     int grid = 0;
-    const hipError_t e = qm::gemm_tile_phases(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, a_layout, b_layout,
+    const hipError_t e = qm::gemm_tile_phases(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, a_layout, b_layout, maskbits,
                                               reinterpret_cast<unsigned long long*>(stamps), stamps_bytes, &grid,
                                               reinterpret_cast<hipStream_t>(stream));
     if (e == hipErrorInvalidValue && grid == 0)
@@ -291,6 +291,36 @@ int qm_masked_hadamard_bwd(const void* g, int g_dtype, int64_t rows, int64_t col
                                             make_signs(sign_bits, hadamard_dim), maskbits, out, out_dtype, false,
                                             reinterpret_cast<hipStream_t>(stream)),
                     "qm_masked_hadamard_bwd");
+}
+
+int qm_gemm_fuses_rotation(const uint8_t* a_scales, const uint8_t* b_scales, int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || K % 32) return 0;
+    // offered the workspace the plain product would use: a shape it would cut into K ranges is not served
+    const size_t ws = qm::gemm_workspace_bytes(M, N, K);
+    return ws == 0 && qm::gemm_will_rotate(a_scales, b_scales, M, N, K, QM_BF16, nullptr, 0) ? 1 : 0;
+}
+
+int qm_gemm_mxfp4_tn_rotated(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
+                             int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout,
+                             const uint8_t* maskbits, const uint32_t* sign_bits, int scale_dtype, void* stream) {
+    if (!valid_layout(a_layout) || !valid_layout(b_layout))
+        return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn_rotated: unknown layout %d / %d", a_layout, b_layout);
+    if (!valid_dtype(scale_dtype)) return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn_rotated: scale_dtype %d", scale_dtype);
+    if (M < 0 || N < 0 || K < 0) return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn_rotated: negative extent");
+    if (M == 0 || N == 0) return 0;
+    if (!c || !a_codes || !a_scales || !b_codes || !b_scales || !maskbits) return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn_rotated: null tensor");
+    if (!qm_gemm_fuses_rotation(a_scales, b_scales, M, N, K))
+        return fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn_rotated: shape M=%lld N=%lld K=%lld is not served with the rotation fused "
+                                    "(see qm_gemm_fuses_rotation); call qm_gemm_mxfp4_tn and qm_masked_hadamard_bwd",
+                    (long long)M, (long long)N, (long long)K);
+    if (!aligned(a_codes, 16) || !aligned(b_codes, 16) || !aligned(a_scales, 4) || !aligned(b_scales, 4) || !aligned(c, 16) || !aligned(maskbits, 4))
+        return fail(QM_ERR_UNALIGNED, "qm_gemm_mxfp4_tn_rotated: codes and c need 16-byte, scales and mask bits 4-byte alignment");
+    bool rotated = false;
+    const int rc = from_hip(qm::gemm_mxfp4_tn_rotated(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, QM_BF16, a_layout, b_layout,
+                                                      nullptr, 0, maskbits, sign_bits ? sign_bits[0] : 0u, scale_dtype, &rotated,
+                                                      reinterpret_cast<hipStream_t>(stream)), "qm_gemm_mxfp4_tn_rotated");
+    if (rc) return rc;
+    return rotated ? 0 : fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn_rotated: the product did not run as planned");
 }
 
 int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, int64_t C, float post, void* out,
@@ -515,14 +545,25 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
         const qm::RequantArgs rx{px + lx.c, px + lx.s, T, I, x_val_dtype, seeds[3], k + wl.xtc, k + wl.xts};
         rc = from_hip(qm::requantize_transposed_hd32_tiled_pair(rx, rw, sg, g_mode, seed_base, hs), "qm_linear_backward");
         if (rc) return rc;
-        rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, gx_product, mid_dtype, codes_layout,
-                              codes_layout, gws, wl.gemm_ws_bytes, stream);
+        // B3 + B7 and B6 + B8: where the product runs on the persistent kernel's bf16 epilogue, the masked inverse rotation is
+        // applied to the tile before it is stored and the product lands in gx / gw directly
+        const bool fuse_x = !gx_rotated && qm::gemm_will_rotate(k + wl.es, k + wl.wts, T, I, O, mid_dtype, gws, wl.gemm_ws_bytes);
+        const bool fuse_w = !gw_rotated && gw_dtype == mid_dtype &&
+                            qm::gemm_will_rotate(k + wl.ets, k + wl.xts, O, I, T, mid_dtype, gws, wl.gemm_ws_bytes);
+        bool done = false;
+        rc = from_hip(qm::gemm_mxfp4_tn_rotated(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, fuse_x ? gx : gx_product, mid_dtype,
+                                                codes_layout, codes_layout, gws, wl.gemm_ws_bytes, fuse_x ? px + lx.m : nullptr,
+                                                signs_x ? signs_x[0] : 0u, x_scale_dtype, &done, hs), "qm_linear_backward");
         if (rc) return rc;
-        rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, gw_product, mid_dtype, codes_layout,
-                              codes_layout, gws, wl.gemm_ws_bytes, stream);
+        if (done != fuse_x) return fail(QM_ERR_INVALID, "qm_linear_backward: the grad-input product did not run as planned");
+        rc = from_hip(qm::gemm_mxfp4_tn_rotated(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, fuse_w ? gw : gw_product, mid_dtype,
+                                                codes_layout, codes_layout, gws, wl.gemm_ws_bytes, fuse_w ? pw + lw.m : nullptr,
+                                                signs_w ? signs_w[0] : 0u, w_scale_dtype, &done, hs), "qm_linear_backward");
         if (rc) return rc;
-        if (gx_rotated) return rotate_gw();
-        if (gw_rotated)
+        if (done != fuse_w) return fail(QM_ERR_INVALID, "qm_linear_backward: the grad-weight product did not run as planned");
+        const bool need_x = !gx_rotated && !fuse_x, need_w = !gw_rotated && !fuse_w;
+        if (!need_x) return need_w ? rotate_gw() : 0;
+        if (!need_w)
             return qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, px + lx.m, gx, mid_dtype, stream);
         return from_hip(qm::masked_hadamard_bwd_hd32_pair(k + wl.gxq, T * I, x_scale_dtype,
                                                           signs_x ? signs_x[0] : 0u, px + lx.m, gx, k + wl.gwq, O * I,

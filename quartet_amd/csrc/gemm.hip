@@ -678,7 +678,7 @@ struct Big4State {
 // requests into the stage it has just freed, `soff` (Q = 0 only) the byte offset of the scale block it requests;
 // `sw` = 16, or 0 for a step whose scale bytes are to read as zero (2^-127: its products vanish); `par` selects the
 // scale buffer the current block lives in.
-template <int Q, bool SWAP, bool FIRST = false>
+template <int Q, bool SWAP, bool FIRST = false, int EXTRA = 0>
 __device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_bytes, int lks, int soff, int sw, int par, int a_off0,
                                           int a_off1, int b_off0, int b_off1, int a_sc_off, int b_sc_off, int sh,
                                           Big4State& st, v16f (&acc)[4][4]) {
@@ -694,7 +694,9 @@ __device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_by
     __builtin_amdgcn_sched_barrier(0);
     // loads younger than the codes of the next step: the codes of the two steps after it (16) and, for Q = 1, 2,
     // the two scale loads issued since; for Q = 3 the scale block read below is older than those and must be in
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm((Q == 1 || Q == 2) ? 18 : 16));
+    // EXTRA: requests of another kind issued since the awaited stage's (the fused epilogue's mask words, which a tile
+    // requests at its first K step and which may stay pending through its first three)
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(((Q == 1 || Q == 2) ? 18 : 16) + EXTRA));
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (Q == 3) big4_read_scales(smem_bytes + kScaleAreaOff + (par ^ 1) * kScaleBufBytes, a_sc_off, b_sc_off, st.sr);
@@ -743,9 +745,25 @@ __device__ __forceinline__ void big4_step(const Big4Plan& plan, uint8_t* smem_by
 // columns per wave through a private 4 KiB LDS stage outside the operand ring, so the next tile's operands
 // keep streaming in underneath; 16-byte chunks are XOR-swizzled by row so that writes and reads spread over
 // all banks.
+// ROT: the masked inverse Hadamard rotation of the layer's backward pass (groups of 32 along n) applied to the tile before it
+// is stored: out[m][n'] = c * sum_n (bf16(alpha * acc[m][n]) * keep[m][n]) * S[n'][n] * sign[n], S the 32 x 32 Sylvester
+// matrix.  With the operand roles swapped a lane holds 16 of a group's 32 n for one m, which is the layout the bf16
+// matrix instruction reads its second operand in (k along the registers, column = lane % 32); its first operand is the
+// +-1 matrix, rebuilt per tile from the sign word.  The sums are fp32 sums of bf16 values in the instruction's order
+// (the stand-alone kernel adds them as a butterfly), the factor c and the final rounding are the same.
+struct RotEpilogue {
+    const uint8_t* mask;  // [M][N / 8] clip-mask bits, bit n % 8 of byte n / 8
+    uint32_t signs;       // bit n: column n of the Hadamard block negated
+    float c;              // 32^-1/2, rounded to the scale dtype
+};
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <bool ROT = false>
 __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alpha, uint16_t* __restrict__ c, int64_t m0,
                                                    int64_t n0, int64_t N, int wm, int wn, int wave, int lane_in,
-                                                   uint8_t* smem_bytes, int rows_valid, int cols_valid) {
+                                                   uint8_t* smem_bytes, int rows_valid, int cols_valid,
+                                                   [[maybe_unused]] const RotEpilogue& rot, [[maybe_unused]] const u32x4 (&keep)[4],
+                                                   [[maybe_unused]] bool keep_shifted) {
     // The opaque copy keeps the address arithmetic below inside the (rarely executed) epilogue instead of being
     // hoisted out of the K loop, where it would hold dozens of registers across the MFMA schedule.
     // the lane index straight from the hardware, so that no copy of it has to stay alive through the K loop
@@ -760,6 +778,32 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
     const uint8_t* rd = region + rsub * 128 + ((chunk ^ rsub) * 16);  // rows rsub + 8k share rsub's swizzle
     const int64_t pitch8 = N * 16;                                   // eight rows of bf16
     uint8_t* out = reinterpret_cast<uint8_t*>(c + (m0 + wm * 128 + rsub) * N + n0 + wn * 128) + chunk * 16;
+    // ROT: `keep[i]` holds the four mask words of the lane's row in block row i (one per 32 x 32 block: its group of 32 n),
+    // requested at the tile's first K step.  The +-1 matrix: lane (n' = lane % 32, half h) holds, for instruction q,
+    // S[n'][n] sign[n] at n = 8 (2 q + rho) + 4 h + e
+    [[maybe_unused]] v8bf hmat[2];
+    // a factor c that bf16 holds exactly (the bf16 scale dtype) rides in the matrix entries: the products stay exact in fp32
+    // and the multiplication after the sums falls away
+    [[maybe_unused]] const bool c_in_matrix = ROT && (f2u(rot.c) & 0xffffu) == 0u;
+    if constexpr (ROT) {
+        const uint32_t one = c_in_matrix ? f2u(rot.c) >> 16 : 0x3f80u;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            uint32_t w[4];
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr) {   // pair pr: rho = pr / 2, e = 2 (pr % 2), +1
+                uint32_t bits = 0u;
+#pragma unroll
+                for (int k = 0; k < 2; ++k) {
+                    const int n = 8 * (2 * q + pr / 2) + 4 * half + 2 * (pr & 1) + k;
+                    const uint32_t neg = ((uint32_t)__builtin_popcount((uint32_t)(lrow & n)) ^ (rot.signs >> n)) & 1u;
+                    bits |= (one | (neg << 15)) << (16 * k);
+                }
+                w[pr] = bits;
+            }
+            hmat[q] = __builtin_bit_cast(v8bf, u32x4{w[0], w[1], w[2], w[3]});
+        }
+    }
     acc_settle();
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -767,16 +811,59 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
         for (int jp = 0; jp < 2; ++jp) {
             if (i * 32 >= rows_valid || jp * 64 >= cols_valid) continue;  // uniform: this pass lies outside the matrix
 #pragma unroll
-            for (int jj = 0; jj < 2; ++jj)
+            for (int jj = 0; jj < 2; ++jj) {
+                if constexpr (!ROT) {
 #pragma unroll
-                for (int b = 0; b < 4; ++b) {
+                    for (int b = 0; b < 4; ++b) {
+                        const v16f& t = acc[i][2 * jp + jj];
+                        const float t0 = acc_read(t[4 * b]), t1 = acc_read(t[4 * b + 1]), t2 = acc_read(t[4 * b + 2]), t3 = acc_read(t[4 * b + 3]);
+                        const v2bf p0 = __builtin_convertvector(v2f{t0 * alpha, t1 * alpha}, v2bf);
+                        const v2bf p1 = __builtin_convertvector(v2f{t2 * alpha, t3 * alpha}, v2bf);
+                        *reinterpret_cast<uint2*>(wr + (((jj * 4 + b) * 16) ^ wsw)) =
+                            make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
+                    }
+                } else {
                     const v16f& t = acc[i][2 * jp + jj];
-                    const float t0 = acc_read(t[4 * b]), t1 = acc_read(t[4 * b + 1]), t2 = acc_read(t[4 * b + 2]), t3 = acc_read(t[4 * b + 3]);
-                    const v2bf p0 = __builtin_convertvector(v2f{t0 * alpha, t1 * alpha}, v2bf);
-                    const v2bf p1 = __builtin_convertvector(v2f{t2 * alpha, t3 * alpha}, v2bf);
-                    *reinterpret_cast<uint2*>(wr + (((jj * 4 + b) * 16) ^ wsw)) =
-                        make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
+                    // the block rounded to bf16 and masked: register pair 2 b + k holds n = 8 b + 4 half + 2 k, + 1
+                    // the block's mask word: word j of the row's four, or word j + 2 where the wave requested the row's last
+                    // 16 bytes (its columns hang over the edge of N; blocks 2 and 3 are then outside and skipped)
+                    const uint32_t kword = keep_shifted ? keep[i][(2 * jp + jj + 2) & 3] : keep[i][2 * jp + jj];
+                    const uint32_t kw = kword >> (4 * half);
+                    uint32_t pk[8];
+#pragma unroll
+                    for (int b = 0; b < 4; ++b)
+#pragma unroll
+                        for (int k = 0; k < 2; ++k) {
+                            const float t0 = acc_read(t[4 * b + 2 * k]), t1 = acc_read(t[4 * b + 2 * k + 1]);
+                            const uint32_t p = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{t0 * alpha, t1 * alpha}, v2bf));
+                            const uint32_t lo = (uint32_t)__builtin_amdgcn_sbfe((int)kw, 8 * b + 2 * k, 1);       // 0 or ~0
+                            const uint32_t hi = (uint32_t)__builtin_amdgcn_sbfe((int)kw, 8 * b + 2 * k + 1, 1);
+                            pk[2 * b + k] = p & ((lo & 0xffffu) | (hi & 0xffff0000u));
+                        }
+                    v16f r;
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) r[e] = 0.0f;
+                    r = __builtin_amdgcn_mfma_f32_32x32x16_bf16(hmat[0], __builtin_bit_cast(v8bf, u32x4{pk[0], pk[1], pk[2], pk[3]}), r, 0, 0, 0);
+                    r = __builtin_amdgcn_mfma_f32_32x32x16_bf16(hmat[1], __builtin_bit_cast(v8bf, u32x4{pk[4], pk[5], pk[6], pk[7]}), r, 0, 0, 0);
+                    if (c_in_matrix) {
+#pragma unroll
+                        for (int b = 0; b < 4; ++b) {
+                            const v2bf p0 = __builtin_convertvector(v2f{r[4 * b], r[4 * b + 1]}, v2bf);
+                            const v2bf p1 = __builtin_convertvector(v2f{r[4 * b + 2], r[4 * b + 3]}, v2bf);
+                            *reinterpret_cast<uint2*>(wr + (((jj * 4 + b) * 16) ^ wsw)) =
+                                make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
+                        }
+                    } else {
+#pragma unroll
+                        for (int b = 0; b < 4; ++b) {
+                            const v2bf p0 = __builtin_convertvector(v2f{r[4 * b] * rot.c, r[4 * b + 1] * rot.c}, v2bf);
+                            const v2bf p1 = __builtin_convertvector(v2f{r[4 * b + 2] * rot.c, r[4 * b + 3] * rot.c}, v2bf);
+                            *reinterpret_cast<uint2*>(wr + (((jj * 4 + b) * 16) ^ wsw)) =
+                                make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
+                        }
+                    }
                 }
+            }
             // the region is private to the wave; LDS operations of one wave complete in order
 #pragma unroll
             for (int r8 = 0; r8 < 4; ++r8) {
@@ -808,11 +895,13 @@ __device__ __forceinline__ unsigned long long shader_clock() {
 // Persistent: the grid is one workgroup per CU (or fewer); each workgroup walks tiles bid, bid + grid, ... as one
 // flat stream of K steps.  The loads that refill a freed ring stage simply continue into the next tile, so the
 // pipeline never drains between tiles and the epilogue runs while the next tile's first four stages arrive.
-template <typename OutT, bool STAMP = false>
+template <typename OutT, bool STAMP = false, bool ROT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mxfp4_tn_big4_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ b_codes,
     const uint8_t* __restrict__ b_scales, int M, int N, int K, float alpha, OutT* __restrict__ c, int a_tiled,
-    int b_tiled, int splits, int late, [[maybe_unused]] unsigned long long* __restrict__ stamps) {
+    int b_tiled, int splits, int late, [[maybe_unused]] unsigned long long* __restrict__ stamps,
+    [[maybe_unused]] RotEpilogue rot = RotEpilogue{}) {
+    static_assert(!ROT || sizeof(OutT) == 2, "the fused inverse rotation is part of the bf16 epilogue");
     extern __shared__ uint32_t smem[];
     uint8_t* smem_bytes = reinterpret_cast<uint8_t*>(smem);
     const uint32_t smem_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)smem;
@@ -924,8 +1013,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         // One block of four K steps.  The load stream is four K steps ahead and rolls over into the next tile;
         // after the last tile it re-requests the current steps (never consumed), which keeps the outstanding-load
         // counts uniform.  FIRST: the tile's first products overwrite the accumulators instead of adding to them.
+        // the fused epilogue's mask words: one per 32 x 32 block of the lane's row, requested here -- ahead of the tile's
+        // first K step, so that the K loop hides their latency -- into registers the epilogue reads.  A row's four words
+        // (the wave's 128 columns) are 16 contiguous bytes: one request per block row.  A wave whose columns hang over the
+        // edge of N by half requests the row's last 16 bytes (its own two words come second there); rows below M and
+        // waves wholly outside read the matrix's last row / columns and store nothing.
+        // Nothing may read these registers before the epilogue (the data is in flight): the words are picked there.
+        [[maybe_unused]] u32x4 keep[4];
+        [[maybe_unused]] bool keep_shifted = false;
+        if constexpr (ROT) {
+            const int64_t mask_pitch = N / 8;
+            int64_t ncol = n0 + wn * 128;
+            keep_shifted = ncol + 128 > N;   // wave-uniform; N >= 256
+            ncol = keep_shifted ? (int64_t)N - 128 : ncol;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                int64_t mrow = m0 + wm * 128 + i * 32 + lrow;
+                mrow = mrow < M ? mrow : (int64_t)M - 1;
+                const uint8_t* src = rot.mask + mrow * mask_pitch + ncol / 8;
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(keep[i]) : "v"(src) : "memory");
+            }
+        }
         auto block4 = [&](int ks, auto first) {
             constexpr bool FIRST = decltype(first)::value;
+            // the four mask-word requests are younger than the stages the first block's steps 0..2 wait for
+            constexpr int EX = (FIRST && ROT) ? 4 : 0;
             int lks = ks + 4;
             if (lks == nk) {
                 if (t + stride < total_items) {
@@ -938,9 +1050,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             const int lbase = lks + 4 <= nk_real ? lks : nk_real - 4;    // a short last block: the row's final four steps
             const int first_live = ks + 4 > nk_real ? muted : 0;         // this block's steps below it are muted
             const auto sw = [&](int q) { return q < first_live ? 0 : 16; };
-            big4_step<0, sizeof(OutT) == 2, FIRST>(plan, smem_bytes, lbase, lbase * 4, sw(0), par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
-            big4_step<1, sizeof(OutT) == 2>(plan, smem_bytes, lbase + 1, 0, sw(1), par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
-            big4_step<2, sizeof(OutT) == 2>(plan, smem_bytes, lbase + 2, 0, sw(2), par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+            big4_step<0, sizeof(OutT) == 2, FIRST, EX>(plan, smem_bytes, lbase, lbase * 4, sw(0), par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+            big4_step<1, sizeof(OutT) == 2, false, EX>(plan, smem_bytes, lbase + 1, 0, sw(1), par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
+            big4_step<2, sizeof(OutT) == 2, false, EX>(plan, smem_bytes, lbase + 2, 0, sw(2), par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
             big4_step<3, sizeof(OutT) == 2>(plan, smem_bytes, lbase + 3, 0, sw(3), par, a_off0, a_off1, b_off0, b_off1, a_sc_off, b_sc_off, sh, st, acc);
             par ^= 1;
         };
@@ -948,8 +1060,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         for (int ks = 4; ks < nk; ks += 4) block4(ks, std::false_type{});
         stamp();
         if constexpr (sizeof(OutT) == 2) {
-            big4_epilogue_bf16(acc, alpha, reinterpret_cast<uint16_t*>(c), m0, n0, N, wm, wn, wave, lane, smem_bytes,
-                               rows_valid, cols_valid);
+            big4_epilogue_bf16<ROT>(acc, alpha, reinterpret_cast<uint16_t*>(c), m0, n0, N, wm, wn, wave, lane, smem_bytes,
+                                    rows_valid, cols_valid, rot, keep, keep_shifted);
         } else {
             OutT* dst = splits > 1 ? c + (int64_t)cur_split * M * N : c;
             const float a_eff = splits > 1 ? 1.0f : alpha;
@@ -1077,11 +1189,11 @@ int choose_splits(int64_t M, int64_t N, int64_t K, int cus) {
 // item, where the tile boundary is a third or more of a tile; longer ones neither gain nor lose (within 0.7 %)
 int big4_late_start(int64_t K, int splits) { return K / kBK / splits <= 16 ? 6 : 0; }
 
-template <typename OutT>
+template <typename OutT, bool ROT = false>
 hipError_t launch_big4(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                        const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_tiled,
-                       int b_tiled, int splits, int cus, hipStream_t stream) {
-    auto kern = gemm_mxfp4_tn_big4_kernel<OutT>;
+                       int b_tiled, int splits, int cus, hipStream_t stream, const RotEpilogue& rot = RotEpilogue{}) {
+    auto kern = gemm_mxfp4_tn_big4_kernel<OutT, false, ROT>;
     static std::atomic<bool> lds_allowed[kMaxDevices];
     hipError_t e = allow_dynamic_lds(kern, kBig4SmemBytes, lds_allowed);
     if (e != hipSuccess) return e;
@@ -1091,7 +1203,7 @@ hipError_t launch_big4(const uint8_t* a_codes, const uint8_t* a_scales, const ui
     if (g > 8) g -= g % 8;
     dim3 grid((unsigned)g), block(256);
     kern<<<grid, block, kBig4SmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
-                                                  reinterpret_cast<OutT*>(c), a_tiled, b_tiled, splits, big4_late_start(K, splits), nullptr);
+                                                  reinterpret_cast<OutT*>(c), a_tiled, b_tiled, splits, big4_late_start(K, splits), nullptr, rot);
     return hipGetLastError();
 }
 
@@ -1144,11 +1256,12 @@ hipError_t launch_gemm(const uint8_t* a_codes, const uint8_t* a_scales, const ui
 int gemm_phase_stamps_per_group() { return kPhaseStamps; }
 hipError_t gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
                             int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout,
-                            unsigned long long* stamps, size_t stamps_bytes, int* grid_out, hipStream_t stream) {
+                            const uint8_t* rot_mask, unsigned long long* stamps, size_t stamps_bytes, int* grid_out, hipStream_t stream) {
     *grid_out = 0;
     if (!gemm_supports_tiled(M, N, K) || K % 512 || ((reinterpret_cast<uintptr_t>(a_scales) | reinterpret_cast<uintptr_t>(b_scales)) & 15))
         return hipErrorInvalidValue;
-    auto kern = gemm_mxfp4_tn_big4_kernel<uint16_t, true>;
+    // rot_mask: the instantiation whose epilogue carries the masked inverse rotation (no sign flips, bf16 scale)
+    auto kern = rot_mask ? gemm_mxfp4_tn_big4_kernel<uint16_t, true, true> : gemm_mxfp4_tn_big4_kernel<uint16_t, true, false>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kBig4SmemBytes);
     if (e != hipSuccess) return e;
     const int64_t items = ((M + kBigM - 1) / kBigM) * ((N + kBigN - 1) / kBigN);
@@ -1158,7 +1271,8 @@ hipError_t gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, con
     if (stamps_bytes < (size_t)g * kPhaseStamps * sizeof(unsigned long long)) return hipErrorInvalidValue;
     kern<<<dim3((unsigned)g), dim3(256), kBig4SmemBytes, stream>>>(a_codes, a_scales, b_codes, b_scales, (int)M, (int)N, (int)K, alpha,
                                                                   reinterpret_cast<uint16_t*>(c), a_layout == LAYOUT_TILED,
-                                                                  b_layout == LAYOUT_TILED, 1, big4_late_start(K, 1), stamps);
+                                                                  b_layout == LAYOUT_TILED, 1, big4_late_start(K, 1), stamps,
+                                                                  RotEpilogue{rot_mask, 0u, hadamard_scale(32, BF16)});
     *grid_out = (int)g;
     return hipGetLastError();
 }
@@ -1187,6 +1301,31 @@ size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                          const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
                          int a_layout, int b_layout, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    return gemm_mxfp4_tn_rotated(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, c_dtype, a_layout, b_layout, workspace,
+                                 workspace_bytes, nullptr, 0u, F32, nullptr, stream);
+}
+
+// whether gemm_mxfp4_tn_rotated would apply the rotation in the product's epilogue for these arguments
+bool gemm_will_rotate(const uint8_t* a_scales, const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, int c_dtype, const void* workspace,
+                      size_t workspace_bytes) {
+    if (c_dtype != BF16 || !gemm_supports_tiled(M, N, K) || K <= kDuoMaxK) return false;
+    const int64_t nk_real = K / kBK, nk_pad = (nk_real + 3) & ~(int64_t)3;
+    const bool persistent_ok = K % 512 == 0 ? ((reinterpret_cast<uintptr_t>(a_scales) | reinterpret_cast<uintptr_t>(b_scales)) & 15) == 0
+                                            : (nk_real >= 4 && (nk_pad - nk_real) * 3 <= nk_real);
+    if (!persistent_ok) return false;
+    int sp = workspace && K % 512 == 0 ? choose_splits(M, N, K, device_cus()) : 1;
+    if (sp > 1 && ((size_t)sp * M * N * sizeof(float) > workspace_bytes || (reinterpret_cast<uintptr_t>(workspace) & 15))) sp = 1;
+    return sp == 1;
+}
+
+// The product, with the layer's masked inverse Hadamard rotation (blocks of 32 along N) applied to the result before it is
+// stored when `rot_mask` is given and the shape runs on the persistent kernel's bf16 epilogue without a cut into K ranges:
+// *rotated tells which (false: c holds the plain product and the caller runs the rotation as a kernel of its own).
+hipError_t gemm_mxfp4_tn_rotated(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                                 const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
+                                 int a_layout, int b_layout, void* workspace, size_t workspace_bytes, const uint8_t* rot_mask,
+                                 uint32_t rot_signs, int rot_scale_dtype, bool* rotated, hipStream_t stream) {
+    if (rotated) *rotated = false;
     if (M == 0 || N == 0) return hipSuccess;
     const int at = a_layout == LAYOUT_TILED, bt = b_layout == LAYOUT_TILED;
     const bool big_ok = gemm_supports_tiled(M, N, K);
@@ -1232,6 +1371,11 @@ hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const 
             else
                 splitk_reduce_kernel<float><<<grid, block, 0, stream>>>(static_cast<const float*>(workspace), sp, mn, alpha, static_cast<float*>(c));
             return hipGetLastError();
+        }
+        if (c_dtype == BF16 && rot_mask && rotated) {
+            *rotated = true;
+            const RotEpilogue rot{rot_mask, rot_signs, hadamard_scale(32, rot_scale_dtype)};
+            return launch_big4<uint16_t, true>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, 1, cus, stream, rot);
         }
         if (c_dtype == BF16) return launch_big4<uint16_t>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, 1, cus, stream);
         return launch_big4<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, 1, cus, stream);

@@ -122,6 +122,14 @@ hipError_t requantize_transposed_mxfp4(const uint8_t* codes_in, const uint8_t* s
 hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                          const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
                          int a_layout, int b_layout, void* workspace, size_t workspace_bytes, hipStream_t stream);
+// the same product with the masked inverse Hadamard rotation of the layer's backward pass (hd 32, along N) fused into the
+// store of the result where the kernel serving the shape can do it; *rotated reports whether it was
+bool gemm_will_rotate(const uint8_t* a_scales, const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, int c_dtype, const void* workspace,
+                      size_t workspace_bytes);
+hipError_t gemm_mxfp4_tn_rotated(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                                 const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
+                                 int a_layout, int b_layout, void* workspace, size_t workspace_bytes, const uint8_t* rot_mask,
+                                 uint32_t rot_signs, int rot_scale_dtype, bool* rotated, hipStream_t stream);
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 // C = alpha * A (packed MXFP4 [M, K]) x B (bf16 [K, N] row-major): K % 64 == 0, N % 8 == 0
 bool gemm_fp4_bf16_nn_supported(int64_t M, int64_t N, int64_t K);
@@ -131,7 +139,7 @@ hipError_t gemm_fp4_bf16_nn(const uint8_t* a_codes, const uint8_t* a_scales, con
 int gemm_phase_stamps_per_group();
 hipError_t gemm_tile_phases(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
                             int64_t M, int64_t N, int64_t K, float alpha, void* c, int a_layout, int b_layout,
-                            unsigned long long* stamps, size_t stamps_bytes, int* grid_out, hipStream_t stream);
+                            const uint8_t* rot_mask, unsigned long long* stamps, size_t stamps_bytes, int* grid_out, hipStream_t stream);
 // measurement aid: the FP4 matrix instruction alone (see gemm.hip)
 int mfma_only_blocks();
 hipError_t mfma_only(const uint8_t* operands, float* sink, int iters, hipStream_t stream);

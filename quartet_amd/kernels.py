@@ -164,6 +164,30 @@ def gemm_mxfp4_tn(a_codes, a_scales, b_codes, b_scales, alpha=1.0, out_dtype=tor
     return c
 
 
+def gemm_fuses_rotation(a_scales, b_scales, M, N, K):
+    """Whether gemm_mxfp4_tn_rotated serves this product (the persistent kernel, no cut into K ranges)."""
+    return bool(_lib.lib().qm_gemm_fuses_rotation(_ptr(a_scales), _ptr(b_scales), M, N, K))
+
+
+def gemm_mxfp4_tn_rotated(a_codes, a_scales, b_codes, b_scales, maskbits, alpha=1.0, scale_dtype=torch.bfloat16, sign_bits=None,
+                          a_tiled=False, b_tiled=False):
+    """masked_hadamard_bwd(gemm_mxfp4_tn(..., bf16), 32, scale_dtype, sign_bits, maskbits) in one launch: the product's
+    epilogue rounds the tile to bf16, masks it and rotates it on the matrix pipe.  [M,N] bf16.  Raises for shapes the
+    fused kernel does not serve (gemm_fuses_rotation tells)."""
+    _require_cuda(a_codes, a_scales, b_codes, b_scales, maskbits)
+    M, K = a_codes.shape[0], a_codes.shape[1] * 2
+    N = b_codes.shape[0]
+    if b_codes.shape[1] * 2 != K:
+        raise _lib.QuartetHipError(f"gemm_mxfp4_tn_rotated: contraction sizes differ ({K} vs {b_codes.shape[1] * 2})")
+    assert maskbits.shape == (M, N // 8) and maskbits.is_contiguous()
+    c = torch.empty((M, N), dtype=torch.bfloat16, device=a_codes.device)
+    rc = _lib.lib().qm_gemm_mxfp4_tn_rotated(_ptr(a_codes), _ptr(a_scales), _ptr(b_codes), _ptr(b_scales), M, N, K, alpha, _ptr(c),
+                                             _layout(a_tiled), _layout(b_tiled), _ptr(maskbits), sign_words(sign_bits),
+                                             _dtype_code(scale_dtype), _stream())
+    _lib.check(rc, "qm_gemm_mxfp4_tn_rotated")
+    return c
+
+
 def gemm_mxfp4_bf16_nn_supported(M, N, K):
     return K > 0 and K % 64 == 0 and N % 8 == 0 and M > 0 and N > 0
 
@@ -214,18 +238,19 @@ def gemm_mxfp4_tn_noalloc(a_codes, a_scales, b_codes, b_scales, alpha, out):
 PHASE_STAMPS = 32   # QM_DIAG_PHASE_STAMPS
 
 
-def gemm_tile_phases(a_codes, a_scales, b_codes, b_scales, alpha=1.0, a_tiled=False, b_tiled=False):
+def gemm_tile_phases(a_codes, a_scales, b_codes, b_scales, alpha=1.0, a_tiled=False, b_tiled=False, maskbits=None):
     """Measurement aid: one launch of the persistent tile kernel's stamping instantiation.  Returns (c [M,N] bf16,
     stamps int64 [workgroups, 32] on the host): per workgroup the shader clock at entry, at the start of its tile loop,
-    then after the K loop and after the epilogue of each of its tiles (unused slots are zero)."""
-    _require_cuda(a_codes, a_scales, b_codes, b_scales)
+    then after the K loop and after the epilogue of each of its tiles (unused slots are zero).  With `maskbits` [M, N/8]
+    the instantiation whose epilogue carries the masked inverse rotation (c is then the rotated product)."""
+    _require_cuda(a_codes, a_scales, b_codes, b_scales, maskbits)
     M, K = a_codes.shape[0], a_codes.shape[1] * 2
     N = b_codes.shape[0]
     assert b_codes.shape[1] * 2 == K
     c = torch.empty((M, N), dtype=torch.bfloat16, device=a_codes.device)
     stamps = torch.zeros((1024, PHASE_STAMPS), dtype=torch.int64, device=a_codes.device)
     groups = _lib.lib().qm_diag_gemm_tile_phases(_ptr(a_codes), _ptr(a_scales), _ptr(b_codes), _ptr(b_scales), M, N, K, alpha,
-                                                 _ptr(c), _layout(a_tiled), _layout(b_tiled), _ptr(stamps),
+                                                 _ptr(c), _layout(a_tiled), _layout(b_tiled), _ptr(maskbits), _ptr(stamps),
                                                  stamps.numel() * 8, _stream())
     if groups < 0:
         _lib.check(int(groups), "qm_diag_gemm_tile_phases")

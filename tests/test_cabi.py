@@ -29,7 +29,7 @@ def test_library_exports_every_declared_function():
 
 def test_host_only_entry_points():
     L = _lib.lib()
-    assert L.qm_version() == 14
+    assert L.qm_version() == 15
     T, I, O = 256, 128, 384
     off = (ctypes.c_size_t * 3)()
     for rows, cols in ((T, I), (O, I)):
@@ -69,6 +69,13 @@ def test_host_only_entry_points():
     (lambda L: L.qm_gemm_mxfp4_bf16_nn(None, None, None, 64, 64, 128, 1.0, None, 0, None), b"null tensor"),
     (lambda L: L.qm_gemm_mxfp4_bf16_nn(0x1000, 0x2000, 0x3008, 64, 64, 128, 1.0, 0x4000, 0, None), b"16-byte"),
     (lambda L: L.qm_gemm_mxfp4_bf16_nn(0x1000, 0x2000, 0x3000, 64, 64, 128, 1.0, 0x4000, 9, None), b"c_dtype"),
+    # the product with the inverse rotation in its epilogue: null tensors, shapes the persistent kernel does not serve (a short
+    # contraction), misaligned mask bits
+    (lambda L: L.qm_gemm_mxfp4_tn_rotated(None, None, None, None, 256, 256, 1024, 1.0, None, 0, 0, None, None, 0, None), b"null tensor"),
+    (lambda L: L.qm_gemm_mxfp4_tn_rotated(0x1000, 0x2000, 0x3000, 0x4000, 256, 256, 512, 1.0, 0x5000, 0, 0, 0x6000, None, 0, None), b"not served"),
+    (lambda L: L.qm_gemm_mxfp4_tn_rotated(0x1000, 0x2000, 0x3000, 0x4000, 256, 200, 1024, 1.0, 0x5000, 0, 0, 0x6000, None, 0, None), b"not served"),
+    (lambda L: L.qm_gemm_mxfp4_tn_rotated(0x1000, 0x2000, 0x3000, 0x4000, 256, 256, 1024, 1.0, 0x5000, 0, 0, 0x6002, None, 0, None), b"4-byte"),
+    (lambda L: L.qm_gemm_mxfp4_tn_rotated(0x1000, 0x2000, 0x3000, 0x4000, 256, 256, 1024, 1.0, 0x5000, 0, 0, 0x6000, None, 5, None), b"scale_dtype"),
     (lambda L: L.qm_quantize_mxfp4_dense(None, 0, 4, 40, None, 1, 0, 0, None, None, None, None, 0, None), b"multiple of 32"),
     (lambda L: L.qm_quantize_mxfp4_dense(None, 0, 4, 64, None, 1, 0, 0, None, None, None, None, 0, None), b"non-null"),
     (lambda L: L.qm_quantize_mxfp4_dense(0x1000, 0, 64, 64, 0x2000, 1, 1, 0, 0x3000, 0x4000, None, None, 0, None), b"transposed input needs"),
@@ -103,6 +110,7 @@ def test_empty_shapes_are_accepted_without_touching_pointers():
     assert L.qm_quantize_mxfp4(None, 0, 0, 64, 32, None, 0, 0, None, 0, None, None, None, None, 0, None) == 0
     assert L.qm_gemm_mxfp4_tn(None, None, None, None, 0, 64, 64, 1.0, None, 0, 0, 0, None, 0, None) == 0
     assert L.qm_gemm_mxfp4_bf16_nn(None, None, None, 0, 64, 64, 1.0, None, 0, None) == 0
+    assert L.qm_gemm_mxfp4_tn_rotated(None, None, None, None, 0, 256, 1024, 1.0, None, 0, 0, None, None, 0, None) == 0
     assert L.qm_linear_forward(None, 0, None, 0, 0, 64, 64, 32, None, 32, None, None, 0, None, 0, 0, None, 0, 0, None) == 0
     assert L.qm_rmsnorm_quantize_mxfp4(None, 0, None, 0, None, None, 1e-5, 0, 64, None, None, 0, None, 0, None) == 0
     assert L.qm_swiglu_quantize_mxfp4(None, 0, 0, 64, None, None, 0, 0, None) == 0

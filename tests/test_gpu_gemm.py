@@ -177,6 +177,59 @@ def test_gemm_scale_arrays_off_16_byte_alignment(K, tiled):
     assert rel <= 1e-6, rel
 
 
+# the product with the masked inverse rotation in its epilogue: one tile, several tiles per workgroup, tiles over the edge of
+# M and N, K with padding steps, both operand layouts
+@pytest.mark.parametrize("M,N,K_", [(256, 256, 1024), (512, 768, 1536), (4352, 4608, 1024), (320, 448, 1920), (8192, 4096, 2048)])
+@pytest.mark.parametrize("tiled", [False, True])
+def test_product_with_the_inverse_rotation_in_its_epilogue(oracle, K, M, N, K_, tiled):
+    """qm_gemm_mxfp4_tn_rotated against the two calls it replaces (bf16 product, then masked_hadamard_bwd): the same
+    bf16-rounded, masked tile is rotated, only the fp32 arithmetic inside a group's sum differs (the matrix instruction's
+    order; with a bf16 scale dtype the factor 32^-1/2 multiplies the terms, as in the reference's bf16 product, instead of
+    the sum), so all but a few elements in a million are identical; and against the float64 evaluation of the definition."""
+    print(f"case rotated product {M}x{N}x{K_} tiled={tiled}", flush=True)
+    if tiled and (M % 128 or N % 128):
+        pytest.skip("the tiled layout needs rows in blocks of 128")
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(M + 3 * N + K_)
+    ac = torch.randint(0, 256, (M, K_ // 2), generator=g, dtype=torch.uint8).to(dev)
+    bc = torch.randint(0, 256, (N, K_ // 2), generator=g, dtype=torch.uint8).to(dev)
+    as_ = torch.randint(118, 132, (M, K_ // 32), generator=g, dtype=torch.uint8).to(dev)
+    bs = torch.randint(120, 136, (N, K_ // 32), generator=g, dtype=torch.uint8).to(dev)
+    keep = torch.randint(0, 256, (M, N // 8), generator=g, dtype=torch.uint8)
+    keep |= torch.randint(0, 256, (M, N // 8), generator=g, dtype=torch.uint8)      # three quarters of the bits set
+    keep = keep.to(dev)
+    signs = int(torch.randint(0, 2 ** 31, (1,), generator=g)) * 2 + 1
+    alpha = 16.0 / 9.0
+    assert K.gemm_fuses_rotation(as_, bs, M, N, K_)
+    at, bt = (K.tile_codes(ac), K.tile_codes(bc)) if tiled else (ac, bc)
+    for sd in (torch.bfloat16, torch.float32):
+        got = K.gemm_mxfp4_tn_rotated(at, as_, bt, bs, keep, alpha, sd, signs, a_tiled=tiled, b_tiled=tiled)
+        plain = K.gemm_mxfp4_tn(at, as_, bt, bs, alpha, torch.bfloat16, a_tiled=tiled, b_tiled=tiled)
+        two = K.masked_hadamard_bwd(plain, 32, sd, signs, keep)
+        torch.cuda.synchronize()
+        differ = got != two
+        frac = float(differ.float().mean())
+        print(f"  scale dtype {sd}: {int(differ.sum())} of {differ.numel()} elements differ from the two-call result", flush=True)
+        assert frac < 1e-4
+        # where they differ: by a bf16 rounding step at the element's size, or -- where a group's terms cancel -- by the fp32
+        # rounding of its partial sums, which is tiny against the terms themselves
+        step = two.float().abs() * 2.0 ** -7 + float(plain.float().abs().max()) * 2.0 ** -18
+        assert bool(((got.float() - two.float()).abs() <= step)[differ].all())
+        # the definition in float64 on sampled rows: bf16(alpha A B^T) * keep, groups of 32 times the signed Sylvester matrix
+        rows = torch.cat([torch.tensor([0, M - 1]), torch.randint(0, M, (14,), generator=g)]).to(dev)
+        A = _torch_dequant(ac[rows], as_[rows])
+        B = _torch_dequant(bc, bs)
+        y = (alpha * (A @ B.T)).to(torch.float32).to(torch.bfloat16).double()
+        bits = ((keep[rows].long()[:, :, None] >> torch.arange(8, device=dev)) & 1).reshape(len(rows), N).double()
+        n = torch.arange(32, device=dev)
+        syl = 1.0 - 2.0 * (torch.tensor([[bin(int(a & b)).count("1") & 1 for b in range(32)] for a in range(32)], device=dev)).double()
+        sgn = 1.0 - 2.0 * ((signs >> n) & 1).double()
+        c = float(torch.tensor(32 ** -0.5).to(sd))
+        want = (((y * bits).view(len(rows), N // 32, 32) * sgn) @ syl.T).reshape(len(rows), N) * c
+        rel = float((got[rows].double() - want).norm() / want.norm())
+        assert rel < 4e-3, rel     # the bf16 rounding of the result: 2^-9 relative per element
+
+
 def test_split_k_is_offered_and_reproducible(K):
     from quartet_amd import _lib
     L = _lib.lib()
@@ -234,6 +287,11 @@ def test_tile_phase_stamps_of_the_persistent_kernel():
         want = K.gemm_mxfp4_tn(ac, as_, bc, bs, 1.5, torch.bfloat16, split_k=False)
         got, stamps = K.gemm_tile_phases(ac, as_, bc, bs, 1.5)
         assert torch.equal(got, want)
+        # the instantiation with the masked inverse rotation in its epilogue: the fused product, bit for bit
+        keep = torch.randint(0, 256, (M, N // 8), generator=g, dtype=torch.uint8).to(dev)
+        got_rot, stamps_rot = K.gemm_tile_phases(ac, as_, bc, bs, 1.5, maskbits=keep)
+        assert torch.equal(got_rot, K.gemm_mxfp4_tn_rotated(ac, as_, bc, bs, keep, 1.5, torch.bfloat16, None))
+        assert stamps_rot.shape == stamps.shape
         tiles = 0
         for row in stamps.tolist():
             assert 0 < row[0] <= row[1]
