@@ -608,7 +608,9 @@ def counters_to_json(fetch_dir, write_dir, sq_dir=None):
         copies = [v for k, vs in agg.items() if "copyBuffer" in k for v in vs]
         return copy_bytes / max(copies)
     fu, wu = unit(fetch), unit(write)
-    groups = {"gemm_mxfp4_tn": lambda k: "gemm_mxfp4_tn" in k and "splitk" not in k,
+    groups = {"gemm_mxfp4_tn": lambda k: "gemm_mxfp4_tn" in k and "splitk" not in k and "false, true>" not in k,
+              # the instantiation with the masked inverse rotation in its epilogue (the step's two gradient products)
+              "gemm_mxfp4_tn_rotated": lambda k: "gemm_mxfp4_tn_big4_kernel" in k and "false, true>" in k,
               "quantize_x_quest_rtn_mask_alone": lambda k: k.startswith("void qm::job_kernel<qm::RowmajorTiledJob") or k.startswith("qm::job_kernel<qm::RowmajorTiledJob"),
               "forward_quantizer_pair": lambda k: "job_pair_kernel<qm::RowmajorTiledJob" in k,
               "gradient_quantizer_pair": lambda k: "job_pair_kernel<qm::TransposedJob" in k,
@@ -960,6 +962,11 @@ def main():
         gemm_ms = diff.pop("ms")
         gemm_tf = 2.0 * T_TOKENS * IN_F * out_f / gemm_ms / 1e9
         traffic, source = _traffic_entry(prof, "gemm_mxfp4_tn")
+        if fused and traffic is not None:
+            t_rot, _ = _traffic_entry(prof, "gemm_mxfp4_tn_rotated")
+            if t_rot is not None:   # per launch, as the step runs them: one plain product, two with the rotation (these also read mask bits)
+                source = {**source, "plain_product_bytes": traffic, "rotated_product_bytes": t_rot}
+                traffic = round((traffic + 2.0 * t_rot) / 3.0, 1)
         what = "mean of the step's three products, timed inside the step"
         if fused:
             what += ("; the two gradient products carry the masked inverse rotation in their epilogue (flops counted: the product's "
