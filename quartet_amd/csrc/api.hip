@@ -506,6 +506,32 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
                                                 gw_dtype, true, hs), "qm_linear_backward");
     };
     if (gx_rotated && hd_x != 32) return fail(QM_ERR_INVALID, "qm_linear_backward: gx_rotated needs hd_x == 32");
+    // B3 + B7 and B6 + B8: where a gradient product runs on the persistent kernel's bf16 epilogue, the masked inverse
+    // rotation of the forward quantizer is applied to the tile before it is stored and the product lands in gx / gw
+    // directly (`fused` reports it); otherwise the product goes to the workspace and the rotation is a kernel of its own.
+    const auto grad_product = [&](const uint8_t* ac, const uint8_t* as, const uint8_t* bc, const uint8_t* bs, int64_t M, int64_t N,
+                                  int64_t K, void* plain_dst, void* final_dst, bool want_rotation, int hd, int final_dtype,
+                                  const uint8_t* mask, const uint32_t* signs, int scale_dtype, bool& fused) -> int {
+        fused = want_rotation && hd == 32 && final_dtype == mid_dtype && final_dst && aligned(final_dst, 16) && valid_dtype(scale_dtype) &&
+                qm::gemm_will_rotate(as, bs, M, N, K, mid_dtype, gws, wl.gemm_ws_bytes);
+        if (!fused)
+            return qm_gemm_mxfp4_tn(ac, as, bc, bs, M, N, K, alpha, plain_dst, mid_dtype, codes_layout, codes_layout, gws, wl.gemm_ws_bytes, stream);
+        bool done = false;
+        const int r = from_hip(qm::gemm_mxfp4_tn_rotated(ac, as, bc, bs, M, N, K, alpha, final_dst, mid_dtype, codes_layout, codes_layout, gws,
+                                                         wl.gemm_ws_bytes, mask, signs ? signs[0] : 0u, scale_dtype, &done, hs),
+                               "qm_linear_backward");
+        if (r) return r;
+        return done ? 0 : fail(QM_ERR_INVALID, "qm_linear_backward: a gradient product did not run as planned");
+    };
+    bool gx_fused = false, gw_fused = false;
+    const auto product_gx = [&]() {
+        return grad_product(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, gx_product, gx, !gx_rotated, hd_x, mid_dtype, px + lx.m,
+                            signs_x, x_scale_dtype, gx_fused);
+    };
+    const auto product_gw = [&]() {
+        return grad_product(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, gw_product, gw, !gw_rotated, hd_w, gw_dtype, pw + lw.m,
+                            signs_w, w_scale_dtype, gw_fused);
+    };
     if (g_matrix) {
         // a dense rotation in the gradient quantizer (rerotate="O32"): the same eight steps on the dense-rotation kernels
         if (hd_g != 32 || T % 128 || I % 128 || O % 128)
@@ -516,22 +542,20 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
         rc = qm_requantize_transposed_mxfp4_dense(pw + lw.c, pw + lw.s, O, I, 1.0f, w_val_dtype, g_matrix, g_mode, seeds[1], k + wl.wtc,
                                                   k + wl.wts, nullptr, codes_layout, codes_layout, stream);
         if (rc) return rc;
-        rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, gx_product, mid_dtype, codes_layout,
-                              codes_layout, gws, wl.gemm_ws_bytes, stream);
+        rc = product_gx();
         if (rc) return rc;
         rc = qm_quantize_mxfp4_dense(e, e_dtype, O, T, g_matrix, g_mode, 1, seeds[2], k + wl.etc, k + wl.ets, nullptr, nullptr, codes_layout, stream);
         if (rc) return rc;
         rc = qm_requantize_transposed_mxfp4_dense(px + lx.c, px + lx.s, T, I, 1.0f, x_val_dtype, g_matrix, g_mode, seeds[3], k + wl.xtc,
                                                   k + wl.xts, nullptr, codes_layout, codes_layout, stream);
         if (rc) return rc;
-        rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, gw_product, mid_dtype, codes_layout,
-                              codes_layout, gws, wl.gemm_ws_bytes, stream);
+        rc = product_gw();
         if (rc) return rc;
-        if (!gx_rotated) {
+        if (!gx_rotated && !gx_fused) {
             rc = qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, px + lx.m, gx, mid_dtype, stream);
             if (rc) return rc;
         }
-        return rotate_gw();
+        return gw_fused ? 0 : rotate_gw();
     }
     if (pair_launches(codes_layout, T, I, O, hd_x, hd_w, hd_g) && e && gx && gw && valid_dtype(e_dtype) && aligned(e, 16) &&
         aligned(gx, 16) && aligned(gw, 16) && valid_dtype(x_val_dtype) && valid_dtype(w_val_dtype) &&
@@ -545,23 +569,11 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
         const qm::RequantArgs rx{px + lx.c, px + lx.s, T, I, x_val_dtype, seeds[3], k + wl.xtc, k + wl.xts};
         rc = from_hip(qm::requantize_transposed_hd32_tiled_pair(rx, rw, sg, g_mode, seed_base, hs), "qm_linear_backward");
         if (rc) return rc;
-        // B3 + B7 and B6 + B8: where the product runs on the persistent kernel's bf16 epilogue, the masked inverse rotation is
-        // applied to the tile before it is stored and the product lands in gx / gw directly
-        const bool fuse_x = !gx_rotated && qm::gemm_will_rotate(k + wl.es, k + wl.wts, T, I, O, mid_dtype, gws, wl.gemm_ws_bytes);
-        const bool fuse_w = !gw_rotated && gw_dtype == mid_dtype &&
-                            qm::gemm_will_rotate(k + wl.ets, k + wl.xts, O, I, T, mid_dtype, gws, wl.gemm_ws_bytes);
-        bool done = false;
-        rc = from_hip(qm::gemm_mxfp4_tn_rotated(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, fuse_x ? gx : gx_product, mid_dtype,
-                                                codes_layout, codes_layout, gws, wl.gemm_ws_bytes, fuse_x ? px + lx.m : nullptr,
-                                                signs_x ? signs_x[0] : 0u, x_scale_dtype, &done, hs), "qm_linear_backward");
+        rc = product_gx();
         if (rc) return rc;
-        if (done != fuse_x) return fail(QM_ERR_INVALID, "qm_linear_backward: the grad-input product did not run as planned");
-        rc = from_hip(qm::gemm_mxfp4_tn_rotated(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, fuse_w ? gw : gw_product, mid_dtype,
-                                                codes_layout, codes_layout, gws, wl.gemm_ws_bytes, fuse_w ? pw + lw.m : nullptr,
-                                                signs_w ? signs_w[0] : 0u, w_scale_dtype, &done, hs), "qm_linear_backward");
+        rc = product_gw();
         if (rc) return rc;
-        if (done != fuse_w) return fail(QM_ERR_INVALID, "qm_linear_backward: the grad-weight product did not run as planned");
-        const bool need_x = !gx_rotated && !fuse_x, need_w = !gw_rotated && !fuse_w;
+        const bool need_x = !gx_rotated && !gx_fused, need_w = !gw_rotated && !gw_fused;
         if (!need_x) return need_w ? rotate_gw() : 0;
         if (!need_w)
             return qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, px + lx.m, gx, mid_dtype, stream);
@@ -577,8 +589,7 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
     rc = qm_requantize_transposed_mxfp4(pw + lw.c, pw + lw.s, O, I, 1.0f, w_val_dtype, hd_g, signs_g, g_mode, nullptr, seeds[1],
                                         k + wl.wtc, k + wl.wts, nullptr, codes_layout, codes_layout, stream);
     if (rc) return rc;
-    rc = qm_gemm_mxfp4_tn(k + wl.ec, k + wl.es, k + wl.wtc, k + wl.wts, T, I, O, alpha, gx_product, mid_dtype, codes_layout,
-                          codes_layout, gws, wl.gemm_ws_bytes, stream);
+    rc = product_gx();
     if (rc) return rc;
     rc = qm_quantize_mxfp4(e, e_dtype, O, T, hd_g, signs_g, g_mode, 1, nullptr, seeds[2], k + wl.etc, k + wl.ets, nullptr, nullptr,
                            codes_layout, stream);
@@ -586,14 +597,13 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
     rc = qm_requantize_transposed_mxfp4(px + lx.c, px + lx.s, T, I, 1.0f, x_val_dtype, hd_g, signs_g, g_mode, nullptr, seeds[3],
                                         k + wl.xtc, k + wl.xts, nullptr, codes_layout, codes_layout, stream);
     if (rc) return rc;
-    rc = qm_gemm_mxfp4_tn(k + wl.etc, k + wl.ets, k + wl.xtc, k + wl.xts, O, I, T, alpha, gw_product, mid_dtype, codes_layout,
-                          codes_layout, gws, wl.gemm_ws_bytes, stream);
+    rc = product_gw();
     if (rc) return rc;
-    if (!gx_rotated) {
+    if (!gx_rotated && !gx_fused) {
         rc = qm_masked_hadamard_bwd(k + wl.gxq, mid_dtype, T, I, hd_x, x_scale_dtype, signs_x, px + lx.m, gx, mid_dtype, stream);
         if (rc) return rc;
     }
-    return rotate_gw();
+    return gw_fused ? 0 : rotate_gw();
 }
 
 int qm_rmsnorm_quantize_mxfp4(const void* x, int x_dtype, const void* add, int add_dtype, void* x_sum, const float* gain, float eps,
