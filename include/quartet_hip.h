@@ -62,7 +62,8 @@ const char* qm_last_error(void);
  *                random rotation of rerotate="O32", mxfp4.py:61-64, applied by the caller): groups of 32 are
  *                quantized as they are; row-major input and codes only, sign_bits == NULL, u == NULL
  *   u            SR modes: device floats in [0,1) indexed by logical flat offset, or NULL to draw
- *                them in-kernel from Philox4x32-10 keyed by (seed, offset)
+ *                them in-kernel from Philox4x32-7 keyed by (seed, offset / 16): element j of a call takes the top
+ *                22 bits of word j / 4 rotated left by 8 (j % 4) bits
  *   codes/scales outputs (required); maskbits, dequant optional (NULL to skip); dequant has
  *                x_dtype and logical shape and holds what the reference kernel returns
  *   codes_layout QM_LAYOUT_TILED needs hadamard_dim 32, rows % 16 == 0, cols % 128 == 0, u == NULL for
@@ -263,6 +264,9 @@ int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, 
  *                     QM_GW_ROTATED: the same for gw and the weight quantizer (second product, B6; gw_dtype == mid_dtype)
  * codes_layout applies to every packed tensor inside; QM_LAYOUT_TILED needs T, I, O multiples of 128 and at
  * least 256, and all Hadamard blocks 32.  T, I, O must be multiples of 32 for the backward pass.
+ * Where a gradient product runs as qm_gemm_fuses_rotation describes (bf16 mid_dtype, Hadamard block 32, for gw also
+ * gw_dtype == mid_dtype), the forward quantizer's masked inverse rotation is applied in that product's epilogue
+ * (qm_gemm_mxfp4_tn_rotated) and the product is not staged in the workspace; elsewhere it is a launch of its own.
  */
 size_t qm_packed_operand_bytes(int64_t rows, int64_t cols);
 /* offsets: HOST array of three (codes, scales, mask bits); returns 0, or QM_ERR_INVALID unless cols % 32 == 0 */
