@@ -280,6 +280,55 @@ def test_linear_step_rows_against_oracle_pipeline(oracle, K, out_features):
     assert np.linalg.norm(gw - gw_ref) / np.linalg.norm(gw_ref) < 1e-2
 
 
+@pytest.mark.parametrize("out_features", OUTS)
+@pytest.mark.parametrize("rerotate", [None, "signs"])
+def test_linear_step_equals_the_composition_of_its_kernels(K, out_features, rerotate):
+    """End to end at full size, bit for bit: the layer's y, grad_x and grad_W equal what the same kernels give when they
+    are called one by one through their own entry points with the layer's sign flips and seeds (two forward quantizers,
+    the product; two gradient quantizers, two re-quantizers, and the two products with the inverse rotation in their
+    epilogue).  Each of those entry points is checked against the oracle on its own, at full size on sampled rows and
+    exhaustively at small sizes, so every element of the layer's results is tied to the oracle through them."""
+    print(f"case fullsize linear step against its kernels out={out_features} rerotate={rerotate}", flush=True)
+    import random
+    import quartet_amd as q
+    dev = torch.device("cuda:0")
+    Of = out_features
+    x, dy = _make_data(Of)
+    g = torch.Generator().manual_seed(11)
+    w = (0.02 * torch.randn(Of, I, generator=g)).to(torch.bfloat16)
+    layer = q.QuantizedLinear(I, Of, bias=False, weight_quantizer=q.QuestMXFP4Quantizer(),
+                              activation_quantizer=q.QuestMXFP4Quantizer(),
+                              gradient_quantizer=q.AlbertTsengQuantizer(stochastic=True, rerotate=rerotate),
+                              backward_scheme=q.BACKWARD_SCHEMES["Q(E)Q(Wt)t_Q(Et)Q(Xt)t"]()).to(dev, torch.bfloat16)
+    with torch.no_grad():
+        layer.weight.copy_(w.to(dev))
+    xd = x.to(dev).requires_grad_(True)
+    torch.manual_seed(77)      # the sign flips of re_randomize
+    random.seed(4242)          # the four stochastic-rounding seeds
+    y = layer(xd)
+    y.backward(dy.to(dev))
+    torch.cuda.synchronize()
+    random.seed(4242)
+    seeds = [random.getrandbits(63) for _ in range(4)]
+    signs = layer.backward_scheme.g_quantizer.sign_bits or None
+    assert (signs is not None) == (rerotate == "signs")
+    tl = True
+    alpha = float(torch.tensor(K.FOUR_THIRDS, dtype=torch.float32) * torch.tensor(K.FOUR_THIRDS, dtype=torch.float32))
+    xq, wq, e = x.to(dev), w.to(dev), dy.to(dev)
+    xc, xs, xm, _ = K.quantize_mxfp4(xq, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)
+    wc, ws, wm, _ = K.quantize_mxfp4(wq, 32, None, K.QM_QUEST_RTN, want_mask=True, tiled=tl)
+    assert torch.equal(y.detach(), K.gemm_mxfp4_tn(xc, xs, wc, ws, 1.0, torch.bfloat16, a_tiled=tl, b_tiled=tl))
+    ec, es, _, _ = K.quantize_mxfp4(e, 32, signs, K.QM_ABSMAX_SR, seed=seeds[0], tiled=tl)
+    wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=seeds[1], tiled_in=tl, tiled_out=tl)
+    etc, ets, _, _ = K.quantize_mxfp4(e, 32, signs, K.QM_ABSMAX_SR, transposed_in=True, seed=seeds[2], tiled=tl)
+    xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, torch.bfloat16, 32, signs, K.QM_ABSMAX_SR, seed=seeds[3], tiled_in=tl, tiled_out=tl)
+    assert K.gemm_fuses_rotation(es, wts, T, I, Of) and K.gemm_fuses_rotation(ets, xts, Of, I, T)
+    gx = K.gemm_mxfp4_tn_rotated(ec, es, wtc, wts, xm, alpha, torch.bfloat16, None, a_tiled=tl, b_tiled=tl)
+    gw = K.gemm_mxfp4_tn_rotated(etc, ets, xtc, xts, wm, alpha, torch.bfloat16, None, a_tiled=tl, b_tiled=tl)
+    assert torch.equal(xd.grad, gx)
+    assert torch.equal(layer.weight.grad, gw)
+
+
 def _signs_from_word(word):
     return np.array([-1 if (word >> j) & 1 else 1 for j in range(32)])
 
