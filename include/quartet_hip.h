@@ -266,7 +266,9 @@ int qm_dequantize_mxfp4(const uint8_t* codes, const uint8_t* scales, int64_t R, 
  * least 256, and all Hadamard blocks 32.  T, I, O must be multiples of 32 for the backward pass.
  * Where a gradient product runs as qm_gemm_fuses_rotation describes (bf16 mid_dtype, Hadamard block 32, for gw also
  * gw_dtype == mid_dtype), the forward quantizer's masked inverse rotation is applied in that product's epilogue
- * (qm_gemm_mxfp4_tn_rotated) and the product is not staged in the workspace; elsewhere it is a launch of its own.
+ * (qm_gemm_mxfp4_tn_rotated) and the product is not staged in the workspace.  Where a gradient product is cut into K
+ * ranges (Hadamard block 32, any mid_dtype / gw_dtype), the rotation is applied by the ordered reduction of the ranges,
+ * with the arithmetic and roundings of the separate launches.  Elsewhere it is a launch of its own.
  */
 size_t qm_packed_operand_bytes(int64_t rows, int64_t cols);
 /* offsets: HOST array of three (codes, scales, mask bits); returns 0, or QM_ERR_INVALID unless cols % 32 == 0 */

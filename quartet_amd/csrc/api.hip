@@ -297,7 +297,7 @@ int qm_gemm_fuses_rotation(const uint8_t* a_scales, const uint8_t* b_scales, int
     if (M <= 0 || N <= 0 || K <= 0 || K % 32) return 0;
     // offered the workspace the plain product would use: a shape it would cut into K ranges is not served
     const size_t ws = qm::gemm_workspace_bytes(M, N, K);
-    return ws == 0 && qm::gemm_will_rotate(a_scales, b_scales, M, N, K, QM_BF16, nullptr, 0) ? 1 : 0;
+    return ws == 0 && qm::gemm_will_rotate(a_scales, b_scales, M, N, K, QM_BF16, QM_BF16, nullptr, 0) ? 1 : 0;
 }
 
 int qm_gemm_mxfp4_tn_rotated(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes, const uint8_t* b_scales,
@@ -317,7 +317,7 @@ int qm_gemm_mxfp4_tn_rotated(const uint8_t* a_codes, const uint8_t* a_scales, co
         return fail(QM_ERR_UNALIGNED, "qm_gemm_mxfp4_tn_rotated: codes and c need 16-byte, scales and mask bits 4-byte alignment");
     bool rotated = false;
     const int rc = from_hip(qm::gemm_mxfp4_tn_rotated(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, QM_BF16, a_layout, b_layout,
-                                                      nullptr, 0, maskbits, sign_bits ? sign_bits[0] : 0u, scale_dtype, &rotated,
+                                                      nullptr, 0, maskbits, sign_bits ? sign_bits[0] : 0u, scale_dtype, QM_BF16, &rotated,
                                                       reinterpret_cast<hipStream_t>(stream)), "qm_gemm_mxfp4_tn_rotated");
     if (rc) return rc;
     return rotated ? 0 : fail(QM_ERR_INVALID, "qm_gemm_mxfp4_tn_rotated: the product did not run as planned");
@@ -512,13 +512,13 @@ int qm_linear_backward_seeded(const void* e, int e_dtype, int64_t T, int64_t I, 
     const auto grad_product = [&](const uint8_t* ac, const uint8_t* as, const uint8_t* bc, const uint8_t* bs, int64_t M, int64_t N,
                                   int64_t K, void* plain_dst, void* final_dst, bool want_rotation, int hd, int final_dtype,
                                   const uint8_t* mask, const uint32_t* signs, int scale_dtype, bool& fused) -> int {
-        fused = want_rotation && hd == 32 && final_dtype == mid_dtype && final_dst && aligned(final_dst, 16) && valid_dtype(scale_dtype) &&
-                qm::gemm_will_rotate(as, bs, M, N, K, mid_dtype, gws, wl.gemm_ws_bytes);
+        fused = want_rotation && hd == 32 && final_dst && aligned(final_dst, 16) && valid_dtype(scale_dtype) && mask &&
+                qm::gemm_will_rotate(as, bs, M, N, K, mid_dtype, final_dtype, gws, wl.gemm_ws_bytes);
         if (!fused)
             return qm_gemm_mxfp4_tn(ac, as, bc, bs, M, N, K, alpha, plain_dst, mid_dtype, codes_layout, codes_layout, gws, wl.gemm_ws_bytes, stream);
         bool done = false;
         const int r = from_hip(qm::gemm_mxfp4_tn_rotated(ac, as, bc, bs, M, N, K, alpha, final_dst, mid_dtype, codes_layout, codes_layout, gws,
-                                                         wl.gemm_ws_bytes, mask, signs ? signs[0] : 0u, scale_dtype, &done, hs),
+                                                         wl.gemm_ws_bytes, mask, signs ? signs[0] : 0u, scale_dtype, final_dtype, &done, hs),
                                "qm_linear_backward");
         if (r) return r;
         return done ? 0 : fail(QM_ERR_INVALID, "qm_linear_backward: a gradient product did not run as planned");

@@ -1302,29 +1302,32 @@ hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const 
                          const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
                          int a_layout, int b_layout, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     return gemm_mxfp4_tn_rotated(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, c_dtype, a_layout, b_layout, workspace,
-                                 workspace_bytes, nullptr, 0u, F32, nullptr, stream);
+                                 workspace_bytes, nullptr, 0u, F32, c_dtype, nullptr, stream);
 }
 
-// whether gemm_mxfp4_tn_rotated would apply the rotation in the product's epilogue for these arguments
-bool gemm_will_rotate(const uint8_t* a_scales, const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, int c_dtype, const void* workspace,
-                      size_t workspace_bytes) {
-    if (c_dtype != BF16 || !gemm_supports_tiled(M, N, K) || K <= kDuoMaxK) return false;
+// whether gemm_mxfp4_tn_rotated would apply the rotation itself for these arguments: in the epilogue of an uncut product
+// (bf16 in and out), or in the reduction of a product it cuts into K ranges
+bool gemm_will_rotate(const uint8_t* a_scales, const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, int c_dtype, int rot_out_dtype,
+                      const void* workspace, size_t workspace_bytes) {
+    if (!gemm_supports_tiled(M, N, K) || K <= kDuoMaxK) return false;
+    if (rot_out_dtype != c_dtype && !(c_dtype == BF16 && rot_out_dtype == F32)) return false;
     const int64_t nk_real = K / kBK, nk_pad = (nk_real + 3) & ~(int64_t)3;
     const bool persistent_ok = K % 512 == 0 ? ((reinterpret_cast<uintptr_t>(a_scales) | reinterpret_cast<uintptr_t>(b_scales)) & 15) == 0
                                             : (nk_real >= 4 && (nk_pad - nk_real) * 3 <= nk_real);
     if (!persistent_ok) return false;
     int sp = workspace && K % 512 == 0 ? choose_splits(M, N, K, device_cus()) : 1;
     if (sp > 1 && ((size_t)sp * M * N * sizeof(float) > workspace_bytes || (reinterpret_cast<uintptr_t>(workspace) & 15))) sp = 1;
-    return sp == 1;
+    return sp > 1 || (c_dtype == BF16 && rot_out_dtype == BF16);
 }
 
 // The product, with the layer's masked inverse Hadamard rotation (blocks of 32 along N) applied to the result before it is
-// stored when `rot_mask` is given and the shape runs on the persistent kernel's bf16 epilogue without a cut into K ranges:
-// *rotated tells which (false: c holds the plain product and the caller runs the rotation as a kernel of its own).
+// stored when `rot_mask` is given and gemm_will_rotate() holds: in the persistent kernel's bf16 epilogue, or in the ordered
+// reduction of the K ranges.  *rotated tells which (true: c holds the rotated result in rot_out_dtype; false: c holds the
+// plain product in c_dtype and the caller runs the rotation as a kernel of its own).
 hipError_t gemm_mxfp4_tn_rotated(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                                  const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
                                  int a_layout, int b_layout, void* workspace, size_t workspace_bytes, const uint8_t* rot_mask,
-                                 uint32_t rot_signs, int rot_scale_dtype, bool* rotated, hipStream_t stream) {
+                                 uint32_t rot_signs, int rot_scale_dtype, int rot_out_dtype, bool* rotated, hipStream_t stream) {
     if (rotated) *rotated = false;
     if (M == 0 || N == 0) return hipSuccess;
     const int at = a_layout == LAYOUT_TILED, bt = b_layout == LAYOUT_TILED;
@@ -1365,6 +1368,11 @@ hipError_t gemm_mxfp4_tn_rotated(const uint8_t* a_codes, const uint8_t* a_scales
             hipError_t e = launch_big4<float>(a_codes, a_scales, b_codes, b_scales, M, N, K, 1.0f, workspace, at, bt, sp, cus, stream);
             if (e != hipSuccess) return e;
             const int64_t mn = M * N;
+            if (rot_mask && rotated && (rot_out_dtype == c_dtype || (c_dtype == BF16 && rot_out_dtype == F32))) {
+                *rotated = true;
+                return splitk_reduce_rotated(static_cast<const float*>(workspace), sp, mn, alpha, c_dtype, rot_mask, rot_signs, rot_scale_dtype,
+                                             c, rot_out_dtype, stream);
+            }
             dim3 grid((unsigned)((mn / 4 + 255) / 256)), block(256);
             if (c_dtype == BF16)
                 splitk_reduce_kernel<uint16_t><<<grid, block, 0, stream>>>(static_cast<const float*>(workspace), sp, mn, alpha, static_cast<uint16_t*>(c));
@@ -1372,7 +1380,7 @@ hipError_t gemm_mxfp4_tn_rotated(const uint8_t* a_codes, const uint8_t* a_scales
                 splitk_reduce_kernel<float><<<grid, block, 0, stream>>>(static_cast<const float*>(workspace), sp, mn, alpha, static_cast<float*>(c));
             return hipGetLastError();
         }
-        if (c_dtype == BF16 && rot_mask && rotated) {
+        if (c_dtype == BF16 && rot_out_dtype == BF16 && rot_mask && rotated) {
             *rotated = true;
             const RotEpilogue rot{rot_mask, rot_signs, hadamard_scale(32, rot_scale_dtype)};
             return launch_big4<uint16_t, true>(a_codes, a_scales, b_codes, b_scales, M, N, K, alpha, c, at, bt, 1, cus, stream, rot);

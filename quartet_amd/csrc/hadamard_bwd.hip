@@ -44,9 +44,62 @@ __device__ __forceinline__ void cross_lane_stage(float (&v)[8], int lane_in_chun
     }
 }
 
+// Eight values of one octet (already loaded into v) -> mask, sign flips, butterfly within the Hadamard block (whose other
+// octets sit in the neighbouring lanes), c, store.  ROUND_OUT (fp32 out): the result is rounded to bf16 and then widened --
+// what a bf16 result converted to fp32 afterwards holds, without the separate conversion pass.
+template <typename TOut, int HD, bool ROUND_OUT>
+__device__ __forceinline__ void rotate_octet(float (&v)[8], uint32_t keep, int64_t octet, float c, const SignBits& sb, TOut* __restrict__ out) {
+    const int lic = (int)(octet & (HD / 8 - 1));
+    const int j0 = lic * 8;
+    const uint32_t sign8 = (sb.w[j0 >> 5] >> (j0 & 31)) & 0xffu;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        // g * mask as the reference multiplies: the factor is the float 1.0 or 0.0 built from the bit
+        const uint32_t all = (uint32_t)__builtin_amdgcn_sbfe((int)keep, i, 1);  // 0 or ~0
+        const float x = v[i] * u2f(all & 0x3f800000u);
+        v[i] = u2f(f2u(x) ^ (((sign8 >> i) & 1u) << 31));
+    }
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (i & h) continue;
+            float a = v[i], b = v[i + h];
+            v[i] = a + b;
+            v[i + h] = a - b;
+        }
+    }
+    cross_lane_stage<1>(v, lic);
+    cross_lane_stage<2>(v, lic);
+    if constexpr (HD >= 64) cross_lane_stage<4>(v, lic);
+    if constexpr (HD >= 128) cross_lane_stage<8>(v, lic);
+    if constexpr (sizeof(TOut) == 2) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // v_cvt_pk_bf16_f32: round to nearest even, the same rounding as f32_to_bf16
+            const v2bf p = __builtin_convertvector(v2f{v[2 * i] * c, v[2 * i + 1] * c}, v2bf);
+            w[i] = __builtin_bit_cast(uint32_t, p);
+        }
+        *reinterpret_cast<uint4*>(out + octet * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = v[i] * c;
+        if constexpr (ROUND_OUT) {
+#pragma unroll
+            for (int i = 0; i < 8; i += 2) {
+                const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[i], v[i + 1]}, v2bf));
+                v[i] = u2f(w << 16);
+                v[i + 1] = u2f(w & 0xffff0000u);
+            }
+        }
+        *reinterpret_cast<float4*>(out + octet * 8) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4*>(out + octet * 8 + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+}
+
 // The work of one launch as a job (qm_jobs.h): two independent inverse rotations can share a grid.
-// ROUND_IN (bf16 in, fp32 out): the result is rounded to bf16 and then widened -- what a bf16 result converted to fp32
-// afterwards holds, without the separate conversion pass.
+// ROUND_IN (bf16 in, fp32 out): the result is rounded to bf16 before it is widened.
 template <typename TIn, typename TOut, int HD, bool ROUND_IN = false>
 struct HadamardBwdJob {
     const TIn* g;
@@ -64,7 +117,6 @@ struct HadamardBwdJob {
     __device__ __forceinline__ void run(unsigned bid) const {
         const int64_t octet = (int64_t)bid * 256 + threadIdx.x;
         if (octet >= n_octets) return;
-        const int lic = (int)(octet & (HD / 8 - 1));
         float v[8];
         if constexpr (sizeof(TIn) == 2) {
             uint4 raw = *reinterpret_cast<const uint4*>(g + octet * 8);
@@ -82,52 +134,49 @@ struct HadamardBwdJob {
         }
         const uint32_t keep = maskbits ? (uint32_t)maskbits[octet] : 0xffu;
         job_requests_issued();
-        const int j0 = lic * 8;
-        const uint32_t sign8 = (sb.w[j0 >> 5] >> (j0 & 31)) & 0xffu;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            // g * mask as the reference multiplies: the factor is the float 1.0 or 0.0 built from the bit
-            const uint32_t all = (uint32_t)__builtin_amdgcn_sbfe((int)keep, i, 1);  // 0 or ~0
-            const float x = v[i] * u2f(all & 0x3f800000u);
-            v[i] = u2f(f2u(x) ^ (((sign8 >> i) & 1u) << 31));
+        rotate_octet<TOut, HD, ROUND_IN>(v, keep, octet, c, sb, out);
+    }
+};
+
+// The same rotation on a product that was cut into K ranges: the input element is alpha * (p[0][i] + p[1][i] + ...)
+// summed in slab order (what the ordered reduction of the partial sums stores), rounded to bf16 when the product's own
+// dtype is bf16 (MID_BF16).  One pass in place of the reduction followed by the rotation, with the same arithmetic.
+template <bool MID_BF16, typename TOut>
+struct SplitKRotateJob {
+    const float* partial;
+    int splits;
+    int64_t mn;
+    float alpha, c;
+    SignBits sb;
+    const uint8_t* maskbits;
+    TOut* out;
+    unsigned blocks;
+
+    SplitKRotateJob(const float* partial_, int splits_, int64_t mn_, float alpha_, float c_, const SignBits& sb_, const uint8_t* maskbits_,
+                    void* out_)
+        : partial(partial_), splits(splits_), mn(mn_), alpha(alpha_), c(c_), sb(sb_), maskbits(maskbits_),
+          out(reinterpret_cast<TOut*>(out_)), blocks((unsigned)((mn_ / 8 + 255) / 256)) {}
+
+    __device__ __forceinline__ void run(unsigned bid) const {
+        const int64_t octet = (int64_t)bid * 256 + threadIdx.x;
+        if (octet >= mn / 8) return;
+        const float* p = partial + octet * 8;
+        float4 a = *reinterpret_cast<const float4*>(p);
+        float4 b = *reinterpret_cast<const float4*>(p + 4);
+        const uint32_t keep = (uint32_t)maskbits[octet];
+        for (int s = 1; s < splits; ++s) {
+            const float4 x = *reinterpret_cast<const float4*>(p + (int64_t)s * mn);
+            const float4 y = *reinterpret_cast<const float4*>(p + (int64_t)s * mn + 4);
+            a.x += x.x; a.y += x.y; a.z += x.z; a.w += x.w;
+            b.x += y.x; b.y += y.y; b.z += y.z; b.w += y.w;
         }
+        job_requests_issued();
+        float v[8] = {a.x * alpha, a.y * alpha, a.z * alpha, a.w * alpha, b.x * alpha, b.y * alpha, b.z * alpha, b.w * alpha};
+        if constexpr (MID_BF16) {
 #pragma unroll
-        for (int h = 1; h < 8; h <<= 1) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                if (i & h) continue;
-                float a = v[i], b = v[i + h];
-                v[i] = a + b;
-                v[i + h] = a - b;
-            }
+            for (int i = 0; i < 8; ++i) v[i] = u2f((uint32_t)f32_to_bf16(v[i]) << 16);
         }
-        cross_lane_stage<1>(v, lic);
-        cross_lane_stage<2>(v, lic);
-        if constexpr (HD >= 64) cross_lane_stage<4>(v, lic);
-        if constexpr (HD >= 128) cross_lane_stage<8>(v, lic);
-        if constexpr (sizeof(TOut) == 2) {
-            uint32_t w[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                // v_cvt_pk_bf16_f32: round to nearest even, the same rounding as f32_to_bf16
-                const v2bf p = __builtin_convertvector(v2f{v[2 * i] * c, v[2 * i + 1] * c}, v2bf);
-                w[i] = __builtin_bit_cast(uint32_t, p);
-            }
-            *reinterpret_cast<uint4*>(out + octet * 8) = make_uint4(w[0], w[1], w[2], w[3]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = v[i] * c;
-            if constexpr (ROUND_IN) {
-#pragma unroll
-                for (int i = 0; i < 8; i += 2) {
-                    const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[i], v[i + 1]}, v2bf));
-                    v[i] = u2f(w << 16);
-                    v[i + 1] = u2f(w & 0xffff0000u);
-                }
-            }
-            *reinterpret_cast<float4*>(out + octet * 8) = make_float4(v[0], v[1], v[2], v[3]);
-            *reinterpret_cast<float4*>(out + octet * 8 + 4) = make_float4(v[4], v[5], v[6], v[7]);
-        }
+        rotate_octet<TOut, 32, MID_BF16 && sizeof(TOut) == 4>(v, keep, octet, c, sb, out);
     }
 };
 
@@ -200,6 +249,19 @@ hipError_t masked_hadamard_bwd_hd32_pair(const void* ga, int64_t na, int scale_d
         using J = HadamardBwdJob<float, float, 32>;
         launch_job_pair(J(ga, na, ca, sa, mask_a, out_a), J(gb, nb, cb, sb, mask_b, out_b), stream);
     }
+    return hipGetLastError();
+}
+
+// c = masked inverse rotation (blocks of 32 along the rows) of the reduced product alpha * sum_s partial[s]; see SplitKRotateJob
+hipError_t splitk_reduce_rotated(const float* partial, int splits, int64_t mn, float alpha, int mid_dtype, const uint8_t* maskbits,
+                                 uint32_t sign_word, int scale_dtype, void* out, int out_dtype, hipStream_t stream) {
+    if (mn == 0) return hipSuccess;
+    if (mn % 32 || !maskbits || splits < 1 || (mid_dtype == F32 && out_dtype != F32)) return hipErrorInvalidValue;
+    const SignBits sb{{sign_word, 0, 0, 0}};
+    const float c = hadamard_scale(32, scale_dtype);
+    if (mid_dtype == BF16 && out_dtype == BF16) launch_job(SplitKRotateJob<true, uint16_t>(partial, splits, mn, alpha, c, sb, maskbits, out), stream);
+    else if (mid_dtype == BF16) launch_job(SplitKRotateJob<true, float>(partial, splits, mn, alpha, c, sb, maskbits, out), stream);
+    else launch_job(SplitKRotateJob<false, float>(partial, splits, mn, alpha, c, sb, maskbits, out), stream);
     return hipGetLastError();
 }
 

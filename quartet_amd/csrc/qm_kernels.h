@@ -123,13 +123,19 @@ hipError_t gemm_mxfp4_tn(const uint8_t* a_codes, const uint8_t* a_scales, const 
                          const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
                          int a_layout, int b_layout, void* workspace, size_t workspace_bytes, hipStream_t stream);
 // the same product with the masked inverse Hadamard rotation of the layer's backward pass (hd 32, along N) fused into the
-// store of the result where the kernel serving the shape can do it; *rotated reports whether it was
-bool gemm_will_rotate(const uint8_t* a_scales, const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, int c_dtype, const void* workspace,
-                      size_t workspace_bytes);
+// store of the result where the kernel serving the shape can do it: in the persistent kernel's bf16 epilogue (c_dtype and
+// rot_out_dtype both BF16), or in the ordered reduction of a product cut into K ranges (the product rounded to c_dtype,
+// the rotated result stored in rot_out_dtype: c_dtype, or F32 holding the bf16-rounded result).  *rotated reports whether
+// it was; c then holds rot_out_dtype elements, otherwise the plain product in c_dtype.
+bool gemm_will_rotate(const uint8_t* a_scales, const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, int c_dtype, int rot_out_dtype,
+                      const void* workspace, size_t workspace_bytes);
 hipError_t gemm_mxfp4_tn_rotated(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
                                  const uint8_t* b_scales, int64_t M, int64_t N, int64_t K, float alpha, void* c, int c_dtype,
                                  int a_layout, int b_layout, void* workspace, size_t workspace_bytes, const uint8_t* rot_mask,
-                                 uint32_t rot_signs, int rot_scale_dtype, bool* rotated, hipStream_t stream);
+                                 uint32_t rot_signs, int rot_scale_dtype, int rot_out_dtype, bool* rotated, hipStream_t stream);
+// the reduction of a product cut into K ranges with that rotation applied to the reduced values (hadamard_bwd.hip)
+hipError_t splitk_reduce_rotated(const float* partial, int splits, int64_t mn, float alpha, int mid_dtype, const uint8_t* maskbits,
+                                 uint32_t sign_word, int scale_dtype, void* out, int out_dtype, hipStream_t stream);
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 // C = alpha * A (packed MXFP4 [M, K]) x B (bf16 [K, N] row-major): K % 64 == 0, N % 8 == 0
 bool gemm_fp4_bf16_nn_supported(int64_t M, int64_t N, int64_t K);

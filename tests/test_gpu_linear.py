@@ -486,6 +486,41 @@ def test_weight_gradient_widened_in_the_kernel(q, T, I, O):
     assert torch.equal(K.masked_hadamard_bwd(gx2, 32, torch.bfloat16, 0x5A5A5A5A, mask), gx0)
 
 
+@pytest.mark.parametrize("mid_dtype,gw_dtype", [(torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                                (torch.float32, torch.float32)])
+def test_backward_with_products_cut_into_k_ranges(q, mid_dtype, gw_dtype):
+    """Few output tiles and a long contraction: both gradient products are cut into K ranges, and the ordered reduction of
+    the ranges applies the masked inverse rotation in the same pass.  Bit for bit what the kernels give one by one
+    (quantizers, re-quantizers, the products with their plain reduction, the inverse rotation as a kernel of its own)."""
+    print(f"case backward with split products mid={mid_dtype} gw={gw_dtype}", flush=True)
+    from quartet_amd import kernels as K
+    from quartet_amd import _lib
+    T, I, O = 4096, 512, 2048
+    assert _lib.lib().qm_gemm_workspace_bytes(T, I, O) > 0 and _lib.lib().qm_gemm_workspace_bytes(O, I, T) > 0
+    dev = "cuda:0"
+    x = make_input(T, I, mid_dtype, seed=21).to(dev)
+    w = make_input(O, I, mid_dtype, seed=22, scale=0.02).to(dev)
+    e = make_input(T, O, mid_dtype, seed=23, scale=1e-2, outlier_frac=0).to(dev)
+    sx, sw, sg, seeds, tl = 0x5A5A5A5A, 0x0F0F1234, 0x13572468, [11, 12, 13, 14], True
+    _, px, pw = K.linear_forward(x, w, 32, sx, 32, sw, mid_dtype, tl)
+    gx, gw = K.linear_backward(e, px, pw, T, I, O, 32, sx, 32, sw, 32, sg, K.QM_ABSMAX_SR, seeds, mid_dtype, mid_dtype, mid_dtype,
+                               mid_dtype, mid_dtype, tl, gw_dtype=gw_dtype)
+    assert gx.dtype == mid_dtype and gw.dtype == gw_dtype
+    alpha = float(torch.tensor(K.FOUR_THIRDS, dtype=torch.float32) * torch.tensor(K.FOUR_THIRDS, dtype=torch.float32))
+    xc, xs, xm, _ = K.quantize_mxfp4(x, 32, sx, K.QM_QUEST_RTN, want_mask=True, tiled=tl)
+    wc, ws, wm, _ = K.quantize_mxfp4(w, 32, sw, K.QM_QUEST_RTN, want_mask=True, tiled=tl)
+    ec, es, _, _ = K.quantize_mxfp4(e, 32, sg, K.QM_ABSMAX_SR, seed=seeds[0], tiled=tl)
+    wtc, wts, _ = K.requantize_transposed_mxfp4(wc, ws, 1.0, mid_dtype, 32, sg, K.QM_ABSMAX_SR, seed=seeds[1], tiled_in=tl, tiled_out=tl)
+    etc, ets, _, _ = K.quantize_mxfp4(e, 32, sg, K.QM_ABSMAX_SR, transposed_in=True, seed=seeds[2], tiled=tl)
+    xtc, xts, _ = K.requantize_transposed_mxfp4(xc, xs, 1.0, mid_dtype, 32, sg, K.QM_ABSMAX_SR, seed=seeds[3], tiled_in=tl, tiled_out=tl)
+    gxq = K.gemm_mxfp4_tn(ec, es, wtc, wts, alpha, mid_dtype, a_tiled=tl, b_tiled=tl, split_k=True)
+    gwq = K.gemm_mxfp4_tn(etc, ets, xtc, xts, alpha, mid_dtype, a_tiled=tl, b_tiled=tl, split_k=True)
+    assert torch.equal(gx, K.masked_hadamard_bwd(gxq, 32, mid_dtype, sx, xm))
+    want_gw = K.masked_hadamard_bwd(gwq, 32, mid_dtype, sw, wm)
+    assert torch.equal(gw, want_gw.to(gw_dtype))
+    assert gw.abs().max() > 0 and gx.abs().max() > 0
+
+
 @pytest.mark.parametrize("three_d", [False, True])
 @pytest.mark.parametrize("stochastic", [False, True])
 def test_error_only_scheme_against_oracle(oracle, q, three_d, stochastic):
