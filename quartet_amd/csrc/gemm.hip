@@ -810,9 +810,9 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
 #pragma unroll
         for (int jp = 0; jp < 2; ++jp) {
             if (i * 32 >= rows_valid || jp * 64 >= cols_valid) continue;  // uniform: this pass lies outside the matrix
+            if constexpr (!ROT) {
 #pragma unroll
-            for (int jj = 0; jj < 2; ++jj) {
-                if constexpr (!ROT) {
+                for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
                     for (int b = 0; b < 4; ++b) {
                         const v16f& t = acc[i][2 * jp + jj];
@@ -822,7 +822,14 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
                         *reinterpret_cast<uint2*>(wr + (((jj * 4 + b) * 16) ^ wsw)) =
                             make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
                     }
-                } else {
+                }
+            } else {
+                // Both blocks of the pass go through the matrix pipe before either result is read: the second block's
+                // conversion and masking run while the first block's instructions are in flight (the opaque copies below
+                // keep the read-out of the results behind both blocks' matrix instructions).  Per tile 15.9 k -> 14.7 k cycles.
+                v16f r[2];
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
                     const v16f& t = acc[i][2 * jp + jj];
                     // the block rounded to bf16 and masked: register pair 2 b + k holds n = 8 b + 4 half + 2 k, + 1
                     // the block's mask word: word j of the row's four, or word j + 2 where the wave requested the row's last
@@ -840,29 +847,30 @@ __device__ __forceinline__ void big4_epilogue_bf16(v16f (&acc)[4][4], float alph
                             const uint32_t hi = (uint32_t)__builtin_amdgcn_sbfe((int)kw, 8 * b + 2 * k + 1, 1);
                             pk[2 * b + k] = p & ((lo & 0xffffu) | (hi & 0xffff0000u));
                         }
-                    v16f r;
+                    v16f z;
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) r[e] = 0.0f;
-                    r = __builtin_amdgcn_mfma_f32_32x32x16_bf16(hmat[0], __builtin_bit_cast(v8bf, u32x4{pk[0], pk[1], pk[2], pk[3]}), r, 0, 0, 0);
-                    r = __builtin_amdgcn_mfma_f32_32x32x16_bf16(hmat[1], __builtin_bit_cast(v8bf, u32x4{pk[4], pk[5], pk[6], pk[7]}), r, 0, 0, 0);
-                    if (c_in_matrix) {
+                    for (int e = 0; e < 16; ++e) z[e] = 0.0f;
+                    z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(hmat[0], __builtin_bit_cast(v8bf, u32x4{pk[0], pk[1], pk[2], pk[3]}), z, 0, 0, 0);
+                    r[jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(hmat[1], __builtin_bit_cast(v8bf, u32x4{pk[4], pk[5], pk[6], pk[7]}), z, 0, 0, 0);
+                }
+                const auto emit = [&](auto scaled) {
 #pragma unroll
-                        for (int b = 0; b < 4; ++b) {
-                            const v2bf p0 = __builtin_convertvector(v2f{r[4 * b], r[4 * b + 1]}, v2bf);
-                            const v2bf p1 = __builtin_convertvector(v2f{r[4 * b + 2], r[4 * b + 3]}, v2bf);
-                            *reinterpret_cast<uint2*>(wr + (((jj * 4 + b) * 16) ^ wsw)) =
-                                make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
-                        }
-                    } else {
+                    for (int jj = 0; jj < 2; ++jj) {
+                        asm volatile("" : "+v"(r[jj]));
 #pragma unroll
                         for (int b = 0; b < 4; ++b) {
-                            const v2bf p0 = __builtin_convertvector(v2f{r[4 * b] * rot.c, r[4 * b + 1] * rot.c}, v2bf);
-                            const v2bf p1 = __builtin_convertvector(v2f{r[4 * b + 2] * rot.c, r[4 * b + 3] * rot.c}, v2bf);
+                            float q[4];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) q[e] = decltype(scaled)::value ? r[jj][4 * b + e] * rot.c : r[jj][4 * b + e];
+                            const v2bf p0 = __builtin_convertvector(v2f{q[0], q[1]}, v2bf);
+                            const v2bf p1 = __builtin_convertvector(v2f{q[2], q[3]}, v2bf);
                             *reinterpret_cast<uint2*>(wr + (((jj * 4 + b) * 16) ^ wsw)) =
                                 make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
                         }
                     }
-                }
+                };
+                if (c_in_matrix) emit(std::false_type{});
+                else emit(std::true_type{});
             }
             // the region is private to the wave; LDS operations of one wave complete in order
 #pragma unroll
